@@ -1,0 +1,95 @@
+#!/usr/bin/env python3
+"""Writes the golden vectors that only the compiled reference can pin (run in the build container, where
+oracle/_ref/libqtip_ref.so exists; the GPU box only reads the committed outputs).
+
+  ref_rng.json            first 64 next() / sign() / normal() of the splitmix stream for seeds 0 and 7
+  ref_vit_raw_x.bin       64 tiles of raw (not fp16-representable) fp32 N(0,1), seed 1234 (first 64 of config 1)
+  ref_vit_raw_hyb.bin     their states under the built-in HYB tlut            (u16 [64][128])
+  ref_vit_raw_syn.bin     their states under the synthetic unit-rms tlut, seed 1 (u16 [64][128])
+  ref_vit_raw_cost.bin    pass-2 path metrics returned by the reference (f64 [2][64]: hyb, syn)
+  ref_config1.json        FNV-1a 64 of the packed words of all 4096 config-1 tiles (synthetic tlut)
+  ref_config1_packed.bin  those packed words (u16 [4096][32], pack_trellis layout, not swizzled)
+  ref_ldl_1024.bin        rows 1000..1007 of L (fp32) from block_ldl_to_L on a seeded n=1024 SPD matrix
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+from oracle import binding as ob  # noqa: E402
+
+
+def fnv1a64(buf):
+    h = 0xcbf29ce484222325
+    for b in bytes(buf):
+        h = ((h ^ b) * 0x100000001b3) & 0xffffffffffffffff
+    return h
+
+
+def ref_quantize(R, X):
+    st = np.zeros((X.shape[0], 128), np.uint16)
+    cost = np.zeros(X.shape[0])
+    hat = np.zeros(256, np.float32)
+    for b in range(X.shape[0]):
+        cost[b] = R.ref_quantize_seq(X[b], st[b], hat)
+    return st, cost
+
+
+def ldl_case(n=1024, seed=3):
+    g = ob.rng_normal(seed, n * 64).reshape(n, 64)
+    H = g @ g.T / 64 + 0.05 * np.eye(n)
+    return H
+
+
+def main():
+    R = ob.ref_lib()
+    assert R is not None, "build oracle/_ref first (make -C oracle ref)"
+    out = {}
+    for seed in (0, 7):
+        u = np.zeros(64, np.uint64)
+        f = np.zeros(64)
+        g = np.zeros(64)
+        R.ref_rng(seed, 0, 64, None, u.ctypes.data)
+        R.ref_rng(seed, 3, 64, f.ctypes.data, None)
+        R.ref_rng(seed, 2, 64, g.ctypes.data, None)
+        out[str(seed)] = {"next": [int(v) for v in u], "sign": [int(v) for v in f], "normal": [float.hex(float(v)) for v in g]}
+    json.dump(out, open(os.path.join(HERE, "ref_rng.json"), "w"))
+
+    X = ob.rng_normal(1234, 4096 * 256).astype(np.float32).reshape(4096, 256)
+    X[:64].tofile(os.path.join(HERE, "ref_vit_raw_x.bin"))
+    hyb = ob.Codebook()
+    syn = ob.Codebook(ob.synthetic_tlut(1))
+    st_h, c_h = ref_quantize(R, X[:64])
+    R.ref_override_codebook(syn.lut0, syn.lut1, syn.lut_h2, syn.lut_rms)
+    st_s, c_s = ref_quantize(R, X[:64])
+    st_h.tofile(os.path.join(HERE, "ref_vit_raw_hyb.bin"))
+    st_s.tofile(os.path.join(HERE, "ref_vit_raw_syn.bin"))
+    np.stack([c_h, c_s]).tofile(os.path.join(HERE, "ref_vit_raw_cost.bin"))
+
+    # all of config 1 under the synthetic tlut, the reference's code on 8 threads through a process pool-free loop
+    import concurrent.futures as cf
+    def chunk(lo):
+        return ref_quantize(R, X[lo:lo + 128])[0]
+    with cf.ThreadPoolExecutor(8) as ex:   # ctypes releases the GIL
+        parts = list(ex.map(chunk, range(0, 4096, 128)))
+    st_all = np.concatenate(parts)
+    packed = np.zeros((4096, 32), np.uint16)
+    R.ref_pack_trellis(st_all.reshape(-1), 4096, packed.reshape(-1))
+    packed.tofile(os.path.join(HERE, "ref_config1_packed.bin"))
+    json.dump({"tiles": 4096, "x_seed": 1234, "tlut_seed": 1, "fnv1a64_packed": "%016x" % fnv1a64(packed.tobytes()),
+               "fnv1a64_states": "%016x" % fnv1a64(st_all.tobytes())},
+              open(os.path.join(HERE, "ref_config1.json"), "w"))
+
+    H = ldl_case()
+    A = H.copy()
+    L = np.zeros((1024, 1024), np.float32)
+    assert R.ref_block_ldl(A.reshape(-1), 1024, L.reshape(-1), 8) == 1
+    L[1000:1008].tofile(os.path.join(HERE, "ref_ldl_1024.bin"))
+    print("wrote golden vectors to", HERE)
+
+
+if __name__ == "__main__":
+    main()

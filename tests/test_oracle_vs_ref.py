@@ -1,0 +1,132 @@
+"""Pins oracle/ against the reference's own CPU core compiled in place (oracle/_ref, built only where
+/root/reference exists) and against the vectors that build wrote into tests/golden.  No GPU."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from conftest import GOLDEN
+
+
+def g(name, dt):
+    return np.fromfile(os.path.join(GOLDEN, name), dtype=dt)
+
+
+# ------------------------------------------------------------------ committed vectors (run everywhere)
+def test_rng_golden(oracle):
+    want = json.load(open(os.path.join(GOLDEN, "ref_rng.json")))
+    for seed in (0, 7):
+        w = want[str(seed)]
+        assert [int(v) for v in oracle.rng_next(seed, 64)] == w["next"]
+        assert [int(v) for v in oracle.rng_sign(seed, 64)] == w["sign"]
+        assert [float.hex(float(v)) for v in oracle.rng_normal(seed, 64)] == w["normal"]
+
+
+def test_viterbi_raw_inputs_golden(oracle, hyb, syn):
+    X = g("ref_vit_raw_x.bin", np.float32).reshape(64, 256)
+    assert np.array_equal(X, oracle.rng_normal(1234, 64 * 256).astype(np.float32).reshape(64, 256))
+    assert not np.array_equal(X, X.astype(np.float16).astype(np.float32))   # inputs are NOT fp16-representable
+    cost = g("ref_vit_raw_cost.bin", np.float64).reshape(2, 64)
+    for k, (cb, name) in enumerate(((hyb, "ref_vit_raw_hyb.bin"), (syn, "ref_vit_raw_syn.bin"))):
+        want = g(name, np.uint16).reshape(64, 128)
+        for fast in (True, False):
+            got = oracle.quantize_tiles(cb, X, fast=fast)
+            assert np.array_equal(got, want)
+        st = np.zeros(128, np.uint16)
+        hat = np.zeros(256, np.float32)
+        for b in range(0, 64, 7):   # returned path metric, bit for bit
+            c = oracle.lib().qo_quantize_seq(cb.lut0, cb.lut1, X[b], st, hat)
+            assert c == cost[k, b]
+
+
+def test_ldl_1024_golden(oracle):
+    n = 1024
+    gm = oracle.rng_normal(3, n * 64).reshape(n, 64)
+    H = gm @ gm.T / 64 + 0.05 * np.eye(n)
+    L = oracle.block_ldl(H)
+    want = g("ref_ldl_1024.bin", np.float32).reshape(8, n)
+    got = L[1000:1008]
+    # different summation order than the blocked reference: equal to fp32 rounding
+    assert np.max(np.abs(got - want)) <= 2e-7 * np.max(np.abs(want))
+    assert np.mean(got.view(np.uint32) != want.view(np.uint32)) < 0.01
+
+
+# ------------------------------------------------------------------ live comparison (build container only)
+@pytest.fixture(scope="module")
+def ref(oracle):
+    R = oracle.ref_lib()
+    if R is None:
+        pytest.skip("oracle/_ref not built (the reference tree is absent here)")
+    return R
+
+
+def test_ref_codebook_perm_formats(oracle, ref, hyb):
+    l0 = np.zeros(65536, np.float32)
+    l1 = np.zeros(65536, np.float32)
+    h2 = np.zeros(65536, np.uint32)
+    import ctypes
+    rms = ctypes.c_double()
+    tl = np.zeros(1024, np.float32)
+    ref.ref_codebook(l0.ctypes.data, l1.ctypes.data, h2.ctypes.data, ctypes.addressof(rms), tl.ctypes.data)
+    assert np.array_equal(l0, hyb.lut0) and np.array_equal(l1, hyb.lut1) and np.array_equal(h2, hyb.lut_h2)
+    assert rms.value == hyb.lut_rms
+    assert np.array_equal(tl, hyb.tlut.reshape(-1))
+    p = np.zeros(256, np.int32)
+    q = np.zeros(256, np.int32)
+    ref.ref_perm256(p, q)
+    op, oq = oracle.perm256()
+    assert np.array_equal(p, op) and np.array_equal(q, oq)
+    rng = np.random.default_rng(0)
+    vals = np.concatenate([rng.normal(size=3000), rng.normal(size=1000) * 1e-6, rng.normal(size=300) * 1e5]).astype(np.float32)
+    L = oracle.lib()
+    for v in vals:
+        assert L.qo_f32_to_fp16(float(v)) == ref.ref_f32_to_fp16(float(v))
+        assert L.qo_f32_to_bf16(float(v)) == ref.ref_f32_to_bf16(float(v))
+    for n in (96, 1024, 3000, 12288, 28672, 57344, 2304, 100, 640):
+        assert L.qo_had_K(n) == ref.ref_had_K(n)
+
+
+def test_ref_viterbi_live(oracle, ref, hyb):
+    # single passes with and without the constraint, returned metrics bit for bit, raw fp32 inputs
+    X = oracle.rng_normal(77, 6 * 256).astype(np.float32).reshape(6, 256) * np.float32(1.3)
+    L = oracle.lib()
+    for b in range(6):
+        for ov in (-1, 17, 4000):
+            s1 = np.zeros(128, np.uint16)
+            s2 = np.zeros(128, np.uint16)
+            c1 = ref.ref_viterbi(X[b], ov, s1)
+            c2 = L.qo_viterbi(hyb.lut0, hyb.lut1, X[b], ov, s2)
+            assert c1 == c2 and np.array_equal(s1, s2)
+            assert ref.ref_path_cost(X[b], s1) == L.qo_path_cost(hyb.lut0, hyb.lut1, X[b], s2)
+
+
+def test_ref_hadamard_pack_ldl_live(oracle, ref):
+    rng = np.random.default_rng(1)
+    L = oracle.lib()
+    for n in (96, 1024, 12288):
+        x = rng.normal(size=(2, n + 8))
+        for t in (0, 1):
+            a = x.reshape(-1).copy()
+            b = x.reshape(-1).copy()
+            ref.ref_hadamard_rows(a, 2, n, n + 8, t)
+            L.qo_hadamard_rows(b, 2, n, n + 8, t)
+            assert np.array_equal(a, b)
+    st = rng.integers(0, 65536, (24, 128)).astype(np.uint16)
+    a = np.zeros(24 * 32, np.uint16)
+    ref.ref_pack_trellis(st.reshape(-1), 24, a)
+    assert np.array_equal(a, oracle.pack_trellis(st).reshape(-1))
+    sw = np.zeros_like(a)
+    ref.ref_swizzle(a, 64, 96, sw)
+    assert np.array_equal(sw, oracle.swizzle(a, 64, 96))
+    un = np.zeros((24, 128), np.uint16)
+    ref.ref_unpack_trellis(a, 24, un.reshape(-1))
+    assert np.array_equal(un, oracle.unpack_trellis(a))
+    n = 272
+    G = rng.normal(size=(n, 400))
+    H = G @ G.T / 400 + 0.02 * np.eye(n)
+    A = H.copy()
+    Lr = np.zeros((n, n), np.float32)
+    assert ref.ref_block_ldl(A.reshape(-1), n, Lr.reshape(-1), 4) == 1
+    Lo = oracle.block_ldl(H)
+    assert np.max(np.abs(Lr - Lo)) <= 2e-7 * np.max(np.abs(Lr))
