@@ -1,0 +1,387 @@
+"""Python host side of the MI355X QTIP group quantizer.
+
+A thin ctypes binding of libqtip_mi355.so (C ABI: include/qtip_mi355.h) plus a mirror of the reference's
+operator interface for this path (src/quantizer.hpp:11-78 of the reference: QuantOpts, LinearIn, LinearOut,
+GroupTiming, HessPrep, rotate_hessian, ldl_hessian, quantize_group, ldlq_gpu).  There is no CPU fallback:
+importing works everywhere, but every compute call needs the HIP library and a gfx950 device and raises
+otherwise.
+"""
+import ctypes as C
+import os
+import subprocess
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_PATH = os.path.join(CSRC, "libqtip_mi355.so")
+
+QTIP_OK, QTIP_E_ARG, QTIP_E_HIP, QTIP_E_NOT_PD, QTIP_E_NOMEM = 0, -1, -2, -3, -4
+
+
+class QtipError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("qtip error %d: %s" % (code, msg))
+        self.code = code
+
+
+def build(jobs=8):
+    """Compile the HIP extension for gfx950 in-tree (hipcc cross-compiles without a GPU)."""
+    subprocess.check_call(["make", "-C", CSRC, "-B", "-j%d" % jobs])
+    return LIB_PATH
+
+
+class _LinearInC(C.Structure):
+    _fields_ = [("m", C.c_int), ("w_f32", C.c_void_p), ("w_bf16", C.c_void_p), ("w_fp8", C.c_void_p),
+                ("scale_bf16", C.c_void_p), ("on_device", C.c_int)]
+
+
+class _LinearOutC(C.Structure):
+    _fields_ = [("trellis", C.c_void_p), ("su_bf16", C.c_void_p), ("sv", C.c_void_p), ("hatW", C.c_void_p),
+                ("wscale", C.c_float), ("proxy", C.c_double), ("proxy_rot_reg", C.c_double), ("seconds", C.c_double)]
+
+
+class _OptsC(C.Structure):
+    _fields_ = [("sigma_reg", C.c_double), ("scale_override", C.c_double), ("ldl_threads", C.c_int),
+                ("feedback", C.c_int), ("skip_proxy", C.c_int)]
+
+
+class _TimingC(C.Structure):
+    _fields_ = [(k, C.c_double) for k in ("load", "rht", "ldl_cpu", "ldlq", "viterbi", "proxy", "pack", "total")]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded C-ABI library.  Raises if it has not been built: there is no other implementation."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise QtipError(QTIP_E_HIP, "%s is missing: build it with __graft_entry__.build() or make -C %s"
+                        % (LIB_PATH, CSRC))
+    # A process must hold ONE HIP runtime.  PyTorch-ROCm ships its own libamdhip64 and asks for it by the
+    # unversioned name, so if this library (linked against libamdhip64.so.7) were loaded first, torch would
+    # bring in a second runtime that finds no GPU.  Loaded after torch, the soname resolves to torch's copy.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
+    L = C.CDLL(LIB_PATH)
+    vp, i, l, d, u64 = C.c_void_p, C.c_int, C.c_long, C.c_double, C.c_uint64
+    L.qtip_last_error.restype = C.c_char_p
+    L.qtip_create.argtypes = [i, C.POINTER(vp)]
+    L.qtip_destroy.argtypes = [vp]
+    L.qtip_destroy.restype = None
+    L.qtip_stream.argtypes = [vp]
+    L.qtip_stream.restype = vp
+    L.qtip_synchronize.argtypes = [vp]
+    L.qtip_set_tlut.argtypes = [vp, vp]
+    L.qtip_lut_rms.argtypes = [vp]
+    L.qtip_lut_rms.restype = d
+    L.qtip_get_lut.argtypes = [vp, vp, vp]
+    L.qtip_viterbi_tiles.argtypes = [vp, vp, l, vp, vp]
+    L.qtip_viterbi_tiles_dev.argtypes = [vp, vp, l, vp, vp]
+    L.qtip_decode_states_dev.argtypes = [vp, vp, l, vp]
+    L.qtip_hadamard_rows_dev.argtypes = [vp, vp, l, i, l, i]
+    L.qtip_had_K.argtypes = [i]
+    L.qtip_sign_vector.argtypes = [u64, l, vp]
+    L.qtip_sign_vector.restype = None
+    L.qtip_rotate_hessian.argtypes = [vp, vp, i, i, u64, d, vp, C.POINTER(d), vp]
+    L.qtip_ldl_hessian.argtypes = [vp, i, i, vp]
+    L.qtip_ldlq_dev.argtypes = [vp, vp, vp, l, l, vp, vp, C.POINTER(d)]
+    L.qtip_default_opts.argtypes = [C.POINTER(_OptsC)]
+    L.qtip_default_opts.restype = None
+    L.qtip_quantize_group.argtypes = [vp, i, C.POINTER(_LinearInC), i, u64, vp, d, vp, vp, C.POINTER(_OptsC),
+                                      C.POINTER(_LinearOutC), C.POINTER(_TimingC)]
+    L.qtip_quantize_group_h.argtypes = [vp, i, C.POINTER(_LinearInC), i, vp, i, u64, C.POINTER(_OptsC),
+                                        C.POINTER(_LinearOutC), C.POINTER(_TimingC)]
+    L.qtip_pack_trellis.argtypes = [vp, l, vp]
+    L.qtip_pack_trellis.restype = None
+    L.qtip_unpack_trellis.argtypes = [vp, l, vp]
+    L.qtip_unpack_trellis.restype = None
+    L.qtip_swizzle_for_kernel.argtypes = [vp, i, i, vp]
+    L.qtip_unswizzle_for_kernel.argtypes = [vp, i, i, vp]
+    _lib = L
+    return L
+
+
+def _check(rc):
+    if rc != 0:
+        raise QtipError(rc, lib().qtip_last_error().decode("utf-8", "replace"))
+
+
+def _ptr(a):
+    """Address of a numpy array, a torch tensor (host or device) or a raw integer address."""
+    if a is None:
+        return None
+    if isinstance(a, int):
+        return a
+    if isinstance(a, np.ndarray):
+        assert a.flags["C_CONTIGUOUS"]
+        return a.ctypes.data
+    if hasattr(a, "data_ptr"):
+        assert a.is_contiguous()
+        return a.data_ptr()
+    raise TypeError(type(a))
+
+
+# ---------------------------------------------------------------- mirror of src/quantizer.hpp
+@dataclass
+class QuantOpts:  # src/quantizer.hpp:11-19
+    sigma_reg: float = 1e-2
+    scale_override: float = 0.9
+    vit_batch: int = 1024      # accepted for source compatibility; the tile kernel sizes its own workspace
+    ldl_threads: int = 16
+    share_su: bool = True      # False is refused, as in the reference (src/quantizer.cpp:209-211)
+    want_hatW: bool = False
+    feedback: int = 0          # 0: fp64 feedback (default), 1: fp32 feedback + bf16 hi/lo split MFMA
+    skip_proxy: bool = False
+
+
+@dataclass
+class LinearIn:  # src/quantizer.hpp:21-28; exactly one weight representation is set
+    name: str
+    m: int
+    w_f32: Optional[object] = None
+    w_bf16: Optional[object] = None
+    w_fp8: Optional[object] = None
+    scale_bf16: Optional[object] = None
+
+
+@dataclass
+class LinearOut:  # src/quantizer.hpp:30-43
+    name: str = ""
+    m: int = 0
+    n: int = 0
+    trellis: Optional[np.ndarray] = None
+    su_bf16: Optional[np.ndarray] = None
+    sv: Optional[np.ndarray] = None
+    wscale: float = 0.0
+    proxy: float = 0.0
+    proxy_rot_reg: float = 0.0
+    seconds: float = 0.0
+    hatW: Optional[np.ndarray] = None
+
+
+@dataclass
+class GroupTiming:  # src/quantizer.hpp:45-47
+    load: float = 0.0
+    rht: float = 0.0
+    ldl_cpu: float = 0.0
+    ldlq: float = 0.0
+    viterbi: float = 0.0
+    proxy: float = 0.0
+    pack: float = 0.0
+    total: float = 0.0
+
+
+@dataclass
+class HessPrep:  # src/quantizer.hpp:51-59
+    n: int = 0
+    seed: int = 0
+    su: Optional[np.ndarray] = None
+    creg: float = 0.0
+    HRr: Optional[np.ndarray] = None
+    L: Optional[np.ndarray] = None
+    t_rot: float = 0.0
+    t_ldl: float = 0.0
+
+
+def _is_device(a):
+    return hasattr(a, "is_cuda") and a.is_cuda
+
+
+class Quantizer:
+    """One context: device, private stream, codebook (the reference's per-worker state)."""
+
+    def __init__(self, device=0, tlut=None):
+        self._h = C.c_void_p()
+        _check(lib().qtip_create(device, C.byref(self._h)))
+        if tlut is not None:
+            self.set_tlut(tlut)
+
+    def close(self):
+        if self._h:
+            lib().qtip_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def stream(self):
+        return lib().qtip_stream(self._h)
+
+    def synchronize(self):
+        _check(lib().qtip_synchronize(self._h))
+
+    def set_tlut(self, tlut):
+        t = None if tlut is None else np.ascontiguousarray(tlut, np.float32).reshape(1024)
+        _check(lib().qtip_set_tlut(self._h, _ptr(t)))
+
+    @property
+    def lut_rms(self):
+        return lib().qtip_lut_rms(self._h)
+
+    def lut(self):
+        a = np.zeros(65536, np.float32)
+        b = np.zeros(65536, np.float32)
+        _check(lib().qtip_get_lut(self._h, _ptr(a), _ptr(b)))
+        return a, b
+
+    # ---- Viterbi of independent tiles
+    def viterbi_tiles(self, X, want_states=True, want_packed=True):
+        X = np.ascontiguousarray(X, np.float32).reshape(-1, 256)
+        B = X.shape[0]
+        st = np.zeros((B, 128), np.uint16) if want_states else None
+        pk = np.zeros((B, 32), np.uint16) if want_packed else None
+        _check(lib().qtip_viterbi_tiles(self._h, _ptr(X), B, _ptr(st), _ptr(pk)))
+        return st, pk
+
+    def viterbi_tiles_dev(self, dX, B, d_states=None, d_packed=None):
+        _check(lib().qtip_viterbi_tiles_dev(self._h, _ptr(dX), B, _ptr(d_states), _ptr(d_packed)))
+
+    def decode_states_dev(self, d_states, B, d_hat):
+        _check(lib().qtip_decode_states_dev(self._h, _ptr(d_states), B, _ptr(d_hat)))
+
+    def hadamard_rows_dev(self, dX, rows, n, ld, transpose):
+        _check(lib().qtip_hadamard_rows_dev(self._h, _ptr(dX), rows, n, ld, 1 if transpose else 0))
+
+    # ---- the group path
+    def rotate_hessian(self, H, n, seed, opt: QuantOpts = None) -> HessPrep:
+        import time
+        opt = opt or QuantOpts()
+        t0 = time.time()
+        hp = HessPrep(n=n, seed=seed)
+        hp.su = np.zeros(n, np.float32)
+        hp.HRr = np.zeros((n, n), np.float32)
+        creg = C.c_double()
+        if not _is_device(H):
+            H = np.ascontiguousarray(H, np.float32)
+        _check(lib().qtip_rotate_hessian(self._h, _ptr(H), 1 if _is_device(H) else 0, n, seed, opt.sigma_reg,
+                                         _ptr(hp.su), C.byref(creg), _ptr(hp.HRr)))
+        hp.creg = creg.value
+        hp.t_rot = time.time() - t0
+        return hp
+
+    @staticmethod
+    def ldl_hessian(hp: HessPrep, threads=16, tag=""):
+        import time
+        t0 = time.time()
+        hp.L = np.zeros((hp.n, hp.n), np.float32)
+        rc = lib().qtip_ldl_hessian(_ptr(hp.HRr), hp.n, threads, _ptr(hp.L))
+        if rc != 0:
+            hp.L = None
+            _check(rc)
+        hp.t_ldl = time.time() - t0
+
+    def ldlq_dev(self, dWT, dL, n, m, d_hatWT, dQ, time_viterbi=False):
+        vs = C.c_double()
+        _check(lib().qtip_ldlq_dev(self._h, _ptr(dWT), _ptr(dL), n, m, _ptr(d_hatWT), _ptr(dQ),
+                                   C.byref(vs) if time_viterbi else None))
+        return vs.value
+
+    def _marshal(self, lins, n, opt):
+        if not opt.share_su:
+            raise QtipError(QTIP_E_ARG, "share_su=false not supported (one LDL per group)")
+        cin = (_LinearInC * len(lins))()
+        cout = (_LinearOutC * len(lins))()
+        outs, keep = [], []
+        for k, li in enumerate(lins):
+            cin[k].m = li.m
+            dev = 0
+            for fld in ("w_f32", "w_bf16", "w_fp8", "scale_bf16"):
+                v = getattr(li, fld)
+                if v is not None:
+                    if _is_device(v):
+                        dev = 1
+                    elif not isinstance(v, int):
+                        v = np.ascontiguousarray(v)
+                    keep.append(v)
+                    setattr(cin[k], fld, _ptr(v))
+            cin[k].on_device = dev
+            o = LinearOut(name=li.name, m=li.m, n=n)
+            o.trellis = np.zeros((li.m // 16) * (n // 16) * 32, np.uint16)
+            o.su_bf16 = np.zeros(n, np.uint16)
+            o.sv = np.zeros(li.m, np.float32)
+            o.hatW = np.zeros((li.m, n), np.float32) if opt.want_hatW else None
+            cout[k].trellis, cout[k].su_bf16, cout[k].sv = _ptr(o.trellis), _ptr(o.su_bf16), _ptr(o.sv)
+            cout[k].hatW = _ptr(o.hatW)
+            outs.append(o)
+        co = _OptsC(opt.sigma_reg, opt.scale_override, opt.ldl_threads, opt.feedback, 1 if opt.skip_proxy else 0)
+        return cin, cout, outs, co, keep
+
+    @staticmethod
+    def _finish(cout, outs, tm):
+        for k, o in enumerate(outs):
+            o.wscale, o.proxy = cout[k].wscale, cout[k].proxy
+            o.proxy_rot_reg, o.seconds = cout[k].proxy_rot_reg, cout[k].seconds
+        return outs, GroupTiming(**{k: getattr(tm, k) for k, _ in _TimingC._fields_})
+
+    def quantize_group(self, lins: List[LinearIn], hp: HessPrep, opt: QuantOpts = None):
+        """quantize_group(s, gemm, lins, hp, opt, tm, tag), src/quantizer.cpp:176-346.  Consumes hp.L."""
+        opt = opt or QuantOpts()
+        cin, cout, outs, co, keep = self._marshal(lins, hp.n, opt)
+        tm = _TimingC()
+        tm.rht, tm.ldl_cpu = hp.t_rot, hp.t_ldl
+        _check(lib().qtip_quantize_group(self._h, len(lins), cin, hp.n, hp.seed, _ptr(hp.su), hp.creg, _ptr(hp.HRr),
+                                         _ptr(hp.L), C.byref(co), cout, C.byref(tm)))
+        hp.L = None
+        return self._finish(cout, outs, tm)
+
+    def quantize_group_h(self, lins: List[LinearIn], n, H, seed, opt: QuantOpts = None):
+        """quantize_group(s, gemm, lins, n, H, seed, opt, tm, tag), src/quantizer.cpp:167-174."""
+        opt = opt or QuantOpts()
+        cin, cout, outs, co, keep = self._marshal(lins, n, opt)
+        tm = _TimingC()
+        if not _is_device(H):
+            H = np.ascontiguousarray(H, np.float32)
+        _check(lib().qtip_quantize_group_h(self._h, len(lins), cin, n, _ptr(H), 1 if _is_device(H) else 0, seed,
+                                           C.byref(co), cout, C.byref(tm)))
+        return self._finish(cout, outs, tm)
+
+
+# ---------------------------------------------------------------- host packers
+def pack_trellis(states):
+    states = np.ascontiguousarray(states, np.uint16).reshape(-1, 128)
+    out = np.zeros((states.shape[0], 32), np.uint16)
+    lib().qtip_pack_trellis(_ptr(states), states.shape[0], _ptr(out))
+    return out
+
+
+def unpack_trellis(packed):
+    packed = np.ascontiguousarray(packed, np.uint16).reshape(-1, 32)
+    out = np.zeros((packed.shape[0], 128), np.uint16)
+    lib().qtip_unpack_trellis(_ptr(packed), packed.shape[0], _ptr(out))
+    return out
+
+
+def swizzle_for_kernel(packed, m, n):
+    packed = np.ascontiguousarray(packed, np.uint16).reshape(-1)
+    out = np.zeros_like(packed)
+    _check(lib().qtip_swizzle_for_kernel(_ptr(packed), m, n, _ptr(out)))
+    return out
+
+
+def unswizzle_for_kernel(tr, m, n):
+    tr = np.ascontiguousarray(tr, np.uint16).reshape(-1)
+    out = np.zeros_like(tr)
+    _check(lib().qtip_unswizzle_for_kernel(_ptr(tr), m, n, _ptr(out)))
+    return out
+
+
+def had_K(n):
+    return lib().qtip_had_K(n)
+
+
+def sign_vector(seed, count):
+    out = np.zeros(count, np.float32)
+    lib().qtip_sign_vector(seed, count, _ptr(out))
+    return out

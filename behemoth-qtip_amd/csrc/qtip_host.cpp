@@ -1,0 +1,185 @@
+// Host-side pieces of the group quantizer: number formats, sign streams, codebook expansion, Hadamard factor
+// selection, trellis packing.  Semantics follow the reference files named at each function.
+#include <cmath>
+#include <cstring>
+
+#include "data/qtip_tables.h"
+#include "qtip_internal.hpp"
+
+namespace qtipmi {
+
+static thread_local std::string g_last_error;
+void set_last_error(const std::string& m) { g_last_error = m; }
+const std::string& last_error_ref() { return g_last_error; }
+void fail(int code, const char* fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  std::vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  throw Error(code, buf);
+}
+
+// IEEE binary16 <-> binary32, round to nearest even (src/common.hpp:49-78 of the reference)
+uint16_t f32_to_fp16(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  const uint32_t sign = (u >> 16) & 0x8000u, mag = u & 0x7fffffffu;
+  if (mag >= 0x7f800000u) return uint16_t(sign | 0x7c00u | (mag > 0x7f800000u ? 0x200u : 0u));
+  if (mag >= 0x477ff000u) return uint16_t(sign | 0x7c00u);  // rounds to infinity
+  if (mag < 0x38800000u) {                                  // below the smallest normal half: fixed point in 2^-24
+    const uint32_t e = mag >> 23;
+    if (e < 102) return uint16_t(sign);                     // < 2^-25: rounds to zero (2^-25 itself ties to even = 0)
+    const uint32_t sig = (mag & 0x7fffffu) | 0x800000u;     // 24-bit significand, value = sig * 2^(e-150)
+    const int shift = int(126 - e);                         // result = sig >> shift, in units of 2^-24
+    const uint32_t q = sig >> shift, rem = sig & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    uint32_t r = q;
+    if (rem > half || (rem == half && (q & 1u))) ++r;
+    return uint16_t(sign | r);
+  }
+  uint32_t h = (((mag >> 23) - 112u) << 10) | ((mag & 0x7fffffu) >> 13);
+  const uint32_t rem = mag & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h;
+  return uint16_t(sign | h);
+}
+float fp16_to_f32(uint16_t h) {
+  const uint32_t s = (h >> 15) & 1u, e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+  float v;
+  if (e == 0) v = std::ldexp(float(m), -24);
+  else if (e == 31) v = m ? NAN : INFINITY;
+  else v = std::ldexp(float(m | 0x400u), int(e) - 25);
+  return s ? -v : v;
+}
+uint16_t f32_to_bf16(float f) {  // src/common.hpp:42-48
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return uint16_t(u >> 16);
+}
+float bf16_to_f32(uint16_t h) {
+  const uint32_t u = uint32_t(h) << 16;
+  float f;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+// splitmix64 stream of the reference (src/common.hpp:91-107)
+SplitMix::SplitMix(uint64_t seed) : s(seed * 0x9E3779B97F4A7C15ull + 0x1234567ull) {}
+uint64_t SplitMix::next() {
+  uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+float SplitMix::sign() { return (next() >> 63) ? -1.0f : 1.0f; }
+
+// get_hadK (src/qtip_core.cpp:77-81): the first factor size of the fixed order that divides n decides
+int had_K(int n) {
+  auto pow2 = [](long v) { return v > 0 && (v & (v - 1)) == 0; };
+  if (n <= 0) return 0;
+  for (int i = 0; i < QTIP_NUM_HAD; ++i) {
+    const int K = qtip_had_order[i];
+    if (n % K == 0) return pow2(n / K) ? K : 0;
+  }
+  return pow2(n) ? 1 : 0;
+}
+std::vector<int8_t> had_matrix(int K, bool transpose) {
+  const uint32_t* bits = qtip_had_bits(K);
+  if (!bits) fail(QTIP_E_ARG, "no Hadamard factor of size %d", K);
+  std::vector<int8_t> m(size_t(K) * K);
+  for (int r = 0; r < K; ++r)
+    for (int k = 0; k < K; ++k)
+      m[size_t(r) * K + k] = int8_t(transpose ? qtip_had_entry(bits, K, k, r) : qtip_had_entry(bits, K, r, k));
+  return m;
+}
+
+// quantlut_sym expansion (src/qtip_core.cpp:18-46): state s reads entry e(s) = bits 6..15 of s*(s+1);
+// bit 9 of e is the sign fold of component 0, the low 9 bits index the fp16-rounded tlut.
+void HostCodebook::build(const float* t) {
+  for (int i = 0; i < 512; ++i)
+    for (int v = 0; v < 2; ++v) {
+      float f;
+      if (t) f = t[i * 2 + v];
+      else std::memcpy(&f, &qtip_hyb_tlut_bits[i * 2 + v], 4);
+      tlut[i][v] = f;
+      tlut_h[i][v] = f32_to_fp16(f);
+    }
+  for (int e = 0; e < kLutEntries; ++e) {
+    const int idx = e & 511;
+    uint16_t h0 = tlut_h[idx][0];
+    if (e >> 9) h0 ^= 0x8000u;
+    entry_f[e][0] = fp16_to_f32(h0);
+    entry_f[e][1] = fp16_to_f32(tlut_h[idx][1]);
+    entry_d[e][0] = entry_f[e][0];
+    entry_d[e][1] = entry_f[e][1];
+  }
+  double ss = 0;  // same accumulation order as the reference: ascending state
+  for (uint32_t s = 0; s < uint32_t(kStates); ++s) {
+    const uint32_t e = entry_of_state(s);
+    ss += double(entry_f[e][0]) * entry_f[e][0] + double(entry_f[e][1]) * entry_f[e][1];
+  }
+  lut_rms = std::sqrt(ss / (2.0 * kStates));
+}
+
+// Bit stream of one trellis, MSB first: the 16 bits of state 0, then the 4 new bits of states 1..127, cut at
+// 512 bits (src/qtip_core.cpp:194-208).  Written nibble-wise: word w holds stream nibbles 4w..4w+3.
+void pack_trellis_host(const uint16_t* states, long B, uint16_t* packed) {
+#pragma omp parallel for schedule(static) if (B > 4096)
+  for (long b = 0; b < B; ++b) {
+    const uint16_t* st = states + b * kSteps;
+    uint16_t* out = packed + b * kWords;
+    out[0] = st[0];
+    for (int w = 1; w < kWords; ++w) {
+      uint32_t v = 0;
+      for (int k = 0; k < 4; ++k) v = (v << 4) | (st[4 * w + k - 3] & 15u);  // stream nibble q (q >= 4) is state q-3
+      out[w] = uint16_t(v);
+    }
+  }
+}
+void unpack_trellis_host(const uint16_t* packed, long B, uint16_t* states) {
+#pragma omp parallel for schedule(static) if (B > 4096)
+  for (long b = 0; b < B; ++b) {
+    const uint16_t* in = packed + b * kWords;
+    uint16_t* st = states + b * kSteps;
+    auto nib = [&](int q) -> uint32_t {
+      q &= 127;  // the stream wraps (tail-biting)
+      return (in[q >> 2] >> (12 - 4 * (q & 3))) & 15u;
+    };
+    for (int t = 0; t < kSteps; ++t) st[t] = uint16_t((nib(t) << 12) | (nib(t + 1) << 8) | (nib(t + 2) << 4) | nib(t + 3));
+  }
+}
+// Kernel layout (src/qtip_core.cpp:230-253): word c of tile (2*i0+i1, 2*j0+j1) goes to
+// out[(((i0*(n/32)+j0)*32 + c)*2 + j1)*2 + i1]
+bool swizzle_host(const uint16_t* packed, int m, int n, uint16_t* out) {
+  if (m % 32 || n % 32) return false;
+  const long nb = n / 16, M2 = m / 32, N2 = n / 32;
+#pragma omp parallel for schedule(static)
+  for (long i0 = 0; i0 < M2; ++i0)
+    for (long j0 = 0; j0 < N2; ++j0) {
+      uint16_t* o = out + (i0 * N2 + j0) * 128;
+      for (int i1 = 0; i1 < 2; ++i1)
+        for (int j1 = 0; j1 < 2; ++j1) {
+          const uint16_t* src = packed + ((2 * i0 + i1) * nb + 2 * j0 + j1) * 32;
+          for (int c = 0; c < 32; ++c) o[(c * 2 + j1) * 2 + i1] = src[c];
+        }
+    }
+  return true;
+}
+bool unswizzle_host(const uint16_t* in, int m, int n, uint16_t* packed) {
+  if (m % 32 || n % 32) return false;
+  const long nb = n / 16, M2 = m / 32, N2 = n / 32;
+#pragma omp parallel for schedule(static)
+  for (long i0 = 0; i0 < M2; ++i0)
+    for (long j0 = 0; j0 < N2; ++j0) {
+      const uint16_t* o = in + (i0 * N2 + j0) * 128;
+      for (int i1 = 0; i1 < 2; ++i1)
+        for (int j1 = 0; j1 < 2; ++j1) {
+          uint16_t* dst = packed + ((2 * i0 + i1) * nb + 2 * j0 + j1) * 32;
+          for (int c = 0; c < 32; ++c) dst[c] = o[(c * 2 + j1) * 2 + i1];
+        }
+    }
+  return true;
+}
+
+}  // namespace qtipmi

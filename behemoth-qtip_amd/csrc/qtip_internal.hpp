@@ -1,0 +1,130 @@
+// Internal declarations shared by the host side and the HIP translation units of libqtip_mi355.so.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/qtip_mi355.h"
+
+namespace qtipmi {
+
+constexpr int kSeq = 256;      // weights per trellis (one 16x16 tile)
+constexpr int kSteps = 128;    // trellis steps, 2 weights each
+constexpr int kStates = 65536; // L = 16
+constexpr int kGroups = 4096;  // states sharing a successor group
+constexpr int kWords = 32;     // packed u16 words per trellis
+constexpr int kLutEntries = 1024;  // distinct codebook entries: bits 6..15 of s*(s+1)
+
+struct Error : std::runtime_error {
+  int code;
+  Error(int c, const std::string& m) : std::runtime_error(m), code(c) {}
+};
+[[noreturn]] void fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void set_last_error(const std::string& m);
+
+#define QTIP_HIP(expr)                                                                              \
+  do {                                                                                              \
+    hipError_t e_ = (expr);                                                                         \
+    if (e_ != hipSuccess)                                                                           \
+      ::qtipmi::fail(QTIP_E_HIP, "%s:%d: %s -> %s", __FILE__, __LINE__, #expr, hipGetErrorString(e_)); \
+  } while (0)
+#define QTIP_REQUIRE(cond, ...)                              \
+  do {                                                       \
+    if (!(cond)) ::qtipmi::fail(QTIP_E_ARG, __VA_ARGS__);    \
+  } while (0)
+
+// Device buffer released on scope exit.
+template <class T>
+struct DBuf {
+  T* p = nullptr;
+  size_t n = 0;
+  DBuf() = default;
+  explicit DBuf(size_t count) { alloc(count); }
+  DBuf(const DBuf&) = delete;
+  DBuf& operator=(const DBuf&) = delete;
+  ~DBuf() { release(); }
+  void alloc(size_t count) {
+    release();
+    n = count;
+    if (count) QTIP_HIP(hipMalloc(reinterpret_cast<void**>(&p), count * sizeof(T)));
+  }
+  void ensure(size_t count) {
+    if (count > n) alloc(count);
+  }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    n = 0;
+  }
+  size_t bytes() const { return n * sizeof(T); }
+  operator T*() const { return p; }
+};
+
+// ---- host-side number formats / streams (qtip_host.cpp)
+uint16_t f32_to_fp16(float f);
+float fp16_to_f32(uint16_t h);
+uint16_t f32_to_bf16(float f);
+float bf16_to_f32(uint16_t h);
+struct SplitMix {
+  uint64_t s;
+  explicit SplitMix(uint64_t seed);
+  uint64_t next();
+  float sign();
+};
+int had_K(int n);
+// K x K mixing matrix as +-1 int8: row k2 holds hadK[k2][k] (transpose=false) or hadK[k][k2] (transpose=true)
+std::vector<int8_t> had_matrix(int K, bool transpose);
+
+struct HostCodebook {
+  float tlut[512][2];
+  uint16_t tlut_h[512][2];
+  // per distinct entry e = flip << 9 | idx: the two decoded components
+  double entry_d[kLutEntries][2];
+  float entry_f[kLutEntries][2];
+  double lut_rms = 0;
+  void build(const float* tlut_or_null);
+  static inline uint32_t entry_of_state(uint32_t s) { return ((s * (s + 1)) >> 6) & 1023u; }
+};
+
+void pack_trellis_host(const uint16_t* states, long B, uint16_t* packed);
+void unpack_trellis_host(const uint16_t* packed, long B, uint16_t* states);
+bool swizzle_host(const uint16_t* packed, int m, int n, uint16_t* out);
+bool unswizzle_host(const uint16_t* in, int m, int n, uint16_t* packed);
+
+// fp64 block LDL on the host (host_ldl.cpp). A: n x n fp64, lower triangle used, destroyed. Returns false if not PD.
+bool block_ldl_host(double* A, int n, float* L_out, int threads);
+
+// ---- GPU launchers (viterbi.hip, rht.hip, ldlq.hip)
+struct TileJob {
+  // inputs: either X (tiles x 256 fp32, sequence order) or the LDLQ feedback operands
+  const float* X = nullptr;
+  long tiles = 0;
+  // outputs (any may be null)
+  uint16_t* states = nullptr;  // state words of tile t at states[(t * q_tile_stride + q_offset) * 128]
+  long q_tile_stride = 1, q_offset = 0;
+  uint16_t* packed = nullptr;  // tiles x 32, pack_trellis layout
+  float* hatWT = nullptr;      // scatter of decoded values: hatWT[(col0 + c) * ldw + 16 * t + r]
+  long ldw = 0, col0 = 0;
+};
+size_t viterbi_workspace_bytes(int slots);
+int viterbi_max_slots(int device);
+void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const float* d_entry_f, void* workspace,
+                          int slots, hipStream_t s);
+void launch_decode_states(const uint16_t* states, long B, float* hat, const float* d_entry_f, hipStream_t s);
+
+}  // namespace qtipmi
+
+struct qtip_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  qtipmi::HostCodebook cb;
+  qtipmi::DBuf<double> d_entry_d;  // [1024][2]
+  qtipmi::DBuf<float> d_entry_f;   // [1024][2]
+  qtipmi::DBuf<unsigned char> vit_ws;
+  int vit_slots = 0;
+};

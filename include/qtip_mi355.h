@@ -1,0 +1,139 @@
+/* C ABI of the MI355X (gfx950) QTIP group quantizer: libqtip_mi355.so.
+ *
+ * Plain pointers and sizes only.  Every call returns 0 on success or a negative QTIP_E_* code;
+ * qtip_last_error() returns the message of the calling thread's last failure.  Nothing here aborts
+ * the process; the C++ shim (behemoth-qtip_amd/csrc/quantizer.hpp) that mirrors the reference's
+ * C++ API restores its abort-on-error behaviour on top of these calls.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the reference root).
+ * Pointers named host_* are host memory, dev_* device memory of the context's device.
+ */
+#ifndef QTIP_MI355_H_
+#define QTIP_MI355_H_
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  QTIP_OK = 0,
+  QTIP_E_ARG = -1,     /* bad argument / unsupported shape (the reference's QCHECK preconditions) */
+  QTIP_E_HIP = -2,     /* a HIP runtime call failed */
+  QTIP_E_NOT_PD = -3,  /* block LDL failed: Hessian not positive definite or not finite */
+  QTIP_E_NOMEM = -4
+};
+
+typedef struct qtip_ctx qtip_ctx;
+
+/* One context per worker thread and device (the reference's worker does hipSetDevice + a private
+ * non-blocking stream + device_lut(), src/pipeline.cpp:237-238,806-812, src/quantizer.cpp:14-28).
+ * The context owns its stream, the codebook tables on the device and reusable workspaces. */
+int qtip_create(int device, qtip_ctx** out);
+void qtip_destroy(qtip_ctx* ctx);
+const char* qtip_last_error(void);
+/* hipStream_t of the context, as an opaque pointer */
+void* qtip_stream(qtip_ctx* ctx);
+int qtip_synchronize(qtip_ctx* ctx);
+
+/* Codebook (replaces the hard-wired codebook(), src/qtip_core.cpp:18-50, and device_lut(),
+ * src/quantizer.cpp:14-28).  tlut: 512 x 2 fp32, NULL selects the built-in HYB table.  The table is
+ * rounded to fp16 (RNE) and expanded by quantlut_sym as the reference does. */
+int qtip_set_tlut(qtip_ctx* ctx, const float* host_tlut);
+double qtip_lut_rms(qtip_ctx* ctx);
+/* decoded 65536-entry LUT (fp16 values as fp32), either pointer may be NULL */
+int qtip_get_lut(qtip_ctx* ctx, float* host_lut0, float* host_lut1);
+
+/* Two-pass tail-biting Viterbi of B independent 256-value sequences (replaces the launch chain
+ * k_viterbi_fwd(roll) -> k_viterbi_overlap -> k_viterbi_fwd(overlap) -> k_viterbi_finish of
+ * tests/test_gpu.cpp:67-88 / src/quantizer.cpp:57-62; result equals quantize_seq_ref,
+ * src/qtip_core.cpp:180-191, bit for bit: fp64 path metrics, no input rounding).
+ * X: B x 256 fp32 in sequence order.  states: B x 128 u16 and/or packed: B x 32 u16 (pack_trellis
+ * layout, src/qtip_core.cpp:194-208); either may be NULL. */
+int qtip_viterbi_tiles(qtip_ctx* ctx, const float* host_X, long B, uint16_t* host_states, uint16_t* host_packed);
+/* Same with device pointers; asynchronous on the context's stream. */
+int qtip_viterbi_tiles_dev(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* dev_states, uint16_t* dev_packed);
+
+/* hat[i] = lut[state[i]] (k_decode_states, src/viterbi.hip:231-238): B x 128 states -> B x 256 fp32 */
+int qtip_decode_states_dev(qtip_ctx* ctx, const uint16_t* dev_states, long B, float* dev_hat);
+
+/* In-place row transform x <- (hadK^(T) (x) H_{n/K}) x / sqrt(n) of `rows` rows of length n, row stride ld
+ * (k_hadamard_rows, src/kernels.hip:293-313; same fp32 dataflow, so results are bit-identical to it). */
+int qtip_hadamard_rows_dev(qtip_ctx* ctx, float* dev_X, long rows, int n, long ld, int transpose);
+int qtip_had_K(int n); /* get_hadK, src/qtip_core.cpp:77-81: K, or 0 if unsupported */
+
+/* Sign vector from the splitmix stream (Rng::sign, src/common.hpp:91-107) */
+void qtip_sign_vector(uint64_t seed, long count, float* host_out);
+
+/* rotate_hessian, src/quantizer.cpp:124-152.  H: n x n fp32 (host, or device when h_on_device != 0; never
+ * written).  Outputs (host): su[n] (+-1), *creg, HRr[n*n]. */
+int qtip_rotate_hessian(qtip_ctx* ctx, const float* H, int h_on_device, int n, uint64_t seed, double sigma_reg,
+                        float* host_su, double* creg, float* host_HRr);
+
+/* ldl_hessian, src/quantizer.cpp:154-165 (+ block_ldl_to_L, src/qtip_core.cpp:444-487): host only, fp64,
+ * uses its own OpenMP team of `threads`; safe to call from a side thread while the GPU works.
+ * HRr n x n fp32 in, L n x n fp32 out (strictly block-lower). */
+int qtip_ldl_hessian(const float* host_HRr, int n, int threads, float* host_L);
+
+/* ldlq_gpu, src/quantizer.cpp:30-89.  WT n x m fp32 (scaled), L n x n fp32, both on the device;
+ * outputs hatWT n x m fp32 and Q[(m/16)*(n/16)][128] u16 on the device.  vit_seconds may be NULL. */
+int qtip_ldlq_dev(qtip_ctx* ctx, const float* dev_WT, const float* dev_L, long n, long m, float* dev_hatWT,
+                  uint16_t* dev_Q, double* vit_seconds);
+
+/* One linear of a group (LinearIn, src/quantizer.hpp:21-28): exactly one weight pointer is set. */
+typedef struct {
+  int m;                     /* out features */
+  const float* w_f32;        /* [m][n] fp32 */
+  const uint16_t* w_bf16;    /* [m][n] raw bf16 bits */
+  const uint8_t* w_fp8;      /* [m][n] FP8 E4M3 with ... */
+  const uint16_t* scale_bf16;/* ... [m] per-output-channel bf16 scale */
+  int on_device;             /* 0: pointers are host memory, 1: device memory */
+} qtip_linear_in;
+
+/* Results for one linear (LinearOut, src/quantizer.hpp:30-43); buffers are caller-allocated host memory. */
+typedef struct {
+  uint16_t* trellis;   /* [(m/16)*(n/16)][32] u16, kernel layout */
+  uint16_t* su_bf16;   /* [n] */
+  float* sv;           /* [m] +-1 */
+  float* hatW;         /* [m][n] or NULL (want_hatW) */
+  float wscale;
+  double proxy;
+  double proxy_rot_reg;
+  double seconds;
+} qtip_linear_out;
+
+typedef struct { /* QuantOpts, src/quantizer.hpp:11-19 */
+  double sigma_reg;      /* 1e-2 */
+  double scale_override; /* 0.9 */
+  int ldl_threads;       /* 16 */
+  int feedback;          /* 0: fp64 feedback + fp64 MFMA prod cache (default); 1: fp32 feedback + bf16 hi/lo split MFMA */
+  int skip_proxy;        /* 1: leave proxy fields 0 */
+} qtip_opts;
+void qtip_default_opts(qtip_opts* o);
+
+typedef struct { /* GroupTiming, src/quantizer.hpp:45-47 */
+  double load, rht, ldl_cpu, ldlq, viterbi, proxy, pack, total;
+} qtip_timing;
+
+/* quantize_group(s, gemm, lins, hp, opt, tm, tag), src/quantizer.cpp:176-346, with the HessPrep fields passed
+ * flat: su[n], creg, HRr[n*n], L[n*n] (host; L is read, never freed).  seed gives the SV streams. */
+int qtip_quantize_group(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, int n, uint64_t seed,
+                        const float* host_su, double creg, const float* host_HRr, const float* host_L,
+                        const qtip_opts* opts, qtip_linear_out* outs, qtip_timing* timing);
+
+/* quantize_group(s, gemm, lins, n, H, seed, opt, tm, tag), src/quantizer.cpp:167-174: rotate + LDL + quantize. */
+int qtip_quantize_group_h(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, int n, const float* H,
+                          int h_on_device, uint64_t seed, const qtip_opts* opts, qtip_linear_out* outs,
+                          qtip_timing* timing);
+
+/* Host packers (pack_trellis / unpack_trellis / swizzle_for_kernel / unswizzle_for_kernel,
+ * src/qtip_core.cpp:194-253) */
+void qtip_pack_trellis(const uint16_t* states, long B, uint16_t* packed);
+void qtip_unpack_trellis(const uint16_t* packed, long B, uint16_t* states);
+int qtip_swizzle_for_kernel(const uint16_t* packed, int m, int n, uint16_t* out);
+int qtip_unswizzle_for_kernel(const uint16_t* in, int m, int n, uint16_t* packed);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
