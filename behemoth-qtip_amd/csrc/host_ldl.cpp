@@ -1,0 +1,307 @@
+// Host-side fp64 block LDL of the rotated Hessian (the reference keeps this step in fp64 on the CPU:
+// ldl_hessian, src/quantizer.cpp:154-165; block_ldl_to_L / cholesky_inplace, src/qtip_core.cpp:321-487).
+//
+//   A = C C^T (lower Cholesky, fp64)  ->  L = C * blockdiag(C_bb^-1) with the 16x16 diagonal blocks and the
+//   upper triangle zeroed, stored as fp32.
+//
+// Own layout of the work: right-looking panels of width NB; the diagonal block is factored in place, the rows
+// below are solved eight at a time (one SIMD lane per row), and the trailing symmetric update runs as a packed
+// register-blocked rank-NB kernel over lower-triangular tiles handed out dynamically to an OpenMP team.  The
+// micro-kernels are written with GCC vector extensions and compiled twice (AVX2 baseline, AVX-512 clone);
+// the clone is picked at run time so one binary serves any x86-64-v3 host.
+#include <omp.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+#include "qtip_internal.hpp"
+
+namespace qtipmi {
+namespace {
+
+typedef double v8d __attribute__((vector_size(64), aligned(8)));
+typedef double v4d __attribute__((vector_size(32), aligned(8)));
+
+constexpr int NB = 256;  // panel width
+constexpr int TILE = 192;  // rows / columns of one trailing-update task (multiple of every MR and NR below)
+
+// ---- rank-kc update of an MR x NR tile: Cij -= sum_p a[p][i] * b[p][j], a packed [kc][MR], b packed [kc][NR]
+// AVX-512: 8 x 24 (24 accumulators of 8 doubles, named so that they stay in registers)
+#define QTIP_ROWS8(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7)
+#define QTIP_ROWS4(X) X(0) X(1) X(2) X(3)
+__attribute__((target("avx512f"))) static void micro_8x24(int kc, const double* __restrict__ a,
+                                                          const double* __restrict__ b, double* __restrict__ C,
+                                                          long ldc, int mr, int nr) {
+  const v8d z = {0, 0, 0, 0, 0, 0, 0, 0};
+#define QTIP_DECL(i) v8d c##i##0 = z, c##i##1 = z, c##i##2 = z;
+  QTIP_ROWS8(QTIP_DECL)
+#undef QTIP_DECL
+  for (int p = 0; p < kc; ++p) {
+    const v8d b0 = *reinterpret_cast<const v8d*>(b + p * 24), b1 = *reinterpret_cast<const v8d*>(b + p * 24 + 8),
+              b2 = *reinterpret_cast<const v8d*>(b + p * 24 + 16);
+#define QTIP_FMA(i)                   \
+  {                                   \
+    const double ai = a[p * 8 + i];   \
+    c##i##0 += ai * b0;               \
+    c##i##1 += ai * b1;               \
+    c##i##2 += ai * b2;               \
+  }
+    QTIP_ROWS8(QTIP_FMA)
+#undef QTIP_FMA
+  }
+  if (mr == 8 && nr == 24) {
+#define QTIP_STORE(i)                                   \
+  {                                                     \
+    double* ci = C + i * ldc;                           \
+    *reinterpret_cast<v8d*>(ci) -= c##i##0;             \
+    *reinterpret_cast<v8d*>(ci + 8) -= c##i##1;         \
+    *reinterpret_cast<v8d*>(ci + 16) -= c##i##2;        \
+  }
+    QTIP_ROWS8(QTIP_STORE)
+#undef QTIP_STORE
+  } else {
+    v8d t[8][3];
+#define QTIP_SPILL(i) t[i][0] = c##i##0, t[i][1] = c##i##1, t[i][2] = c##i##2;
+    QTIP_ROWS8(QTIP_SPILL)
+#undef QTIP_SPILL
+    for (int i = 0; i < mr; ++i)
+      for (int j = 0; j < nr; ++j) C[i * ldc + j] -= t[i][j >> 3][j & 7];
+  }
+}
+// AVX2: 4 x 12
+static void micro_4x12(int kc, const double* __restrict__ a, const double* __restrict__ b, double* __restrict__ C,
+                       long ldc, int mr, int nr) {
+  const v4d z = {0, 0, 0, 0};
+#define QTIP_DECL(i) v4d c##i##0 = z, c##i##1 = z, c##i##2 = z;
+  QTIP_ROWS4(QTIP_DECL)
+#undef QTIP_DECL
+  for (int p = 0; p < kc; ++p) {
+    const v4d b0 = *reinterpret_cast<const v4d*>(b + p * 12), b1 = *reinterpret_cast<const v4d*>(b + p * 12 + 4),
+              b2 = *reinterpret_cast<const v4d*>(b + p * 12 + 8);
+#define QTIP_FMA(i)                   \
+  {                                   \
+    const double ai = a[p * 4 + i];   \
+    c##i##0 += ai * b0;               \
+    c##i##1 += ai * b1;               \
+    c##i##2 += ai * b2;               \
+  }
+    QTIP_ROWS4(QTIP_FMA)
+#undef QTIP_FMA
+  }
+  v4d t[4][3];
+#define QTIP_SPILL(i) t[i][0] = c##i##0, t[i][1] = c##i##1, t[i][2] = c##i##2;
+  QTIP_ROWS4(QTIP_SPILL)
+#undef QTIP_SPILL
+  for (int i = 0; i < mr; ++i)
+    for (int j = 0; j < nr; ++j) C[i * ldc + j] -= t[i][j >> 2][j & 3];
+}
+
+// ---- eight rows of the panel solve  X * L11^T = A21, one lane per row (x holds the rows transposed: x[p][lane])
+__attribute__((target("avx512f"))) static void solve8_avx512(int kb, const double* __restrict__ L11 /*kb x kb*/,
+                                                              const double* __restrict__ rdiag, v8d* __restrict__ x) {
+  for (int j = 0; j < kb; ++j) {
+    const double* lj = L11 + size_t(j) * kb;
+    v8d s0 = x[j], s1 = v8d{0, 0, 0, 0, 0, 0, 0, 0}, s2 = s1, s3 = s1;
+    int p = 0;
+    for (; p + 4 <= j; p += 4) {
+      s0 -= lj[p] * x[p];
+      s1 -= lj[p + 1] * x[p + 1];
+      s2 -= lj[p + 2] * x[p + 2];
+      s3 -= lj[p + 3] * x[p + 3];
+    }
+    for (; p < j; ++p) s0 -= lj[p] * x[p];
+    x[j] = ((s0 + s1) + (s2 + s3)) * rdiag[j];
+  }
+}
+static void solve8_avx2(int kb, const double* __restrict__ L11, const double* __restrict__ rdiag,
+                        v8d* __restrict__ x) {
+  for (int j = 0; j < kb; ++j) {
+    const double* lj = L11 + size_t(j) * kb;
+    v8d s0 = x[j], s1 = v8d{0, 0, 0, 0, 0, 0, 0, 0};
+    int p = 0;
+    for (; p + 2 <= j; p += 2) {
+      s0 -= lj[p] * x[p];
+      s1 -= lj[p + 1] * x[p + 1];
+    }
+    for (; p < j; ++p) s0 -= lj[p] * x[p];
+    x[j] = (s0 + s1) * rdiag[j];
+  }
+}
+
+struct Kernels {
+  int MR, NR;
+  void (*micro)(int, const double*, const double*, double*, long, int, int);
+  void (*solve8)(int, const double*, const double*, v8d*);
+};
+static Kernels pick_kernels() {
+  __builtin_cpu_init();
+  if (__builtin_cpu_supports("avx512f")) return Kernels{8, 24, micro_8x24, solve8_avx512};
+  return Kernels{4, 12, micro_4x12, solve8_avx2};
+}
+
+// unblocked lower Cholesky of the kb x kb diagonal block at A (row stride n); false if not positive definite
+static bool factor_diagonal(double* A, long n, int kb) {
+  for (int j = 0; j < kb; ++j) {
+    double* aj = A + long(j) * n;
+    double d = aj[j];
+    for (int p = 0; p < j; ++p) d -= aj[p] * aj[p];
+    if (!(d > 0) || !std::isfinite(d)) return false;
+    d = std::sqrt(d);
+    aj[j] = d;
+    const double rd = 1.0 / d;
+    for (int i = j + 1; i < kb; ++i) {
+      double* ai = A + long(i) * n;
+      double s0 = ai[j], s1 = 0;
+      int p = 0;
+      for (; p + 2 <= j; p += 2) {
+        s0 -= ai[p] * aj[p];
+        s1 -= ai[p + 1] * aj[p + 1];
+      }
+      if (p < j) s0 -= ai[p] * aj[p];
+      ai[j] = (s0 + s1) * rd;
+    }
+  }
+  return true;
+}
+
+bool cholesky_lower(double* A, int n, int threads) {
+  double tdiag = 0, tsolve = 0, tupd = 0, tq;
+  const Kernels kn = pick_kernels();
+  const int MR = kn.MR, NR = kn.NR;
+  std::vector<double> packA, packB, L11(size_t(NB) * NB), rdiag(NB);
+  for (int k = 0; k < n; k += NB) {
+    const int kb = std::min(NB, n - k);
+    tq = omp_get_wtime();
+    if (!factor_diagonal(A + long(k) * n + k, n, kb)) return false;
+    tdiag += omp_get_wtime() - tq;
+    tq = omp_get_wtime();
+    const int r0 = k + kb, nr = n - r0;
+    if (nr <= 0) break;
+    for (int j = 0; j < kb; ++j) {
+      for (int p = 0; p < kb; ++p) L11[size_t(j) * kb + p] = p <= j ? A[long(k + j) * n + k + p] : 0.0;
+      rdiag[j] = 1.0 / L11[size_t(j) * kb + j];
+    }
+    const int nPA = (nr + MR - 1) / MR, nPB = (nr + NR - 1) / NR;
+    packA.assign(size_t(nPA) * MR * kb, 0.0);
+    packB.assign(size_t(nPB) * NR * kb, 0.0);
+    // panel solve, fused with packing the solved panel in both micro-panel layouts
+#pragma omp parallel for schedule(dynamic, 4) num_threads(threads)
+    for (int g = 0; g < (nr + 7) / 8; ++g) {
+      const int rb = g * 8, rows = std::min(8, nr - rb);
+      alignas(64) v8d x[NB];
+      for (int p = 0; p < kb; ++p) {
+        v8d v = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int r = 0; r < rows; ++r) v[r] = A[long(r0 + rb + r) * n + k + p];
+        x[p] = v;
+      }
+      kn.solve8(kb, L11.data(), rdiag.data(), x);
+      for (int r = 0; r < rows; ++r) {
+        const int i = rb + r;
+        double* dst = A + long(r0 + i) * n + k;
+        double* pa = packA.data() + size_t(i / MR) * MR * kb + (i % MR);
+        double* pb = packB.data() + size_t(i / NR) * NR * kb + (i % NR);
+        for (int p = 0; p < kb; ++p) {
+          const double v = x[p][r];
+          dst[p] = v;
+          pa[size_t(p) * MR] = v;
+          pb[size_t(p) * NR] = v;
+        }
+      }
+    }
+    tsolve += omp_get_wtime() - tq;
+    tq = omp_get_wtime();
+    // trailing update of the lower triangle, tiles (bi, bj <= bi) largest rows first
+    const int nT = (nr + TILE - 1) / TILE;
+    const long ntask = long(nT) * (nT + 1) / 2;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
+    for (long task = 0; task < ntask; ++task) {
+      // enumerate from the bottom row block upwards: row block bi has bi+1 tiles
+      long rem = task;
+      int bi = nT - 1;
+      while (rem > bi) {
+        rem -= bi + 1;
+        --bi;
+      }
+      const int bj = int(rem);
+      const int i0 = bi * TILE, i1 = std::min(nr, i0 + TILE), j0 = bj * TILE, j1 = std::min(nr, j0 + TILE);
+      for (int jj = j0; jj < j1; jj += NR) {
+        const double* pb = packB.data() + size_t(jj / NR) * NR * kb;
+        const int nrr = std::min(NR, nr - jj);
+        for (int ii = i0; ii < i1; ii += MR) {
+          if (jj > ii + MR - 1) continue;  // micro tile entirely above the diagonal
+          const int mrr = std::min(MR, nr - ii);
+          kn.micro(kb, packA.data() + size_t(ii / MR) * MR * kb, pb, A + long(r0 + ii) * n + r0 + jj, n, mrr, nrr);
+        }
+      }
+    }
+    tupd += omp_get_wtime() - tq;
+  }
+  if (getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "chol: diag %.3f solve+pack %.3f update %.3f\n", tdiag, tsolve, tupd);
+  return true;
+}
+
+}  // namespace
+
+bool block_ldl_host(double* A, int n, float* L_out, int threads) {
+  if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
+  if (threads <= 0) threads = omp_get_max_threads();
+  double tq = omp_get_wtime();
+  if (!cholesky_lower(A, n, threads)) return false;
+  const double t_chol = omp_get_wtime() - tq;
+  tq = omp_get_wtime();
+  const int nb = n / 16;
+  // inverse of every 16x16 lower-triangular diagonal block (column by column, forward substitution)
+  std::vector<double> inv(size_t(nb) * 256);
+#pragma omp parallel for schedule(static) num_threads(threads)
+  for (int b = 0; b < nb; ++b) {
+    double D[16][16], V[16][16];
+    for (int i = 0; i < 16; ++i)
+      for (int j = 0; j < 16; ++j) D[i][j] = j <= i ? A[long(b * 16 + i) * n + b * 16 + j] : 0.0;
+    for (int c = 0; c < 16; ++c)
+      for (int i = 0; i < 16; ++i) {
+        double s = i == c ? 1.0 : 0.0;
+        for (int p = 0; p < i; ++p) s -= D[i][p] * V[p][c];
+        V[i][c] = s / D[i][i];
+      }
+    std::memcpy(&inv[size_t(b) * 256], V, sizeof V);
+  }
+  int finite = 1;
+#pragma omp parallel for schedule(dynamic, 16) num_threads(threads) reduction(&& : finite)
+  for (int r = 0; r < n; ++r) {
+    const double* ar = A + long(r) * n;
+    float* lr = L_out + long(r) * n;
+    const int rb = r / 16;
+    for (int bj = 0; bj < rb; ++bj) {
+      const double* a = ar + bj * 16;
+      const double* iv = &inv[size_t(bj) * 256];
+      for (int j = 0; j < 16; ++j) {
+        double s = 0;
+        for (int p = j; p < 16; ++p) s += a[p] * iv[p * 16 + j];
+        lr[bj * 16 + j] = float(s);
+        finite = finite && std::isfinite(s);
+      }
+    }
+    std::memset(lr + long(rb) * 16, 0, sizeof(float) * size_t(n - rb * 16));  // diagonal block and everything right of it
+  }
+  if (getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "block_ldl: cholesky %.3f, L assembly %.3f\n", t_chol, omp_get_wtime() - tq);
+  return finite != 0;
+}
+
+// A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle (tiled so both reads stay in cache)
+void symmetrize_lower_host(const float* HRr, int n, double* A, int threads) {
+  if (threads <= 0) threads = omp_get_max_threads();
+  constexpr int T = 64;
+  const int nt = (n + T - 1) / T;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
+  for (int bi = 0; bi < nt; ++bi)
+    for (int bj = 0; bj <= bi; ++bj) {
+      const int i1 = std::min(n, (bi + 1) * T), j1 = std::min(n, (bj + 1) * T);
+      for (int i = bi * T; i < i1; ++i)
+        for (int j = bj * T; j < j1 && j <= i; ++j)
+          A[size_t(i) * n + j] = 0.5 * (double(HRr[size_t(i) * n + j]) + double(HRr[size_t(j) * n + i]));
+    }
+}
+
+}  // namespace qtipmi

@@ -1,0 +1,194 @@
+// LDLQ kernels for gfx950 (reference: ldlq_gpu, src/quantizer.cpp:30-89; ldlq_prep_kernel,
+// src/viterbi.hip:241-267; the CPU form of the algorithm, tests/test_gpu.cpp:180-225).
+//
+//  * ldlq_prep: in-buffer error feedback for one 16-column block; one thread per weight row keeps the 16
+//    column targets in registers, the <= 112 rows of L of the open buffer sit in LDS.  fp64 accumulation (the
+//    CPU algorithm's precision: fp64 is full rate on CDNA4 VALUs), result rounded fp64 -> fp32 -> fp16 like
+//    the CPU path and written in trellis sequence order.
+//  * gemm_tn: C[M][N] (+)= sum_k A[k][i] * (B1 - B2)[k][j] on the fp64 matrix cores
+//    (v_mfma_f64_16x16x4_f64), fp32 operands widened while staging through LDS.  Two epilogues: accumulate
+//    into C (the cross-buffer prod cache), or reduce sum(acc * (B1 - B2)[i][j]) for tr(X^T H X) (the proxy).
+#include <hip/hip_fp16.h>
+
+#include "ldlq.hpp"
+#include "qtip_internal.hpp"
+
+namespace qtipmi {
+namespace {
+
+__device__ __forceinline__ int perm_inv(int q) {  // tile index 16*r + c -> sequence position
+  const int a = q >> 7, b = (q >> 4) & 7, c = (q >> 3) & 1, d = (q >> 1) & 3, e = q & 1;
+  return (((b * 4 + d) * 2 + c) * 2 + a) * 2 + e;
+}
+
+template <typename ProdT>
+__global__ __launch_bounds__(256) void ldlq_prep_kernel(const float* __restrict__ WT, const float* __restrict__ hatWT,
+                                                        const ProdT* __restrict__ prod, const float* __restrict__ L,
+                                                        long n, long m, int col0, int bufend, float* __restrict__ X) {
+  __shared__ ProdT Ls[112][16];
+  const int k0 = col0 + 16, nk = bufend - k0;
+  for (int idx = threadIdx.x; idx < nk * 16; idx += blockDim.x) {
+    const int kk = idx >> 4, c = idx & 15;
+    Ls[kk][c] = ProdT(L[long(k0 + kk) * n + col0 + c]);
+  }
+  __syncthreads();
+  const long j = long(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (j >= m) return;
+  ProdT acc[16];
+#pragma unroll
+  for (int c = 0; c < 16; ++c) acc[c] = ProdT(WT[long(col0 + c) * m + j]) + prod[long(col0 + c) * m + j];
+  for (int kk = 0; kk < nk; ++kk) {
+    const long o = long(k0 + kk) * m + j;
+    const ProdT dk = ProdT(WT[o]) - ProdT(hatWT[o]);
+#pragma unroll
+    for (int c = 0; c < 16; ++c) acc[c] += Ls[kk][c] * dk;
+  }
+  const long bt = j >> 4;
+  const int r = int(j & 15);
+  float* xb = X + bt * 256;
+#pragma unroll
+  for (int c = 0; c < 16; ++c) xb[perm_inv(r * 16 + c)] = __half2float(__float2half_rn(float(acc[c])));
+}
+
+// ---------------------------------------------------------------- fp64 MFMA GEMM
+typedef double double4_t __attribute__((ext_vector_type(4)));
+constexpr int BM = 64, BN = 64, KC = 32;
+
+// MODE 0: C += acc.  MODE 1: partial[block] = sum_ij acc[i][j] * (B1 - B2)[i][j]  (square case M == K rows of B)
+template <int MODE>
+__global__ __launch_bounds__(256) void gemm_tn_f64_kernel(int M, int N, int K, const float* __restrict__ A, long lda,
+                                                          const float* __restrict__ B1, const float* __restrict__ B2,
+                                                          long ldb, double* __restrict__ C, long ldc,
+                                                          double* __restrict__ partial) {
+  __shared__ double As[KC][BM];
+  __shared__ double Bs[KC][BN];
+  __shared__ double red[4];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const long i0 = long(blockIdx.y) * BM, j0 = long(blockIdx.x) * BN;
+  double4_t acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
+
+  for (int kc = 0; kc < K; kc += KC) {
+    for (int idx = t; idx < KC * BM; idx += 256) {
+      const int k = idx / BM, i = idx % BM;
+      const long gi = i0 + i;
+      As[k][i] = (kc + k < K && gi < M) ? double(A[long(kc + k) * lda + gi]) : 0.0;
+    }
+    for (int idx = t; idx < KC * BN; idx += 256) {
+      const int k = idx / BN, j = idx % BN;
+      const long gj = j0 + j;
+      double v = 0.0;
+      if (kc + k < K && gj < N) {
+        const long o = long(kc + k) * ldb + gj;
+        v = double(B1[o]);
+        if (B2) v -= double(B2[o]);
+      }
+      Bs[k][j] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KC; kk += 4) {
+      const int kr = kk + (lane >> 4), c = lane & 15;
+      double a[2], b[2];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi) a[mi] = As[kr][wm * 32 + mi * 16 + c];
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) b[ni] = Bs[kr][wn * 32 + ni * 16 + c];
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+          acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  // accumulator element v of a lane: row (lane / 16) + 4 v, column lane % 16 of the 16x16 tile
+  double local = 0.0;
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const long gi = i0 + wm * 32 + mi * 16 + (lane >> 4) + 4 * v;
+        const long gj = j0 + wn * 32 + ni * 16 + (lane & 15);
+        if (gi < M && gj < N) {
+          if (MODE == 0) {
+            C[gi * ldc + gj] += acc[mi][ni][v];
+          } else {
+            const long o = gi * ldb + gj;
+            double x = double(B1[o]);
+            if (B2) x -= double(B2[o]);
+            local += acc[mi][ni][v] * x;
+          }
+        }
+      }
+  if (MODE == 1) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off, 64);
+    if (lane == 0) red[wave] = local;
+    __syncthreads();
+    if (t == 0) partial[long(blockIdx.y) * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+  }
+}
+
+__global__ __launch_bounds__(256) void sum_partials_kernel(const double* __restrict__ partial, long count,
+                                                           double* __restrict__ out) {
+  __shared__ double red[256];
+  double acc = 0;
+  for (long i = threadIdx.x; i < count; i += 256) acc += partial[i];
+  red[threadIdx.x] = acc;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if (int(threadIdx.x) < s) red[threadIdx.x] += red[threadIdx.x + s];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *out = red[0];
+}
+
+}  // namespace
+
+void launch_ldlq_prep_f64(const float* WT, const float* hatWT, const double* prod, const float* L, long n, long m,
+                          int col0, int bufend, float* X, hipStream_t s) {
+  QTIP_REQUIRE(bufend - col0 - 16 <= 112 && bufend - col0 - 16 >= 0, "ldlq_prep: block outside its buffer");
+  ldlq_prep_kernel<double><<<dim3(unsigned((m + 255) / 256)), dim3(256), 0, s>>>(WT, hatWT, prod, L, n, m, col0,
+                                                                                 bufend, X);
+  QTIP_HIP(hipGetLastError());
+}
+void launch_ldlq_prep_f32(const float* WT, const float* hatWT, const float* prod, const float* L, long n, long m,
+                          int col0, int bufend, float* X, hipStream_t s) {
+  QTIP_REQUIRE(bufend - col0 - 16 <= 112 && bufend - col0 - 16 >= 0, "ldlq_prep: block outside its buffer");
+  ldlq_prep_kernel<float><<<dim3(unsigned((m + 255) / 256)), dim3(256), 0, s>>>(WT, hatWT, prod, L, n, m, col0,
+                                                                                bufend, X);
+  QTIP_HIP(hipGetLastError());
+}
+
+void launch_gemm_tn_f64_acc(int M, int N, int K, const float* A, long lda, const float* B1, const float* B2, long ldb,
+                            double* C, long ldc, hipStream_t s) {
+  if (M <= 0 || N <= 0 || K <= 0) return;
+  dim3 grid(unsigned((N + BN - 1) / BN), unsigned((M + BM - 1) / BM));
+  gemm_tn_f64_kernel<0><<<grid, dim3(256), 0, s>>>(M, N, K, A, lda, B1, B2, ldb, C, ldc, nullptr);
+  QTIP_HIP(hipGetLastError());
+}
+
+double quad_trace_f64(int n, int N, const float* H, const float* B1, const float* B2, long ldb, DBuf<double>& scratch,
+                      hipStream_t s) {
+  if (n <= 0 || N <= 0) return 0.0;
+  dim3 grid(unsigned((N + BN - 1) / BN), unsigned((n + BM - 1) / BM));
+  const long blocks = long(grid.x) * grid.y;
+  scratch.ensure(size_t(blocks) + 1);
+  gemm_tn_f64_kernel<1><<<grid, dim3(256), 0, s>>>(n, N, n, H, n, B1, B2, ldb, nullptr, 0, scratch);
+  QTIP_HIP(hipGetLastError());
+  sum_partials_kernel<<<dim3(1), dim3(256), 0, s>>>(scratch, blocks, scratch + blocks);
+  QTIP_HIP(hipGetLastError());
+  double h = 0;
+  QTIP_HIP(hipMemcpyAsync(&h, scratch + blocks, sizeof(double), hipMemcpyDeviceToHost, s));
+  QTIP_HIP(hipStreamSynchronize(s));
+  return h;
+}
+
+}  // namespace qtipmi

@@ -1,0 +1,9 @@
+#pragma once
+#include "qtip_internal.hpp"
+namespace qtipmi {
+void launch_bf16_to_f32(const uint16_t* in, float* out, long count, hipStream_t s);
+void launch_fp8_to_f32(const uint8_t* w, const uint16_t* scale_bf16, float* out, long rows, long cols, hipStream_t s);
+void launch_scale_rc(float* X, long rows, long cols, long ld, const float* rs, const float* cs, hipStream_t s);
+// states of one linear (m x n weights, tiles row-major) -> kernel-layout trellis words
+void launch_pack_swizzle(const uint16_t* Q, long m, long n, uint16_t* out, hipStream_t s);
+}  // namespace qtipmi

@@ -1,11 +1,12 @@
 // extern "C" surface of libqtip_mi355.so (declared in include/qtip_mi355.h).  Exceptions thrown by the
 // implementation stop here and become return codes plus a thread-local message.
+#include <chrono>
 #include <cstring>
 #include <exception>
+#include <vector>
 #include <memory>
 #include <new>
 
-#include "qtip_internal.hpp"
 #include "quantizer_impl.hpp"
 
 namespace qtipmi {
@@ -77,6 +78,7 @@ int qtip_create(int device, qtip_ctx** out) {
     QTIP_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
     c->cb.build(nullptr);
     upload_codebook(c.get());
+    c->rht.init(device, c->stream);
     (void)hipSetDevice(prev);
     *out = c.release();
   });
@@ -199,15 +201,73 @@ int qtip_unswizzle_for_kernel(const uint16_t* in, int m, int n, uint16_t* packed
 
 }  // extern "C"
 
-// ---- TEMPORARY: entry points still to be implemented
+
 extern "C" {
-#define QTIP_TODO(name) \
-  qtipmi::set_last_error(#name ": not implemented yet"); \
-  return QTIP_E_ARG
-int qtip_hadamard_rows_dev(qtip_ctx*, float*, long, int, long, int) { QTIP_TODO(qtip_hadamard_rows_dev); }
-int qtip_rotate_hessian(qtip_ctx*, const float*, int, int, uint64_t, double, float*, double*, float*) { QTIP_TODO(qtip_rotate_hessian); }
-int qtip_ldl_hessian(const float*, int, int, float*) { QTIP_TODO(qtip_ldl_hessian); }
-int qtip_ldlq_dev(qtip_ctx*, const float*, const float*, long, long, float*, uint16_t*, double*) { QTIP_TODO(qtip_ldlq_dev); }
-int qtip_quantize_group(qtip_ctx*, int, const qtip_linear_in*, int, uint64_t, const float*, double, const float*, const float*, const qtip_opts*, qtip_linear_out*, qtip_timing*) { QTIP_TODO(qtip_quantize_group); }
-int qtip_quantize_group_h(qtip_ctx*, int, const qtip_linear_in*, int, const float*, int, uint64_t, const qtip_opts*, qtip_linear_out*, qtip_timing*) { QTIP_TODO(qtip_quantize_group_h); }
+
+int qtip_hadamard_rows_dev(qtip_ctx* ctx, float* dev_X, long rows, int n, long ld, int transpose) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && (rows == 0 || dev_X != nullptr), "hadamard_rows: bad arguments");
+    DeviceGuard g(ctx);
+    ctx->rht.hadamard_rows(dev_X, rows, n, ld, transpose != 0);
+  });
 }
+
+int qtip_rotate_hessian(qtip_ctx* ctx, const float* H, int h_on_device, int n, uint64_t seed, double sigma_reg,
+                        float* host_su, double* creg, float* host_HRr) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "null context");
+    DeviceGuard g(ctx);
+    rotate_hessian_impl(ctx, H, h_on_device != 0, n, seed, sigma_reg, host_su, creg, host_HRr);
+  });
+}
+
+int qtip_ldl_hessian(const float* host_HRr, int n, int threads, float* host_L) {
+  return guarded([&] { ldl_hessian_impl(host_HRr, n, threads, host_L); });
+}
+
+int qtip_ldlq_dev(qtip_ctx* ctx, const float* dev_WT, const float* dev_L, long n, long m, float* dev_hatWT,
+                  uint16_t* dev_Q, double* vit_seconds) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && dev_WT && dev_L && dev_hatWT && dev_Q, "ldlq: bad arguments");
+    DeviceGuard g(ctx);
+    ldlq_impl(ctx, dev_WT, dev_L, n, m, dev_hatWT, dev_Q, 0, vit_seconds);
+  });
+}
+
+int qtip_quantize_group(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, int n, uint64_t seed,
+                        const float* host_su, double creg, const float* host_HRr, const float* host_L,
+                        const qtip_opts* opts, qtip_linear_out* outs, qtip_timing* timing) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "null context");
+    DeviceGuard g(ctx);
+    qtip_opts o;
+    qtip_default_opts(&o);
+    if (opts) o = *opts;
+    quantize_group_impl(ctx, nlin, lins, n, seed, host_su, creg, host_HRr, host_L, o, outs, timing);
+  });
+}
+
+int qtip_quantize_group_h(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, int n, const float* H, int h_on_device,
+                          uint64_t seed, const qtip_opts* opts, qtip_linear_out* outs, qtip_timing* timing) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && n > 0, "quantize_group: bad arguments");
+    DeviceGuard g(ctx);
+    qtip_opts o;
+    qtip_default_opts(&o);
+    if (opts) o = *opts;
+    std::vector<float> su(static_cast<size_t>(n)), HRr(size_t(n) * n), L(size_t(n) * n);
+    double creg = 0;
+    qtip_timing T{};
+    auto t0 = std::chrono::steady_clock::now();
+    rotate_hessian_impl(ctx, H, h_on_device != 0, n, seed, o.sigma_reg, su.data(), &creg, HRr.data());
+    auto t1 = std::chrono::steady_clock::now();
+    ldl_hessian_impl(HRr.data(), n, o.ldl_threads, L.data());
+    auto t2 = std::chrono::steady_clock::now();
+    T.rht = std::chrono::duration<double>(t1 - t0).count();
+    T.ldl_cpu = std::chrono::duration<double>(t2 - t1).count();
+    quantize_group_impl(ctx, nlin, lins, n, seed, su.data(), creg, HRr.data(), L.data(), o, outs, &T);
+    if (timing) *timing = T;
+  });
+}
+
+}  // extern "C"

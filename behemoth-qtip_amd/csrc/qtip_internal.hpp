@@ -98,6 +98,8 @@ bool unswizzle_host(const uint16_t* in, int m, int n, uint16_t* packed);
 
 // fp64 block LDL on the host (host_ldl.cpp). A: n x n fp64, lower triangle used, destroyed. Returns false if not PD.
 bool block_ldl_host(double* A, int n, float* L_out, int threads);
+// A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle
+void symmetrize_lower_host(const float* HRr, int n, double* A, int threads);
 
 // ---- GPU launchers (viterbi.hip, rht.hip, ldlq.hip)
 struct TileJob {
@@ -119,12 +121,3 @@ void launch_decode_states(const uint16_t* states, long B, float* hat, const floa
 
 }  // namespace qtipmi
 
-struct qtip_ctx {
-  int device = 0;
-  hipStream_t stream = nullptr;
-  qtipmi::HostCodebook cb;
-  qtipmi::DBuf<double> d_entry_d;  // [1024][2]
-  qtipmi::DBuf<float> d_entry_f;   // [1024][2]
-  qtipmi::DBuf<unsigned char> vit_ws;
-  int vit_slots = 0;
-};

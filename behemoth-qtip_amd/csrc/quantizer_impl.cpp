@@ -1,0 +1,311 @@
+// Group quantizer: Hessian rotation, host LDL, weight RHT + scaling, LDLQ driver, proxy, packing.
+// Operation order, seeds and formulas follow the reference's src/quantizer.cpp:30-346 (cited per step).
+#include "quantizer_impl.hpp"
+
+#include <chrono>
+#include <cmath>
+#include <sys/mman.h>
+
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+namespace qtipmi {
+namespace {
+// Large host work buffers, kept for the life of the process and handed out one caller at a time.
+struct HostPool {
+  struct Slot {
+    void* p;
+    size_t cap;
+    bool busy;
+  };
+  std::mutex mu;
+  std::vector<Slot> slots;
+  void* acquire(size_t bytes) {
+    std::lock_guard<std::mutex> lk(mu);
+    for (auto& s : slots)
+      if (!s.busy && s.cap >= bytes) {
+        s.busy = true;
+        return s.p;
+      }
+    for (auto& s : slots)  // an idle but smaller buffer is replaced rather than kept beside the new one
+      if (!s.busy) {
+        std::free(s.p);
+        s.p = nullptr;
+        s.cap = 0;
+      }
+    void* p = nullptr;
+    const size_t huge = size_t(2) << 20;
+    const size_t cap = (bytes + huge - 1) / huge * huge;
+    if (posix_memalign(&p, huge, cap) != 0 || !p) throw Error(QTIP_E_NOMEM, "out of host memory for the LDL work matrix");
+    (void)madvise(p, cap, MADV_HUGEPAGE);
+    for (auto& s : slots)
+      if (!s.p) {
+        s = Slot{p, cap, true};
+        return p;
+      }
+    slots.push_back(Slot{p, cap, true});
+    return p;
+  }
+  void release(void* p) {
+    std::lock_guard<std::mutex> lk(mu);
+    for (auto& s : slots)
+      if (s.p == p) s.busy = false;
+  }
+};
+HostPool& host_pool() {
+  static HostPool pool;
+  return pool;
+}
+struct HostScratch {
+  void* p;
+  explicit HostScratch(size_t bytes) : p(host_pool().acquire(bytes)) {}
+  ~HostScratch() { host_pool().release(p); }
+  void* get() const { return p; }
+};
+
+double now_s() {
+  using namespace std::chrono;
+  return duration<double>(steady_clock::now().time_since_epoch()).count();
+}
+}  // namespace
+
+// ---------------------------------------------------------------- rotate_hessian, src/quantizer.cpp:124-152
+void rotate_hessian_impl(qtip_ctx* c, const float* H, bool on_device, int n, uint64_t seed, double sigma_reg,
+                         float* host_su, double* creg, float* host_HRr) {
+  QTIP_REQUIRE(n > 0 && H && host_su && creg && host_HRr, "rotate_hessian: bad arguments");
+  QTIP_REQUIRE(had_K(n) > 0, "unsupported hadamard dim %d", n);
+  hipStream_t s = c->stream;
+  SplitMix rng(seed);
+  for (int i = 0; i < n; ++i) host_su[i] = rng.sign();
+  DBuf<float> d_su{size_t(n)};
+  QTIP_HIP(hipMemcpyAsync(d_su, host_su, size_t(n) * 4, hipMemcpyHostToDevice, s));
+  DBuf<float> Ht(size_t(n) * n), HR(size_t(n) * n);
+  QTIP_HIP(hipMemcpyAsync(Ht, H, size_t(n) * n * 4, on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, s));
+  // regularize_H: H += sigma_reg * mean(diag(H)) * I, before the rotation
+  const double dsum = c->rht.reduce(Ht, n, nullptr, 0, n, n, 3);
+  *creg = sigma_reg * dsum / n;
+  c->rht.add_diag(Ht, n, float(*creg));
+  // HRr = hadUt(hadUt(H * su su^T)^T)
+  c->rht.hadamard_rows(Ht, n, n, n, true, d_su, d_su);
+  c->rht.transpose(Ht, n, n, n, HR, n);
+  c->rht.hadamard_rows(HR, n, n, n, true);
+  QTIP_HIP(hipMemcpyAsync(host_HRr, HR, size_t(n) * n * 4, hipMemcpyDeviceToHost, s));
+  QTIP_HIP(hipStreamSynchronize(s));
+}
+
+// ---------------------------------------------------------------- ldl_hessian, src/quantizer.cpp:154-165
+void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L) {
+  QTIP_REQUIRE(n > 0 && n % 16 == 0 && host_HRr && host_L, "ldl_hessian: bad arguments (n = %d)", n);
+  // n x n fp64 work matrix (6.6 GB at n = 28672): taken from a process-wide pool so that repeated groups do not
+  // pay for mapping and faulting it in again
+  HostScratch A(size_t(n) * n * sizeof(double));
+  double* a = static_cast<double*>(A.get());
+  symmetrize_lower_host(host_HRr, n, a, threads);
+  if (!block_ldl_host(a, n, host_L, threads)) throw Error(QTIP_E_NOT_PD, "block LDL failed (H not PD)");
+}
+
+// ---------------------------------------------------------------- ldlq_gpu, src/quantizer.cpp:30-89
+void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, float* hatWT, uint16_t* Q, int feedback,
+               double* vit_seconds) {
+  QTIP_REQUIRE(n % 128 == 0, "LDLQ needs n %% 128 == 0 (n = %ld)", n);
+  QTIP_REQUIRE(m % 16 == 0 && m > 0, "LDLQ needs m %% 16 == 0 (m = %ld)", m);
+  QTIP_REQUIRE(feedback == 0, "feedback mode %d is not available", feedback);
+  hipStream_t s = c->stream;
+  ensure_viterbi_workspace(c);
+  const long ntr = m / 16, nblk = n / 16;
+  DBuf<double> prod(size_t(n) * m);
+  DBuf<float> X(size_t(ntr) * 256);
+  QTIP_HIP(hipMemsetAsync(prod, 0, prod.bytes(), s));
+  QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
+  std::vector<hipEvent_t> ev;
+  auto mark = [&] {
+    hipEvent_t e;
+    QTIP_HIP(hipEventCreate(&e));
+    QTIP_HIP(hipEventRecord(e, s));
+    ev.push_back(e);
+  };
+  for (long cur = nblk; cur > 0; cur -= 8) {
+    const int bufend = int(16 * cur), c0 = bufend - 128;
+    for (int i = 7; i >= 0; --i) {
+      const int col0 = c0 + 16 * i;
+      launch_ldlq_prep_f64(WT, hatWT, prod, L, n, m, col0, bufend, X, s);
+      if (vit_seconds) mark();
+      TileJob job;
+      job.X = X;
+      job.tiles = ntr;
+      job.states = Q;
+      job.q_tile_stride = nblk;
+      job.q_offset = col0 / 16;
+      job.hatWT = hatWT;
+      job.ldw = m;
+      job.col0 = col0;
+      launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws, c->vit_slots, s);
+      if (vit_seconds) mark();
+    }
+    if (c0 > 0)  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
+      launch_gemm_tn_f64_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m, prod, m, s);
+  }
+  QTIP_HIP(hipStreamSynchronize(s));
+  if (vit_seconds) {
+    double t = 0;
+    for (size_t i = 0; i + 1 < ev.size(); i += 2) {
+      float ms = 0;
+      QTIP_HIP(hipEventElapsedTime(&ms, ev[i], ev[i + 1]));
+      t += ms * 1e-3;
+    }
+    *vit_seconds = t;
+  }
+  for (auto e : ev) (void)hipEventDestroy(e);
+}
+
+// ---------------------------------------------------------------- quantize_group, src/quantizer.cpp:176-346
+void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
+                         double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
+                         qtip_linear_out* outs, qtip_timing* tm) {
+  QTIP_REQUIRE(nlin > 0 && lins && outs && host_su && host_L, "quantize_group: bad arguments");
+  QTIP_REQUIRE(n % 128 == 0, "LDLQ needs n %% 128 == 0 (n = %d)", n);
+  QTIP_REQUIRE(had_K(n) > 0 && n / had_K(n) <= 8192, "unsupported hadamard dim %d", n);
+  QTIP_REQUIRE(opt.skip_proxy || host_HRr, "quantize_group: HRr is needed for the proxy");
+  hipStream_t s = c->stream;
+  qtip_timing T{};
+  if (tm) T.rht = tm->rht, T.ldl_cpu = tm->ldl_cpu;
+  const double t_start = now_s();
+  double t0 = t_start;
+  long mt = 0, maxm = 0;
+  std::vector<long> off;
+  for (int li = 0; li < nlin; ++li) {
+    const qtip_linear_in& l = lins[li];
+    QTIP_REQUIRE(l.m > 0 && l.m % 32 == 0 && n % 32 == 0, "kernel layout needs m, n multiples of 32 (m=%d n=%d)", l.m, n);
+    QTIP_REQUIRE(had_K(l.m) > 0 && l.m / had_K(l.m) <= 8192, "unsupported hadamard dim %d", l.m);
+    QTIP_REQUIRE((l.w_f32 != nullptr) + (l.w_bf16 != nullptr) + (l.w_fp8 != nullptr) == 1,
+                 "linear %d: exactly one of w_f32 / w_bf16 / w_fp8 must be set", li);
+    QTIP_REQUIRE(outs[li].trellis && outs[li].su_bf16 && outs[li].sv, "linear %d: output buffers missing", li);
+    off.push_back(mt);
+    mt += l.m;
+    maxm = std::max<long>(maxm, l.m);
+  }
+  DBuf<float> d_su{size_t(n)}, d_sv{size_t(mt)};
+  QTIP_HIP(hipMemcpyAsync(d_su, host_su, size_t(n) * 4, hipMemcpyHostToDevice, s));
+
+  // ---- weights -> Wr^T (n x mt), each linear's column block scaled by 1/Wscale (src/quantizer.cpp:195-249)
+  DBuf<float> WT(size_t(n) * mt);
+  {
+    DBuf<float> Wt(size_t(maxm) * n);
+    DBuf<uint8_t> raw;
+    DBuf<uint16_t> sc;
+    for (int li = 0; li < nlin; ++li) {
+      const qtip_linear_in& l = lins[li];
+      qtip_linear_out& O = outs[li];
+      const long m = l.m;
+      SplitMix r2(seed * 1000003ull + uint64_t(li) + 1);
+      for (long i = 0; i < m; ++i) O.sv[i] = r2.sign();
+      for (int i = 0; i < n; ++i) O.su_bf16[i] = f32_to_bf16(host_su[i]);
+      QTIP_HIP(hipMemcpyAsync(d_sv + off[li], O.sv, size_t(m) * 4, hipMemcpyHostToDevice, s));
+      const hipMemcpyKind kind = l.on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice;
+      if (l.w_fp8) {
+        raw.ensure(size_t(m) * n);
+        QTIP_HIP(hipMemcpyAsync(raw, l.w_fp8, size_t(m) * n, kind, s));
+        if (l.scale_bf16) {
+          sc.ensure(size_t(m));
+          QTIP_HIP(hipMemcpyAsync(sc, l.scale_bf16, size_t(m) * 2, kind, s));
+        }
+        launch_fp8_to_f32(raw, l.scale_bf16 ? sc.p : nullptr, Wt, m, n, s);
+      } else if (l.w_bf16) {
+        raw.ensure(size_t(m) * n * 2);
+        QTIP_HIP(hipMemcpyAsync(raw, l.w_bf16, size_t(m) * n * 2, kind, s));
+        launch_bf16_to_f32(reinterpret_cast<const uint16_t*>(raw.p), Wt, m * n, s);
+      } else {
+        QTIP_HIP(hipMemcpyAsync(Wt, l.w_f32, size_t(m) * n * 4, kind, s));
+      }
+      QTIP_HIP(hipStreamSynchronize(s));
+      T.load += now_s() - t0;
+      t0 = now_s();
+      // Wr^T = hadUt_m( hadUt_n( diag(SV) W diag(SU) )^T )
+      c->rht.hadamard_rows(Wt, m, n, n, true, d_sv + off[li], d_su);
+      c->rht.transpose(Wt, m, n, n, WT + off[li], mt);
+      c->rht.hadamard_rows(WT + off[li], n, int(m), mt, true);
+      const double ss = c->rht.reduce(WT + off[li], mt, nullptr, 0, n, m, 0);
+      const double rms = std::sqrt(ss / (double(n) * double(m)));
+      O.wscale = float(rms / (double(float(c->cb.lut_rms)) * opt.scale_override));
+      c->rht.scale(WT + off[li], n, m, mt, 1.0f / O.wscale);
+      QTIP_HIP(hipStreamSynchronize(s));
+      T.rht += now_s() - t0;
+      t0 = now_s();
+    }
+  }
+
+  DBuf<float> Ld(size_t(n) * n);
+  QTIP_HIP(hipMemcpyAsync(Ld, host_L, size_t(n) * n * 4, hipMemcpyHostToDevice, s));
+  QTIP_HIP(hipStreamSynchronize(s));
+  T.load += now_s() - t0;
+  t0 = now_s();
+
+  // ---- LDLQ + Viterbi
+  DBuf<float> hatWT(size_t(n) * mt);
+  DBuf<uint16_t> Q(size_t(mt / 16) * (n / 16) * 128);
+  double vit = 0;
+  ldlq_impl(c, WT, Ld, n, mt, hatWT, Q, opt.feedback, &vit);
+  T.ldlq += now_s() - t0;
+  T.viterbi += vit;
+  t0 = now_s();
+  Ld.release();
+
+  // ---- proxy (rotated, scaled domain; Wscale cancels), src/quantizer.cpp:268-303
+  if (!opt.skip_proxy) {
+    DBuf<float> HR(size_t(n) * n);
+    QTIP_HIP(hipMemcpyAsync(HR, host_HRr, HR.bytes(), hipMemcpyHostToDevice, s));
+    for (int li = 0; li < nlin; ++li) {
+      const long m = lins[li].m;
+      const double den = quad_trace_f64(n, int(m), HR, WT + off[li], nullptr, mt, c->scratch, s);
+      const double num = quad_trace_f64(n, int(m), HR, WT + off[li], hatWT + off[li], mt, c->scratch, s);
+      const double wn2 = c->rht.reduce(WT + off[li], mt, nullptr, 0, n, m, 0);
+      const double dn2 = c->rht.reduce(WT + off[li], mt, hatWT + off[li], mt, n, m, 2);
+      outs[li].proxy_rot_reg = num / den;
+      outs[li].proxy = (num - creg * dn2) / (den - creg * wn2);
+    }
+  } else {
+    for (int li = 0; li < nlin; ++li) outs[li].proxy = outs[li].proxy_rot_reg = 0;
+  }
+  QTIP_HIP(hipStreamSynchronize(s));
+  T.proxy += now_s() - t0;
+  t0 = now_s();
+
+  // ---- states -> packed trellis in kernel layout, src/quantizer.cpp:305-320 (packed on the device)
+  {
+    const long nblk = n / 16;
+    DBuf<uint16_t> tr(size_t(mt / 16) * nblk * 32);
+    for (int li = 0; li < nlin; ++li) {
+      const long m = lins[li].m;
+      const size_t tile0 = size_t(off[li] / 16) * nblk;
+      launch_pack_swizzle(Q + tile0 * 128, m, n, tr + tile0 * 32, s);
+      QTIP_HIP(hipMemcpyAsync(outs[li].trellis, tr + tile0 * 32, size_t(m / 16) * nblk * 32 * 2, hipMemcpyDeviceToHost, s));
+    }
+    QTIP_HIP(hipStreamSynchronize(s));
+  }
+  // ---- optional reconstruction in the original domain, src/quantizer.cpp:321-338:
+  //      hatW = diag(SV) U_m (hatWr * Wscale) U_n^T diag(SU)
+  for (int li = 0; li < nlin; ++li) {
+    if (!outs[li].hatW) continue;
+    const long m = lins[li].m;
+    DBuf<float> a(size_t(n) * m), b(size_t(m) * n);
+    QTIP_HIP(hipMemcpy2DAsync(a, size_t(m) * 4, hatWT + off[li], size_t(mt) * 4, size_t(m) * 4, size_t(n),
+                              hipMemcpyDeviceToDevice, s));
+    c->rht.hadamard_rows(a, n, int(m), m, false);
+    c->rht.transpose(a, n, m, m, b, n);
+    c->rht.hadamard_rows(b, m, n, n, false);
+    c->rht.scale(b, m, n, n, outs[li].wscale);
+    launch_scale_rc(b, m, n, n, d_sv + off[li], d_su, s);
+    QTIP_HIP(hipMemcpyAsync(outs[li].hatW, b, size_t(m) * n * 4, hipMemcpyDeviceToHost, s));
+    QTIP_HIP(hipStreamSynchronize(s));
+  }
+  T.pack += now_s() - t0;
+  T.total = (now_s() - t_start) + (tm ? tm->rht : 0.0) + T.ldl_cpu;
+  double wsum = 0;
+  for (int li = 0; li < nlin; ++li) wsum += double(lins[li].m) * n;
+  for (int li = 0; li < nlin; ++li) outs[li].seconds = T.total * double(lins[li].m) * n / wsum;
+  if (tm) *tm = T;
+}
+
+}  // namespace qtipmi

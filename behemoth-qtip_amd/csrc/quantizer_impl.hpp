@@ -1,3 +1,30 @@
-// group quantizer internals (filled in by quantizer_impl.cpp)
+// The context behind the C ABI and the group-quantizer entry points implemented in quantizer_impl.cpp.
 #pragma once
+#include "ldlq.hpp"
+#include "misc.hpp"
 #include "qtip_internal.hpp"
+#include "rht.hpp"
+
+struct qtip_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  qtipmi::HostCodebook cb;
+  qtipmi::DBuf<double> d_entry_d;  // [1024][2] decoded codebook entries, fp64
+  qtipmi::DBuf<float> d_entry_f;   // [1024][2] the same as fp32
+  qtipmi::DBuf<unsigned char> vit_ws;  // back-pointer slots of the resident Viterbi workgroups
+  int vit_slots = 0;
+  qtipmi::Rht rht;
+  qtipmi::DBuf<double> scratch;
+};
+
+namespace qtipmi {
+void ensure_viterbi_workspace(qtip_ctx* c);
+void rotate_hessian_impl(qtip_ctx* c, const float* H, bool on_device, int n, uint64_t seed, double sigma_reg,
+                         float* host_su, double* creg, float* host_HRr);
+void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L);
+void ldlq_impl(qtip_ctx* c, const float* dWT, const float* dL, long n, long m, float* d_hatWT, uint16_t* dQ,
+               int feedback, double* vit_seconds);
+void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
+                         double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
+                         qtip_linear_out* outs, qtip_timing* tm);
+}  // namespace qtipmi
