@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Benchmark of the QTIP per-Hessian-group quantize path on one MI355X.
+
+A step is one pass of the hot path over one synthetic group: Hessian rotation (GPU), fp64 block LDL (host),
+weight RHT + Wscale, LDLQ with the two-pass Viterbi, packing to the kernel-layout trellis.  Default workload:
+BASELINE configuration 5, the 12288 x 28672 down-proj group.  The K timed steps are K groups handled the way the
+reference's scheduler handles consecutive groups (src/pipeline.cpp:254-290): all Hessians are rotated first, a
+side thread factors them in order, and the GPU quantizes group k as soon as its factor is ready, so the host
+LDL of group k+1 overlaps the GPU work of group k.  Nothing is precomputed outside the timed region.
+
+Prints ONE JSON line (see the keys below).  `value` is weights quantized per second over the whole timed region.
+"""
+import argparse
+import json
+import os
+import sys
+import threading
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FLOP_PER_WEIGHT = 393216.0      # 2^16 add-compare-selects per weight, 6 flop each (survey figure for the Viterbi)
+PEAK_FP64_TFLOPS = 78.6         # MI355X vector fp64
+
+
+def load_pkg():
+    from __graft_entry__ import _pkg
+    return _pkg()
+
+
+def load_synth():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("qtip_synth", os.path.join(ROOT, "behemoth-qtip_amd", "synth.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def cpu_baseline(seconds_budget=15.0, threads=16):
+    """Reference CPU Viterbi (oracle/_ref when present, else the oracle port) on a bounded sample of tiles."""
+    import concurrent.futures as cf
+    import numpy as np
+    from oracle import binding as ob
+    R = ob.ref_lib()
+    kind = "reference" if R is not None else "port"
+    cb = ob.Codebook()
+    X = ob.rng_normal(77, 4096 * 256).astype(np.float32).astype(np.float16).astype(np.float32).reshape(4096, 256)
+    done = [0]
+    lock = threading.Lock()
+    deadline = time.time() + seconds_budget
+
+    def work(lo):
+        st = np.zeros(128, np.uint16)
+        hat = np.zeros(256, np.float32)
+        n = 0
+        for b in range(lo, 4096, threads):
+            if time.time() > deadline:
+                break
+            if R is not None:
+                R.ref_quantize_seq(X[b], st, hat)
+            else:
+                ob.lib().qo_quantize_seq(cb.lut0, cb.lut1, X[b], st, hat)
+            n += 1
+        with lock:
+            done[0] += n
+
+    t0 = time.time()
+    with cf.ThreadPoolExecutor(threads) as ex:
+        list(ex.map(work, range(threads)))
+    dt = time.time() - t0
+    return {"value": done[0] * 256 / dt / 1e6, "unit": "Mweights/s", "cores": threads, "kind": kind,
+            "sample": "%d tiles of 256 fp16-rounded N(0,1) weights, two-pass Viterbi only (the dominant stage), "
+                      "%.1f s on %d threads" % (done[0], dt, threads)}
+
+
+def run_viterbi_only(args, pkg):
+    """Configuration 1: 4096 independent tiles, Viterbi only."""
+    import numpy as np
+    import torch
+    from oracle import binding as ob
+    q = pkg.Quantizer(0, tlut=ob.synthetic_tlut(1))
+    X = torch.from_numpy(ob.rng_normal(1234, 4096 * 256).astype(np.float32).reshape(4096, 256)).cuda()
+    S = torch.zeros((4096, 128), dtype=torch.int16, device="cuda")
+    P = torch.zeros((4096, 32), dtype=torch.int16, device="cuda")
+    for _ in range(args.warmup):
+        q.viterbi_tiles_dev(X, 4096, S, P)
+    q.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.time()
+    for _ in range(args.steps):
+        q.viterbi_tiles_dev(X, 4096, S, P)
+    q.synchronize()
+    torch.cuda.synchronize()
+    dt = time.time() - t0
+    weights = 4096 * 256 * args.steps
+    per_launch = dt / args.steps
+    return dict(weights=weights, wall=dt, vit_launch_s=per_launch, vit_launch_weights=4096 * 256,
+                workload="config1: 4096 independent 16x16 tiles, Viterbi only", extra={})
+
+
+def run_group(args, pkg):
+    import numpy as np
+    import torch
+    synth = load_synth()
+    q = pkg.Quantizer(0)
+    cfg = args.config
+    if cfg == 2:
+        Ws_h, H_h = synth.config2()
+        Ws = [torch.from_numpy(w).cuda() for w in Ws_h]
+        H = torch.from_numpy(H_h).cuda()
+    else:
+        Ws, H = synth.large_config(cfg)
+    n = H.shape[0]
+    ms = [int(w.shape[0]) for w in Ws]
+    lins = [pkg.LinearIn("w%d" % i, m, w_f32=w) for i, (m, w) in enumerate(zip(ms, Ws))]
+    opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=True)
+    weights_per_step = sum(ms) * n
+
+    def pinned(shape):
+        return torch.empty(shape, dtype=torch.float32, pin_memory=True).numpy()
+
+    nbuf = max(args.steps, args.warmup, 1)
+    su = [np.zeros(n, np.float32) for _ in range(nbuf)]
+    HRr = [pinned((n, n)) for _ in range(nbuf)]
+    Lb = [pinned((n, n)) for _ in range(nbuf)]
+    stats = {}
+
+    def run_steps(K, record):
+        """K groups, pipelined like consecutive groups of a layer: rotate all, LDL on a side thread, quantize in order."""
+        import ctypes as C
+        L = pkg.lib()
+        creg = [C.c_double() for _ in range(K)]
+        ready = [threading.Event() for _ in range(K)]
+        ldl_t = [0.0] * K
+        err = []
+        t_rot0 = time.time()
+        for k in range(K):
+            rc = L.qtip_rotate_hessian(q._h, H.data_ptr(), 1, n, 3 + k, opt.sigma_reg, su[k].ctypes.data,
+                                       C.byref(creg[k]), HRr[k].ctypes.data)
+            if rc:
+                raise RuntimeError(L.qtip_last_error())
+        t_rot = time.time() - t_rot0
+
+        def ldl_side():
+            for k in range(K):
+                t0 = time.time()
+                rc = L.qtip_ldl_hessian(HRr[k].ctypes.data, n, args.ldl_threads, Lb[k].ctypes.data)
+                ldl_t[k] = time.time() - t0
+                if rc:
+                    err.append(L.qtip_last_error())
+                ready[k].set()
+
+        th = threading.Thread(target=ldl_side)
+        th.start()
+        tms, waits = [], []
+        for k in range(K):
+            t0 = time.time()
+            ready[k].wait()
+            waits.append(time.time() - t0)
+            if err:
+                raise RuntimeError(err[0])
+            hp = pkg.HessPrep(n=n, seed=3 + k, su=su[k], creg=creg[k].value, HRr=HRr[k], L=Lb[k])
+            outs, tm = q.quantize_group(lins, hp, opt)
+            tms.append(tm)
+        th.join()
+        if record:
+            stats.update(rot_s=t_rot / K, ldl_s=sum(ldl_t) / K, ldl_wait_s=sum(waits) / K,
+                         ldlq_s=sum(t.ldlq for t in tms) / K, viterbi_s=sum(t.viterbi for t in tms) / K,
+                         rht_w_s=sum(t.rht for t in tms) / K, load_s=sum(t.load for t in tms) / K,
+                         pack_s=sum(t.pack for t in tms) / K, wscale=float(outs[0].wscale))
+
+    if args.warmup > 0:
+        run_steps(args.warmup, False)
+    q.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.time()
+    run_steps(args.steps, True)
+    q.synchronize()
+    torch.cuda.synchronize()
+    wall = time.time() - t0
+    ntr = sum(ms) // 16
+    launches = n // 16
+    gpu_s = stats["rot_s"] + stats["rht_w_s"] + stats["load_s"] + stats["ldlq_s"] + stats["pack_s"]
+    extra = dict(stats)
+    extra.update(gpu_only_Mweights_s=weights_per_step / gpu_s / 1e6,
+                 serial_Mweights_s=weights_per_step / (gpu_s + stats["ldl_s"]) / 1e6,
+                 viterbi_only_Mweights_s=weights_per_step / stats["viterbi_s"] / 1e6,
+                 proxy_in_timed_region=False, ldl_threads=args.ldl_threads)
+    names = {2: "config2: 1024x1024 group", 3: "config3: 12288x12288 q-proj group",
+             4: "config4: gate+up 2x(28672x12288) group", 5: "config5: 12288x28672 down-proj group"}
+    return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
+                vit_launch_weights=ntr * 256, workload=names[cfg] + " (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)",
+                extra=extra)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--config", type=int, default=5, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--ldl-threads", type=int, default=16)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="first run one plain 1 GiB device copy kernel (known traffic, scales the rocprof byte counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (every tile row is independent, "
+              "see DESIGN.md for how the path would shard)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    pkg = load_pkg()
+    if args.pmc_calibration:
+        a = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        b = torch.empty_like(a)
+        torch.cuda.synchronize()
+        b.copy_(a)          # 1 GiB read + 1 GiB written by one elementwise kernel
+        torch.cuda.synchronize()
+        del a, b
+    res = run_viterbi_only(args, pkg) if args.config == 1 else run_group(args, pkg)
+    value = res["weights"] / res["wall"] / 1e6
+    achieved = res["vit_launch_weights"] * FLOP_PER_WEIGHT / res["vit_launch_s"] / 1e12
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "viterbi_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("config%d_bytes_per_launch" % args.config)
+        except Exception:
+            traffic = None
+    out = {
+        "metric": "Mweights/s quantized (RHT+LDLQ+2-pass Viterbi) 12288x28672; % VALU/LDS peak",
+        "value": value, "unit": "Mweights/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": res["wall"] / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": dict({"workload": res["workload"]}, **res["extra"]),
+        "roofline": {"bound": "valu", "kernel": "viterbi_tiles_kernel", "achieved": achieved, "peak": PEAK_FP64_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_FP64_TFLOPS, "traffic": traffic,
+                     "launch_ms": res["vit_launch_s"] * 1e3, "weights_per_launch": res["vit_launch_weights"],
+                     "flop_per_weight": FLOP_PER_WEIGHT},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(threads=min(16, os.cpu_count() or 1))
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
