@@ -1,0 +1,186 @@
+// C++ shim with the reference's own interface for the group quantizer (src/quantizer.hpp:11-78 of the
+// reference: same names, argument meaning and abort-on-error behaviour), implemented on the C ABI of
+// libqtip_mi355.so.  A caller such as run_qtip_groups (src/pipeline.cpp:229-312) compiles against this header
+// instead of the reference's quantizer.hpp and links libqtip_mi355.so instead of quantizer.cpp + its kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/qtip_mi355.h"
+
+namespace qtip {
+
+// The reference passes its hipBLASLt wrapper through these calls; the MFMA contractions live inside the
+// library here, so the type only keeps the signatures source-compatible.
+class Gemm {
+ public:
+  Gemm() = default;
+  explicit Gemm(hipStream_t) {}
+};
+
+struct QuantOpts {  // src/quantizer.hpp:11-19
+  double sigma_reg = 1e-2;
+  double scale_override = 0.9;
+  int vit_batch = 1024;  // accepted, unused: the tile kernel sizes its own back-pointer workspace
+  int ldl_threads = 16;
+  bool share_su = true;
+  std::string dump_dir;  // not supported by the shim (must stay empty)
+  bool want_hatW = false;
+};
+
+struct LinearIn {  // src/quantizer.hpp:21-28
+  std::string name;
+  int m = 0;
+  const uint8_t* w_fp8 = nullptr;
+  const uint16_t* scale_bf16 = nullptr;
+  const uint16_t* w_bf16 = nullptr;
+  const float* w_f32 = nullptr;
+};
+
+struct LinearOut {  // src/quantizer.hpp:30-43
+  std::string name;
+  int m = 0, n = 0;
+  std::vector<uint16_t> trellis;
+  std::vector<uint16_t> su_bf16;
+  std::vector<float> sv;
+  float wscale = 0;
+  double proxy = 0;
+  double proxy_rot_reg = 0;
+  double seconds = 0;
+  std::vector<float> hatW;
+};
+
+struct GroupTiming {  // src/quantizer.hpp:45-47
+  double load = 0, rht = 0, ldl_cpu = 0, ldlq = 0, viterbi = 0, proxy = 0, pack = 0, total = 0;
+};
+
+struct HessPrep {  // src/quantizer.hpp:51-59
+  int n = 0;
+  uint64_t seed = 0;
+  std::vector<float> su;
+  double creg = 0;
+  std::vector<float> HRr;
+  std::vector<float> L;
+  double t_rot = 0, t_ldl = 0;
+};
+
+namespace detail {
+[[noreturn]] inline void die(const std::string& msg) {  // src/common.hpp:24-28
+  std::fprintf(stderr, "fatal: %s\n", msg.c_str());
+  std::fflush(stderr);
+  std::abort();
+}
+inline void check(int rc, const char* what) {
+  if (rc != QTIP_OK) die(std::string(what) + ": " + qtip_last_error());
+}
+inline double now_s() {
+  using namespace std::chrono;
+  return duration<double>(steady_clock::now().time_since_epoch()).count();
+}
+// one context per device, created on first use by the worker thread that has made the device current
+inline qtip_ctx* context() {
+  static std::mutex mu;
+  static std::map<int, qtip_ctx*> cache;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) die("hipGetDevice failed");
+  std::lock_guard<std::mutex> lk(mu);
+  auto it = cache.find(dev);
+  if (it != cache.end()) return it->second;
+  qtip_ctx* c = nullptr;
+  check(qtip_create(dev, &c), "qtip_create");
+  cache[dev] = c;
+  return c;
+}
+}  // namespace detail
+
+inline void rotate_hessian(hipStream_t, const float* H, int n, uint64_t seed, const QuantOpts& opt, HessPrep& hp) {
+  const double t0 = detail::now_s();
+  hp.n = n;
+  hp.seed = seed;
+  hp.su.resize(size_t(n));
+  hp.HRr.resize(size_t(n) * n);
+  detail::check(qtip_rotate_hessian(detail::context(), H, 0, n, seed, opt.sigma_reg, hp.su.data(), &hp.creg,
+                                    hp.HRr.data()),
+                "rotate_hessian");
+  hp.t_rot = detail::now_s() - t0;
+}
+
+inline void ldl_hessian(HessPrep& hp, int threads, const std::string& tag) {
+  const double t0 = detail::now_s();
+  hp.L.resize(size_t(hp.n) * hp.n);
+  const int rc = qtip_ldl_hessian(hp.HRr.data(), hp.n, threads, hp.L.data());
+  if (rc != QTIP_OK) detail::die("block LDL failed (H not PD) for " + tag + ": " + qtip_last_error());
+  hp.t_ldl = detail::now_s() - t0;
+}
+
+inline std::vector<LinearOut> quantize_group(hipStream_t, Gemm&, const std::vector<LinearIn>& lins, HessPrep& hp,
+                                             const QuantOpts& opt, GroupTiming* tm, const std::string& tag) {
+  if (!opt.share_su) detail::die("share_su=false not supported (one LDL per group)");
+  if (!opt.dump_dir.empty()) detail::die("dump_dir is not supported by this build (" + tag + ")");
+  const int n = hp.n;
+  std::vector<qtip_linear_in> cin(lins.size());
+  std::vector<qtip_linear_out> cout(lins.size());
+  std::vector<LinearOut> out(lins.size());
+  for (size_t i = 0; i < lins.size(); ++i) {
+    const LinearIn& l = lins[i];
+    cin[i] = qtip_linear_in{l.m, l.w_f32, l.w_bf16, l.w_fp8, l.scale_bf16, 0};
+    LinearOut& o = out[i];
+    o.name = l.name, o.m = l.m, o.n = n;
+    if (l.m <= 0 || l.m % 16 || n % 16) detail::die("bad linear shape for " + tag);
+    o.trellis.resize(size_t(l.m / 16) * (n / 16) * 32);
+    o.su_bf16.resize(size_t(n));
+    o.sv.resize(size_t(l.m));
+    if (opt.want_hatW) o.hatW.resize(size_t(l.m) * n);
+    cout[i] = qtip_linear_out{o.trellis.data(), o.su_bf16.data(), o.sv.data(), opt.want_hatW ? o.hatW.data() : nullptr,
+                              0.f, 0.0, 0.0, 0.0};
+  }
+  qtip_opts co;
+  qtip_default_opts(&co);
+  co.sigma_reg = opt.sigma_reg, co.scale_override = opt.scale_override, co.ldl_threads = opt.ldl_threads;
+  qtip_timing ct{};
+  ct.rht = hp.t_rot, ct.ldl_cpu = hp.t_ldl;
+  detail::check(qtip_quantize_group(detail::context(), int(lins.size()), cin.data(), n, hp.seed, hp.su.data(), hp.creg,
+                                    hp.HRr.data(), hp.L.data(), &co, cout.data(), &ct),
+                ("quantize_group " + tag).c_str());
+  hp.L.clear();  // consumed, as in the reference (src/quantizer.cpp:256-257)
+  hp.L.shrink_to_fit();
+  for (size_t i = 0; i < lins.size(); ++i) {
+    out[i].wscale = cout[i].wscale, out[i].proxy = cout[i].proxy;
+    out[i].proxy_rot_reg = cout[i].proxy_rot_reg, out[i].seconds = cout[i].seconds;
+  }
+  if (tm) *tm = GroupTiming{ct.load, ct.rht, ct.ldl_cpu, ct.ldlq, ct.viterbi, ct.proxy, ct.pack, ct.total};
+  return out;
+}
+
+inline std::vector<LinearOut> quantize_group(hipStream_t s, Gemm& gemm, const std::vector<LinearIn>& lins, int n,
+                                             const float* H, uint64_t seed, const QuantOpts& opt, GroupTiming* tm,
+                                             const std::string& tag) {
+  HessPrep hp;
+  rotate_hessian(s, H, n, seed, opt, hp);
+  ldl_hessian(hp, opt.ldl_threads, tag);
+  return quantize_group(s, gemm, lins, hp, opt, tm, tag);
+}
+
+// WT n x m, L n x n, hatWT n x m, Q on the device (src/quantizer.hpp:70-73); vit_batch and the LUT pointer are
+// accepted for source compatibility (the library holds its own codebook tables).
+inline void ldlq_gpu(hipStream_t, Gemm&, const float* WT, const float* L, long n, long m, float* hatWT, uint16_t* Q,
+                     int /*vit_batch*/, const uint32_t* /*lut_h2_dev*/, double* vit_s) {
+  detail::check(qtip_ldlq_dev(detail::context(), WT, L, n, m, hatWT, Q, vit_s), "ldlq_gpu");
+}
+
+// The reference returns its device half2 LUT; the library keeps its tables private, so this only makes sure the
+// context (and with it the tables) exists on the current device.
+inline const uint32_t* device_lut() {
+  (void)detail::context();
+  return nullptr;
+}
+
+}  // namespace qtip

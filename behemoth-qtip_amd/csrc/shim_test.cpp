@@ -1,0 +1,65 @@
+// Exercises the C++ shim the way the reference's own GPU test drives quantize_group
+// (tests/test_gpu.cpp:301-372): two linears sharing one Hessian, then a CPU decode of the packed output.
+// Prints one line per linear; exit code 0 on success.  Built by the Makefile as qtip_shim_test.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "quantizer.hpp"
+
+using namespace qtip;
+
+int main() {
+  if (hipSetDevice(0) != hipSuccess) {
+    std::fprintf(stderr, "no GPU\n");
+    return 2;
+  }
+  hipStream_t S;
+  if (hipStreamCreate(&S) != hipSuccess) return 2;
+  Gemm g(S);
+  const int n = 256;
+  std::mt19937_64 rng(33);
+  std::normal_distribution<double> N01(0.0, 1.0);
+  std::vector<float> W1(size_t(64) * n), W2(size_t(32) * n), H(size_t(n) * n);
+  for (auto& v : W1) v = float(N01(rng) * 0.02);
+  for (auto& v : W2) v = float(N01(rng) * 0.05);
+  std::vector<double> G(size_t(n) * 3 * n);
+  for (auto& x : G) x = N01(rng);
+  for (int i = 0; i < n; ++i)
+    for (int j = 0; j <= i; ++j) {
+      double s = 0;
+      for (int p = 0; p < 3 * n; ++p) s += G[size_t(i) * 3 * n + p] * G[size_t(j) * 3 * n + p];
+      H[size_t(i) * n + j] = H[size_t(j) * n + i] = float(s / (3 * n));
+    }
+  std::vector<LinearIn> lins(2);
+  lins[0].name = "a", lins[0].m = 64, lins[0].w_f32 = W1.data();
+  lins[1].name = "b", lins[1].m = 32, lins[1].w_f32 = W2.data();
+  QuantOpts o;
+  o.ldl_threads = 4;
+  o.want_hatW = true;
+  GroupTiming tm;
+  auto out = quantize_group(S, g, lins, n, H.data(), 7, o, &tm, "shim_test");
+  int fail = 0;
+  for (size_t li = 0; li < out.size(); ++li) {
+    const LinearOut& lo = out[li];
+    const std::vector<float>& W = li == 0 ? W1 : W2;
+    // proxy of the returned reconstruction with the unregularised H, in fp64 on the host
+    double num = 0, den = 0;
+    for (int i = 0; i < lo.m; ++i) {
+      std::vector<double> d(n), w(n);
+      for (int j = 0; j < n; ++j) d[j] = double(W[size_t(i) * n + j]) - lo.hatW[size_t(i) * n + j], w[j] = W[size_t(i) * n + j];
+      for (int a = 0; a < n; ++a)
+        for (int b = 0; b < n; ++b) num += d[a] * H[size_t(a) * n + b] * d[b], den += w[a] * H[size_t(a) * n + b] * w[b];
+    }
+    const double p = num / den;
+    std::printf("%s: proxy %.6f host-recomputed %.6f proxy_rot_reg %.6f wscale %.6f words %zu\n", lo.name.c_str(),
+                lo.proxy, p, lo.proxy_rot_reg, lo.wscale, lo.trellis.size());
+    if (!(lo.proxy > 0 && lo.proxy < 0.2)) ++fail;
+    if (std::fabs(p - lo.proxy) / lo.proxy > 1e-3) ++fail;
+    if (lo.trellis.size() != size_t(lo.m / 16) * (n / 16) * 32) ++fail;
+  }
+  std::printf(fail ? "SHIM TEST FAILED\n" : "SHIM TEST PASSED\n");
+  return fail ? 1 : 0;
+}
