@@ -25,10 +25,12 @@
 namespace qtipmi {
 namespace {
 
+#include "data/viterbi_layout.h"
+
 constexpr int kThreads = 256;
-constexpr int kRowStride = 33;                   // doubles per E row: 2 x 16 entries + 1 pad
-constexpr int kESlots = 64 * kRowStride;         // 2112
-constexpr int kMSlots = 256 * 16 + 32;           // 4128: column c at c*16 + (c >> 3)
+constexpr int kRowStride = QTIP_VIT_ROW_STRIDE;  // doubles per E row: 2 x 16 entries + padding
+constexpr int kESlots = 64 * kRowStride + (kRowStride - 32);
+constexpr int kMSlots = 256 * 17;                // metric of (column c, digit d) at c*17 + d
 constexpr int kBpWordsPerTile = 127 * kThreads;  // u64 words
 
 struct Smem {
@@ -61,39 +63,36 @@ __device__ __forceinline__ uint32_t bp_lookup(const unsigned long long* step_wor
 // is left in sm.final_state.
 __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict__ entry_d, int roll, int ov,
                                              unsigned long long* __restrict__ bp, int bp_first) {
-  const int u = threadIdx.x;
+  const int tid = threadIdx.x;
+  const int u = kOctetOfLane[tid];  // which octet of groups this lane owns (placement tuned against LDS bank conflicts)
   const double INF = __builtin_inf();
 
-  // this thread's 4 codebook entries for the per-step error table: e = u + 256*q -> row u & 63, k = (u >> 6) + 4q
-  double l0[4], l1[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    l0[q] = entry_d[2 * (u + 256 * q)];
-    l1[q] = entry_d[2 * (u + 256 * q) + 1];
-  }
-  const int e_wr = (u & 63) * kRowStride + (u >> 6);
+  // this thread's 4 codebook entries for the per-step error table: e = tid + 256*q -> row tid & 63, k = (tid >> 6) + 4q
+  // (re-read from the 16 KB global table every step: it stays in the CU's vector L1 and the registers are needed)
+  const double2* __restrict__ entries = reinterpret_cast<const double2*>(entry_d) + tid;
+  const int e_wr = (tid & 63) * kRowStride + kRowPad[tid & 63] + (tid >> 6);
 
   // per-pair E row base (in doubles): row * stride + b4
   int ebase[8];
 #pragma unroll
   for (int m = 0; m < 8; ++m) {
     const uint32_t j = 8u * u + m, p = j * (j + 1u);
-    ebase[m] = int((p >> 6) & 63u) * kRowStride + int((p >> 12) & 15u);
+    const int row = int((p >> 6) & 63u);
+    ebase[m] = row * kRowStride + kRowPad[row] + int((p >> 12) & 15u);
   }
   const int colA = u >> 1, colB = 255 - colA;
-  const int rA = colA * 16 + (colA >> 3), rB = colB * 16 + (colB >> 3);
-  const int wA = 128 * (u & 31) + (u >> 5) + (u & 31);
-  const int wB = (255 - 8 * (u & 31)) * 16 + 15 - (u >> 5) + 31 - (u & 31);
+  const int rA = colA * 17, rB = colB * 17;
+  const int wA = 136 * (u & 31) + (u >> 5);                    // slot of group 8u + m: wA + 17 m
+  const int wB = (255 - 8 * (u & 31)) * 17 + 15 - (u >> 5);    // slot of group 4095 - 8u - m: wB - 17 m
 
   // initial metrics: M_0[g] = 0, or +inf outside group ov
-  for (int g = u; g < kGroups; g += kThreads) {
+  for (int g = tid; g < kGroups; g += kThreads) {
     const int col = g & 255, d = g >> 8;
-    sm.M[col * 16 + d + (col >> 3)] = (ov < 0 || g == ov) ? 0.0 : INF;
+    sm.M[col * 17 + d] = (ov < 0 || g == ov) ? 0.0 : INF;
   }
   __syncthreads();
 
-  double bestc = INF;
-  uint32_t bests = 0xffffffffu;
+  unsigned long long word = 0;
   for (int it = 0; it < kSteps; ++it) {
     // ---- phase R: metric columns -> registers, error table of this step -> LDS
     double MA[16], MB[16];
@@ -107,7 +106,8 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
       const double x0 = double(sm.x[t]), x1 = double(sm.x[t + 1]);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const double a = l0[q] - x0, b = l1[q] - x1;
+        const double2 l = entries[256 * q];
+        const double a = l.x - x0, b = l.y - x1;
         const double err = __builtin_fma(a, a, b * b);
         sm.E[e_wr + 4 * q] = err;
         sm.E[e_wr + 4 * q + 16] = err;
@@ -115,8 +115,7 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
     }
     __syncthreads();
     // ---- phase C: 16 groups x 16 candidates
-    unsigned long long word = 0;
-    const bool last = it == kSteps - 1;
+    word = 0;
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
       const int g = 2 * m + 1;
@@ -130,45 +129,55 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
       for (int d = 1; d < 16; ++d) {
         const double ca = e[d] + MA[d];
         const double cb = e[15 - d] + MB[d];
-        if (ca < ba) ba = ca, da = d;
-        if (cb < bb) bb = cb, db = d;
+        da = ca < ba ? uint32_t(d) : da;  // strict: the first minimum in ascending d wins ties
+        db = cb < bb ? uint32_t(d) : db;
+        ba = __builtin_fmin(ba, ca);
+        bb = __builtin_fmin(bb, cb);
       }
-      sm.M[wA + 16 * m] = ba;
-      sm.M[wB - 16 * m] = bb;
+      sm.M[wA + 17 * m] = ba;
+      sm.M[wB - 17 * m] = bb;
       word |= (unsigned long long)(da) << (4 * m);
       word |= (unsigned long long)(db) << (32 + 4 * m);
-      if (last) {  // candidates for the final state: smallest metric, then smallest state
-        const uint32_t ja = 8u * u + m, jb = 4095u - ja;
-        const uint32_t sa = (da << 12) | ja, sb = (db << 12) | jb;
-        if (ov < 0) {
-          if (ba < bestc || (ba == bestc && sa < bests)) bestc = ba, bests = sa;
-          if (bb < bestc || (bb == bestc && sb < bests)) bestc = bb, bests = sb;
-        } else {
-          if (int(ja) == ov) sm.final_state = sa;
-          if (int(jb) == ov) sm.final_state = sb;
-        }
-      }
+      __builtin_amdgcn_sched_barrier(0);  // keep one row of the error table in flight at a time (register budget)
     }
     if (it >= bp_first && it < kSteps - 1)
       __hip_atomic_store(bp + size_t(it) * kThreads + u, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
   }
+  // final state: smallest metric, then smallest state, over the metrics of the last step (each lane re-reads the
+  // 16 values it has just written; their predecessor digits are the nibbles of the last back-pointer word)
   if (ov < 0) {
-    // lexicographic (metric, state) minimum over the workgroup
+    double bestc = INF;
+    uint32_t bests = 0xffffffffu;
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+      const uint32_t ja = 8u * u + m, jb = 4095u - ja;
+      const uint32_t sa = (uint32_t(word >> (4 * m)) & 15u) << 12 | ja;
+      const uint32_t sb = (uint32_t(word >> (32 + 4 * m)) & 15u) << 12 | jb;
+      const double ca = sm.M[wA + 17 * m], cb = sm.M[wB - 17 * m];
+      if (ca < bestc || (ca == bestc && sa < bests)) bestc = ca, bests = sa;
+      if (cb < bestc || (cb == bestc && sb < bests)) bestc = cb, bests = sb;
+    }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
       const double oc = __shfl_xor(bestc, off, 64);
       const uint32_t os = __shfl_xor(bests, off, 64);
       if (oc < bestc || (oc == bestc && os < bests)) bestc = oc, bests = os;
     }
-    if ((u & 63) == 0) sm.red_c[u >> 6] = bestc, sm.red_s[u >> 6] = bests;
+    if ((tid & 63) == 0) sm.red_c[tid >> 6] = bestc, sm.red_s[tid >> 6] = bests;
     __syncthreads();
-    if (u == 0) {
+    if (tid == 0) {
       double c = sm.red_c[0];
       uint32_t s = sm.red_s[0];
       for (int w = 1; w < 4; ++w)
         if (sm.red_c[w] < c || (sm.red_c[w] == c && sm.red_s[w] < s)) c = sm.red_c[w], s = sm.red_s[w];
       sm.final_state = s;
+    }
+  } else {
+    const uint32_t j = uint32_t(ov), jj = j < 2048u ? j : 4095u - j;
+    if (jj >> 3 == uint32_t(u)) {
+      const uint32_t shift = (jj & 7u) * 4u + (j < 2048u ? 0u : 32u);
+      sm.final_state = (uint32_t(word >> shift) & 15u) << 12 | j;
     }
   }
   __syncthreads();
