@@ -65,6 +65,16 @@ struct HostScratch {
   void* get() const { return p; }
 };
 
+// Waits for the stream without spinning on a core: the host LDL of the next group runs on all cores meanwhile.
+void wait_stream_sleeping(hipStream_t s) {
+  hipEvent_t e;
+  QTIP_HIP(hipEventCreateWithFlags(&e, hipEventBlockingSync | hipEventDisableTiming));
+  hipError_t rc = hipEventRecord(e, s);
+  if (rc == hipSuccess) rc = hipEventSynchronize(e);
+  (void)hipEventDestroy(e);
+  QTIP_HIP(rc);
+}
+
 double now_s() {
   using namespace std::chrono;
   return duration<double>(steady_clock::now().time_since_epoch()).count();
@@ -102,7 +112,9 @@ void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L) 
   // pay for mapping and faulting it in again
   HostScratch A(size_t(n) * n * sizeof(double));
   double* a = static_cast<double*>(A.get());
+  const double ts0 = now_s();
   symmetrize_lower_host(host_HRr, n, a, threads);
+  if (getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "ldl_hessian: symmetrize %.3f\n", now_s() - ts0);
   if (!block_ldl_host(a, n, host_L, threads)) throw Error(QTIP_E_NOT_PD, "block LDL failed (H not PD)");
 }
 
@@ -147,7 +159,7 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
     if (c0 > 0)  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
       launch_gemm_tn_f64_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m, prod, m, s);
   }
-  QTIP_HIP(hipStreamSynchronize(s));
+  wait_stream_sleeping(s);
   if (vit_seconds) {
     double t = 0;
     for (size_t i = 0; i + 1 < ev.size(); i += 2) {
