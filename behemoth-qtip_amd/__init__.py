@@ -92,7 +92,7 @@ def lib():
     L.qtip_sign_vector.restype = None
     L.qtip_rotate_hessian.argtypes = [vp, vp, i, i, u64, d, vp, C.POINTER(d), vp]
     L.qtip_ldl_hessian.argtypes = [vp, i, i, vp]
-    L.qtip_ldlq_dev.argtypes = [vp, vp, vp, l, l, vp, vp, C.POINTER(d)]
+    L.qtip_ldlq_dev.argtypes = [vp, vp, vp, l, l, vp, vp, i, C.POINTER(d)]
     L.qtip_default_opts.argtypes = [C.POINTER(_OptsC)]
     L.qtip_default_opts.restype = None
     L.qtip_quantize_group.argtypes = [vp, i, C.POINTER(_LinearInC), i, u64, vp, d, vp, vp, C.POINTER(_OptsC),
@@ -282,9 +282,9 @@ class Quantizer:
             _check(rc)
         hp.t_ldl = time.time() - t0
 
-    def ldlq_dev(self, dWT, dL, n, m, d_hatWT, dQ, time_viterbi=False):
+    def ldlq_dev(self, dWT, dL, n, m, d_hatWT, dQ, time_viterbi=False, feedback=0):
         vs = C.c_double()
-        _check(lib().qtip_ldlq_dev(self._h, _ptr(dWT), _ptr(dL), n, m, _ptr(d_hatWT), _ptr(dQ),
+        _check(lib().qtip_ldlq_dev(self._h, _ptr(dWT), _ptr(dL), n, m, _ptr(d_hatWT), _ptr(dQ), feedback,
                                    C.byref(vs) if time_viterbi else None))
         return vs.value
 

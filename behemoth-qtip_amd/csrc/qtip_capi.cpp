@@ -226,11 +226,11 @@ int qtip_ldl_hessian(const float* host_HRr, int n, int threads, float* host_L) {
 }
 
 int qtip_ldlq_dev(qtip_ctx* ctx, const float* dev_WT, const float* dev_L, long n, long m, float* dev_hatWT,
-                  uint16_t* dev_Q, double* vit_seconds) {
+                  uint16_t* dev_Q, int feedback, double* vit_seconds) {
   return guarded([&] {
     QTIP_REQUIRE(ctx != nullptr && dev_WT && dev_L && dev_hatWT && dev_Q, "ldlq: bad arguments");
     DeviceGuard g(ctx);
-    ldlq_impl(ctx, dev_WT, dev_L, n, m, dev_hatWT, dev_Q, 0, vit_seconds);
+    ldlq_impl(ctx, dev_WT, dev_L, n, m, dev_hatWT, dev_Q, feedback, vit_seconds);
   });
 }
 

@@ -173,7 +173,7 @@ inline std::vector<LinearOut> quantize_group(hipStream_t s, Gemm& gemm, const st
 // accepted for source compatibility (the library holds its own codebook tables).
 inline void ldlq_gpu(hipStream_t, Gemm&, const float* WT, const float* L, long n, long m, float* hatWT, uint16_t* Q,
                      int /*vit_batch*/, const uint32_t* /*lut_h2_dev*/, double* vit_s) {
-  detail::check(qtip_ldlq_dev(detail::context(), WT, L, n, m, hatWT, Q, vit_s), "ldlq_gpu");
+  detail::check(qtip_ldlq_dev(detail::context(), WT, L, n, m, hatWT, Q, 0, vit_s), "ldlq_gpu");
 }
 
 // The reference returns its device half2 LUT; the library keeps its tables private, so this only makes sure the

@@ -123,13 +123,17 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
                double* vit_seconds) {
   QTIP_REQUIRE(n % 128 == 0, "LDLQ needs n %% 128 == 0 (n = %ld)", n);
   QTIP_REQUIRE(m % 16 == 0 && m > 0, "LDLQ needs m %% 16 == 0 (m = %ld)", m);
-  QTIP_REQUIRE(feedback == 0, "feedback mode %d is not available", feedback);
+  QTIP_REQUIRE(feedback == 0 || feedback == 1, "unknown feedback mode %d", feedback);
   hipStream_t s = c->stream;
   ensure_viterbi_workspace(c);
   const long ntr = m / 16, nblk = n / 16;
-  DBuf<double> prod(size_t(n) * m);
+  // feedback 0: fp64 feedback sums and fp64 prod cache; feedback 1: fp32 sums, fp32 prod cache updated by the
+  // bf16 hi/lo split MFMA product
+  DBuf<double> prod(feedback == 0 ? size_t(n) * m : 0);
+  DBuf<float> prod32(feedback == 1 ? size_t(n) * m : 0);
   DBuf<float> X(size_t(ntr) * 256);
-  QTIP_HIP(hipMemsetAsync(prod, 0, prod.bytes(), s));
+  if (feedback == 0) QTIP_HIP(hipMemsetAsync(prod, 0, prod.bytes(), s));
+  else QTIP_HIP(hipMemsetAsync(prod32, 0, prod32.bytes(), s));
   QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
   std::vector<hipEvent_t> ev;
   auto mark = [&] {
@@ -142,7 +146,8 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
     const int bufend = int(16 * cur), c0 = bufend - 128;
     for (int i = 7; i >= 0; --i) {
       const int col0 = c0 + 16 * i;
-      launch_ldlq_prep_f64(WT, hatWT, prod, L, n, m, col0, bufend, X, s);
+      if (feedback == 0) launch_ldlq_prep_f64(WT, hatWT, prod, L, n, m, col0, bufend, X, s);
+      else launch_ldlq_prep_f32(WT, hatWT, prod32, L, n, m, col0, bufend, X, s);
       if (vit_seconds) mark();
       TileJob job;
       job.X = X;
@@ -156,8 +161,13 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
       launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws, c->vit_slots, s);
       if (vit_seconds) mark();
     }
-    if (c0 > 0)  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
-      launch_gemm_tn_f64_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m, prod, m, s);
+    if (c0 > 0) {  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
+      if (feedback == 0)
+        launch_gemm_tn_f64_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m, prod, m, s);
+      else
+        launch_gemm_tn_bf16x3_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m,
+                                  prod32, m, s);
+    }
   }
   wait_stream_sleeping(s);
   if (vit_seconds) {

@@ -114,7 +114,7 @@ def run_group(args, pkg):
     n = H.shape[0]
     ms = [int(w.shape[0]) for w in Ws]
     lins = [pkg.LinearIn("w%d" % i, m, w_f32=w) for i, (m, w) in enumerate(zip(ms, Ws))]
-    opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=True)
+    opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=True, feedback=args.feedback)
     weights_per_step = sum(ms) * n
 
     def pinned(shape):
@@ -186,7 +186,7 @@ def run_group(args, pkg):
     extra.update(gpu_only_Mweights_s=weights_per_step / gpu_s / 1e6,
                  serial_Mweights_s=weights_per_step / (gpu_s + stats["ldl_s"]) / 1e6,
                  viterbi_only_Mweights_s=weights_per_step / stats["viterbi_s"] / 1e6,
-                 proxy_in_timed_region=False, ldl_threads=args.ldl_threads)
+                 proxy_in_timed_region=False, ldl_threads=args.ldl_threads, feedback=args.feedback)
     names = {2: "config2: 1024x1024 group", 3: "config3: 12288x12288 q-proj group",
              4: "config4: gate+up 2x(28672x12288) group", 5: "config5: 12288x28672 down-proj group"}
     return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
@@ -202,6 +202,8 @@ def main():
     ap.add_argument("--config", type=int, default=5, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--ldl-threads", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--feedback", type=int, default=0, choices=[0, 1],
+                    help="0: fp64 LDLQ feedback (default); 1: fp32 feedback + bf16 hi/lo split MFMA prod cache")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="first run one plain 1 GiB device copy kernel (known traffic, scales the rocprof byte counters)")
     args = ap.parse_args()

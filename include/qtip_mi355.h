@@ -76,9 +76,10 @@ int qtip_rotate_hessian(qtip_ctx* ctx, const float* H, int h_on_device, int n, u
 int qtip_ldl_hessian(const float* host_HRr, int n, int threads, float* host_L);
 
 /* ldlq_gpu, src/quantizer.cpp:30-89.  WT n x m fp32 (scaled), L n x n fp32, both on the device;
- * outputs hatWT n x m fp32 and Q[(m/16)*(n/16)][128] u16 on the device.  vit_seconds may be NULL. */
+ * outputs hatWT n x m fp32 and Q[(m/16)*(n/16)][128] u16 on the device.  feedback as in qtip_opts;
+ * vit_seconds may be NULL. */
 int qtip_ldlq_dev(qtip_ctx* ctx, const float* dev_WT, const float* dev_L, long n, long m, float* dev_hatWT,
-                  uint16_t* dev_Q, double* vit_seconds);
+                  uint16_t* dev_Q, int feedback, double* vit_seconds);
 
 /* One linear of a group (LinearIn, src/quantizer.hpp:21-28): exactly one weight pointer is set. */
 typedef struct {
@@ -106,7 +107,8 @@ typedef struct { /* QuantOpts, src/quantizer.hpp:11-19 */
   double sigma_reg;      /* 1e-2 */
   double scale_override; /* 0.9 */
   int ldl_threads;       /* 16 */
-  int feedback;          /* 0: fp64 feedback + fp64 MFMA prod cache (default); 1: fp32 feedback + bf16 hi/lo split MFMA */
+  int feedback;          /* 0: fp64 feedback sums + fp64 MFMA prod cache (default, tracks the fp64 CPU form);
+                            1: fp32 feedback sums + bf16 hi/lo split MFMA prod cache (the reference GPU's arithmetic) */
   int skip_proxy;        /* 1: leave proxy fields 0 */
 } qtip_opts;
 void qtip_default_opts(qtip_opts* o);

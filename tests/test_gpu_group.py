@@ -103,6 +103,44 @@ def test_ldlq_matches_cpu_algorithm(qz, oracle, hyb, m, n):
             assert np.array_equal(tile[perm], h)
 
 
+def test_ldlq_split_bf16_feedback(qz, oracle, hyb):
+    """feedback = 1 (fp32 sums in the buffer, prod cache by the bf16 hi/lo split MFMA product, the arithmetic of the
+    reference's GPU path): not bit-tracking the fp64 CPU form, so the bar is the reference's own for this
+    arithmetic (tests/test_gpu.cpp:295-296): proxy within 1 %, decode(states) == hatW."""
+    import torch
+    say("case: ldlq feedback=1 m=64 n=512")
+    qz.set_tlut(None)
+    m, n = 64, 512
+    rng = np.random.default_rng(77)
+    Wr = rng.normal(size=(m, n)).astype(np.float32)
+    H = _spd(n, 6)
+    L = oracle.block_ldl(H)
+    hat_o, Q_o = oracle.ldlq(hyb, Wr, L)
+    dWT = torch.from_numpy(np.ascontiguousarray(Wr.T)).cuda()
+    dL = torch.from_numpy(L).cuda()
+    dH = torch.zeros((n, m), device="cuda")
+    dQ = torch.zeros(((m // 16) * (n // 16), 128), dtype=torch.int16, device="cuda")
+    torch.cuda.synchronize()
+    qz.ldlq_dev(dWT, dL, n, m, dH, dQ, feedback=1)
+    hat_g = dH.cpu().numpy().T.copy()
+    Q_g = dQ.cpu().numpy().view(np.uint16)
+    H32 = H.astype(np.float32)
+    po = oracle.lib().qo_proxy(Wr.reshape(-1), hat_o.reshape(-1), H32.reshape(-1), m, n, 0)
+    pg = oracle.lib().qo_proxy(Wr.reshape(-1), np.ascontiguousarray(hat_g).reshape(-1), H32.reshape(-1), m, n, 0)
+    same = np.all(Q_g == Q_o, axis=1).mean()
+    say("  identical trellises %.4f, proxy cpu %.6f gpu %.6f" % (same, po, pg))
+    assert abs(pg - po) / po < 0.01
+    perm, _ = oracle.perm256()
+    l0, l1 = qz.lut()
+    for b in range(m // 16):
+        for blk in range(n // 16):
+            st = Q_g[b * (n // 16) + blk]
+            h = np.stack([l0[st], l1[st]], axis=-1).reshape(-1)
+            assert np.array_equal(hat_g[16 * b:16 * b + 16, 16 * blk:16 * blk + 16].reshape(-1)[perm], h)
+    with pytest.raises(Exception):
+        qz.ldlq_dev(dWT, dL, n, m, dH, dQ, feedback=7)
+
+
 def test_ldlq_rejects_bad_shapes(qz, pkg):
     import torch
     z = torch.zeros(1, device="cuda")
@@ -251,3 +289,11 @@ def test_group_config2(qz, oracle, pkg, hyb, synth):
     assert agree >= 0.99
     assert rel < 0.01
     assert lo.wscale == ref["wscale"][0]
+    # the same group with the reference GPU's arithmetic (fp32 feedback, split-bf16 prod cache): reported, and held
+    # to the proxy bar only -- one flipped fp16 rounding changes every later tile of its tile row
+    outs1, _ = qz.quantize_group_h([pkg.LinearIn("w", n, w_f32=Ws[0])], n, H, 11, pkg.QuantOpts(ldl_threads=16, feedback=1))
+    got1 = pkg.unswizzle_for_kernel(outs1[0].trellis, n, n).reshape(-1, 32)
+    agree1 = np.all(got1 == want, axis=1).mean()
+    rel1 = abs(outs1[0].proxy - ref["proxy"][0]) / ref["proxy"][0]
+    say("  feedback=1: code agreement %.4f, proxy %.6f (rel %.2e)" % (agree1, outs1[0].proxy, rel1))
+    assert rel1 < 0.01
