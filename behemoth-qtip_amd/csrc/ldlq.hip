@@ -52,56 +52,66 @@ __global__ __launch_bounds__(256) void ldlq_prep_kernel(const float* __restrict_
 
 // ---------------------------------------------------------------- fp64 MFMA GEMM
 typedef double double4_t __attribute__((ext_vector_type(4)));
-constexpr int BM = 64, BN = 64, KC = 32;
+constexpr int BM = 128, BN = 128, KC = 16;
 
-// MODE 0: C += acc.  MODE 1: partial[block] = sum_ij acc[i][j] * (B1 - B2)[i][j]  (square case M == K rows of B)
+// 128 x 128 outputs per workgroup, 4 waves of 64 x 64 (4 x 4 tiles of v_mfma_f64_16x16x4_f64), K in slices of 16
+// staged through LDS as fp64.  M and K are multiples of 16 and of 4 here (multiples of 128 in the LDLQ), N a
+// multiple of 4; rows and columns beyond M / N are masked.
+// MODE 0: C += acc.  MODE 1: partial[block] = sum_ij acc[i][j] * (B1 - B2)[i][j]  (square case: M rows of B)
 template <int MODE>
-__global__ __launch_bounds__(256) void gemm_tn_f64_kernel(int M, int N, int K, const float* __restrict__ A, long lda,
-                                                          const float* __restrict__ B1, const float* __restrict__ B2,
-                                                          long ldb, double* __restrict__ C, long ldc,
-                                                          double* __restrict__ partial) {
-  __shared__ double As[KC][BM];
-  __shared__ double Bs[KC][BN];
+__global__ __launch_bounds__(256, 2) void gemm_tn_f64_kernel(int M, int N, int K, const float* __restrict__ A,
+                                                             long lda, const float* __restrict__ B1,
+                                                             const float* __restrict__ B2, long ldb,
+                                                             double* __restrict__ C, long ldc,
+                                                             double* __restrict__ partial) {
+  __shared__ __attribute__((aligned(16))) double As[KC][BM];
+  __shared__ __attribute__((aligned(16))) double Bs[KC][BN];
   __shared__ double red[4];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const long i0 = long(blockIdx.y) * BM, j0 = long(blockIdx.x) * BN;
-  double4_t acc[2][2];
+  double4_t acc[4][4];
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < 4; ++a)
 #pragma unroll
-    for (int b = 0; b < 2; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
+    for (int b = 0; b < 4; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
+  const int lk = t >> 5, lc = (t & 31) * 4;  // this thread stages rows lk and lk + 8 of a slice, 4 columns at lc
+  const bool a_ok = i0 + lc + 3 < M, b_ok = j0 + lc + 3 < N;
 
   for (int kc = 0; kc < K; kc += KC) {
-    for (int idx = t; idx < KC * BM; idx += 256) {
-      const int k = idx / BM, i = idx % BM;
-      const long gi = i0 + i;
-      As[k][i] = (kc + k < K && gi < M) ? double(A[long(kc + k) * lda + gi]) : 0.0;
-    }
-    for (int idx = t; idx < KC * BN; idx += 256) {
-      const int k = idx / BN, j = idx % BN;
-      const long gj = j0 + j;
-      double v = 0.0;
-      if (kc + k < K && gj < N) {
-        const long o = long(kc + k) * ldb + gj;
-        v = double(B1[o]);
-        if (B2) v -= double(B2[o]);
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int k = lk + 8 * r;
+      float4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+      if (kc + k < K) {
+        if (a_ok) a = *reinterpret_cast<const float4*>(A + long(kc + k) * lda + i0 + lc);
+        if (b_ok) {
+          b = *reinterpret_cast<const float4*>(B1 + long(kc + k) * ldb + j0 + lc);
+        }
       }
-      Bs[k][j] = v;
+      double bx = b.x, by = b.y, bz = b.z, bw = b.w;
+      if (B2 && b_ok && kc + k < K) {
+        const float4 c = *reinterpret_cast<const float4*>(B2 + long(kc + k) * ldb + j0 + lc);
+        bx -= double(c.x), by -= double(c.y), bz -= double(c.z), bw -= double(c.w);
+      }
+      *reinterpret_cast<double2*>(&As[k][lc]) = double2{double(a.x), double(a.y)};
+      *reinterpret_cast<double2*>(&As[k][lc + 2]) = double2{double(a.z), double(a.w)};
+      *reinterpret_cast<double2*>(&Bs[k][lc]) = double2{bx, by};
+      *reinterpret_cast<double2*>(&Bs[k][lc + 2]) = double2{bz, bw};
     }
     __syncthreads();
 #pragma unroll
     for (int kk = 0; kk < KC; kk += 4) {
       const int kr = kk + (lane >> 4), c = lane & 15;
-      double a[2], b[2];
+      double a[4], b[4];
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi) a[mi] = As[kr][wm * 32 + mi * 16 + c];
+      for (int mi = 0; mi < 4; ++mi) a[mi] = As[kr][wm * 64 + mi * 16 + c];
 #pragma unroll
-      for (int ni = 0; ni < 2; ++ni) b[ni] = Bs[kr][wn * 32 + ni * 16 + c];
+      for (int ni = 0; ni < 4; ++ni) b[ni] = Bs[kr][wn * 64 + ni * 16 + c];
 #pragma unroll
-      for (int mi = 0; mi < 2; ++mi)
+      for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
+        for (int ni = 0; ni < 4; ++ni)
           acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
     }
     __syncthreads();
@@ -109,13 +119,13 @@ __global__ __launch_bounds__(256) void gemm_tn_f64_kernel(int M, int N, int K, c
   // accumulator element v of a lane: row (lane / 16) + 4 v, column lane % 16 of the 16x16 tile
   double local = 0.0;
 #pragma unroll
-  for (int mi = 0; mi < 2; ++mi)
+  for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-    for (int ni = 0; ni < 2; ++ni)
+    for (int ni = 0; ni < 4; ++ni)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const long gi = i0 + wm * 32 + mi * 16 + (lane >> 4) + 4 * v;
-        const long gj = j0 + wn * 32 + ni * 16 + (lane & 15);
+        const long gi = i0 + wm * 64 + mi * 16 + (lane >> 4) + 4 * v;
+        const long gj = j0 + wn * 64 + ni * 16 + (lane & 15);
         if (gi < M && gj < N) {
           if (MODE == 0) {
             C[gi * ldc + gj] += acc[mi][ni][v];
@@ -281,6 +291,7 @@ void launch_ldlq_prep_f32(const float* WT, const float* hatWT, const float* prod
 void launch_gemm_tn_f64_acc(int M, int N, int K, const float* A, long lda, const float* B1, const float* B2, long ldb,
                             double* C, long ldc, hipStream_t s) {
   if (M <= 0 || N <= 0 || K <= 0) return;
+  QTIP_REQUIRE(M % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0, "fp64 GEMM needs 16-byte aligned fp32 rows");
   dim3 grid(unsigned((N + BN - 1) / BN), unsigned((M + BM - 1) / BM));
   gemm_tn_f64_kernel<0><<<grid, dim3(256), 0, s>>>(M, N, K, A, lda, B1, B2, ldb, C, ldc, nullptr);
   QTIP_HIP(hipGetLastError());
@@ -299,6 +310,7 @@ void launch_gemm_tn_bf16x3_acc(int M, int N, int K, const float* A, long lda, co
 double quad_trace_f64(int n, int N, const float* H, const float* B1, const float* B2, long ldb, DBuf<double>& scratch,
                       hipStream_t s) {
   if (n <= 0 || N <= 0) return 0.0;
+  QTIP_REQUIRE(n % 4 == 0 && N % 4 == 0 && ldb % 4 == 0, "fp64 GEMM needs 16-byte aligned fp32 rows");
   dim3 grid(unsigned((N + BN - 1) / BN), unsigned((n + BM - 1) / BM));
   const long blocks = long(grid.x) * grid.y;
   scratch.ensure(size_t(blocks) + 1);
