@@ -8,6 +8,8 @@
 //  * gemm_tn: C[M][N] (+)= sum_k A[k][i] * (B1 - B2)[k][j] on the fp64 matrix cores
 //    (v_mfma_f64_16x16x4_f64), fp32 operands widened while staging through LDS.  Two epilogues: accumulate
 //    into C (the cross-buffer prod cache), or reduce sum(acc * (B1 - B2)[i][j]) for tr(X^T H X) (the proxy).
+//  * gemm_tn_bf16x3: the same prod-cache update with fp32 C and the operands split into bf16 hi + lo
+//    (v_mfma_f32_32x32x16_bf16, three terms), the arithmetic of the reference's GPU path.
 #include <hip/hip_fp16.h>
 
 #include "ldlq.hpp"
