@@ -5,7 +5,8 @@
 //   upper triangle zeroed, stored as fp32.
 //
 // Own layout of the work: right-looking panels of width NB; the diagonal block is factored in place, the rows
-// below are solved eight at a time (one SIMD lane per row), and the trailing symmetric update runs as a packed
+// below are solved in chunks of NR rows held transposed (64-column sub-blocks: rank update through the micro-kernel
+// plus a small triangular substitution), and the trailing symmetric update runs as a packed
 // register-blocked rank-NB kernel over lower-triangular tiles handed out dynamically to an OpenMP team.  The
 // micro-kernels are written with GCC vector extensions and compiled twice (AVX2 baseline, AVX-512 clone);
 // the clone is picked at run time so one binary serves any x86-64-v3 host.
@@ -98,47 +99,40 @@ static void micro_4x12(int kc, const double* __restrict__ a, const double* __res
     for (int j = 0; j < nr; ++j) C[i * ldc + j] -= t[i][j >> 2][j & 3];
 }
 
-// ---- eight rows of the panel solve  X * L11^T = A21, one lane per row (x holds the rows transposed: x[p][lane])
-__attribute__((target("avx512f"))) static void solve8_avx512(int kb, const double* __restrict__ L11 /*kb x kb*/,
-                                                              const double* __restrict__ rdiag, v8d* __restrict__ x) {
-  for (int j = 0; j < kb; ++j) {
-    const double* lj = L11 + size_t(j) * kb;
-    v8d s0 = x[j], s1 = v8d{0, 0, 0, 0, 0, 0, 0, 0}, s2 = s1, s3 = s1;
-    int p = 0;
-    for (; p + 4 <= j; p += 4) {
-      s0 -= lj[p] * x[p];
-      s1 -= lj[p + 1] * x[p + 1];
-      s2 -= lj[p + 2] * x[p + 2];
-      s3 -= lj[p + 3] * x[p + 3];
-    }
-    for (; p < j; ++p) s0 -= lj[p] * x[p];
-    x[j] = ((s0 + s1) + (s2 + s3)) * rdiag[j];
+// ---- panel solve  X * L11^T = A21 on a chunk of NR rows held transposed, x[p][NR] (the layout of one packed
+// B micro-panel).  The panel depth is cut into sub-blocks of SUB columns: the contribution of the columns already
+// solved goes through the rank-update micro-kernel, only the SUB x SUB triangle is substituted here.
+constexpr int SUB = 64;
+#define QTIP_TRI_SOLVE(NAME, NRC)                                                                              \
+  static void NAME(int nb, const double* __restrict__ Lbb, int ldl, const double* __restrict__ rdiag,          \
+                   double* __restrict__ x) {                                                                   \
+    for (int j = 0; j < nb; ++j) {                                                                             \
+      double acc[NRC];                                                                                         \
+      double* xj = x + size_t(j) * NRC;                                                                        \
+      for (int c = 0; c < NRC; ++c) acc[c] = xj[c];                                                            \
+      const double* lj = Lbb + size_t(j) * ldl;                                                                \
+      for (int q = 0; q < j; ++q) {                                                                            \
+        const double l = lj[q];                                                                                \
+        const double* xq = x + size_t(q) * NRC;                                                                \
+        for (int c = 0; c < NRC; ++c) acc[c] -= l * xq[c];                                                     \
+      }                                                                                                        \
+      const double rd = rdiag[j];                                                                              \
+      for (int c = 0; c < NRC; ++c) xj[c] = acc[c] * rd;                                                       \
+    }                                                                                                          \
   }
-}
-static void solve8_avx2(int kb, const double* __restrict__ L11, const double* __restrict__ rdiag,
-                        v8d* __restrict__ x) {
-  for (int j = 0; j < kb; ++j) {
-    const double* lj = L11 + size_t(j) * kb;
-    v8d s0 = x[j], s1 = v8d{0, 0, 0, 0, 0, 0, 0, 0};
-    int p = 0;
-    for (; p + 2 <= j; p += 2) {
-      s0 -= lj[p] * x[p];
-      s1 -= lj[p + 1] * x[p + 1];
-    }
-    for (; p < j; ++p) s0 -= lj[p] * x[p];
-    x[j] = (s0 + s1) * rdiag[j];
-  }
-}
+__attribute__((target("avx512f"))) QTIP_TRI_SOLVE(tri_solve_24, 24)
+QTIP_TRI_SOLVE(tri_solve_12, 12)
+#undef QTIP_TRI_SOLVE
 
 struct Kernels {
   int MR, NR;
   void (*micro)(int, const double*, const double*, double*, long, int, int);
-  void (*solve8)(int, const double*, const double*, v8d*);
+  void (*tri_solve)(int, const double*, int, const double*, double*);
 };
 static Kernels pick_kernels() {
   __builtin_cpu_init();
-  if (__builtin_cpu_supports("avx512f")) return Kernels{8, 24, micro_8x24, solve8_avx512};
-  return Kernels{4, 12, micro_4x12, solve8_avx2};
+  if (__builtin_cpu_supports("avx512f")) return Kernels{8, 24, micro_8x24, tri_solve_24};
+  return Kernels{4, 12, micro_4x12, tri_solve_12};
 }
 
 // unblocked lower Cholesky of the kb x kb diagonal block at A (row stride n); false if not positive definite
@@ -170,7 +164,12 @@ bool cholesky_lower(double* A, int n, int threads) {
   double tdiag = 0, tsolve = 0, tupd = 0, tq;
   const Kernels kn = pick_kernels();
   const int MR = kn.MR, NR = kn.NR;
-  std::vector<double> packA, packB, L11(size_t(NB) * NB), rdiag(NB);
+  std::vector<double> packL, L11(size_t(NB) * NB), rdiag(NB);
+  // packed copies of the solved panel (A side: MR-row micro-panels, B side: NR-row micro-panels), first panel largest
+  const size_t capA = size_t((n + MR - 1) / MR) * MR * NB, capB = size_t((n + NR - 1) / NR) * NR * NB;
+  HostScratch packs((capA + capB) * sizeof(double));
+  double* const packA = static_cast<double*>(packs.get());
+  double* const packB = packA + capA;
   for (int k = 0; k < n; k += NB) {
     const int kb = std::min(NB, n - k);
     tq = omp_get_wtime();
@@ -184,29 +183,55 @@ bool cholesky_lower(double* A, int n, int threads) {
       rdiag[j] = 1.0 / L11[size_t(j) * kb + j];
     }
     const int nPA = (nr + MR - 1) / MR, nPB = (nr + NR - 1) / NR;
-    packA.assign(size_t(nPA) * MR * kb, 0.0);
-    packB.assign(size_t(nPB) * NR * kb, 0.0);
-    // panel solve, fused with packing the solved panel in both micro-panel layouts
-#pragma omp parallel for schedule(dynamic, 4) num_threads(threads)
-    for (int g = 0; g < (nr + 7) / 8; ++g) {
-      const int rb = g * 8, rows = std::min(8, nr - rb);
-      alignas(64) v8d x[NB];
-      for (int p = 0; p < kb; ++p) {
-        v8d v = {0, 0, 0, 0, 0, 0, 0, 0};
-        for (int r = 0; r < rows; ++r) v[r] = A[long(r0 + rb + r) * n + k + p];
-        x[p] = v;
+    // only the padding rows of the last micro-panels need zeroing
+    for (int i = nr; i < nPA * MR; ++i)
+      for (int p = 0; p < kb; ++p) packA[size_t(i / MR) * MR * kb + size_t(p) * MR + (i % MR)] = 0.0;
+    for (int i = nr; i < nPB * NR; ++i)
+      for (int p = 0; p < kb; ++p) packB[size_t(i / NR) * NR * kb + size_t(p) * NR + (i % NR)] = 0.0;
+    // L11 sub-block rows packed for the micro-kernel's A side: for sub-block b, tile it: [q < 64 b][MR] holding
+    // L11[64 b + MR it + i][q]
+    const int nsb = (kb + SUB - 1) / SUB;
+    size_t offL[NB / SUB + 1];
+    {
+      size_t o = 0;
+      for (int b = 0; b < nsb; ++b) {
+        offL[b] = o;
+        const int p0 = b * SUB, pb = std::min(SUB, kb - p0);
+        o += size_t((pb + MR - 1) / MR) * MR * p0;
       }
-      kn.solve8(kb, L11.data(), rdiag.data(), x);
+      packL.assign(o, 0.0);
+      for (int b = 1; b < nsb; ++b) {
+        const int p0 = b * SUB, pb = std::min(SUB, kb - p0);
+        for (int i = 0; i < pb; ++i)
+          for (int q = 0; q < p0; ++q)
+            packL[offL[b] + size_t(i / MR) * MR * p0 + size_t(q) * MR + (i % MR)] = L11[size_t(p0 + i) * kb + q];
+      }
+    }
+    // panel solve in place in the packed B micro-panels (one chunk = NR rows), then write back and pack the A side
+#pragma omp parallel for schedule(dynamic, 2) num_threads(threads)
+    for (int g = 0; g < nPB; ++g) {
+      const int rb = g * NR, rows = std::min(NR, nr - rb);
+      double* x = packB + size_t(g) * NR * kb;  // [p][NR], rows beyond `rows` stay zero
+      for (int r = 0; r < rows; ++r) {
+        const double* src = A + long(r0 + rb + r) * n + k;
+        for (int p = 0; p < kb; ++p) x[size_t(p) * NR + r] = src[p];
+      }
+      for (int b = 0; b < nsb; ++b) {
+        const int p0 = b * SUB, pb = std::min(SUB, kb - p0);
+        if (b > 0)
+          for (int it = 0; it * MR < pb; ++it)
+            kn.micro(p0, packL.data() + offL[b] + size_t(it) * MR * p0, x, x + size_t(p0 + it * MR) * NR, NR,
+                     std::min(MR, pb - it * MR), NR);
+        kn.tri_solve(pb, L11.data() + size_t(p0) * kb + p0, kb, rdiag.data() + p0, x + size_t(p0) * NR);
+      }
       for (int r = 0; r < rows; ++r) {
         const int i = rb + r;
         double* dst = A + long(r0 + i) * n + k;
-        double* pa = packA.data() + size_t(i / MR) * MR * kb + (i % MR);
-        double* pb = packB.data() + size_t(i / NR) * NR * kb + (i % NR);
+        double* pa = packA + size_t(i / MR) * MR * kb + (i % MR);
         for (int p = 0; p < kb; ++p) {
-          const double v = x[p][r];
+          const double v = x[size_t(p) * NR + r];
           dst[p] = v;
           pa[size_t(p) * MR] = v;
-          pb[size_t(p) * NR] = v;
         }
       }
     }
@@ -227,12 +252,12 @@ bool cholesky_lower(double* A, int n, int threads) {
       const int bj = int(rem);
       const int i0 = bi * TILE, i1 = std::min(nr, i0 + TILE), j0 = bj * TILE, j1 = std::min(nr, j0 + TILE);
       for (int jj = j0; jj < j1; jj += NR) {
-        const double* pb = packB.data() + size_t(jj / NR) * NR * kb;
+        const double* pb = packB + size_t(jj / NR) * NR * kb;
         const int nrr = std::min(NR, nr - jj);
         for (int ii = i0; ii < i1; ii += MR) {
           if (jj > ii + MR - 1) continue;  // micro tile entirely above the diagonal
           const int mrr = std::min(MR, nr - ii);
-          kn.micro(kb, packA.data() + size_t(ii / MR) * MR * kb, pb, A + long(r0 + ii) * n + r0 + jj, n, mrr, nrr);
+          kn.micro(kb, packA + size_t(ii / MR) * MR * kb, pb, A + long(r0 + ii) * n + r0 + jj, n, mrr, nrr);
         }
       }
     }

@@ -1,7 +1,11 @@
 // Host-side pieces of the group quantizer: number formats, sign streams, codebook expansion, Hadamard factor
 // selection, trellis packing.  Semantics follow the reference files named at each function.
+#include <sys/mman.h>
+
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "data/qtip_tables.h"
 #include "qtip_internal.hpp"
@@ -181,5 +185,57 @@ bool unswizzle_host(const uint16_t* in, int m, int n, uint16_t* packed) {
     }
   return true;
 }
+
+namespace {
+// Large host work buffers, kept for the life of the process and handed out one caller at a time.
+struct HostPool {
+  struct Slot {
+    void* p;
+    size_t cap;
+    bool busy;
+  };
+  std::mutex mu;
+  std::vector<Slot> slots;
+  void* acquire(size_t bytes) {
+    std::lock_guard<std::mutex> lk(mu);
+    Slot* fit = nullptr;  // smallest idle buffer that is large enough
+    for (auto& s : slots)
+      if (!s.busy && s.p && s.cap >= bytes && (!fit || s.cap < fit->cap)) fit = &s;
+    if (fit) {
+      fit->busy = true;
+      return fit->p;
+    }
+    for (auto& s : slots)  // an idle but smaller buffer is replaced rather than kept beside the new one
+      if (!s.busy) {
+        std::free(s.p);
+        s.p = nullptr;
+        s.cap = 0;
+      }
+    void* p = nullptr;
+    const size_t huge = size_t(2) << 20;
+    const size_t cap = (bytes + huge - 1) / huge * huge;
+    if (posix_memalign(&p, huge, cap) != 0 || !p) throw Error(QTIP_E_NOMEM, "out of host memory for the LDL work matrix");
+    (void)madvise(p, cap, MADV_HUGEPAGE);
+    for (auto& s : slots)
+      if (!s.p) {
+        s = Slot{p, cap, true};
+        return p;
+      }
+    slots.push_back(Slot{p, cap, true});
+    return p;
+  }
+  void release(void* p) {
+    std::lock_guard<std::mutex> lk(mu);
+    for (auto& s : slots)
+      if (s.p == p) s.busy = false;
+  }
+};
+HostPool& host_pool() {
+  static HostPool pool;
+  return pool;
+}
+}  // namespace
+HostScratch::HostScratch(size_t bytes) : p(host_pool().acquire(bytes)) {}
+HostScratch::~HostScratch() { host_pool().release(p); }
 
 }  // namespace qtipmi

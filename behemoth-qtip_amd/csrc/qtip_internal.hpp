@@ -96,6 +96,18 @@ void unpack_trellis_host(const uint16_t* packed, long B, uint16_t* states);
 bool swizzle_host(const uint16_t* packed, int m, int n, uint16_t* out);
 bool unswizzle_host(const uint16_t* in, int m, int n, uint16_t* packed);
 
+// Large host work buffer from a process-wide pool (2 MB aligned, huge-page advised, kept for the life of the
+// process and handed out to one caller at a time): the fp64 LDL work matrix (6.6 GB at n = 28672) and its packed
+// panels are not mapped and faulted in again for every group.  Contents are whatever the last user left.
+struct HostScratch {
+  void* p;
+  explicit HostScratch(size_t bytes);
+  ~HostScratch();
+  HostScratch(const HostScratch&) = delete;
+  HostScratch& operator=(const HostScratch&) = delete;
+  void* get() const { return p; }
+};
+
 // fp64 block LDL on the host (host_ldl.cpp). A: n x n fp64, lower triangle used, destroyed. Returns false if not PD.
 bool block_ldl_host(double* A, int n, float* L_out, int threads);
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle

@@ -13,58 +13,6 @@
 
 namespace qtipmi {
 namespace {
-// Large host work buffers, kept for the life of the process and handed out one caller at a time.
-struct HostPool {
-  struct Slot {
-    void* p;
-    size_t cap;
-    bool busy;
-  };
-  std::mutex mu;
-  std::vector<Slot> slots;
-  void* acquire(size_t bytes) {
-    std::lock_guard<std::mutex> lk(mu);
-    for (auto& s : slots)
-      if (!s.busy && s.cap >= bytes) {
-        s.busy = true;
-        return s.p;
-      }
-    for (auto& s : slots)  // an idle but smaller buffer is replaced rather than kept beside the new one
-      if (!s.busy) {
-        std::free(s.p);
-        s.p = nullptr;
-        s.cap = 0;
-      }
-    void* p = nullptr;
-    const size_t huge = size_t(2) << 20;
-    const size_t cap = (bytes + huge - 1) / huge * huge;
-    if (posix_memalign(&p, huge, cap) != 0 || !p) throw Error(QTIP_E_NOMEM, "out of host memory for the LDL work matrix");
-    (void)madvise(p, cap, MADV_HUGEPAGE);
-    for (auto& s : slots)
-      if (!s.p) {
-        s = Slot{p, cap, true};
-        return p;
-      }
-    slots.push_back(Slot{p, cap, true});
-    return p;
-  }
-  void release(void* p) {
-    std::lock_guard<std::mutex> lk(mu);
-    for (auto& s : slots)
-      if (s.p == p) s.busy = false;
-  }
-};
-HostPool& host_pool() {
-  static HostPool pool;
-  return pool;
-}
-struct HostScratch {
-  void* p;
-  explicit HostScratch(size_t bytes) : p(host_pool().acquire(bytes)) {}
-  ~HostScratch() { host_pool().release(p); }
-  void* get() const { return p; }
-};
-
 // Waits for the stream without spinning on a core: the host LDL of the next group runs on all cores meanwhile.
 void wait_stream_sleeping(hipStream_t s) {
   hipEvent_t e;
