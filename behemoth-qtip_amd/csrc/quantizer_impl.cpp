@@ -90,8 +90,14 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
     QTIP_HIP(hipEventRecord(e, s));
     ev.push_back(e);
   };
-  for (long cur = nblk; cur > 0; cur -= 8) {
+  // The queue is kept two buffers (16 launches of ~2 ms) ahead of the GPU and no further: beyond that the
+  // submitting thread would spin on a full queue and take a core from the host LDL of the next group.
+  hipEvent_t pace[3];
+  for (auto& e : pace) QTIP_HIP(hipEventCreateWithFlags(&e, hipEventBlockingSync | hipEventDisableTiming));
+  long nbuf_done = 0;
+  for (long cur = nblk; cur > 0; cur -= 8, ++nbuf_done) {
     const int bufend = int(16 * cur), c0 = bufend - 128;
+    if (nbuf_done >= 2) QTIP_HIP(hipEventSynchronize(pace[(nbuf_done - 2) % 3]));
     for (int i = 7; i >= 0; --i) {
       const int col0 = c0 + 16 * i;
       if (feedback == 0) launch_ldlq_prep_f64(WT, hatWT, prod, L, n, m, col0, bufend, X, s);
@@ -116,7 +122,9 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
         launch_gemm_tn_bf16x3_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m,
                                   prod32, m, s);
     }
+    QTIP_HIP(hipEventRecord(pace[nbuf_done % 3], s));
   }
+  for (auto& e : pace) (void)hipEventDestroy(e);
   wait_stream_sleeping(s);
   if (vit_seconds) {
     double t = 0;

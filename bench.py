@@ -202,8 +202,7 @@ def main():
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--config", type=int, default=5, choices=[1, 2, 3, 4, 5])
-    ap.add_argument("--ldl-threads", type=int, default=15,
-                    help="OpenMP team of the host LDL; one of the box's 16 cores is left to the thread feeding the GPU queue")
+    ap.add_argument("--ldl-threads", type=int, default=16, help="OpenMP team of the host LDL")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--feedback", type=int, default=0, choices=[0, 1],
                     help="0: fp64 LDLQ feedback (default); 1: fp32 feedback + bf16 hi/lo split MFMA prod cache")
