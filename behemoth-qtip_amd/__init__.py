@@ -87,6 +87,8 @@ def lib():
     L.qtip_viterbi_tiles_dev.argtypes = [vp, vp, l, vp, vp]
     L.qtip_decode_states_dev.argtypes = [vp, vp, l, vp]
     L.qtip_hadamard_rows_dev.argtypes = [vp, vp, l, i, l, i]
+    L.qtip_decode_trellis_dev.argtypes = [vp, vp, i, i, vp]
+    L.qtip_dequantize_linear.argtypes = [vp, vp, vp, vp, C.c_float, i, i, vp, i]
     L.qtip_had_K.argtypes = [i]
     L.qtip_sign_vector.argtypes = [u64, l, vp]
     L.qtip_sign_vector.restype = None
@@ -250,6 +252,22 @@ class Quantizer:
 
     def decode_states_dev(self, d_states, B, d_hat):
         _check(lib().qtip_decode_states_dev(self._h, _ptr(d_states), B, _ptr(d_hat)))
+
+    def decode_trellis_dev(self, d_trellis, m, n, d_hatWr):
+        """Kernel-layout trellis words (device) -> hatWr m x n fp32 (device); runtime/src/qtip.cpp:83-118."""
+        _check(lib().qtip_decode_trellis_dev(self._h, _ptr(d_trellis), m, n, _ptr(d_hatWr)))
+
+    def dequantize_linear(self, out: "LinearOut", hatW=None):
+        """hatW (m x n fp32) of one quantized linear from its packed output; hatW may be a device tensor to fill."""
+        m, n = out.m, out.n
+        tr = np.ascontiguousarray(out.trellis, dtype=np.uint16)
+        su = np.ascontiguousarray(out.su_bf16, dtype=np.uint16)
+        sv = np.ascontiguousarray(out.sv, dtype=np.float32)
+        if hatW is None:
+            hatW = np.empty((m, n), np.float32)
+        _check(lib().qtip_dequantize_linear(self._h, _ptr(tr), _ptr(su), _ptr(sv), float(out.wscale), m, n, _ptr(hatW),
+                                            1 if _is_device(hatW) else 0))
+        return hatW
 
     def hadamard_rows_dev(self, dX, rows, n, ld, transpose):
         _check(lib().qtip_hadamard_rows_dev(self._h, _ptr(dX), rows, n, ld, 1 if transpose else 0))

@@ -6,4 +6,7 @@ void launch_fp8_to_f32(const uint8_t* w, const uint16_t* scale_bf16, float* out,
 void launch_scale_rc(float* X, long rows, long cols, long ld, const float* rs, const float* cs, hipStream_t s);
 // states of one linear (m x n weights, tiles row-major) -> kernel-layout trellis words
 void launch_pack_swizzle(const uint16_t* Q, long m, long n, uint16_t* out, hipStream_t s);
+// kernel-layout trellis words of one linear -> hatWr (m x n fp32, row stride ld): lookup of every 16-bit window (decode.hip)
+void launch_decode_trellis(const uint16_t* trellis, long m, long n, const float* entry_f, float* out, long ld,
+                           hipStream_t s);
 }  // namespace qtipmi

@@ -170,6 +170,44 @@ int qtip_decode_states_dev(qtip_ctx* ctx, const uint16_t* dev_states, long B, fl
   });
 }
 
+int qtip_decode_trellis_dev(qtip_ctx* ctx, const uint16_t* dev_trellis, int m, int n, float* dev_hatWr) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && dev_trellis && dev_hatWr, "decode_trellis: bad arguments");
+    DeviceGuard g(ctx);
+    launch_decode_trellis(dev_trellis, m, n, ctx->d_entry_f, dev_hatWr, n, ctx->stream);
+  });
+}
+
+int qtip_dequantize_linear(qtip_ctx* ctx, const uint16_t* host_trellis, const uint16_t* host_su_bf16,
+                           const float* host_sv, float wscale, int m, int n, float* hatW, int hatW_on_device) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && host_trellis && host_su_bf16 && host_sv && hatW, "dequantize_linear: bad arguments");
+    QTIP_REQUIRE(m > 0 && n > 0 && m % 32 == 0 && n % 32 == 0, "dequantize_linear: m, n must be multiples of 32 (m=%d n=%d)", m, n);
+    QTIP_REQUIRE(had_K(m) > 0 && had_K(n) > 0, "dequantize_linear: no Hadamard transform of size %d x %d", m, n);
+    DeviceGuard g(ctx);
+    hipStream_t s = ctx->stream;
+    const size_t words = size_t(m / 16) * (n / 16) * 32;
+    DBuf<uint16_t> tr(words);
+    DBuf<float> a(size_t(n) * m), b(size_t(m) * n), d_su(n), d_sv(m);
+    std::vector<float> su(n);
+    for (int i = 0; i < n; ++i) su[i] = bf16_to_f32(host_su_bf16[i]);
+    QTIP_HIP(hipMemcpyAsync(tr, host_trellis, words * 2, hipMemcpyHostToDevice, s));
+    QTIP_HIP(hipMemcpyAsync(d_su, su.data(), size_t(n) * 4, hipMemcpyHostToDevice, s));
+    QTIP_HIP(hipMemcpyAsync(d_sv, host_sv, size_t(m) * 4, hipMemcpyHostToDevice, s));
+    launch_decode_trellis(tr, m, n, ctx->d_entry_f, b, n, s);
+    // same operation order as the reconstruction at the end of quantize_group (src/quantizer.cpp:321-338), starting
+    // from hatWr^T, so that both give the same bits
+    ctx->rht.transpose(b, m, n, n, a, m);
+    ctx->rht.hadamard_rows(a, n, m, m, false);
+    ctx->rht.transpose(a, n, m, m, b, n);
+    ctx->rht.hadamard_rows(b, m, n, n, false);
+    ctx->rht.scale(b, m, n, n, wscale);
+    launch_scale_rc(b, m, n, n, d_sv, d_su, s);
+    QTIP_HIP(hipMemcpyAsync(hatW, b, size_t(m) * n * 4, hatW_on_device ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost, s));
+    QTIP_HIP(hipStreamSynchronize(s));
+  });
+}
+
 int qtip_had_K(int n) { return had_K(n); }
 
 void qtip_sign_vector(uint64_t seed, long count, float* host_out) {

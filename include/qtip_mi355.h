@@ -57,6 +57,18 @@ int qtip_viterbi_tiles_dev(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* 
 /* hat[i] = lut[state[i]] (k_decode_states, src/viterbi.hip:231-238): B x 128 states -> B x 256 fp32 */
 int qtip_decode_states_dev(qtip_ctx* ctx, const uint16_t* dev_states, long B, float* dev_hat);
 
+/* Decoder of the packed output (decode_rows / decode_tile, runtime/src/qtip.cpp:83-118, word addressing of
+ * HostLinear::word, runtime/include/behemoth/qtip.hpp:63-67): kernel-layout trellis u16[(m/16)*(n/16)*32] ->
+ * hatWr m x n fp32 row-major, the rotated and Wscale-free weight (fp16 codebook values).  Asynchronous. */
+int qtip_decode_trellis_dev(qtip_ctx* ctx, const uint16_t* dev_trellis, int m, int n, float* dev_hatWr);
+
+/* Weight of one quantized linear in the original domain from what quantize_group returns for it:
+ * hatW = diag(SV) U_m (hatWr * Wscale) U_n^T diag(SU), the reconstruction of src/quantizer.cpp:321-338 started from
+ * the packed trellis instead of the LDLQ buffer (bit-identical to qtip_linear_out.hatW).  trellis, su_bf16[n], sv[m]
+ * are host memory; hatW m x n fp32 is host memory, or device memory when hatW_on_device != 0.  Synchronous. */
+int qtip_dequantize_linear(qtip_ctx* ctx, const uint16_t* host_trellis, const uint16_t* host_su_bf16,
+                           const float* host_sv, float wscale, int m, int n, float* hatW, int hatW_on_device);
+
 /* In-place row transform x <- (hadK^(T) (x) H_{n/K}) x / sqrt(n) of `rows` rows of length n, row stride ld
  * (k_hadamard_rows, src/kernels.hip:293-313; same fp32 dataflow, so results are bit-identical to it). */
 int qtip_hadamard_rows_dev(qtip_ctx* ctx, float* dev_X, long rows, int n, long ld, int transpose);
