@@ -101,6 +101,15 @@ def lib():
                                       C.POINTER(_LinearOutC), C.POINTER(_TimingC)]
     L.qtip_quantize_group_h.argtypes = [vp, i, C.POINTER(_LinearInC), i, vp, i, u64, C.POINTER(_OptsC),
                                         C.POINTER(_LinearOutC), C.POINTER(_TimingC)]
+    L.qtip_run_groups.argtypes = [vp, i, vp, C.POINTER(_OptsC), vp, vp]
+    L.qtip_reserve_groups.argtypes = [vp, i]
+    L.qtip_st_create.argtypes = [C.POINTER(vp)]
+    L.qtip_st_destroy.argtypes = [vp]
+    L.qtip_st_destroy.restype = None
+    L.qtip_st_add.argtypes = [vp, C.c_char_p, C.c_char_p, vp, i, vp, u64]
+    L.qtip_st_add_qtip_linear.argtypes = [vp, C.c_char_p, vp, i, i, vp]
+    L.qtip_st_write.argtypes = [vp, C.c_char_p, vp, i, C.POINTER(u64)]
+    L.qtip_get_tlut_f16.argtypes = [vp, vp]
     L.qtip_pack_trellis.argtypes = [vp, l, vp]
     L.qtip_pack_trellis.restype = None
     L.qtip_unpack_trellis.argtypes = [vp, l, vp]
@@ -109,6 +118,11 @@ def lib():
     L.qtip_unswizzle_for_kernel.argtypes = [vp, i, i, vp]
     _lib = L
     return L
+
+
+class _GroupC(C.Structure):
+    _fields_ = [("nlin", C.c_int), ("lins", C.c_void_p), ("outs", C.c_void_p), ("n", C.c_int), ("H", C.c_void_p),
+                ("h_on_device", C.c_int), ("seed", C.c_uint64)]
 
 
 def _check(rc):
@@ -364,6 +378,88 @@ class Quantizer:
         _check(lib().qtip_quantize_group_h(self._h, len(lins), cin, n, _ptr(H), 1 if _is_device(H) else 0, seed,
                                            C.byref(co), cout, C.byref(tm)))
         return self._finish(cout, outs, tm)
+
+
+    def reserve_groups(self, n):
+        _check(lib().qtip_reserve_groups(self._h, n))
+
+    def run_groups(self, groups, opt: QuantOpts = None):
+        """Several groups with the host LDL of group g+1 overlapping the GPU work of group g (run_qtip_groups,
+        src/pipeline.cpp:229-312).  groups: list of (lins, n, H, seed).  Returns a list of (outs, timing, ldl_wait)."""
+        opt = opt or QuantOpts()
+        G = (_GroupC * len(groups))()
+        held, keep = [], []
+        co = None
+        for g, (lins, n, H, seed) in enumerate(groups):
+            cin, cout, outs, co, kp = self._marshal(lins, n, opt)
+            if not _is_device(H):
+                H = np.ascontiguousarray(H, np.float32)
+            keep.append((kp, H, cin))
+            held.append((cout, outs))
+            G[g].nlin, G[g].lins, G[g].outs = len(lins), C.addressof(cin), C.addressof(cout)
+            G[g].n, G[g].H, G[g].h_on_device, G[g].seed = n, _ptr(H), 1 if _is_device(H) else 0, seed
+        tms = (_TimingC * len(groups))()
+        waits = (C.c_double * len(groups))()
+        if groups:
+            _check(lib().qtip_run_groups(self._h, len(groups), C.addressof(G), C.byref(co), C.addressof(tms),
+                                         C.addressof(waits)))
+        res = []
+        for g, (cout, outs) in enumerate(held):
+            o, tm = self._finish(cout, outs, tms[g])
+            res.append((o, tm, waits[g]))
+        return res
+
+    def tlut_f16(self):
+        out = np.zeros((512, 2), np.uint16)
+        _check(lib().qtip_get_tlut_f16(self._h, _ptr(out)))
+        return out
+
+
+class LayerFileWriter:
+    """safetensors container of a quantized layer (SafeTensorsWriter, src/safetensors.cpp:93-137; tensor set of
+    write_layer_file, src/pipeline.cpp:315-352).  Host only."""
+
+    def __init__(self):
+        self._h = C.c_void_p()
+        _check(lib().qtip_st_create(C.byref(self._h)))
+
+    def close(self):
+        if self._h:
+            lib().qtip_st_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def add(self, name, dtype, shape, data):
+        data = np.ascontiguousarray(data)
+        sh = (C.c_int64 * max(1, len(shape)))(*shape)
+        _check(lib().qtip_st_add(self._h, name.encode(), dtype.encode(), C.addressof(sh), len(shape), _ptr(data),
+                                 data.nbytes))
+
+    def add_qtip_linear(self, prefix, out: "LinearOut", tlut_f16=None):
+        co = _LinearOutC()
+        tr = np.ascontiguousarray(out.trellis, np.uint16)
+        su = np.ascontiguousarray(out.su_bf16, np.uint16)
+        sv = np.ascontiguousarray(out.sv, np.float32)
+        co.trellis, co.su_bf16, co.sv, co.wscale = _ptr(tr), _ptr(su), _ptr(sv), out.wscale
+        tl = None if tlut_f16 is None else np.ascontiguousarray(tlut_f16, np.uint16)
+        _check(lib().qtip_st_add_qtip_linear(self._h, prefix.encode(), C.addressof(co), out.m, out.n, _ptr(tl)))
+
+    def write(self, path, metadata=None):
+        n = C.c_uint64()
+        if metadata is None:
+            _check(lib().qtip_st_write(self._h, path.encode(), None, 0, C.byref(n)))
+        else:
+            flat = []
+            for k, v in metadata.items():
+                flat += [k.encode(), v.encode()]
+            arr = (C.c_char_p * max(1, len(flat)))(*flat)
+            _check(lib().qtip_st_write(self._h, path.encode(), C.addressof(arr), len(metadata), C.byref(n)))
+        return n.value
 
 
 # ---------------------------------------------------------------- host packers

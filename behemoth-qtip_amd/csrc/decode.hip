@@ -12,7 +12,7 @@
 namespace qtipmi {
 namespace {
 
-constexpr int kPatchCols = 128, kLdsStride = 132;
+constexpr int kLdsStride = 132;  // floats per staged patch row: 128 columns + padding, 16-byte aligned
 
 __global__ __launch_bounds__(256) void decode_trellis_kernel(const uint16_t* __restrict__ trellis, long n2 /* n / 32 */,
                                                             const float* __restrict__ entry_f,

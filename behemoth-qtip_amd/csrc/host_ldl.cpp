@@ -7,20 +7,35 @@
 // Own layout of the work: right-looking panels of width NB; the diagonal block is factored in place, the rows
 // below are solved in chunks of NR rows held transposed (64-column sub-blocks: rank update through the micro-kernel
 // plus a small triangular substitution), and the trailing symmetric update runs as a packed
-// register-blocked rank-NB kernel over lower-triangular tiles handed out dynamically to an OpenMP team.  The
+// register-blocked rank-NB kernel over lower-triangular tiles handed out dynamically to a team of host threads (host_team.hpp).  The
 // micro-kernels are written with GCC vector extensions and compiled twice (AVX2 baseline, AVX-512 clone);
 // the clone is picked at run time so one binary serves any x86-64-v3 host.
-#include <omp.h>
-
 #include <algorithm>
+#include <atomic>
+#include <chrono>
 #include <cmath>
 #include <cstring>
+#include <memory>
+#include <thread>
 #include <vector>
 
+#include "host_team.hpp"
 #include "qtip_internal.hpp"
 
 namespace qtipmi {
 namespace {
+
+double wtime() { return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count(); }
+
+// The team belongs to the calling thread (the factorization may run on a side thread while another thread does
+// other work with a team of its own) and lives until that thread ends or asks for another size.
+HostTeam& team_of_this_thread(int threads) {
+  if (threads <= 0) threads = int(std::thread::hardware_concurrency());
+  if (threads <= 0) threads = 1;
+  static thread_local std::unique_ptr<HostTeam> team;
+  if (!team || team->size() != threads) team.reset(new HostTeam(threads));
+  return *team;
+}
 
 typedef double v8d __attribute__((vector_size(64), aligned(8)));
 typedef double v4d __attribute__((vector_size(32), aligned(8)));
@@ -160,7 +175,7 @@ static bool factor_diagonal(double* A, long n, int kb) {
   return true;
 }
 
-bool cholesky_lower(double* A, int n, int threads) {
+bool cholesky_lower(double* A, int n, HostTeam& team) {
   double tdiag = 0, tsolve = 0, tupd = 0, tq;
   const Kernels kn = pick_kernels();
   const int MR = kn.MR, NR = kn.NR;
@@ -172,10 +187,10 @@ bool cholesky_lower(double* A, int n, int threads) {
   double* const packB = packA + capA;
   for (int k = 0; k < n; k += NB) {
     const int kb = std::min(NB, n - k);
-    tq = omp_get_wtime();
+    tq = wtime();
     if (!factor_diagonal(A + long(k) * n + k, n, kb)) return false;
-    tdiag += omp_get_wtime() - tq;
-    tq = omp_get_wtime();
+    tdiag += wtime() - tq;
+    tq = wtime();
     const int r0 = k + kb, nr = n - r0;
     if (nr <= 0) break;
     for (int j = 0; j < kb; ++j) {
@@ -208,8 +223,8 @@ bool cholesky_lower(double* A, int n, int threads) {
       }
     }
     // panel solve in place in the packed B micro-panels (one chunk = NR rows), then write back and pack the A side
-#pragma omp parallel for schedule(dynamic, 2) num_threads(threads)
-    for (int g = 0; g < nPB; ++g) {
+    team.parallel_for(nPB, 2, [&](long gl) {
+      const int g = int(gl);
       const int rb = g * NR, rows = std::min(NR, nr - rb);
       double* x = packB + size_t(g) * NR * kb;  // [p][NR], rows beyond `rows` stay zero
       for (int r = 0; r < rows; ++r) {
@@ -234,14 +249,13 @@ bool cholesky_lower(double* A, int n, int threads) {
           pa[size_t(p) * MR] = v;
         }
       }
-    }
-    tsolve += omp_get_wtime() - tq;
-    tq = omp_get_wtime();
+    });
+    tsolve += wtime() - tq;
+    tq = wtime();
     // trailing update of the lower triangle, tiles (bi, bj <= bi) largest rows first
     const int nT = (nr + TILE - 1) / TILE;
     const long ntask = long(nT) * (nT + 1) / 2;
-#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
-    for (long task = 0; task < ntask; ++task) {
+    team.parallel_for(ntask, 1, [&](long task) {
       // enumerate from the bottom row block upwards: row block bi has bi+1 tiles
       long rem = task;
       int bi = nT - 1;
@@ -260,8 +274,8 @@ bool cholesky_lower(double* A, int n, int threads) {
           kn.micro(kb, packA + size_t(ii / MR) * MR * kb, pb, A + long(r0 + ii) * n + r0 + jj, n, mrr, nrr);
         }
       }
-    }
-    tupd += omp_get_wtime() - tq;
+    });
+    tupd += wtime() - tq;
   }
   if (getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "chol: diag %.3f solve+pack %.3f update %.3f\n", tdiag, tsolve, tupd);
   return true;
@@ -271,16 +285,16 @@ bool cholesky_lower(double* A, int n, int threads) {
 
 bool block_ldl_host(double* A, int n, float* L_out, int threads) {
   if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
-  if (threads <= 0) threads = omp_get_max_threads();
-  double tq = omp_get_wtime();
-  if (!cholesky_lower(A, n, threads)) return false;
-  const double t_chol = omp_get_wtime() - tq;
-  tq = omp_get_wtime();
+  HostTeam& team = team_of_this_thread(threads);
+  double tq = wtime();
+  if (!cholesky_lower(A, n, team)) return false;
+  const double t_chol = wtime() - tq;
+  tq = wtime();
   const int nb = n / 16;
   // inverse of every 16x16 lower-triangular diagonal block (column by column, forward substitution)
   std::vector<double> inv(size_t(nb) * 256);
-#pragma omp parallel for schedule(static) num_threads(threads)
-  for (int b = 0; b < nb; ++b) {
+  team.parallel_for(nb, (nb + team.size() - 1) / team.size(), [&](long bl) {
+    const int b = int(bl);
     double D[16][16], V[16][16];
     for (int i = 0; i < 16; ++i)
       for (int j = 0; j < 16; ++j) D[i][j] = j <= i ? A[long(b * 16 + i) * n + b * 16 + j] : 0.0;
@@ -291,10 +305,11 @@ bool block_ldl_host(double* A, int n, float* L_out, int threads) {
         V[i][c] = s / D[i][i];
       }
     std::memcpy(&inv[size_t(b) * 256], V, sizeof V);
-  }
-  int finite = 1;
-#pragma omp parallel for schedule(dynamic, 16) num_threads(threads) reduction(&& : finite)
-  for (int r = 0; r < n; ++r) {
+  });
+  std::atomic<int> finite{1};
+  team.parallel_for(n, 16, [&](long rl) {
+    const int r = int(rl);
+    bool ok = true;
     const double* ar = A + long(r) * n;
     float* lr = L_out + long(r) * n;
     const int rb = r / 16;
@@ -305,28 +320,30 @@ bool block_ldl_host(double* A, int n, float* L_out, int threads) {
         double s = 0;
         for (int p = j; p < 16; ++p) s += a[p] * iv[p * 16 + j];
         lr[bj * 16 + j] = float(s);
-        finite = finite && std::isfinite(s);
+        ok = ok && std::isfinite(s);
       }
     }
     std::memset(lr + long(rb) * 16, 0, sizeof(float) * size_t(n - rb * 16));  // diagonal block and everything right of it
-  }
-  if (getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "block_ldl: cholesky %.3f, L assembly %.3f\n", t_chol, omp_get_wtime() - tq);
-  return finite != 0;
+    if (!ok) finite.store(0, std::memory_order_relaxed);
+  });
+  if (getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "block_ldl: cholesky %.3f, L assembly %.3f\n", t_chol, wtime() - tq);
+  return finite.load() != 0;
 }
 
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle (tiled so both reads stay in cache)
 void symmetrize_lower_host(const float* HRr, int n, double* A, int threads) {
-  if (threads <= 0) threads = omp_get_max_threads();
+  HostTeam& team = team_of_this_thread(threads);
   constexpr int T = 64;
   const int nt = (n + T - 1) / T;
-#pragma omp parallel for schedule(dynamic, 1) num_threads(threads)
-  for (int bi = 0; bi < nt; ++bi)
+  team.parallel_for(nt, 1, [&](long bil) {
+    const int bi = int(bil);
     for (int bj = 0; bj <= bi; ++bj) {
       const int i1 = std::min(n, (bi + 1) * T), j1 = std::min(n, (bj + 1) * T);
       for (int i = bi * T; i < i1; ++i)
         for (int j = bj * T; j < j1 && j <= i; ++j)
           A[size_t(i) * n + j] = 0.5 * (double(HRr[size_t(i) * n + j]) + double(HRr[size_t(j) * n + i]));
     }
+  });
 }
 
 }  // namespace qtipmi

@@ -237,6 +237,64 @@ int qtip_unswizzle_for_kernel(const uint16_t* in, int m, int n, uint16_t* packed
   return QTIP_E_ARG;
 }
 
+int qtip_run_groups(qtip_ctx* ctx, int ngroups, const qtip_group* groups, const qtip_opts* opts, qtip_timing* timings,
+                    double* ldl_wait_s) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "run_groups: bad arguments");
+    DeviceGuard g(ctx);
+    qtip_opts o;
+    qtip_default_opts(&o);
+    if (opts) o = *opts;
+    run_groups_impl(ctx, ngroups, groups, o, timings, ldl_wait_s);
+  });
+}
+
+int qtip_reserve_groups(qtip_ctx* ctx, int n) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && n > 0, "reserve_groups: bad arguments");
+    DeviceGuard g(ctx);
+    reserve_group_ring(ctx, n, 3);
+  });
+}
+
+int qtip_st_create(qtip_st_writer** out) {
+  return guarded([&] {
+    QTIP_REQUIRE(out != nullptr, "st_create: bad arguments");
+    *out = st_new();
+  });
+}
+void qtip_st_destroy(qtip_st_writer* w) { st_delete(w); }
+int qtip_st_add(qtip_st_writer* w, const char* name, const char* dtype, const int64_t* shape, int rank,
+                const void* data, uint64_t bytes) {
+  return guarded([&] { st_add(w, name, dtype, shape, rank, data, size_t(bytes)); });
+}
+int qtip_st_add_qtip_linear(qtip_st_writer* w, const char* prefix, const qtip_linear_out* out, int m, int n,
+                            const uint16_t* tlut_f16) {
+  return guarded([&] {
+    if (tlut_f16) {
+      st_add_qtip_linear(w, prefix, out, m, n, tlut_f16);
+    } else {
+      HostCodebook cb;
+      cb.build(nullptr);
+      st_add_qtip_linear(w, prefix, out, m, n, &cb.tlut_h[0][0]);
+    }
+  });
+}
+int qtip_st_write(qtip_st_writer* w, const char* path, const char* const* metadata_kv, int nmeta,
+                  uint64_t* bytes_written) {
+  return guarded([&] {
+    static const char* const kDefault[2] = {"format", "pt"};
+    const size_t b = metadata_kv ? st_write(w, path, metadata_kv, nmeta) : st_write(w, path, kDefault, 1);
+    if (bytes_written) *bytes_written = b;
+  });
+}
+int qtip_get_tlut_f16(qtip_ctx* ctx, uint16_t* host_tlut_f16) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && host_tlut_f16, "get_tlut_f16: bad arguments");
+    std::memcpy(host_tlut_f16, &ctx->cb.tlut_h[0][0], 512 * 2 * 2);
+  });
+}
+
 }  // extern "C"
 
 

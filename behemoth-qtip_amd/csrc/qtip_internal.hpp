@@ -65,6 +65,27 @@ struct DBuf {
   operator T*() const { return p; }
 };
 
+// Page-locked host buffer (staging for HRr / L), released on scope exit.
+template <class T>
+struct HBuf {
+  T* p = nullptr;
+  size_t n = 0;
+  HBuf() = default;
+  HBuf(const HBuf&) = delete;
+  HBuf& operator=(const HBuf&) = delete;
+  ~HBuf() { release(); }
+  void alloc(size_t count) {
+    release();
+    if (count) QTIP_HIP(hipHostMalloc(reinterpret_cast<void**>(&p), count * sizeof(T), hipHostMallocDefault));
+    n = count;
+  }
+  void release() {
+    if (p) (void)hipHostFree(p);
+    p = nullptr;
+    n = 0;
+  }
+};
+
 // ---- host-side number formats / streams (qtip_host.cpp)
 uint16_t f32_to_fp16(float f);
 float fp16_to_f32(uint16_t h);
@@ -112,6 +133,15 @@ struct HostScratch {
 bool block_ldl_host(double* A, int n, float* L_out, int threads);
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle
 void symmetrize_lower_host(const float* HRr, int n, double* A, int threads);
+
+// ---- layer-file writer (layer_file.cpp); the struct behind the C handle is defined there
+qtip_st_writer* st_new();
+void st_delete(qtip_st_writer* w);
+void st_add(qtip_st_writer* w, const char* name, const char* dtype, const int64_t* shape, int rank, const void* data,
+            size_t bytes);
+void st_add_qtip_linear(qtip_st_writer* w, const char* prefix, const qtip_linear_out* out, int m, int n,
+                        const uint16_t* tlut_f16);
+size_t st_write(const qtip_st_writer* w, const char* path, const char* const* meta_kv, int nmeta);
 
 // ---- GPU launchers (viterbi.hip, rht.hip, ldlq.hip)
 struct TileJob {

@@ -15,6 +15,7 @@ struct qtip_ctx {
   int vit_slots = 0;
   qtipmi::Rht rht;
   qtipmi::DBuf<double> scratch;
+  qtipmi::HBuf<float> ring_HRr[3], ring_L[3];  // page-locked staging of run_groups, kept between calls
 };
 
 namespace qtipmi {
@@ -27,4 +28,7 @@ void ldlq_impl(qtip_ctx* c, const float* dWT, const float* dL, long n, long m, f
 void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
                          double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
                          qtip_linear_out* outs, qtip_timing* tm);
+void reserve_group_ring(qtip_ctx* c, int n, int depth);
+void run_groups_impl(qtip_ctx* c, int ngroups, const qtip_group* groups, const qtip_opts& opt, qtip_timing* timings,
+                     double* ldl_wait);
 }  // namespace qtipmi

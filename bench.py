@@ -5,8 +5,9 @@ A step is one pass of the hot path over one synthetic group: Hessian rotation (G
 weight RHT + Wscale, LDLQ with the two-pass Viterbi, packing to the kernel-layout trellis.  Default workload:
 BASELINE configuration 5, the 12288 x 28672 down-proj group.  The K timed steps are K groups handled the way the
 reference's scheduler handles consecutive groups (src/pipeline.cpp:254-290): Hessians are rotated ahead of use
-(here two groups ahead, through a ring of three staging buffers), a side thread factors them in order, and the GPU
-quantizes group k as soon as its factor is ready, so the host LDL of group k+1 overlaps the GPU work of group k.
+(two groups ahead, through a ring of three staging buffers), a side thread factors them in order, and the GPU
+quantizes group k as soon as its factor is ready, so the host LDL of group k+1 overlaps the GPU work of group k;
+the scheduling is the library's own (qtip_run_groups).
 Nothing is precomputed outside the timed region; the first group's LDL is fully exposed.
 
 Prints ONE JSON line (see the keys below).  `value` is weights quantized per second over the whole timed region.
@@ -118,75 +119,21 @@ def run_group(args, pkg):
     opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=True, feedback=args.feedback)
     weights_per_step = sum(ms) * n
 
-    def pinned(shape):
-        # page-locked host buffers for HRr and L; zeroed once so that their pages are mapped on the CPU side before
-        # the clock starts (a caller's staging buffers are long-lived; first touch costs ~1.3 s per 3.3 GB here)
-        return torch.empty(shape, dtype=torch.float32, pin_memory=True).zero_().numpy()
-
-    nbuf = min(3, max(args.steps, args.warmup, 1))     # ring of staging buffers: rotate k+2 | factor k+1 | quantize k
-    su = [np.zeros(n, np.float32) for _ in range(nbuf)]
-    HRr = [pinned((n, n)) for _ in range(nbuf)]
-    Lb = [pinned((n, n)) for _ in range(nbuf)]
     stats = {}
 
     def run_steps(K, record):
-        """K groups, pipelined like consecutive groups of a layer: the Hessian of group k+2 is rotated and the one of
-        group k+1 is factored on a side thread while the GPU quantizes group k."""
-        import ctypes as C
-        L = pkg.lib()
-        creg = [C.c_double() for _ in range(K)]
-        rotated = [threading.Event() for _ in range(K)]
-        ready = [threading.Event() for _ in range(K)]
-        ldl_t = [0.0] * K
-        rot_t = [0.0] * K
-        err = []
-
-        def rotate(k):
-            t0 = time.time()
-            b = k % nbuf
-            rc = L.qtip_rotate_hessian(q._h, H.data_ptr(), 1, n, 3 + k, opt.sigma_reg, su[b].ctypes.data,
-                                       C.byref(creg[k]), HRr[b].ctypes.data)
-            if rc:
-                raise RuntimeError(L.qtip_last_error())
-            rot_t[k] = time.time() - t0
-            rotated[k].set()
-
-        for k in range(min(2, K)):
-            rotate(k)
-
-        def ldl_side():
-            for k in range(K):
-                rotated[k].wait()
-                t0 = time.time()
-                b = k % nbuf
-                rc = L.qtip_ldl_hessian(HRr[b].ctypes.data, n, args.ldl_threads, Lb[b].ctypes.data)
-                ldl_t[k] = time.time() - t0
-                if rc:
-                    err.append(L.qtip_last_error())
-                ready[k].set()
-
-        th = threading.Thread(target=ldl_side)
-        th.start()
-        tms, waits = [], []
-        for k in range(K):
-            t0 = time.time()
-            ready[k].wait()
-            waits.append(time.time() - t0)
-            if err:
-                raise RuntimeError(err[0])
-            if k + 2 < K:
-                rotate(k + 2)   # its buffers were last used by group k-1, which is finished
-            b = k % nbuf
-            hp = pkg.HessPrep(n=n, seed=3 + k, su=su[b], creg=creg[k].value, HRr=HRr[b], L=Lb[b])
-            outs, tm = q.quantize_group(lins, hp, opt)
-            tms.append(tm)
-        th.join()
+        """K groups through the library's scheduler: the Hessian of group k+2 is rotated and the one of group k+1 is
+        factored on a side thread while the GPU quantizes group k."""
+        res = q.run_groups([(lins, n, H, 3 + k) for k in range(K)], opt)
         if record:
-            stats.update(rot_s=sum(rot_t) / K, ldl_s=sum(ldl_t) / K, ldl_wait_s=sum(waits) / K,
+            tms = [r[1] for r in res]
+            stats.update(rht_s=sum(t.rht for t in tms) / K,      # Hessian rotation + weight RHT + Wscale
+                         ldl_s=sum(t.ldl_cpu for t in tms) / K, ldl_wait_s=sum(r[2] for r in res) / K,
                          ldlq_s=sum(t.ldlq for t in tms) / K, viterbi_s=sum(t.viterbi for t in tms) / K,
-                         rht_w_s=sum(t.rht for t in tms) / K, load_s=sum(t.load for t in tms) / K,
-                         pack_s=sum(t.pack for t in tms) / K, wscale=float(outs[0].wscale))
+                         load_s=sum(t.load for t in tms) / K, pack_s=sum(t.pack for t in tms) / K,
+                         wscale=float(res[-1][0][0].wscale))
 
+    q.reserve_groups(n)   # page-locked staging ring (3 x (HRr, L)); a worker keeps it for its lifetime
     if args.warmup > 0:
         run_steps(args.warmup, False)
     q.synchronize()
@@ -198,7 +145,7 @@ def run_group(args, pkg):
     wall = time.time() - t0
     ntr = sum(ms) // 16
     launches = n // 16
-    gpu_s = stats["rot_s"] + stats["rht_w_s"] + stats["load_s"] + stats["ldlq_s"] + stats["pack_s"]
+    gpu_s = stats["rht_s"] + stats["load_s"] + stats["ldlq_s"] + stats["pack_s"]
     extra = dict(stats)
     extra.update(gpu_only_Mweights_s=weights_per_step / gpu_s / 1e6,
                  serial_Mweights_s=weights_per_step / (gpu_s + stats["ldl_s"]) / 1e6,

@@ -140,6 +140,47 @@ int qtip_quantize_group_h(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, i
                           int h_on_device, uint64_t seed, const qtip_opts* opts, qtip_linear_out* outs,
                           qtip_timing* timing);
 
+/* Several groups through one context with the overlap of run_qtip_groups, src/pipeline.cpp:229-312: Hessians are
+ * rotated on the GPU ahead of use, a side thread runs the host fp64 LDL of the groups in order, and group g is
+ * quantized as soon as its factor is ready (the LDL of group g+1 overlaps the GPU work of group g).  HRr and L live
+ * in page-locked staging buffers owned by the context (a ring of three pairs, 6 n^2 floats, kept between calls).
+ * timings / ldl_wait_s (seconds the GPU side waited for each group's factor) may be NULL.  On an error the
+ * groups before the failing one are complete. */
+typedef struct {
+  int nlin;
+  const qtip_linear_in* lins;
+  qtip_linear_out* outs; /* nlin entries, caller-allocated buffers as for qtip_quantize_group */
+  int n;
+  const float* H; /* n x n fp32, host or device */
+  int h_on_device;
+  uint64_t seed;
+} qtip_group;
+int qtip_run_groups(qtip_ctx* ctx, int ngroups, const qtip_group* groups, const qtip_opts* opts, qtip_timing* timings,
+                    double* ldl_wait_s);
+/* Allocates the staging ring of qtip_run_groups for Hessians up to n x n ahead of the first call (optional). */
+int qtip_reserve_groups(qtip_ctx* ctx, int n);
+
+/* Layer file writer: the safetensors container of SafeTensorsWriter, src/safetensors.cpp:93-137 (u64 header length,
+ * JSON header with sorted keys padded to 8 bytes, tensors back to back in name order, written to path + ".tmp" and
+ * renamed).  Host only; no context needed.  dtype strings are safetensors names ("I16", "BF16", "F32", "F16", "I64",
+ * "F8_E4M3", "U8", ...); data is copied by qtip_st_add; adding a name twice replaces the tensor. */
+typedef struct qtip_st_writer qtip_st_writer;
+int qtip_st_create(qtip_st_writer** out);
+void qtip_st_destroy(qtip_st_writer* w);
+int qtip_st_add(qtip_st_writer* w, const char* name, const char* dtype, const int64_t* shape, int rank,
+                const void* data, uint64_t bytes);
+/* The six tensors of one QTIP linear under `prefix` (e.g. "model.layers.3.mlp.down_proj."), as write_layer_file
+ * stores them (src/pipeline.cpp:329-340): trellis I16 [(m/16)(n/16)][32], SU BF16 [n], SV F32 [m] = sv * wscale,
+ * tlut F16 [512][2], rcp I64 = 0, tp_rank I64 = 8.  tlut_f16 NULL takes the built-in HYB table. */
+int qtip_st_add_qtip_linear(qtip_st_writer* w, const char* prefix, const qtip_linear_out* out, int m, int n,
+                            const uint16_t* tlut_f16);
+/* metadata_kv: 2 * nmeta strings (key, value, ...); NULL writes the reference's default {"format": "pt"}.
+ * *bytes_written (may be NULL) receives the file size. */
+int qtip_st_write(qtip_st_writer* w, const char* path, const char* const* metadata_kv, int nmeta,
+                  uint64_t* bytes_written);
+/* fp16 bits of the context's codebook table [512][2] (Codebook::tlut_h, src/qtip_core.hpp:24-31) */
+int qtip_get_tlut_f16(qtip_ctx* ctx, uint16_t* host_tlut_f16);
+
 /* Host packers (pack_trellis / unpack_trellis / swizzle_for_kernel / unswizzle_for_kernel,
  * src/qtip_core.cpp:194-253) */
 void qtip_pack_trellis(const uint16_t* states, long B, uint16_t* packed);

@@ -297,3 +297,38 @@ def test_group_config2(qz, oracle, pkg, hyb, synth):
     rel1 = abs(outs1[0].proxy - ref["proxy"][0]) / ref["proxy"][0]
     say("  feedback=1: code agreement %.4f, proxy %.6f (rel %.2e)" % (agree1, outs1[0].proxy, rel1))
     assert rel1 < 0.01
+
+
+def test_run_groups_equals_group_by_group(qz, oracle, pkg, synth):
+    """The overlapped scheduler (run_qtip_groups, src/pipeline.cpp:229-312) returns, for five groups of three
+    different widths through its ring of three staging buffers, exactly what quantize_group returns one at a time;
+    a Hessian that is not positive definite stops it with the LDL's error code after the groups before it."""
+    say("case: run_groups, 5 groups")
+    qz.set_tlut(None)
+    cases = []
+    for g, (n, ms) in enumerate([(256, (64, 32)), (512, (32,)), (256, (32,)), (1024, (64,)), (512, (32, 64))]):
+        Ws, H = synth.small_group(seed=50 + g, n=n, ms=ms)
+        lins = [pkg.LinearIn("g%d_%d" % (g, k), w.shape[0], w_f32=w) for k, w in enumerate(Ws)]
+        cases.append((lins, n, H, 100 + g))
+    opt = pkg.QuantOpts(ldl_threads=8)
+    res = qz.run_groups(cases, opt)
+    assert len(res) == len(cases)
+    for (lins, n, H, seed), (outs, tm, wait) in zip(cases, res):
+        one, _ = qz.quantize_group_h(lins, n, H, seed, opt)
+        for a, b in zip(outs, one):
+            assert a.name == b.name and a.m == b.m and a.n == n
+            assert np.array_equal(a.trellis, b.trellis) and np.array_equal(a.sv, b.sv)
+            assert np.array_equal(a.su_bf16, b.su_bf16)
+            assert a.wscale == b.wscale and a.proxy == b.proxy and a.proxy_rot_reg == b.proxy_rot_reg
+        assert tm.total > 0 and tm.ldl_cpu > 0 and tm.rht > 0 and wait >= 0
+    assert qz.run_groups([], opt) == []
+    # failure in the third of four groups
+    rng = np.random.default_rng(1)
+    G = rng.standard_normal((256, 8)).astype(np.float32)
+    bad = list(cases[:2]) + [(cases[2][0], 256, G @ G.T, 5), cases[3]]
+    with pytest.raises(pkg.QtipError) as e:
+        qz.run_groups(bad, pkg.QuantOpts(ldl_threads=8, sigma_reg=0.0))
+    assert e.value.code == pkg.QTIP_E_NOT_PD
+    # the context is still usable
+    again = qz.run_groups(cases[:1], opt)
+    assert np.array_equal(again[0][0][0].trellis, res[0][0][0].trellis)
