@@ -183,4 +183,105 @@ inline const uint32_t* device_lut() {
   return nullptr;
 }
 
+// ---------------------------------------------------------------- callers either side of quantize_group
+// One Hessian group of a layer as run_qtip_groups forms it (src/pipeline.cpp:240-246,266-280).
+struct GroupSpec {
+  std::vector<LinearIn> lins;
+  int n = 0;
+  const float* H = nullptr;  // host, n x n
+  uint64_t seed = 0;
+  std::string tag;
+};
+
+// The body of run_qtip_groups (src/pipeline.cpp:247-309): rotation ahead of use, host LDL of the groups on a side
+// thread, quantize_group as factors arrive.  Returns the LinearOuts per group; tms / ldl_wait may be null.
+inline std::vector<std::vector<LinearOut>> run_groups(const std::vector<GroupSpec>& groups, const QuantOpts& opt,
+                                                      std::vector<GroupTiming>* tms = nullptr,
+                                                      std::vector<double>* ldl_wait = nullptr) {
+  if (!opt.share_su) detail::die("share_su=false not supported (one LDL per group)");
+  if (!opt.dump_dir.empty()) detail::die("dump_dir is not supported by this build");
+  const size_t ng = groups.size();
+  std::vector<std::vector<qtip_linear_in>> cin(ng);
+  std::vector<std::vector<qtip_linear_out>> cout(ng);
+  std::vector<std::vector<LinearOut>> out(ng);
+  std::vector<qtip_group> cg(ng);
+  for (size_t g = 0; g < ng; ++g) {
+    const GroupSpec& G = groups[g];
+    cin[g].resize(G.lins.size()), cout[g].resize(G.lins.size()), out[g].resize(G.lins.size());
+    for (size_t i = 0; i < G.lins.size(); ++i) {
+      const LinearIn& l = G.lins[i];
+      if (l.m <= 0 || l.m % 16 || G.n <= 0 || G.n % 16) detail::die("bad linear shape for " + G.tag);
+      cin[g][i] = qtip_linear_in{l.m, l.w_f32, l.w_bf16, l.w_fp8, l.scale_bf16, 0};
+      LinearOut& o = out[g][i];
+      o.name = l.name, o.m = l.m, o.n = G.n;
+      o.trellis.resize(size_t(l.m / 16) * (G.n / 16) * 32);
+      o.su_bf16.resize(size_t(G.n));
+      o.sv.resize(size_t(l.m));
+      if (opt.want_hatW) o.hatW.resize(size_t(l.m) * G.n);
+      cout[g][i] = qtip_linear_out{o.trellis.data(), o.su_bf16.data(), o.sv.data(),
+                                   opt.want_hatW ? o.hatW.data() : nullptr, 0.f, 0.0, 0.0, 0.0};
+    }
+    cg[g] = qtip_group{int(G.lins.size()), cin[g].data(), cout[g].data(), G.n, G.H, 0, G.seed};
+  }
+  qtip_opts co;
+  qtip_default_opts(&co);
+  co.sigma_reg = opt.sigma_reg, co.scale_override = opt.scale_override, co.ldl_threads = opt.ldl_threads;
+  std::vector<qtip_timing> ct(ng);
+  std::vector<double> waits(ng, 0.0);
+  detail::check(qtip_run_groups(detail::context(), int(ng), cg.data(), &co, ct.data(), waits.data()), "run_groups");
+  for (size_t g = 0; g < ng; ++g)
+    for (size_t i = 0; i < out[g].size(); ++i) {
+      out[g][i].wscale = cout[g][i].wscale, out[g][i].proxy = cout[g][i].proxy;
+      out[g][i].proxy_rot_reg = cout[g][i].proxy_rot_reg, out[g][i].seconds = cout[g][i].seconds;
+    }
+  if (tms) {
+    tms->clear();
+    for (auto& t : ct) tms->push_back(GroupTiming{t.load, t.rht, t.ldl_cpu, t.ldlq, t.viterbi, t.proxy, t.pack, t.total});
+  }
+  if (ldl_wait) *ldl_wait = waits;
+  return out;
+}
+
+// hatW (m x n, original domain) of a quantized linear from its packed output (the reconstruction of
+// src/quantizer.cpp:321-338 started from the trellis words; decode as runtime/src/qtip.cpp:83-118).
+inline std::vector<float> dequantize_linear(const LinearOut& lo) {
+  std::vector<float> h(size_t(lo.m) * lo.n);
+  detail::check(qtip_dequantize_linear(detail::context(), lo.trellis.data(), lo.su_bf16.data(), lo.sv.data(), lo.wscale,
+                                       lo.m, lo.n, h.data(), 0),
+                "dequantize_linear");
+  return h;
+}
+
+// src/safetensors.hpp:52-70: same calls, same file bytes.
+class SafeTensorsWriter {
+ public:
+  SafeTensorsWriter() { detail::check(qtip_st_create(&w_), "SafeTensorsWriter"); }
+  ~SafeTensorsWriter() { qtip_st_destroy(w_); }
+  SafeTensorsWriter(const SafeTensorsWriter&) = delete;
+  SafeTensorsWriter& operator=(const SafeTensorsWriter&) = delete;
+  void add(const std::string& name, const std::string& dtype, const std::vector<int64_t>& shape, const void* data,
+           size_t bytes) {
+    detail::check(qtip_st_add(w_, name.c_str(), dtype.c_str(), shape.data(), int(shape.size()), data, bytes),
+                  "SafeTensorsWriter::add");
+  }
+  // the six tensors write_layer_file stores for a QTIP linear (src/pipeline.cpp:329-340); tlut_f16 null = HYB table
+  void add_qtip_linear(const std::string& prefix, const LinearOut& r, const uint16_t* tlut_f16 = nullptr) {
+    qtip_linear_out o{const_cast<uint16_t*>(r.trellis.data()), const_cast<uint16_t*>(r.su_bf16.data()),
+                      const_cast<float*>(r.sv.data()), nullptr, r.wscale, 0.0, 0.0, 0.0};
+    detail::check(qtip_st_add_qtip_linear(w_, prefix.c_str(), &o, r.m, r.n, tlut_f16), "SafeTensorsWriter::add_qtip_linear");
+  }
+  size_t write(const std::string& path, const std::map<std::string, std::string>& metadata = {{"format", "pt"}}) const {
+    std::vector<const char*> kv;
+    for (auto& e : metadata) kv.push_back(e.first.c_str()), kv.push_back(e.second.c_str());
+    static const char* const none[2] = {nullptr, nullptr};
+    uint64_t bytes = 0;
+    detail::check(qtip_st_write(w_, path.c_str(), kv.empty() ? none : kv.data(), int(metadata.size()), &bytes),
+                  "SafeTensorsWriter::write");
+    return size_t(bytes);
+  }
+
+ private:
+  qtip_st_writer* w_ = nullptr;
+};
+
 }  // namespace qtip

@@ -5,6 +5,7 @@
 #include <cstdio>
 #include <cstring>
 #include <random>
+#include <string>
 #include <vector>
 
 #include "quantizer.hpp"
@@ -59,6 +60,38 @@ int main() {
     if (!(lo.proxy > 0 && lo.proxy < 0.2)) ++fail;
     if (std::fabs(p - lo.proxy) / lo.proxy > 1e-3) ++fail;
     if (lo.trellis.size() != size_t(lo.m / 16) * (n / 16) * 32) ++fail;
+  }
+  // the scheduler over three groups returns what quantize_group returns for each, dequantize_linear reproduces the
+  // reconstruction, and the layer file holds the tensors of both linears
+  {
+    std::vector<GroupSpec> gs(3);
+    for (int k = 0; k < 3; ++k) gs[size_t(k)] = GroupSpec{lins, n, H.data(), uint64_t(7 + k), "g" + std::to_string(k)};
+    std::vector<GroupTiming> tms;
+    std::vector<double> waits;
+    auto res = run_groups(gs, o, &tms, &waits);
+    if (res.size() != 3 || tms.size() != 3 || waits.size() != 3) ++fail;
+    for (size_t li = 0; li < out.size() && res.size() == 3; ++li) {
+      if (res[0][li].trellis != out[li].trellis || res[0][li].wscale != out[li].wscale) ++fail;
+      if (res[1][li].trellis == out[li].trellis) ++fail;  // another seed, another sign vector
+      if (dequantize_linear(res[0][li]) != out[li].hatW) ++fail;
+    }
+    std::printf("run_groups: 3 groups, ldl %.3fs ldlq %.3fs, mismatches so far %d\n", tms.empty() ? 0.0 : tms[0].ldl_cpu,
+                tms.empty() ? 0.0 : tms[0].ldlq, fail);
+    SafeTensorsWriter w;
+    w.add_qtip_linear("model.layers.0.a.", out[0]);
+    w.add_qtip_linear("model.layers.0.b.", out[1]);
+    const char* path = "/tmp/qtip_shim_test_layer.safetensors";
+    const size_t bytes = w.write(path);
+    FILE* f = std::fopen(path, "rb");
+    long sz = -1;
+    if (f) {
+      std::fseek(f, 0, SEEK_END);
+      sz = std::ftell(f);
+      std::fclose(f);
+      std::remove(path);
+    }
+    std::printf("layer file: %zu bytes\n", bytes);
+    if (sz != long(bytes) || bytes < out[0].trellis.size() * 2 + out[1].trellis.size() * 2) ++fail;
   }
   std::printf(fail ? "SHIM TEST FAILED\n" : "SHIM TEST PASSED\n");
   return fail ? 1 : 0;
