@@ -40,8 +40,14 @@ HostTeam& team_of_this_thread(int threads) {
 typedef double v8d __attribute__((vector_size(64), aligned(8)));
 typedef double v4d __attribute__((vector_size(32), aligned(8)));
 
-constexpr int NB = 256;  // panel width
-constexpr int TILE = 192;  // rows / columns of one trailing-update task (multiple of every MR and NR below)
+#ifndef QTIP_LDL_NB
+#define QTIP_LDL_NB 512
+#endif
+#ifndef QTIP_LDL_TILE
+#define QTIP_LDL_TILE 384
+#endif
+constexpr int NB = QTIP_LDL_NB;      // panel width
+constexpr int TILE = QTIP_LDL_TILE;  // rows / columns of one trailing-update task (multiple of every MR and NR below)
 
 // ---- rank-kc update of an MR x NR tile: Cij -= sum_p a[p][i] * b[p][j], a packed [kc][MR], b packed [kc][NR]
 // AVX-512: 8 x 24 (24 accumulators of 8 doubles, named so that they stay in registers)
@@ -175,26 +181,35 @@ static bool factor_diagonal(double* A, long n, int kb) {
   return true;
 }
 
-bool cholesky_lower(double* A, int n, HostTeam& team) {
+// Lower Cholesky of the n x n matrix at A (row stride ld) by right-looking panels of width NBT.  With a team the panel
+// solve and the trailing update are shared out; without one (the diagonal blocks of the outer factorization, which
+// are factored by this same routine with narrow panels) everything runs on the calling thread.
+template <int NBT, int TILET>
+bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
   double tdiag = 0, tsolve = 0, tupd = 0, tq;
   const Kernels kn = pick_kernels();
   const int MR = kn.MR, NR = kn.NR;
-  std::vector<double> packL, L11(size_t(NB) * NB), rdiag(NB);
+  std::vector<double> packL;
+  std::vector<double> L11(static_cast<size_t>(NBT) * NBT, 0.0), rdiag(static_cast<size_t>(NBT), 0.0);
   // packed copies of the solved panel (A side: MR-row micro-panels, B side: NR-row micro-panels), first panel largest
-  const size_t capA = size_t((n + MR - 1) / MR) * MR * NB, capB = size_t((n + NR - 1) / NR) * NR * NB;
+  const size_t capA = size_t((n + MR - 1) / MR) * MR * NBT, capB = size_t((n + NR - 1) / NR) * NR * NBT;
   HostScratch packs((capA + capB) * sizeof(double));
   double* const packA = static_cast<double*>(packs.get());
   double* const packB = packA + capA;
-  for (int k = 0; k < n; k += NB) {
-    const int kb = std::min(NB, n - k);
+  for (int k = 0; k < n; k += NBT) {
+    const int kb = std::min(NBT, n - k);
     tq = wtime();
-    if (!factor_diagonal(A + long(k) * n + k, n, kb)) return false;
+    if constexpr (NBT > 64) {
+      if (!cholesky_panels<64, 96>(A + long(k) * ld + k, ld, kb, nullptr, false)) return false;
+    } else {
+      if (!factor_diagonal(A + long(k) * ld + k, ld, kb)) return false;
+    }
     tdiag += wtime() - tq;
     tq = wtime();
     const int r0 = k + kb, nr = n - r0;
     if (nr <= 0) break;
     for (int j = 0; j < kb; ++j) {
-      for (int p = 0; p < kb; ++p) L11[size_t(j) * kb + p] = p <= j ? A[long(k + j) * n + k + p] : 0.0;
+      for (int p = 0; p < kb; ++p) L11[size_t(j) * kb + p] = p <= j ? A[long(k + j) * ld + k + p] : 0.0;
       rdiag[j] = 1.0 / L11[size_t(j) * kb + j];
     }
     const int nPA = (nr + MR - 1) / MR, nPB = (nr + NR - 1) / NR;
@@ -206,7 +221,7 @@ bool cholesky_lower(double* A, int n, HostTeam& team) {
     // L11 sub-block rows packed for the micro-kernel's A side: for sub-block b, tile it: [q < 64 b][MR] holding
     // L11[64 b + MR it + i][q]
     const int nsb = (kb + SUB - 1) / SUB;
-    size_t offL[NB / SUB + 1];
+    size_t offL[NBT / SUB + 1];
     {
       size_t o = 0;
       for (int b = 0; b < nsb; ++b) {
@@ -223,12 +238,12 @@ bool cholesky_lower(double* A, int n, HostTeam& team) {
       }
     }
     // panel solve in place in the packed B micro-panels (one chunk = NR rows), then write back and pack the A side
-    team.parallel_for(nPB, 2, [&](long gl) {
+    auto solve_chunk = [&](long gl) {
       const int g = int(gl);
       const int rb = g * NR, rows = std::min(NR, nr - rb);
       double* x = packB + size_t(g) * NR * kb;  // [p][NR], rows beyond `rows` stay zero
       for (int r = 0; r < rows; ++r) {
-        const double* src = A + long(r0 + rb + r) * n + k;
+        const double* src = A + long(r0 + rb + r) * ld + k;
         for (int p = 0; p < kb; ++p) x[size_t(p) * NR + r] = src[p];
       }
       for (int b = 0; b < nsb; ++b) {
@@ -241,7 +256,7 @@ bool cholesky_lower(double* A, int n, HostTeam& team) {
       }
       for (int r = 0; r < rows; ++r) {
         const int i = rb + r;
-        double* dst = A + long(r0 + i) * n + k;
+        double* dst = A + long(r0 + i) * ld + k;
         double* pa = packA + size_t(i / MR) * MR * kb + (i % MR);
         for (int p = 0; p < kb; ++p) {
           const double v = x[size_t(p) * NR + r];
@@ -249,13 +264,16 @@ bool cholesky_lower(double* A, int n, HostTeam& team) {
           pa[size_t(p) * MR] = v;
         }
       }
-    });
+    };
+    if (team) team->parallel_for(nPB, 2, solve_chunk);
+    else
+      for (long gl = 0; gl < nPB; ++gl) solve_chunk(gl);
     tsolve += wtime() - tq;
     tq = wtime();
     // trailing update of the lower triangle, tiles (bi, bj <= bi) largest rows first
-    const int nT = (nr + TILE - 1) / TILE;
+    const int nT = (nr + TILET - 1) / TILET;
     const long ntask = long(nT) * (nT + 1) / 2;
-    team.parallel_for(ntask, 1, [&](long task) {
+    auto update_tile = [&](long task) {
       // enumerate from the bottom row block upwards: row block bi has bi+1 tiles
       long rem = task;
       int bi = nT - 1;
@@ -264,20 +282,23 @@ bool cholesky_lower(double* A, int n, HostTeam& team) {
         --bi;
       }
       const int bj = int(rem);
-      const int i0 = bi * TILE, i1 = std::min(nr, i0 + TILE), j0 = bj * TILE, j1 = std::min(nr, j0 + TILE);
+      const int i0 = bi * TILET, i1 = std::min(nr, i0 + TILET), j0 = bj * TILET, j1 = std::min(nr, j0 + TILET);
       for (int jj = j0; jj < j1; jj += NR) {
         const double* pb = packB + size_t(jj / NR) * NR * kb;
         const int nrr = std::min(NR, nr - jj);
         for (int ii = i0; ii < i1; ii += MR) {
           if (jj > ii + MR - 1) continue;  // micro tile entirely above the diagonal
           const int mrr = std::min(MR, nr - ii);
-          kn.micro(kb, packA + size_t(ii / MR) * MR * kb, pb, A + long(r0 + ii) * n + r0 + jj, n, mrr, nrr);
+          kn.micro(kb, packA + size_t(ii / MR) * MR * kb, pb, A + long(r0 + ii) * ld + r0 + jj, ld, mrr, nrr);
         }
       }
-    });
+    };
+    if (team) team->parallel_for(ntask, 1, update_tile);
+    else
+      for (long task = 0; task < ntask; ++task) update_tile(task);
     tupd += wtime() - tq;
   }
-  if (getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "chol: diag %.3f solve+pack %.3f update %.3f\n", tdiag, tsolve, tupd);
+  if (top && getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "chol: diag %.3f solve+pack %.3f update %.3f\n", tdiag, tsolve, tupd);
   return true;
 }
 
@@ -287,7 +308,7 @@ bool block_ldl_host(double* A, int n, float* L_out, int threads) {
   if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
   HostTeam& team = team_of_this_thread(threads);
   double tq = wtime();
-  if (!cholesky_lower(A, n, team)) return false;
+  if (!cholesky_panels<NB, TILE>(A, n, n, &team, true)) return false;
   const double t_chol = wtime() - tq;
   tq = wtime();
   const int nb = n / 16;
