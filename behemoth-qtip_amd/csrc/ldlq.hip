@@ -5,9 +5,10 @@
 //    column targets in registers, the <= 112 rows of L of the open buffer sit in LDS.  fp64 accumulation (the
 //    CPU algorithm's precision: fp64 is full rate on CDNA4 VALUs), result rounded fp64 -> fp32 -> fp16 like
 //    the CPU path and written in trellis sequence order.
-//  * gemm_tn: C[M][N] (+)= sum_k A[k][i] * (B1 - B2)[k][j] on the fp64 matrix cores
-//    (v_mfma_f64_16x16x4_f64), fp32 operands widened while staging through LDS.  Two epilogues: accumulate
-//    into C (the cross-buffer prod cache), or reduce sum(acc * (B1 - B2)[i][j]) for tr(X^T H X) (the proxy).
+//  * gemm_tn: sum_k A[k][i] * (B1 - B2)[k][j] on the fp64 matrix cores (v_mfma_f64_16x16x4_f64), fp32 operands
+//    widened while staging through LDS.  The cross-buffer feedback ("prod cache") of a 128-column buffer is gathered
+//    from all rows quantized so far by a K-split kernel; a second kernel reduces sum(acc * (B1 - B2)[i][j]) for
+//    tr(X^T H X) (the proxy).
 //  * gemm_tn_bf16x3: the same prod-cache update with fp32 C and the operands split into bf16 hi + lo
 //    (v_mfma_f32_32x32x16_bf16, three terms), the arithmetic of the reference's GPU path.
 #include <hip/hip_fp16.h>
@@ -26,7 +27,8 @@ __device__ __forceinline__ int perm_inv(int q) {  // tile index 16*r + c -> sequ
 template <typename ProdT>
 __global__ __launch_bounds__(256) void ldlq_prep_kernel(const float* __restrict__ WT, const float* __restrict__ hatWT,
                                                         const ProdT* __restrict__ prod, const float* __restrict__ L,
-                                                        long n, long m, int col0, int bufend, float* __restrict__ X) {
+                                                        long n, long m, int col0, int bufend, int prod_row0,
+                                                        float* __restrict__ X) {
   __shared__ ProdT Ls[112][16];
   const int k0 = col0 + 16, nk = bufend - k0;
   for (int idx = threadIdx.x; idx < nk * 16; idx += blockDim.x) {
@@ -38,7 +40,7 @@ __global__ __launch_bounds__(256) void ldlq_prep_kernel(const float* __restrict_
   if (j >= m) return;
   ProdT acc[16];
 #pragma unroll
-  for (int c = 0; c < 16; ++c) acc[c] = ProdT(WT[long(col0 + c) * m + j]) + prod[long(col0 + c) * m + j];
+  for (int c = 0; c < 16; ++c) acc[c] = ProdT(WT[long(col0 + c) * m + j]) + prod[long(col0 + c - prod_row0) * m + j];
   for (int kk = 0; kk < nk; ++kk) {
     const long o = long(k0 + kk) * m + j;
     const ProdT dk = ProdT(WT[o]) - ProdT(hatWT[o]);
@@ -146,6 +148,95 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_f64_kernel(int M, int N, int K
     __syncthreads();
     if (t == 0) partial[long(blockIdx.y) * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
   }
+}
+
+// ---------------------------------------------------------------- fp64 MFMA GEMM, 128 output rows, K split
+// out[y][i][j] = sum over the K slices of split y of A[k][i] * (B1 - B2)[k][j], i < 128: the cross-buffer feedback
+// of one 128-column LDLQ buffer gathered from all rows already quantized ("left-looking": every product term is
+// read once and nothing is read-modified-written).  K is long and the output small, so the K range is shared out
+// over gridDim.y workgroups per column tile and the partial tiles are summed afterwards in a fixed order.  The next
+// K slice is fetched into registers while the matrix cores work on the current one.
+__global__ __launch_bounds__(256, 2) void gemm_tn_f64_splitk_kernel(int N, long K, const float* __restrict__ A, long lda,
+                                                                    const float* __restrict__ B1,
+                                                                    const float* __restrict__ B2, long ldb,
+                                                                    double* __restrict__ out, long ldo) {
+  __shared__ __attribute__((aligned(16))) double As[KC][BM];
+  __shared__ __attribute__((aligned(16))) double Bs[KC][BN];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const long j0 = long(blockIdx.x) * BN;
+  const long slices = (K + KC - 1) / KC;
+  const long s0 = slices * blockIdx.y / gridDim.y, s1 = slices * (blockIdx.y + 1) / gridDim.y;
+  double4_t acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
+  const int lk = t >> 5, lc = (t & 31) * 4;  // this thread stages rows lk and lk + 8 of a slice, 4 columns at lc
+  const bool b_ok = j0 + lc + 3 < N;
+  float4 ga[2], gb[2], gc[2];
+  auto fetch = [&](long slice) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const long k = slice * KC + lk + 8 * r;
+      ga[r] = gb[r] = gc[r] = float4{0.f, 0.f, 0.f, 0.f};
+      if (k < K) {
+        ga[r] = *reinterpret_cast<const float4*>(A + k * lda + lc);
+        if (b_ok) {
+          gb[r] = *reinterpret_cast<const float4*>(B1 + k * ldb + j0 + lc);
+          gc[r] = *reinterpret_cast<const float4*>(B2 + k * ldb + j0 + lc);
+        }
+      }
+    }
+  };
+  if (s0 < s1) fetch(s0);
+  for (long sl = s0; sl < s1; ++sl) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int k = lk + 8 * r;
+      *reinterpret_cast<double2*>(&As[k][lc]) = double2{double(ga[r].x), double(ga[r].y)};
+      *reinterpret_cast<double2*>(&As[k][lc + 2]) = double2{double(ga[r].z), double(ga[r].w)};
+      *reinterpret_cast<double2*>(&Bs[k][lc]) = double2{double(gb[r].x) - double(gc[r].x), double(gb[r].y) - double(gc[r].y)};
+      *reinterpret_cast<double2*>(&Bs[k][lc + 2]) = double2{double(gb[r].z) - double(gc[r].z), double(gb[r].w) - double(gc[r].w)};
+    }
+    __syncthreads();
+    if (sl + 1 < s1) fetch(sl + 1);
+#pragma unroll
+    for (int kk = 0; kk < KC; kk += 4) {
+      const int kr = kk + (lane >> 4), c = lane & 15;
+      double a[4], b[4];
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) a[mi] = As[kr][wm * 64 + mi * 16 + c];
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) b[ni] = Bs[kr][wn * 64 + ni * 16 + c];
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni)
+          acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  double* o = out + long(blockIdx.y) * BM * ldo;
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const long gi = wm * 64 + mi * 16 + (lane >> 4) + 4 * v;
+        const long gj = j0 + wn * 64 + ni * 16 + (lane & 15);
+        if (gj < N) o[gi * ldo + gj] = acc[mi][ni][v];
+      }
+}
+
+// P[i] = part[0][i] + part[1][i] + ... (in this order), i < count
+__global__ void sum_splits_kernel(const double* __restrict__ part, int splits, long count, double* __restrict__ P) {
+  const long i = long(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  double s = part[i];
+  for (int k = 1; k < splits; ++k) s += part[long(k) * count + i];
+  P[i] = s;
 }
 
 // ---------------------------------------------------------------- bf16 hi/lo split MFMA GEMM (fp32 accumulate)
@@ -275,28 +366,42 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(const double* __restr
 
 }  // namespace
 
-void launch_ldlq_prep_f64(const float* WT, const float* hatWT, const double* prod, const float* L, long n, long m,
-                          int col0, int bufend, float* X, hipStream_t s) {
+void launch_ldlq_prep_f64(const float* WT, const float* hatWT, const double* prod, int prod_row0, const float* L, long n,
+                          long m, int col0, int bufend, float* X, hipStream_t s) {
   QTIP_REQUIRE(bufend - col0 - 16 <= 112 && bufend - col0 - 16 >= 0, "ldlq_prep: block outside its buffer");
+  QTIP_REQUIRE(col0 >= prod_row0, "ldlq_prep: block outside the prod slab");
   ldlq_prep_kernel<double><<<dim3(unsigned((m + 255) / 256)), dim3(256), 0, s>>>(WT, hatWT, prod, L, n, m, col0,
-                                                                                 bufend, X);
+                                                                                 bufend, prod_row0, X);
   QTIP_HIP(hipGetLastError());
 }
 void launch_ldlq_prep_f32(const float* WT, const float* hatWT, const float* prod, const float* L, long n, long m,
                           int col0, int bufend, float* X, hipStream_t s) {
   QTIP_REQUIRE(bufend - col0 - 16 <= 112 && bufend - col0 - 16 >= 0, "ldlq_prep: block outside its buffer");
   ldlq_prep_kernel<float><<<dim3(unsigned((m + 255) / 256)), dim3(256), 0, s>>>(WT, hatWT, prod, L, n, m, col0,
-                                                                                bufend, X);
+                                                                                bufend, 0, X);
   QTIP_HIP(hipGetLastError());
 }
 
-void launch_gemm_tn_f64_acc(int M, int N, int K, const float* A, long lda, const float* B1, const float* B2, long ldb,
-                            double* C, long ldc, hipStream_t s) {
-  if (M <= 0 || N <= 0 || K <= 0) return;
-  QTIP_REQUIRE(M % 4 == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0, "fp64 GEMM needs 16-byte aligned fp32 rows");
-  dim3 grid(unsigned((N + BN - 1) / BN), unsigned((M + BM - 1) / BM));
-  gemm_tn_f64_kernel<0><<<grid, dim3(256), 0, s>>>(M, N, K, A, lda, B1, B2, ldb, C, ldc, nullptr);
+int gemm_splitk_splits(long K) {
+  // 96 column tiles x 5 splits keep every CU's two workgroup slots busy at m = 12288; short K ranges are not split
+  // below 512 rows
+  const long s = K / 512;
+  return int(s < 1 ? 1 : (s > 5 ? 5 : s));
+}
+
+void launch_gemm_tn_f64_gather(int N, long K, const float* A, long lda, const float* B1, const float* B2, long ldb,
+                               double* P, double* partials, hipStream_t s) {
+  QTIP_REQUIRE(N > 0 && K > 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 && B2 != nullptr,
+               "fp64 gather GEMM needs 16-byte aligned fp32 rows");
+  const int S = gemm_splitk_splits(K);
+  dim3 grid(unsigned((N + BN - 1) / BN), unsigned(S));
+  gemm_tn_f64_splitk_kernel<<<grid, dim3(256), 0, s>>>(N, K, A, lda, B1, B2, ldb, S == 1 ? P : partials, N);
   QTIP_HIP(hipGetLastError());
+  if (S > 1) {
+    const long count = long(BM) * N;
+    sum_splits_kernel<<<dim3(unsigned((count + 255) / 256)), dim3(256), 0, s>>>(partials, S, count, P);
+    QTIP_HIP(hipGetLastError());
+  }
 }
 
 void launch_gemm_tn_bf16x3_acc(int M, int N, int K, const float* A, long lda, const float* B1, const float* B2, long ldb,

@@ -77,11 +77,11 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   const long ntr = m / 16, nblk = n / 16;
   // feedback 0: fp64 feedback sums and fp64 prod cache; feedback 1: fp32 sums, fp32 prod cache updated by the
   // bf16 hi/lo split MFMA product
-  DBuf<double> prod(feedback == 0 ? size_t(n) * m : 0);
+  // feedback 0: the feedback of the rows quantized in earlier buffers is gathered per buffer into a 128 x m slab
+  DBuf<double> prod(feedback == 0 ? size_t(128) * m : 0), parts(feedback == 0 ? size_t(5) * 128 * m : 0);
   DBuf<float> prod32(feedback == 1 ? size_t(n) * m : 0);
   DBuf<float> X(size_t(ntr) * 256);
-  if (feedback == 0) QTIP_HIP(hipMemsetAsync(prod, 0, prod.bytes(), s));
-  else QTIP_HIP(hipMemsetAsync(prod32, 0, prod32.bytes(), s));
+  if (feedback == 1) QTIP_HIP(hipMemsetAsync(prod32, 0, prod32.bytes(), s));
   QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
   std::vector<hipEvent_t> ev;
   auto mark = [&] {
@@ -98,9 +98,16 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   for (long cur = nblk; cur > 0; cur -= 8, ++nbuf_done) {
     const int bufend = int(16 * cur), c0 = bufend - 128;
     if (nbuf_done >= 2) QTIP_HIP(hipEventSynchronize(pace[(nbuf_done - 2) % 3]));
+    if (feedback == 0) {  // prod[r][:] = sum_{k >= bufend} L[k][c0 + r] (WT - hatWT)[k][:], r < 128
+      if (bufend < n)
+        launch_gemm_tn_f64_gather(int(m), n - bufend, L + long(bufend) * n + c0, n, WT + long(bufend) * m,
+                                  hatWT + long(bufend) * m, m, prod, parts, s);
+      else
+        QTIP_HIP(hipMemsetAsync(prod, 0, prod.bytes(), s));
+    }
     for (int i = 7; i >= 0; --i) {
       const int col0 = c0 + 16 * i;
-      if (feedback == 0) launch_ldlq_prep_f64(WT, hatWT, prod, L, n, m, col0, bufend, X, s);
+      if (feedback == 0) launch_ldlq_prep_f64(WT, hatWT, prod, c0, L, n, m, col0, bufend, X, s);
       else launch_ldlq_prep_f32(WT, hatWT, prod32, L, n, m, col0, bufend, X, s);
       if (vit_seconds) mark();
       TileJob job;
@@ -115,12 +122,9 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
       launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws, c->vit_slots, s);
       if (vit_seconds) mark();
     }
-    if (c0 > 0) {  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
-      if (feedback == 0)
-        launch_gemm_tn_f64_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m, prod, m, s);
-      else
-        launch_gemm_tn_bf16x3_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m,
-                                  prod32, m, s);
+    if (c0 > 0 && feedback == 1) {  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
+      launch_gemm_tn_bf16x3_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m,
+                                prod32, m, s);
     }
     QTIP_HIP(hipEventRecord(pace[nbuf_done % 3], s));
   }
