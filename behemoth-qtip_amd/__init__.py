@@ -101,6 +101,8 @@ def lib():
                                       C.POINTER(_LinearOutC), C.POINTER(_TimingC)]
     L.qtip_quantize_group_h.argtypes = [vp, i, C.POINTER(_LinearInC), i, vp, i, u64, C.POINTER(_OptsC),
                                         C.POINTER(_LinearOutC), C.POINTER(_TimingC)]
+    L.qtip_hessian_accumulate_dev.argtypes = [vp, vp, l, i, vp]
+    L.qtip_hessian_finish_dev.argtypes = [vp, vp, i, d]
     L.qtip_run_groups.argtypes = [vp, i, vp, C.POINTER(_OptsC), vp, vp]
     L.qtip_reserve_groups.argtypes = [vp, i]
     L.qtip_st_create.argtypes = [C.POINTER(vp)]
@@ -379,6 +381,14 @@ class Quantizer:
                                            C.byref(co), cout, C.byref(tm)))
         return self._finish(cout, outs, tm)
 
+
+    def hessian_accumulate_dev(self, dX_bf16, rows, n, dH):
+        """dH (n x n fp32, device) += X^T X for dX_bf16 (rows x n bf16 bits, device); src/model.cpp:352-363."""
+        _check(lib().qtip_hessian_accumulate_dev(self._h, _ptr(dX_bf16), rows, n, _ptr(dH)))
+
+    def hessian_finish_dev(self, dH, n, scale=1.0):
+        """Mirror the computed triangle and scale (src/model.cpp:260-264, src/pipeline.cpp:160-166)."""
+        _check(lib().qtip_hessian_finish_dev(self._h, _ptr(dH), n, float(scale)))
 
     def reserve_groups(self, n):
         _check(lib().qtip_reserve_groups(self._h, n))

@@ -1,0 +1,205 @@
+// Hessian accumulation, the step that feeds the group quantizer: H (n x n fp32) += X^T X for a batch X of `rows`
+// activation vectors (rows x n bf16, row-major).  Reference: the hess() lambda of LayerRunner::forward_batch,
+// src/model.cpp:352-363 (a bf16 GEMM with fp32 accumulation over the 10 blocks bi <= bj of a 4 x 4 partition),
+// symmetrize_hess / k_symmetrize_blocks (src/model.cpp:260-264, src/kernels.hip:465-474) and the division by the
+// token count (src/pipeline.cpp:160-166).
+//
+// A symmetric rank-`rows` update on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16, fp32 accumulate).  Only the
+// 256 x 256 tiles on or below the diagonal are computed (50.4 % of the square at n = 28672, against 62.5 % for the
+// 4 x 4 block schedule); hessian_finish mirrors them into the other triangle and scales.
+//
+// One 256-thread workgroup per tile, one workgroup per CU: a wave owns 128 x 128 outputs (4 x 4 MFMA tiles, 256
+// accumulator registers).  Both operands are column slices of X and the contraction runs over the rows of X, so the
+// matrix cores want, per lane, 8 consecutive rows of one column, while memory has the columns contiguous: every
+// thread loads an 8 row x 8 column block (eight 16-byte loads, whole 128-byte lines per wave), transposes it in
+// registers (v_perm_b32) and writes eight 16-byte column pieces to LDS ([column][row], 144-byte pitch: conflict-free
+// for the writes and for the lanes' 16-byte fragment reads).  Two LDS stages of 64 rows: the next stage is fetched
+// and written while the matrix cores work on the current one.  Workgroups are numbered so that the 32 that share an
+// XCD (and its L2) at a time form an 8 x 4 patch of tiles, which needs 12 operand slices instead of 33.
+#include "misc.hpp"
+#include "qtip_internal.hpp"
+
+namespace qtipmi {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kTile = 256;    // output tile edge
+constexpr int kStage = 64;    // rows of X per LDS stage
+constexpr int kPitch = 72;    // u16 per LDS row: 64 rows of X + 8 padding (144 bytes)
+constexpr int kSliceU16 = kTile * kPitch;                 // one operand slice in LDS
+constexpr size_t kLdsBytes = size_t(4) * kSliceU16 * 2;   // 2 stages x (A, B)
+constexpr int kPatchRows = 8, kPatchCols = 4;             // tiles per XCD patch
+
+struct Block8x8 {
+  uint4 r[8];  // r[q]: 8 consecutive columns of row q
+};
+
+__device__ __forceinline__ void fetch_block(Block8x8& b, const uint16_t* __restrict__ X, long rows, long n, long row0,
+                                            long col0) {
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    b.r[q] = uint4{0u, 0u, 0u, 0u};
+    if (row0 + q < rows && col0 + 7 < n) b.r[q] = *reinterpret_cast<const uint4*>(X + (row0 + q) * n + col0);
+  }
+}
+
+// column c of the block as 8 consecutive rows (4 dwords), written to dst[c * kPitch .. ]
+__device__ __forceinline__ void store_block_transposed(const Block8x8& b, uint16_t* dst) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const uint32_t w[8] = {d == 0 ? b.r[0].x : d == 1 ? b.r[0].y : d == 2 ? b.r[0].z : b.r[0].w,
+                           d == 0 ? b.r[1].x : d == 1 ? b.r[1].y : d == 2 ? b.r[1].z : b.r[1].w,
+                           d == 0 ? b.r[2].x : d == 1 ? b.r[2].y : d == 2 ? b.r[2].z : b.r[2].w,
+                           d == 0 ? b.r[3].x : d == 1 ? b.r[3].y : d == 2 ? b.r[3].z : b.r[3].w,
+                           d == 0 ? b.r[4].x : d == 1 ? b.r[4].y : d == 2 ? b.r[4].z : b.r[4].w,
+                           d == 0 ? b.r[5].x : d == 1 ? b.r[5].y : d == 2 ? b.r[5].z : b.r[5].w,
+                           d == 0 ? b.r[6].x : d == 1 ? b.r[6].y : d == 2 ? b.r[6].z : b.r[6].w,
+                           d == 0 ? b.r[7].x : d == 1 ? b.r[7].y : d == 2 ? b.r[7].z : b.r[7].w};
+    uint4 even, odd;  // columns 2d and 2d + 1: (row 0, row 1), (2, 3), (4, 5), (6, 7)
+    even.x = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u);
+    even.y = __builtin_amdgcn_perm(w[3], w[2], 0x05040100u);
+    even.z = __builtin_amdgcn_perm(w[5], w[4], 0x05040100u);
+    even.w = __builtin_amdgcn_perm(w[7], w[6], 0x05040100u);
+    odd.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
+    odd.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
+    odd.z = __builtin_amdgcn_perm(w[5], w[4], 0x07060302u);
+    odd.w = __builtin_amdgcn_perm(w[7], w[6], 0x07060302u);
+    *reinterpret_cast<uint4*>(dst + (2 * d) * kPitch) = even;
+    *reinterpret_cast<uint4*>(dst + (2 * d + 1) * kPitch) = odd;
+  }
+}
+
+__global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __restrict__ X, long rows, long n,
+                                                          float* __restrict__ H, int tiles, int patch_cols) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  // workgroup -> tile: ids that differ by 8 run on different XCDs; the 32 ids an XCD holds at a time are one patch
+  const long b = blockIdx.x;
+  const long xcd = b & 7, local = b >> 3;
+  const long patch = (local / (kPatchRows * kPatchCols)) * 8 + xcd, within = local % (kPatchRows * kPatchCols);
+  const long ti = (patch / patch_cols) * kPatchRows + within / kPatchCols;
+  const long tj = (patch % patch_cols) * kPatchCols + within % kPatchCols;
+  if (ti >= tiles || tj > ti) return;  // outside the matrix or above the diagonal
+  const bool diag = ti == tj;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int ro = t & 7, cg = t >> 3;  // this thread stages rows 8 ro .. 8 ro + 7, columns 8 cg .. 8 cg + 7 of a slice
+  const long ci = ti * kTile + 8 * cg, cj = tj * kTile + 8 * cg;
+  uint16_t* const wr = lds + (8 * cg) * kPitch + 8 * ro;  // within a slice
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][c][v] = 0.f;
+
+  const long stages = (rows + kStage - 1) / kStage;
+  Block8x8 ga, gb;
+  fetch_block(ga, X, rows, n, 8 * ro, ci);
+  if (!diag) fetch_block(gb, X, rows, n, 8 * ro, cj);
+  store_block_transposed(ga, wr);
+  if (!diag) store_block_transposed(gb, wr + kSliceU16);
+  __syncthreads();
+
+  const int kq = 8 * (lane >> 5), rl = lane & 31;
+  for (long st = 0; st < stages; ++st) {
+    const uint16_t* As = lds + (st & 1) * 2 * kSliceU16;
+    const uint16_t* Bs = diag ? As : As + kSliceU16;
+    const bool more = st + 1 < stages;
+    if (more) {
+      fetch_block(ga, X, rows, n, (st + 1) * kStage + 8 * ro, ci);
+      if (!diag) fetch_block(gb, X, rows, n, (st + 1) * kStage + 8 * ro, cj);
+    }
+#pragma unroll
+    for (int ks = 0; ks < kStage / 16; ++ks) {
+      bf16x8 fa[4], fb[4];
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+        fa[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + (wm * 128 + mi * 32 + rl) * kPitch + ks * 16 + kq));
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni)
+        fb[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Bs + (wn * 128 + ni * 32 + rl) * kPitch + ks * 16 + kq));
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni)
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
+    }
+    if (more) {
+      uint16_t* nxt = lds + ((st + 1) & 1) * 2 * kSliceU16 + (8 * cg) * kPitch + 8 * ro;
+      store_block_transposed(ga, nxt);
+      if (!diag) store_block_transposed(gb, nxt + kSliceU16);
+    }
+    __syncthreads();
+  }
+  // accumulator element v of a lane: row (v % 4) + 8 (v / 4) + 4 (lane / 32), column lane % 32 of the 32 x 32 tile
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const long gi = ti * kTile + wm * 128 + mi * 32 + (v & 3) + 8 * (v >> 2) + 4 * (lane >> 5);
+        const long gj = tj * kTile + wn * 128 + ni * 32 + rl;
+        if (gi < n && gj < n) H[gi * n + gj] += acc[mi][ni][v];
+      }
+}
+
+// H[i][j] for j > i takes H[j][i] (computed tiles hold the lower triangle and the whole diagonal tiles); everything
+// is scaled.  32 x 32 patches through LDS so both the read and the write are row segments.
+__global__ __launch_bounds__(256) void hessian_finish_kernel(float* __restrict__ H, long n, float scale) {
+  __shared__ float tile[32][33];
+  const long bi = blockIdx.y, bj = blockIdx.x;
+  if (bj > bi) return;  // the patch pair (bi, bj), (bj, bi) is handled by the lower one
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const long i = bi * 32 + ty + 8 * k, j = bj * 32 + tx;
+    float v = 0.f;
+    if (i < n && j < n) {
+      v = H[i * n + j] * scale;
+      if (bi != bj || j <= i) H[i * n + j] = v;
+    }
+    tile[ty + 8 * k][tx] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const long i = bj * 32 + ty + 8 * k, j = bi * 32 + tx;  // element (i, j) of the mirrored patch = lower (j, i)
+    if (i < n && j < n && (bi != bj || j > i)) H[i * n + j] = tile[tx][ty + 8 * k];
+  }
+}
+
+}  // namespace
+
+void launch_hessian_accumulate(const uint16_t* X, long rows, long n, float* H, hipStream_t s) {
+  QTIP_REQUIRE(X != nullptr && H != nullptr && rows >= 0 && n > 0, "hessian_accumulate: bad arguments");
+  QTIP_REQUIRE(n % 8 == 0 && (reinterpret_cast<uintptr_t>(X) & 15) == 0, "hessian_accumulate: rows of X must be 16-byte aligned (n = %ld)", n);
+  if (rows == 0) return;
+  static bool configured = false;  // per process; the attribute belongs to the function, not to a device context
+  if (!configured) {
+    QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 int(kLdsBytes)));
+    configured = true;
+  }
+  const int tiles = int((n + kTile - 1) / kTile);
+  const int patch_rows = (tiles + kPatchRows - 1) / kPatchRows, patch_cols = (tiles + kPatchCols - 1) / kPatchCols;
+  const long patches = long(patch_rows) * patch_cols;
+  const long padded = (patches + 7) / 8 * 8;  // whole rounds over the 8 XCDs
+  const long grid = padded * kPatchRows * kPatchCols;
+  QTIP_REQUIRE(grid < (1l << 31), "hessian_accumulate: n too large (%ld)", n);
+  syrk_bf16_kernel<<<dim3(unsigned(grid)), dim3(256), kLdsBytes, s>>>(X, rows, n, H, tiles, patch_cols);
+  QTIP_HIP(hipGetLastError());
+}
+
+void launch_hessian_finish(float* H, long n, float scale, hipStream_t s) {
+  QTIP_REQUIRE(H != nullptr && n > 0, "hessian_finish: bad arguments");
+  const unsigned nb = unsigned((n + 31) / 32);
+  hessian_finish_kernel<<<dim3(nb, nb), dim3(256), 0, s>>>(H, n, scale);
+  QTIP_HIP(hipGetLastError());
+}
+
+}  // namespace qtipmi

@@ -9,4 +9,7 @@ void launch_pack_swizzle(const uint16_t* Q, long m, long n, uint16_t* out, hipSt
 // kernel-layout trellis words of one linear -> hatWr (m x n fp32, row stride ld): lookup of every 16-bit window (decode.hip)
 void launch_decode_trellis(const uint16_t* trellis, long m, long n, const float* entry_f, float* out, long ld,
                            hipStream_t s);
+// H (n x n fp32) += X^T X for X = rows x n bf16, tiles on or below the diagonal only; then mirror + scale (hessian.hip)
+void launch_hessian_accumulate(const uint16_t* X, long rows, long n, float* H, hipStream_t s);
+void launch_hessian_finish(float* H, long n, float scale, hipStream_t s);
 }  // namespace qtipmi

@@ -237,6 +237,21 @@ int qtip_unswizzle_for_kernel(const uint16_t* in, int m, int n, uint16_t* packed
   return QTIP_E_ARG;
 }
 
+int qtip_hessian_accumulate_dev(qtip_ctx* ctx, const uint16_t* dev_X_bf16, long rows, int n, float* dev_H) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "hessian_accumulate: bad arguments");
+    DeviceGuard g(ctx);
+    launch_hessian_accumulate(dev_X_bf16, rows, n, dev_H, ctx->stream);
+  });
+}
+int qtip_hessian_finish_dev(qtip_ctx* ctx, float* dev_H, int n, double scale) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "hessian_finish: bad arguments");
+    DeviceGuard g(ctx);
+    launch_hessian_finish(dev_H, n, float(scale), ctx->stream);
+  });
+}
+
 int qtip_run_groups(qtip_ctx* ctx, int ngroups, const qtip_group* groups, const qtip_opts* opts, qtip_timing* timings,
                     double* ldl_wait_s) {
   return guarded([&] {

@@ -140,6 +140,15 @@ int qtip_quantize_group_h(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, i
                           int h_on_device, uint64_t seed, const qtip_opts* opts, qtip_linear_out* outs,
                           qtip_timing* timing);
 
+/* Hessian accumulation, the step before the path (hess() in LayerRunner::forward_batch, src/model.cpp:352-363):
+ * dev_H (n x n fp32, row-major) += X^T X for a batch of `rows` activation vectors dev_X (rows x n raw bf16 bits,
+ * row-major), bf16 products with fp32 accumulation on the matrix cores.  Only the 256 x 256 tiles on or below the
+ * diagonal are updated; qtip_hessian_finish_dev mirrors them into the other triangle and multiplies by `scale`
+ * (symmetrize_hess, src/model.cpp:260-264, and the 1 / token count of src/pipeline.cpp:160-166).  n % 8 == 0.
+ * Asynchronous on the context's stream. */
+int qtip_hessian_accumulate_dev(qtip_ctx* ctx, const uint16_t* dev_X_bf16, long rows, int n, float* dev_H);
+int qtip_hessian_finish_dev(qtip_ctx* ctx, float* dev_H, int n, double scale);
+
 /* Several groups through one context with the overlap of run_qtip_groups, src/pipeline.cpp:229-312: Hessians are
  * rotated on the GPU ahead of use, a side thread runs the host fp64 LDL of the groups in order, and group g is
  * quantized as soon as its factor is ready (the LDL of group g+1 overlaps the GPU work of group g).  HRr and L live
