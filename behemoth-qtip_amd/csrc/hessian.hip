@@ -12,8 +12,8 @@
 // accumulator registers).  Both operands are column slices of X and the contraction runs over the rows of X, so the
 // matrix cores want, per lane, 8 consecutive rows of one column, while memory has the columns contiguous: every
 // thread loads an 8 row x 8 column block (eight 16-byte loads, whole 128-byte lines per wave), transposes it in
-// registers (v_perm_b32) and writes eight 16-byte column pieces to LDS ([column][row], 144-byte pitch: conflict-free
-// for the writes and for the lanes' 16-byte fragment reads).  Two LDS stages of 64 rows: the next stage is fetched
+// registers (v_perm_b32) and writes eight 16-byte column pieces to LDS ([column][row], 128-byte pitch with the pieces
+// XOR-swizzled: conflict-free for the writes and for the lanes' 16-byte fragment reads).  Two LDS stages of 64 rows: the next stage is fetched
 // and written while the matrix cores work on the current one.  Workgroups are numbered so that the 32 that share an
 // XCD (and its L2) at a time form an 8 x 4 patch of tiles, which needs 12 operand slices instead of 33.
 #include "misc.hpp"
@@ -27,7 +27,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kTile = 256;    // output tile edge
 constexpr int kStage = 64;    // rows of X per LDS stage
-constexpr int kPitch = 72;    // u16 per LDS row: 64 rows of X + 8 padding (144 bytes)
+constexpr int kPitch = 64;    // u16 per LDS row: the 64 rows of X of one stage (128 bytes), 16-byte pieces XOR-swizzled
 constexpr int kSliceU16 = kTile * kPitch;                 // one operand slice in LDS
 constexpr size_t kLdsBytes = size_t(4) * kSliceU16 * 2;   // 2 stages x (A, B)
 constexpr int kPatchRows = 8, kPatchCols = 4;             // tiles per XCD patch
@@ -36,39 +36,148 @@ struct Block8x8 {
   uint4 r[8];  // r[q]: 8 consecutive columns of row q
 };
 
+// Rows beyond `rows` read as zero (they would add to every output); columns beyond n only feed outputs that are
+// never stored, so their address is clamped instead.  FULL: the caller knows that all 8 rows exist.
+template <bool FULL>
 __device__ __forceinline__ void fetch_block(Block8x8& b, const uint16_t* __restrict__ X, long rows, long n, long row0,
                                             long col0) {
+  const long c = col0 + 7 < n ? col0 : 0;
 #pragma unroll
   for (int q = 0; q < 8; ++q) {
-    b.r[q] = uint4{0u, 0u, 0u, 0u};
-    if (row0 + q < rows && col0 + 7 < n) b.r[q] = *reinterpret_cast<const uint4*>(X + (row0 + q) * n + col0);
+    if (FULL) {
+      b.r[q] = *reinterpret_cast<const uint4*>(X + (row0 + q) * n + c);
+    } else {
+      const bool ok = row0 + q < rows;
+      const uint4 v = *reinterpret_cast<const uint4*>(X + (ok ? row0 + q : 0) * n + c);
+      b.r[q] = ok ? v : uint4{0u, 0u, 0u, 0u};
+    }
   }
 }
 
-// column c of the block as 8 consecutive rows (4 dwords), written to dst[c * kPitch .. ]
-__device__ __forceinline__ void store_block_transposed(const Block8x8& b, uint16_t* dst) {
-#pragma unroll
-  for (int d = 0; d < 4; ++d) {
-    const uint32_t w[8] = {d == 0 ? b.r[0].x : d == 1 ? b.r[0].y : d == 2 ? b.r[0].z : b.r[0].w,
-                           d == 0 ? b.r[1].x : d == 1 ? b.r[1].y : d == 2 ? b.r[1].z : b.r[1].w,
-                           d == 0 ? b.r[2].x : d == 1 ? b.r[2].y : d == 2 ? b.r[2].z : b.r[2].w,
-                           d == 0 ? b.r[3].x : d == 1 ? b.r[3].y : d == 2 ? b.r[3].z : b.r[3].w,
-                           d == 0 ? b.r[4].x : d == 1 ? b.r[4].y : d == 2 ? b.r[4].z : b.r[4].w,
-                           d == 0 ? b.r[5].x : d == 1 ? b.r[5].y : d == 2 ? b.r[5].z : b.r[5].w,
-                           d == 0 ? b.r[6].x : d == 1 ? b.r[6].y : d == 2 ? b.r[6].z : b.r[6].w,
-                           d == 0 ? b.r[7].x : d == 1 ? b.r[7].y : d == 2 ? b.r[7].z : b.r[7].w};
-    uint4 even, odd;  // columns 2d and 2d + 1: (row 0, row 1), (2, 3), (4, 5), (6, 7)
-    even.x = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u);
-    even.y = __builtin_amdgcn_perm(w[3], w[2], 0x05040100u);
-    even.z = __builtin_amdgcn_perm(w[5], w[4], 0x05040100u);
-    even.w = __builtin_amdgcn_perm(w[7], w[6], 0x05040100u);
-    odd.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
-    odd.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
-    odd.z = __builtin_amdgcn_perm(w[5], w[4], 0x07060302u);
-    odd.w = __builtin_amdgcn_perm(w[7], w[6], 0x07060302u);
-    *reinterpret_cast<uint4*>(dst + (2 * d) * kPitch) = even;
-    *reinterpret_cast<uint4*>(dst + (2 * d + 1) * kPitch) = odd;
+// LDS layout of an operand slice: column `col` of X occupies 128 bytes; its 16-byte piece holding rows 8 p .. 8 p + 7 of
+// the stage sits at piece position p ^ (col & 7) ^ ((col >> 3) & 7).  The writers of one instruction are 8 lanes with
+// the same column offset in 8 neighbouring column groups, the readers 8 lanes on 8 neighbouring columns: both then
+// touch 8 different 16-byte bank groups.
+//
+// column c of the block as 8 consecutive rows (4 dwords), written to piece (sw ^ c) of row c of dst; sw = p ^ (group & 7)
+template <int D>
+__device__ __forceinline__ void store_chunk_transposed(const Block8x8& b, uint16_t* dst, int sw) {
+  const uint32_t w[8] = {D == 0 ? b.r[0].x : D == 1 ? b.r[0].y : D == 2 ? b.r[0].z : b.r[0].w,
+                         D == 0 ? b.r[1].x : D == 1 ? b.r[1].y : D == 2 ? b.r[1].z : b.r[1].w,
+                         D == 0 ? b.r[2].x : D == 1 ? b.r[2].y : D == 2 ? b.r[2].z : b.r[2].w,
+                         D == 0 ? b.r[3].x : D == 1 ? b.r[3].y : D == 2 ? b.r[3].z : b.r[3].w,
+                         D == 0 ? b.r[4].x : D == 1 ? b.r[4].y : D == 2 ? b.r[4].z : b.r[4].w,
+                         D == 0 ? b.r[5].x : D == 1 ? b.r[5].y : D == 2 ? b.r[5].z : b.r[5].w,
+                         D == 0 ? b.r[6].x : D == 1 ? b.r[6].y : D == 2 ? b.r[6].z : b.r[6].w,
+                         D == 0 ? b.r[7].x : D == 1 ? b.r[7].y : D == 2 ? b.r[7].z : b.r[7].w};
+  uint4 even, odd;  // columns 2 D and 2 D + 1: (row 0, row 1), (2, 3), (4, 5), (6, 7)
+  even.x = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u);
+  even.y = __builtin_amdgcn_perm(w[3], w[2], 0x05040100u);
+  even.z = __builtin_amdgcn_perm(w[5], w[4], 0x05040100u);
+  even.w = __builtin_amdgcn_perm(w[7], w[6], 0x05040100u);
+  odd.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
+  odd.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
+  odd.z = __builtin_amdgcn_perm(w[5], w[4], 0x07060302u);
+  odd.w = __builtin_amdgcn_perm(w[7], w[6], 0x07060302u);
+  *reinterpret_cast<uint4*>(dst + (2 * D) * kPitch + ((sw ^ (2 * D)) << 3)) = even;
+  *reinterpret_cast<uint4*>(dst + (2 * D + 1) * kPitch + ((sw ^ (2 * D + 1)) << 3)) = odd;
+}
+__device__ __forceinline__ void store_block_transposed(const Block8x8& b, uint16_t* dst, int sw) {
+  store_chunk_transposed<0>(b, dst, sw);
+  store_chunk_transposed<1>(b, dst, sw);
+  store_chunk_transposed<2>(b, dst, sw);
+  store_chunk_transposed<3>(b, dst, sw);
+}
+
+// One 64-row stage of a workgroup: 64 MFMAs per wave on the LDS buffers As / Bs while (FETCH != 0) the next stage
+// travels global memory -> registers -> transpose -> the other LDS buffer.  FETCH: 0 nothing follows, 1 the next
+// stage is complete, 2 it is the ragged last one.  The function is one basic block; the group barriers at its end
+// give the order the instruction scheduler is asked for: loads first, then fragment reads of k-slice ks + 1 between
+// the MFMAs of slice ks, and the transposes and LDS writes of the next stage between the MFMAs of the last slice.
+template <bool DIAG, int FETCH>
+__device__ __forceinline__ void syrk_stage(floatx16 (&acc)[4][4], const uint16_t* As, const uint16_t* Bs, uint16_t* nxt,
+                                           Block8x8& ga, Block8x8& gb, const uint16_t* __restrict__ X, long rows,
+                                           long n, long r0, long ci, long cj, int offA, int offB, int swr, int sww) {
+  if (FETCH) {
+    fetch_block<FETCH == 1>(ga, X, rows, n, r0, ci);
+    if (!DIAG) fetch_block<FETCH == 1>(gb, X, rows, n, r0, cj);
   }
+  bf16x8 fa[2][4], fb[2][4];
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi) {
+    const int piece = (swr ^ (4 * (mi & 1))) << 3;
+    fa[0][mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + offA + mi * 32 * kPitch + piece));
+    fb[0][mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Bs + offB + mi * 32 * kPitch + piece));
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int ks = 0; ks < kStage / 16; ++ks) {
+    if (ks + 1 < kStage / 16) {
+      // the fragments of the next k-slice are requested before the 16 MFMAs of this one are queued
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        const int piece = (swr ^ (2 * (ks + 1)) ^ (4 * (mi & 1))) << 3;
+        fa[(ks + 1) & 1][mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + offA + mi * 32 * kPitch + piece));
+        fb[(ks + 1) & 1][mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Bs + offB + mi * 32 * kPitch + piece));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) {
+        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][mi], fb[ks & 1][ni], acc[mi][ni], 0, 0, 0);
+        if (FETCH && ks == kStage / 16 - 1) {
+          // last k-slice: the next stage's blocks are transposed and written to the other LDS buffer in the shadow of
+          // the matrix instructions, one quarter block (8 permutes, 2 writes) after every second (fourth) MFMA
+          const int i = mi * 4 + ni;
+          if (!DIAG) {
+            if (i == 0) store_chunk_transposed<0>(ga, nxt, sww);
+            if (i == 2) store_chunk_transposed<1>(ga, nxt, sww);
+            if (i == 4) store_chunk_transposed<2>(ga, nxt, sww);
+            if (i == 6) store_chunk_transposed<3>(ga, nxt, sww);
+            if (i == 8) store_chunk_transposed<0>(gb, nxt + kSliceU16, sww);
+            if (i == 10) store_chunk_transposed<1>(gb, nxt + kSliceU16, sww);
+            if (i == 12) store_chunk_transposed<2>(gb, nxt + kSliceU16, sww);
+            if (i == 14) store_chunk_transposed<3>(gb, nxt + kSliceU16, sww);
+          } else {
+            if (i == 0) store_chunk_transposed<0>(ga, nxt, sww);
+            if (i == 4) store_chunk_transposed<1>(ga, nxt, sww);
+            if (i == 8) store_chunk_transposed<2>(ga, nxt, sww);
+            if (i == 12) store_chunk_transposed<3>(ga, nxt, sww);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __syncthreads();
+}
+
+template <bool DIAG>
+__device__ __forceinline__ void syrk_tile(floatx16 (&acc)[4][4], uint16_t* lds, const uint16_t* __restrict__ X, long rows,
+                                          long n, long ci, long cj, int ro, int cg, int offA, int offB, int swr) {
+  const long stages = (rows + kStage - 1) / kStage;
+  Block8x8 ga, gb;
+  uint16_t* const wr = lds + (8 * cg) * kPitch;  // row of this thread's first column within a slice
+  const int sww = ro ^ (cg & 7);
+  fetch_block<false>(ga, X, rows, n, 8 * ro, ci);
+  if (!DIAG) fetch_block<false>(gb, X, rows, n, 8 * ro, cj);
+  store_block_transposed(ga, wr, sww);
+  if (!DIAG) store_block_transposed(gb, wr + kSliceU16, sww);
+  __syncthreads();
+  // stages whose successor is complete run in one loop body; the ragged successor and the last stage follow
+  long st = 0;
+#define QTIP_SYRK_STAGE(F)                                                                                   \
+  syrk_stage<DIAG, F>(acc, lds + (st & 1) * 2 * kSliceU16, lds + (st & 1) * 2 * kSliceU16 + (DIAG ? 0 : kSliceU16), \
+                      wr + ((st + 1) & 1) * 2 * kSliceU16, ga, gb, X, rows, n, (st + 1) * kStage + 8 * ro, ci, cj, offA, offB, swr, sww)
+  for (; (st + 2) * kStage <= rows; ++st) QTIP_SYRK_STAGE(1);
+  if (st + 1 < stages) {
+    QTIP_SYRK_STAGE(2);
+    ++st;
+  }
+  QTIP_SYRK_STAGE(0);
+#undef QTIP_SYRK_STAGE
 }
 
 __global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __restrict__ X, long rows, long n,
@@ -81,12 +190,15 @@ __global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __res
   const long ti = (patch / patch_cols) * kPatchRows + within / kPatchCols;
   const long tj = (patch % patch_cols) * kPatchCols + within % kPatchCols;
   if (ti >= tiles || tj > ti) return;  // outside the matrix or above the diagonal
-  const bool diag = ti == tj;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int ro = t & 7, cg = t >> 3;  // this thread stages rows 8 ro .. 8 ro + 7, columns 8 cg .. 8 cg + 7 of a slice
+  // this thread stages rows 8 ro .. 8 ro + 7, columns 8 cg .. 8 cg + 7 of a slice; 8 neighbouring lanes read one
+  // 128-byte line of a row of X
+  const int ro = (t >> 3) & 7, cg = (t & 7) + 8 * (t >> 6);
   const long ci = ti * kTile + 8 * cg, cj = tj * kTile + 8 * cg;
-  uint16_t* const wr = lds + (8 * cg) * kPitch + 8 * ro;  // within a slice
+  const int rl = lane & 31;
+  const int offA = (wm * 128 + rl) * kPitch, offB = (wn * 128 + rl) * kPitch;
+  const int swr = (lane >> 5) ^ (rl & 7) ^ (rl >> 3);  // piece of k-slice 0, row tile 0; the others differ by constants
 
   floatx16 acc[4][4];
 #pragma unroll
@@ -95,46 +207,21 @@ __global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __res
     for (int c = 0; c < 4; ++c)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][c][v] = 0.f;
-
-  const long stages = (rows + kStage - 1) / kStage;
-  Block8x8 ga, gb;
-  fetch_block(ga, X, rows, n, 8 * ro, ci);
-  if (!diag) fetch_block(gb, X, rows, n, 8 * ro, cj);
-  store_block_transposed(ga, wr);
-  if (!diag) store_block_transposed(gb, wr + kSliceU16);
-  __syncthreads();
-
-  const int kq = 8 * (lane >> 5), rl = lane & 31;
-  for (long st = 0; st < stages; ++st) {
-    const uint16_t* As = lds + (st & 1) * 2 * kSliceU16;
-    const uint16_t* Bs = diag ? As : As + kSliceU16;
-    const bool more = st + 1 < stages;
-    if (more) {
-      fetch_block(ga, X, rows, n, (st + 1) * kStage + 8 * ro, ci);
-      if (!diag) fetch_block(gb, X, rows, n, (st + 1) * kStage + 8 * ro, cj);
-    }
+  {
+    // The accumulators enter the stage loop as results of a matrix instruction (of zero operands): they then live in
+    // the accumulation registers from the start.  Entering as plain zeros, the compiler keeps them in ordinary
+    // registers at the loop head and copies all 256 of them to the accumulation registers and back in every stage.
+    bf16x8 z;
 #pragma unroll
-    for (int ks = 0; ks < kStage / 16; ++ks) {
-      bf16x8 fa[4], fb[4];
+    for (int e = 0; e < 8; ++e) z[e] = __bf16(0.f);
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-        fa[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + (wm * 128 + mi * 32 + rl) * kPitch + ks * 16 + kq));
+    for (int a = 0; a < 4; ++a)
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni)
-        fb[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Bs + (wn * 128 + ni * 32 + rl) * kPitch + ks * 16 + kq));
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
-    }
-    if (more) {
-      uint16_t* nxt = lds + ((st + 1) & 1) * 2 * kSliceU16 + (8 * cg) * kPitch + 8 * ro;
-      store_block_transposed(ga, nxt);
-      if (!diag) store_block_transposed(gb, nxt + kSliceU16);
-    }
-    __syncthreads();
+      for (int c = 0; c < 4; ++c) acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z, z, acc[a][c], 0, 0, 0);
   }
+  if (ti == tj) syrk_tile<true>(acc, lds, X, rows, n, ci, cj, ro, cg, offA, offB, swr);
+  else syrk_tile<false>(acc, lds, X, rows, n, ci, cj, ro, cg, offA, offB, swr);
+
   // accumulator element v of a lane: row (v % 4) + 8 (v / 4) + 4 (lane / 32), column lane % 32 of the 32 x 32 tile
 #pragma unroll
   for (int mi = 0; mi < 4; ++mi)
