@@ -123,8 +123,12 @@ def run_group(args, pkg):
 
     def run_steps(K, record):
         """K groups through the library's scheduler: the Hessian of group k+2 is rotated and the one of group k+1 is
-        factored on a side thread while the GPU quantizes group k."""
-        res = q.run_groups([(lins, n, H, 3 + k) for k in range(K)], opt)
+        factored on a side thread while the GPU quantizes group k.  The untimed warm-up groups also evaluate the proxy
+        (the metric's stages are RHT + LDLQ + Viterbi; the proxy's value and cost are reported beside them)."""
+        o = opt if record else pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback)
+        res = q.run_groups([(lins, n, H, 3 + k) for k in range(K)], o)
+        if not record:
+            stats.update(proxy=float(res[-1][0][0].proxy), proxy_s=float(res[-1][1].proxy))
         if record:
             tms = [r[1] for r in res]
             stats.update(rht_s=sum(t.rht for t in tms) / K,      # Hessian rotation + weight RHT + Wscale
