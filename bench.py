@@ -176,8 +176,9 @@ def main():
                     help="first run one plain 1 GiB device copy kernel (known traffic, scales the rocprof byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (every tile row is independent, "
-              "see DESIGN.md for how the path would shard)" % args.gpus, file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (given SU, L and Wscale every 16-row "
+              "tile row of a group is independent, so the path would shard by tile rows without any exchange)" % args.gpus,
+              file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():
