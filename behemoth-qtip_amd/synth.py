@@ -1,4 +1,4 @@
-"""Seeded synthetic layers for the benchmark configurations (BASELINE.json `configs`).
+"""Seeded synthetic layers for the benchmark configurations (the five benchmark configurations: tiles only, 1024 x 1024, q-proj, gate+up, down-proj).
 
 Small configurations are generated with numpy on the host (bit-stable across machines); the large ones with
 torch on the GPU so that set-up takes seconds, not minutes.  Input synthesis is never timed.

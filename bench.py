@@ -3,7 +3,7 @@
 
 A step is one pass of the hot path over one synthetic group: Hessian rotation (GPU), fp64 block LDL (host),
 weight RHT + Wscale, LDLQ with the two-pass Viterbi, packing to the kernel-layout trellis.  Default workload:
-BASELINE configuration 5, the 12288 x 28672 down-proj group.  The K timed steps are K groups handled the way the
+benchmark configuration 5, the 12288 x 28672 down-proj group.  The K timed steps are K groups handled the way the
 reference's scheduler handles consecutive groups (src/pipeline.cpp:254-290): Hessians are rotated ahead of use
 (two groups ahead, through a ring of three staging buffers), a side thread factors them in order, and the GPU
 quantizes group k as soon as its factor is ready, so the host LDL of group k+1 overlaps the GPU work of group k;

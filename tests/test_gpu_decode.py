@@ -119,7 +119,7 @@ def test_dequantize_equals_group_reconstruction(qz, oracle, pkg, hyb):
 
 
 def test_decode_full_size_sample(qz, hyb):
-    """BASELINE configuration 5 shape (12288 x 28672): random words decoded on the device, a sample of 32-row blocks
+    """Benchmark configuration 5 shape (12288 x 28672): random words decoded on the device, a sample of 32-row blocks
     compared with the CPU decoder, every value a codebook entry; prints the achieved HBM rate."""
     import torch
     say("case: decode 12288x28672 random words")

@@ -1,4 +1,4 @@
-"""Full-size checks (BASELINE configurations 3 and 5) of the GPU group path: agreement with the CPU form on a row
+"""Full-size checks (benchmark configurations 3 and 5) of the GPU group path: agreement with the CPU form on a row
 subset of the rotated weights (LDLQ is row-independent given L), and size-independent properties of the packed
 output (every trellis tail-biting and link-consistent, decode(states) == hatW on sampled tiles)."""
 import os

@@ -271,7 +271,7 @@ def test_group_input_formats_and_errors(qz, oracle, pkg, synth):
 
 
 def test_group_config2(qz, oracle, pkg, hyb, synth):
-    """BASELINE config 2 (1024 x 1024, AR(1) Hessian with outlier channels): code agreement >= 99 % and proxy
+    """Benchmark configuration 2 (1024 x 1024, AR(1) Hessian with outlier channels): code agreement >= 99 % and proxy
     within 1 % relative of the CPU restatement (north-star accuracy targets for full LDLQ groups)."""
     say("case: config 2, 1024x1024")
     qz.set_tlut(None)

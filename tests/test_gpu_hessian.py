@@ -61,7 +61,7 @@ def test_hessian_rejects_bad_shapes(qz, pkg):
 
 
 def test_hessian_config5_shape(qz):
-    """BASELINE configuration 5 width (n = 28672) with 8192 token rows: sampled entries against fp64, exact symmetry,
+    """Benchmark configuration 5 width (n = 28672) with 8192 token rows: sampled entries against fp64, exact symmetry,
     and the achieved matrix-core rate."""
     import torch
     say("case: hessian 8192 x 28672")

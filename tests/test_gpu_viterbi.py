@@ -61,7 +61,7 @@ def test_raw_inputs_golden(qz):
 
 
 def test_config1_full(qz, oracle):
-    """BASELINE config 1: 4096 tiles of raw fp32 N(0,1), synthetic unit-rms tlut; packed words bit-exact against
+    """Benchmark configuration 1: 4096 tiles of raw fp32 N(0,1), synthetic unit-rms tlut; packed words bit-exact against
     the output of the compiled reference (committed fixture)."""
     say("case: config 1, 4096 tiles")
     meta = json.load(open(os.path.join(GOLDEN, "ref_config1.json")))
