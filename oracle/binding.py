@@ -15,6 +15,7 @@ _REF = {}
 f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
 f64p = np.ctypeslib.ndpointer(np.float64, flags="C_CONTIGUOUS")
 u16p = np.ctypeslib.ndpointer(np.uint16, flags="C_CONTIGUOUS")
+u8p = np.ctypeslib.ndpointer(np.uint8, flags="C_CONTIGUOUS")
 u32p = np.ctypeslib.ndpointer(np.uint32, flags="C_CONTIGUOUS")
 u64p = np.ctypeslib.ndpointer(np.uint64, flags="C_CONTIGUOUS")
 i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
@@ -74,6 +75,16 @@ def lib():
     L.qo_quantize_group.argtypes = [f32p, C.c_int, C.POINTER(C.c_void_p), i32p, C.c_int, f32p, C.c_uint64, C.c_double,
                                     C.c_double, u16p, u16p, f32p, f32p, f64p, f64p, C.c_void_p, C.c_void_p,
                                     C.c_void_p, C.c_int]
+    L.qo_f32_to_fp8e4m3.restype = C.c_uint8
+    L.qo_f32_to_fp8e4m3.argtypes = [C.c_float]
+    L.qo_fp8e4m3_to_f32.restype = C.c_float
+    L.qo_fp8e4m3_to_f32.argtypes = [C.c_uint8]
+    L.qo_nvfp4_quantize.argtypes = [f32p, C.c_int, C.c_int, u8p, u8p, C.POINTER(C.c_float)]
+    L.qo_nvfp4_dequantize.argtypes = [u8p, u8p, C.c_float, C.c_int, C.c_int, f32p]
+    L.qo_nvfp4_proxy_error.restype = C.c_double
+    L.qo_nvfp4_proxy_error.argtypes = [f32p, f32p, C.c_int, C.c_int, C.c_void_p]
+    L.qo_nvfp4_prepare.argtypes = [f32p, C.c_int, C.c_double, C.c_int, C.c_void_p, f32p]
+    L.qo_nvfp4_blocks.argtypes = [f32p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_int, u8p, u8p]
     _LIB = L
     return L
 
@@ -113,6 +124,14 @@ def ref_lib(native=False):
     R.ref_f32_to_bf16.restype = C.c_uint16
     R.ref_f32_to_bf16.argtypes = [C.c_float]
     R.ref_rng.argtypes = [C.c_uint64, C.c_int, C.c_long, C.c_void_p, C.c_void_p]
+    if hasattr(R, "ref_nvfp4_quantize"):
+        R.ref_f32_to_fp8e4m3.restype = C.c_uint
+        R.ref_f32_to_fp8e4m3.argtypes = [C.c_float]
+        R.ref_nvfp4_quantize.restype = C.c_float
+        R.ref_nvfp4_quantize.argtypes = [f32p, C.c_int, C.c_int, u8p, u8p]
+        R.ref_nvfp4_dequantize.argtypes = [u8p, u8p, C.c_float, C.c_int, C.c_int, f32p]
+        R.ref_nvfp4_proxy_error.restype = C.c_double
+        R.ref_nvfp4_proxy_error.argtypes = [f32p, f32p, C.c_int, C.c_int, C.c_void_p]
     _REF[name] = R
     return R
 
@@ -249,3 +268,50 @@ def quantize_group(tlut, Ws, H, seed, sigma_reg=1e-2, scale_override=0.9, thread
     assert rc == 0, rc
     return dict(trellis=trellis, su_bf16=su_bf16, sv=sv, wscale=wscale, proxy=proxy, proxy_rot_reg=prr, Q=Q, WT=WT,
                 hatWT=hT, m=ms, n=n)
+
+
+# ---------------------------------------------------------------- NVFP4 fallback quantizer
+def nvfp4_quantize(w):
+    """nvfp4_quantize, src/nvfp4.cpp:12-55 -> (packed [m][n/2], scales [m][n/16], global)."""
+    w = np.ascontiguousarray(w, np.float32)
+    m, n = w.shape
+    packed = np.zeros((m, n // 2), np.uint8)
+    scales = np.zeros((m, n // 16), np.uint8)
+    g = C.c_float()
+    assert lib().qo_nvfp4_quantize(w.reshape(-1), m, n, packed.reshape(-1), scales.reshape(-1), C.byref(g)) == 0
+    return packed, scales, g.value
+
+
+def nvfp4_dequantize(packed, scales, g, m, n):
+    out = np.zeros((m, n), np.float32)
+    lib().qo_nvfp4_dequantize(np.ascontiguousarray(packed).reshape(-1), np.ascontiguousarray(scales).reshape(-1), g, m, n,
+                              out.reshape(-1))
+    return out
+
+
+def nvfp4_proxy_error(w, what, H=None):
+    m, n = w.shape
+    Hp = None if H is None else np.ascontiguousarray(H, np.float32).ctypes.data
+    return lib().qo_nvfp4_proxy_error(np.ascontiguousarray(w, np.float32).reshape(-1),
+                                      np.ascontiguousarray(what, np.float32).reshape(-1), m, n, Hp)
+
+
+def nvfp4_prepare(H, sigma_reg=1e-2, calibrate=True):
+    """src/nvfp4_gpu.hip:181-207 -> (L or None, dw); None when H is not positive definite."""
+    H = np.ascontiguousarray(H, np.float32)
+    n = H.shape[0]
+    L = np.zeros((n, n), np.float32) if calibrate else None
+    dw = np.zeros(n, np.float32)
+    rc = lib().qo_nvfp4_prepare(H.reshape(-1), n, sigma_reg, 1 if calibrate else 0, None if L is None else L.ctypes.data, dw)
+    return None if rc else (L, dw)
+
+
+def nvfp4_blocks(w, L, dw, g, calibrate, search):
+    """The block loop of nvfp4_quantize_group (src/nvfp4_gpu.hip:217-228) -> (packed, scales)."""
+    w = np.ascontiguousarray(w, np.float32)
+    m, n = w.shape
+    packed = np.zeros((m, n // 2), np.uint8)
+    scales = np.zeros((m, n // 16), np.uint8)
+    lib().qo_nvfp4_blocks(w.reshape(-1), m, n, None if L is None else L.ctypes.data, None if dw is None else dw.ctypes.data,
+                          g, 1 if calibrate else 0, 1 if search else 0, packed.reshape(-1), scales.reshape(-1))
+    return packed, scales

@@ -780,3 +780,207 @@ int qo_quantize_group(const float* tlut, int nlin, const float* const* W, const 
   free(lut0), free(lut1), free(su), free(HRr), free(L), free(WT), free(WTd), free(hT), free(Q), free(DT);
   return rc;
 }
+
+/* ================================================================== NVFP4 fallback quantizer */
+static unsigned nv_round_even(float v) { /* src/nvfp4.hpp:19-23 */
+  const float f = floorf(v), r = v - f;
+  unsigned n = (unsigned)f;
+  return n + (unsigned)(r > .5f || (r == .5f && (n & 1u)));
+}
+uint8_t qo_f32_to_fp8e4m3(float x) { /* src/nvfp4.hpp:15-33 */
+  const uint8_t sign = signbit(x) ? 128 : 0;
+  if (isnan(x)) return (uint8_t)(sign | 127);
+  x = fminf(fabsf(x), 448.f);
+  if (x < ldexpf(1.f, -6)) return (uint8_t)(sign | nv_round_even(x * 512.f));
+  int e;
+  const float frac = frexpf(x, &e) * 2;
+  unsigned mant = nv_round_even((frac - 1) * 8);
+  int ee = e + 6;
+  if (mant == 8) {
+    mant = 0;
+    ++ee;
+  }
+  unsigned c = ((unsigned)ee << 3) | mant;
+  return (uint8_t)(sign | (c < 126u ? c : 126u));
+}
+float qo_fp8e4m3_to_f32(uint8_t b) { /* src/common.hpp:81-88 */
+  const uint32_t s = b >> 7, e = (b >> 3) & 0xf, m = b & 7;
+  float v;
+  if (e == 0) v = ldexpf((float)m, -9);
+  else if (e == 15 && m == 7) v = NAN;
+  else v = ldexpf((float)(m | 8), (int)e - 10);
+  return s ? -v : v;
+}
+static const float kNvLevels[8] = {0, .5f, 1, 1.5f, 2, 3, 4, 6};
+/* nearest E2M1 magnitude code, ties to the even code (src/nvfp4.cpp:27-38, src/nvfp4_gpu.hip:47-60) */
+static int nv_fp4_mag(float a) {
+  float best = INFINITY;
+  int code = 0;
+  for (int i = 0; i < 8; ++i) {
+    const float e = fabsf(a - kNvLevels[i]);
+    if (e < best || (e == best && (i % 2 == 0))) {
+      best = e;
+      code = i;
+    }
+  }
+  return code;
+}
+int qo_nvfp4_quantize(const float* w, int m, int n, uint8_t* packed, uint8_t* scales, float* global) {
+  if (m <= 0 || n <= 0 || n % 16) return -1;
+  const size_t numel = (size_t)m * n;
+  float maximum = 0;
+  for (size_t i = 0; i < numel; ++i) maximum = fmaxf(maximum, fabsf(w[i]));
+  const float g = maximum ? maximum / (448.f * 6) : 1.f;
+  *global = g;
+  for (size_t b = 0; b < numel / 16; ++b) {
+    float mx = 0;
+    for (int j = 0; j < 16; ++j) mx = fmaxf(mx, fabsf(w[b * 16 + j]));
+    const uint8_t sc = qo_f32_to_fp8e4m3(mx / (6 * g));
+    scales[b] = sc;
+    const float scale = qo_fp8e4m3_to_f32(sc) * g;
+    for (int j = 0; j < 16; j += 2) {
+      const float x0 = scale ? w[b * 16 + j] / scale : 0, x1 = scale ? w[b * 16 + j + 1] / scale : 0;
+      const uint8_t c0 = (uint8_t)(nv_fp4_mag(fabsf(x0)) | (signbit(x0) ? 8 : 0));
+      const uint8_t c1 = (uint8_t)(nv_fp4_mag(fabsf(x1)) | (signbit(x1) ? 8 : 0));
+      packed[b * 8 + j / 2] = (uint8_t)(c0 | (c1 << 4));
+    }
+  }
+  return 0;
+}
+void qo_nvfp4_dequantize(const uint8_t* packed, const uint8_t* scales, float global, int m, int n, float* out) {
+  const size_t numel = (size_t)m * n;
+  for (size_t i = 0; i < numel; ++i) {
+    const uint8_t code = (packed[i / 2] >> (i % 2 * 4)) & 15;
+    const float s = qo_fp8e4m3_to_f32(scales[i / 16]);
+    const float v = (code & 8 ? -1.f : 1.f) * kNvLevels[code & 7];
+    out[i] = qo_bf16_to_f32(qo_f32_to_bf16(v * s * global));
+  }
+}
+double qo_nvfp4_proxy_error(const float* w, const float* what, int m, int n, const float* H) {
+  double total = 0;
+#pragma omp parallel for reduction(+ : total) schedule(static)
+  for (int r = 0; r < m; ++r) {
+    double* e = (double*)malloc(sizeof(double) * (size_t)n);
+    for (int j = 0; j < n; ++j) e[j] = (double)w[(size_t)r * n + j] - what[(size_t)r * n + j];
+    if (!H) {
+      for (int j = 0; j < n; ++j) total += e[j] * e[j];
+    } else {
+      for (int i = 0; i < n; ++i) {
+        double acc = 0;
+        for (int j = 0; j < n; ++j) acc += (double)H[(size_t)i * n + j] * e[j];
+        total += e[i] * acc;
+      }
+    }
+    free(e);
+  }
+  return total / m;
+}
+int qo_nvfp4_prepare(const float* H, int n, double sigma_reg, int calibrate, float* L, float* dw) {
+  double dsum = 0;
+  for (int i = 0; i < n; ++i) dsum += H[(size_t)i * n + i];
+  const double creg = sigma_reg * dsum / n;
+  if (!calibrate) {
+    for (int i = 0; i < n; ++i) dw[i] = (float)(H[(size_t)i * n + i] + creg);
+    return 0;
+  }
+  double* A = (double*)malloc(sizeof(double) * (size_t)n * n);
+  for (long i = 0; i < n; ++i)
+    for (long j = 0; j <= i; ++j)
+      A[(size_t)i * n + j] = 0.5 * ((double)H[(size_t)i * n + j] + H[(size_t)j * n + i]) + (i == j ? creg : 0.0);
+  if (!qo_cholesky(A, n)) {
+    free(A);
+    return -1;
+  }
+  memset(L, 0, sizeof(float) * (size_t)n * n);
+  for (long j = 0; j < n; ++j) {
+    const double d = A[(size_t)j * n + j];
+    dw[j] = (float)(d * d);
+    for (long i = j + 1; i < n; ++i) L[(size_t)i * n + j] = (float)(A[(size_t)i * n + j] / d);
+  }
+  free(A);
+  return 0;
+}
+/* one row of one 16-column block: nv_block_kernel, src/nvfp4_gpu.hip:66-158 */
+static void nv_block_row(const float* w16, const float* f16, const float Lb[16][16], const float* Dw, float global,
+                         int calibrate, int search, uint8_t* nib, uint8_t* scale_out, float* err_out) {
+  float w[16], base[16], amax = 0;
+  for (int k = 0; k < 16; ++k) {
+    w[k] = w16[k];
+    base[k] = w[k] + (calibrate ? f16[k] : 0.f);
+    amax = fmaxf(amax, fabsf(calibrate ? base[k] : w[k]));
+  }
+  unsigned cand[11];
+  int nc = 0;
+  const unsigned c1 = qo_f32_to_fp8e4m3(amax / (6.f * global)) & 127u;
+  cand[nc++] = c1;
+  if (search) {
+    static const float g[8] = {0.70f, 0.75f, 0.80f, 0.85f, 0.90f, 0.95f, 1.00f, 1.05f};
+    for (int i = 0; i < 8; ++i) cand[nc++] = qo_f32_to_fp8e4m3(amax * g[i] / (6.f * global)) & 127u;
+    cand[nc++] = c1 > 0 ? c1 - 1 : 0;
+    cand[nc++] = c1 < 126 ? c1 + 1 : 126;
+  }
+  float best_cost = INFINITY;
+  unsigned best = c1;
+  for (int ci = 0; ci < nc; ++ci) {
+    const float sd = qo_fp8e4m3_to_f32((uint8_t)cand[ci]), scale = sd * global;
+    float err[16], cost = 0;
+    for (int k = 15; k >= 0; --k) {
+      float t = base[k];
+      if (calibrate)
+        for (int j = k + 1; j < 16; ++j) t += err[j] * Lb[j][k];
+      const float x = scale != 0.f ? t / scale : 0.f;
+      const int code = nv_fp4_mag(fabsf(x));
+      const float q = qo_bf16_to_f32(qo_f32_to_bf16((x < 0 ? -1.f : 1.f) * kNvLevels[code] * sd * global));
+      cost += Dw[k] * (t - q) * (t - q);
+      err[k] = w[k] - q;
+    }
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = cand[ci];
+    }
+  }
+  const float sd = qo_fp8e4m3_to_f32((uint8_t)best), scale = sd * global;
+  for (int k = 15; k >= 0; --k) {
+    float t = base[k];
+    if (calibrate)
+      for (int j = k + 1; j < 16; ++j) t += err_out[j] * Lb[j][k];
+    const float x = scale != 0.f ? t / scale : 0.f;
+    const int code = nv_fp4_mag(fabsf(x));
+    const float q = qo_bf16_to_f32(qo_f32_to_bf16((x < 0 ? -1.f : 1.f) * kNvLevels[code] * sd * global));
+    err_out[k] = w[k] - q;
+    nib[k] = (uint8_t)(code | (signbit(x) ? 8 : 0));
+  }
+  *scale_out = (uint8_t)best;
+}
+void qo_nvfp4_blocks(const float* w, int m, int n, const float* L, const float* dw, float global, int calibrate,
+                     int search, uint8_t* packed, uint8_t* scales) {
+  const int cal = calibrate && L != NULL;
+  float* F = cal ? (float*)calloc((size_t)m * n, sizeof(float)) : NULL;
+  float* E = (float*)malloc(sizeof(float) * (size_t)m * 16);
+  for (int c0 = n - 16; c0 >= 0; c0 -= 16) {
+    float Lb[16][16], Dw[16];
+    for (int a = 0; a < 16; ++a) {
+      Dw[a] = dw ? dw[c0 + a] : 1.f;
+      for (int b = 0; b < 16; ++b) Lb[a][b] = cal ? L[(size_t)(c0 + a) * n + c0 + b] : 0.f;
+    }
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < m; ++r) {
+      uint8_t nib[16], sc;
+      nv_block_row(w + (size_t)r * n + c0, cal ? F + (size_t)r * n + c0 : NULL, Lb, Dw, global, cal, search, nib, &sc,
+                   E + (size_t)r * 16);
+      for (int k = 0; k < 16; k += 2) packed[(size_t)r * (n / 2) + (c0 + k) / 2] = (uint8_t)(nib[k] | (nib[k + 1] << 4));
+      scales[(size_t)r * (n / 16) + c0 / 16] = sc;
+    }
+    if (cal && c0 > 0) { /* nv_feedback_kernel: F[r][col] += sum_j E[r][j] * L[c0 + j][col], col < c0 */
+#pragma omp parallel for schedule(static)
+      for (int r = 0; r < m; ++r)
+        for (int col = 0; col < c0; ++col) {
+          float acc = 0;
+          for (int j = 0; j < 16; ++j) acc += E[(size_t)r * 16 + j] * L[(size_t)(c0 + j) * n + col];
+          F[(size_t)r * n + col] += acc;
+        }
+    }
+  }
+  free(E);
+  free(F);
+}

@@ -87,6 +87,27 @@ int qo_quantize_group(const float* tlut, int nlin, const float* const* W, const 
 /* tr(D H D^T)/tr(W H W^T) in fp64; W, hatW m x n row-major, H n x n */
 double qo_proxy(const float* W, const float* hatW, const float* H, int m, int n, int threads);
 
+/* ---- NVFP4 fallback quantizer (two E2M1 values per byte, one E4M3 scale per 16 input channels, one fp32 global
+ *      scale per matrix).  Format and the plain quantizer: src/nvfp4.hpp:15-33,54-57, src/nvfp4.cpp:12-87.  Scale
+ *      search and Hessian-calibrated rounding: a CPU restatement of the reference's GPU kernels
+ *      (src/nvfp4_gpu.hip:66-228) in the same fp32 operation order, no fused multiply-adds. */
+uint8_t qo_f32_to_fp8e4m3(float x);
+float qo_fp8e4m3_to_f32(uint8_t b);
+/* nvfp4_quantize, src/nvfp4.cpp:12-55: w m x n fp32 -> packed [m][n/2], scales [m][n/16], *global.  -1 if n % 16. */
+int qo_nvfp4_quantize(const float* w, int m, int n, uint8_t* packed, uint8_t* scales, float* global);
+/* nvfp4_dequantize, src/nvfp4.cpp:57-70 (values rounded to bf16) */
+void qo_nvfp4_dequantize(const uint8_t* packed, const uint8_t* scales, float global, int m, int n, float* out);
+/* nvfp4_proxy_error, src/nvfp4.cpp:72-87: tr(E H E^T) / m, H may be NULL (identity) */
+double qo_nvfp4_proxy_error(const float* w, const float* what, int m, int n, const float* H);
+/* Host preparation of nvfp4_quantize_group, src/nvfp4_gpu.hip:181-207: regularised H -> unit-lower L (n x n fp32,
+ * H = L D L^T) and dw = D when calibrate, else dw = diag(H) + creg and L untouched.  0 ok, -1 not positive definite. */
+int qo_nvfp4_prepare(const float* H, int n, double sigma_reg, int calibrate, float* L, float* dw);
+/* The block loop of nvfp4_quantize_group, src/nvfp4_gpu.hip:217-228 with nv_block_kernel :66-158 and
+ * nv_feedback_kernel :161-172: 16-column blocks from the last to the first.  L / dw may be NULL (no calibration /
+ * uniform weights); global as returned by qo_nvfp4_quantize. */
+void qo_nvfp4_blocks(const float* w, int m, int n, const float* L, const float* dw, float global, int calibrate,
+                     int search, uint8_t* packed, uint8_t* scales);
+
 #ifdef __cplusplus
 }
 #endif

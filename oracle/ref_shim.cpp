@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include "nvfp4.hpp"
 #include "qtip_core.hpp"
 
 using namespace qtip;
@@ -71,5 +72,24 @@ void ref_rng(uint64_t seed, int kind, long count, double* out_f, uint64_t* out_u
       default: out_f[i] = r.sign(); break;
     }
   }
+}
+// NVFP4 fallback quantizer, src/nvfp4.hpp / src/nvfp4.cpp
+unsigned ref_f32_to_fp8e4m3(float x) { return f32_to_fp8e4m3(x); }  // src/nvfp4.hpp:15-33
+float ref_nvfp4_quantize(const float* w, int m, int n, uint8_t* packed, uint8_t* scales) {  // src/nvfp4.cpp:12-55
+  Nvfp4Tensor t = nvfp4_quantize(w, m, n);
+  std::memcpy(packed, t.packed.data(), t.packed.size());
+  std::memcpy(scales, t.scales.data(), t.scales.size());
+  return t.global;
+}
+void ref_nvfp4_dequantize(const uint8_t* packed, const uint8_t* scales, float global, int m, int n, float* out) {  // :57-70
+  Nvfp4Tensor t;
+  t.m = m, t.n = n, t.global = global;
+  t.packed.assign(packed, packed + size_t(m) * n / 2);
+  t.scales.assign(scales, scales + size_t(m) * n / 16);
+  std::vector<float> v = nvfp4_dequantize(t);
+  std::memcpy(out, v.data(), v.size() * 4);
+}
+double ref_nvfp4_proxy_error(const float* w, const float* what, int m, int n, const float* H) {  // :72-87
+  return nvfp4_proxy_error(w, what, m, n, H);
 }
 }

@@ -88,6 +88,30 @@ def main():
     L = np.zeros((1024, 1024), np.float32)
     assert R.ref_block_ldl(A.reshape(-1), 1024, L.reshape(-1), 8) == 1
     L[1000:1008].tofile(os.path.join(HERE, "ref_ldl_1024.bin"))
+    # NVFP4: the reference's plain quantizer (src/nvfp4.cpp) on gaussian and heavy-tailed weights (the two cases of
+    # tests/test_nvfp4.cpp:47-57, same shapes, this repo's generator), plus the E4M3 encoder on a sweep of values
+    nv = {}
+    for name, seed, heavy in (("gauss", 5, False), ("heavy", 11, True)):
+        m, n = 96, 256
+        w = ob.rng_normal(seed, m * n) * 0.02
+        if heavy:
+            w = w * np.exp(1.2 * ob.rng_normal(seed + 100, m * n))
+        w = w.astype(np.float32).reshape(m, n)
+        w[3, 16:32] = 0.0                      # an all-zero block
+        packed = np.zeros((m, n // 2), np.uint8)
+        scales = np.zeros((m, n // 16), np.uint8)
+        g = R.ref_nvfp4_quantize(w.reshape(-1), m, n, packed.reshape(-1), scales.reshape(-1))
+        dq = np.zeros((m, n), np.float32)
+        R.ref_nvfp4_dequantize(packed.reshape(-1), scales.reshape(-1), g, m, n, dq.reshape(-1))
+        np.concatenate([packed.reshape(-1), scales.reshape(-1)]).tofile(os.path.join(HERE, "ref_nvfp4_%s.bin" % name))
+        nv[name] = {"m": m, "n": n, "seed": seed, "global": float.hex(float(g)),
+                    "fnv1a64_dequant": "%016x" % fnv1a64(dq.tobytes()),
+                    "mse": float.hex(R.ref_nvfp4_proxy_error(w.reshape(-1), dq.reshape(-1), m, n, None))}
+    xs = np.concatenate([np.float32(2.0) ** np.arange(-12, 10, dtype=np.float32) * s for s in (1.0, 1.0625, 1.25, 1.4375, 1.9375)]
+                        + [np.array([0.0, 448.0, 500.0, 1e-9, 0.015625, 0.0146484375], np.float32)]).astype(np.float32)
+    nv["fp8_inputs"] = [float.hex(float(v)) for v in xs]
+    nv["fp8_codes"] = [int(R.ref_f32_to_fp8e4m3(float(v))) for v in xs]
+    json.dump(nv, open(os.path.join(HERE, "ref_nvfp4.json"), "w"))
     print("wrote golden vectors to", HERE)
 
 
