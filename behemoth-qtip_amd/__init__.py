@@ -103,6 +103,13 @@ def lib():
                                         C.POINTER(_LinearOutC), C.POINTER(_TimingC)]
     L.qtip_hessian_accumulate_dev.argtypes = [vp, vp, l, i, vp]
     L.qtip_hessian_finish_dev.argtypes = [vp, vp, i, d]
+    L.qtip_f32_to_fp8e4m3.restype = C.c_uint8
+    L.qtip_f32_to_fp8e4m3.argtypes = [C.c_float]
+    L.qtip_nvfp4_quantize.argtypes = [vp, i, i, vp, vp, C.POINTER(C.c_float)]
+    L.qtip_nvfp4_dequantize.argtypes = [vp, vp, C.c_float, i, i, vp]
+    L.qtip_nvfp4_prepare.argtypes = [vp, i, d, i, i, vp, vp]
+    L.qtip_nvfp4_quantize_prepared.argtypes = [vp, i, vp, i, vp, vp, i]
+    L.qtip_nvfp4_quantize_group.argtypes = [vp, i, vp, i, vp, C.POINTER(_Nvfp4OptsC), C.POINTER(i)]
     L.qtip_run_groups.argtypes = [vp, i, vp, C.POINTER(_OptsC), vp, vp]
     L.qtip_reserve_groups.argtypes = [vp, i]
     L.qtip_st_create.argtypes = [C.POINTER(vp)]
@@ -125,6 +132,14 @@ def lib():
 class _GroupC(C.Structure):
     _fields_ = [("nlin", C.c_int), ("lins", C.c_void_p), ("outs", C.c_void_p), ("n", C.c_int), ("H", C.c_void_p),
                 ("h_on_device", C.c_int), ("seed", C.c_uint64)]
+
+
+class _Nvfp4MatrixC(C.Structure):
+    _fields_ = [("m", C.c_int), ("w", C.c_void_p), ("packed", C.c_void_p), ("scales", C.c_void_p), ("global_", C.c_float)]
+
+
+class _Nvfp4OptsC(C.Structure):
+    _fields_ = [("scale_search", C.c_int), ("calibrate", C.c_int), ("sigma_reg", C.c_double)]
 
 
 def _check(rc):
@@ -390,6 +405,43 @@ class Quantizer:
         """Mirror the computed triangle and scale (src/model.cpp:260-264, src/pipeline.cpp:160-166)."""
         _check(lib().qtip_hessian_finish_dev(self._h, _ptr(dH), n, float(scale)))
 
+    # ---- NVFP4 fallback quantizer (src/nvfp4_gpu.hpp)
+    @staticmethod
+    def _nvfp4_marshal(ws, n):
+        mats = (_Nvfp4MatrixC * len(ws))()
+        outs, keep = [], []
+        for k, w in enumerate(ws):
+            w = np.ascontiguousarray(w, np.float32)
+            assert w.ndim == 2 and w.shape[1] == n
+            t = Nvfp4Tensor(m=w.shape[0], n=n, packed=np.zeros((w.shape[0], n // 2), np.uint8),
+                            scales=np.zeros((w.shape[0], n // 16), np.uint8))
+            mats[k].m, mats[k].w, mats[k].packed, mats[k].scales = w.shape[0], _ptr(w), _ptr(t.packed), _ptr(t.scales)
+            outs.append(t)
+            keep.append(w)
+        return mats, outs, keep
+
+    def nvfp4_quantize_group(self, ws, n, H=None, scale_search=True, calibrate=True, sigma_reg=1e-2):
+        """nvfp4_quantize_group, src/nvfp4_gpu.hip:174-241 -> (tensors, calibrated)."""
+        mats, outs, keep = self._nvfp4_marshal(ws, n)
+        o = _Nvfp4OptsC(1 if scale_search else 0, 1 if calibrate else 0, sigma_reg)
+        used = C.c_int()
+        Hc = None if H is None else np.ascontiguousarray(H, np.float32)
+        _check(lib().qtip_nvfp4_quantize_group(self._h, len(ws), C.addressof(mats), n, _ptr(Hc), C.byref(o), C.byref(used)))
+        for k, t in enumerate(outs):
+            t.global_scale = mats[k].global_
+        return outs, bool(used.value)
+
+    def nvfp4_quantize_prepared(self, ws, n, L=None, dw=None, scale_search=True):
+        """The device block loop on a prepared factor (L unit-lower n x n or None, dw [n] or None)."""
+        mats, outs, keep = self._nvfp4_marshal(ws, n)
+        Lc = None if L is None else np.ascontiguousarray(L, np.float32)
+        dc = None if dw is None else np.ascontiguousarray(dw, np.float32)
+        _check(lib().qtip_nvfp4_quantize_prepared(self._h, len(ws), C.addressof(mats), n, _ptr(Lc), _ptr(dc),
+                                                  1 if scale_search else 0))
+        for k, t in enumerate(outs):
+            t.global_scale = mats[k].global_
+        return outs
+
     def reserve_groups(self, n):
         _check(lib().qtip_reserve_groups(self._h, n))
 
@@ -425,6 +477,48 @@ class Quantizer:
         return out
 
 
+@dataclass
+class Nvfp4Tensor:  # src/nvfp4.hpp:35-41
+    m: int = 0
+    n: int = 0
+    packed: Optional[np.ndarray] = None   # [m][n/2], low nibble = first of two values
+    scales: Optional[np.ndarray] = None   # [m][n/16] E4M3 block scales
+    global_scale: float = 1.0
+
+
+def nvfp4_quantize(w):
+    """nvfp4_quantize, src/nvfp4.cpp:12-55 (host)."""
+    w = np.ascontiguousarray(w, np.float32)
+    m, n = w.shape
+    t = Nvfp4Tensor(m=m, n=n, packed=np.zeros((m, n // 2), np.uint8), scales=np.zeros((m, max(n // 16, 0)), np.uint8))
+    g = C.c_float()
+    _check(lib().qtip_nvfp4_quantize(_ptr(w), m, n, _ptr(t.packed), _ptr(t.scales), C.byref(g)))
+    t.global_scale = g.value
+    return t
+
+
+def nvfp4_dequantize(t: Nvfp4Tensor):
+    """nvfp4_dequantize, src/nvfp4.cpp:57-70 (host)."""
+    out = np.zeros((t.m, t.n), np.float32)
+    _check(lib().qtip_nvfp4_dequantize(_ptr(np.ascontiguousarray(t.packed)), _ptr(np.ascontiguousarray(t.scales)),
+                                       t.global_scale, t.m, t.n, _ptr(out)))
+    return out
+
+
+def nvfp4_prepare(H, sigma_reg=1e-2, calibrate=True, threads=16):
+    """Host preparation of the calibrated quantizer (src/nvfp4_gpu.hip:181-207) -> (L or None, dw)."""
+    H = np.ascontiguousarray(H, np.float32)
+    n = H.shape[0]
+    L = np.zeros((n, n), np.float32) if calibrate else None
+    dw = np.zeros(n, np.float32)
+    _check(lib().qtip_nvfp4_prepare(_ptr(H), n, sigma_reg, 1 if calibrate else 0, threads, _ptr(L), _ptr(dw)))
+    return L, dw
+
+
+def f32_to_fp8e4m3(x):
+    return int(lib().qtip_f32_to_fp8e4m3(float(x)))
+
+
 class LayerFileWriter:
     """safetensors container of a quantized layer (SafeTensorsWriter, src/safetensors.cpp:93-137; tensor set of
     write_layer_file, src/pipeline.cpp:315-352).  Host only."""
@@ -458,6 +552,12 @@ class LayerFileWriter:
         co.trellis, co.su_bf16, co.sv, co.wscale = _ptr(tr), _ptr(su), _ptr(sv), out.wscale
         tl = None if tlut_f16 is None else np.ascontiguousarray(tlut_f16, np.uint16)
         _check(lib().qtip_st_add_qtip_linear(self._h, prefix.encode(), C.addressof(co), out.m, out.n, _ptr(tl)))
+
+    def add_nvfp4_linear(self, prefix, t: "Nvfp4Tensor"):
+        """weight_packed / weight_scale / weight_global_scale of an NVFP4 linear (src/pipeline.cpp:342-346)."""
+        self.add(prefix + "weight_packed", "U8", [t.m, t.n // 2], t.packed)
+        self.add(prefix + "weight_scale", "F8_E4M3", [t.m, t.n // 16], t.scales)
+        self.add(prefix + "weight_global_scale", "F32", [], np.array([t.global_scale], np.float32))
 
     def write(self, path, metadata=None):
         n = C.c_uint64()

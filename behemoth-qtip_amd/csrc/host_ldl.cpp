@@ -304,6 +304,11 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
 
 }  // namespace
 
+bool cholesky_lower_host(double* A, int n, int threads) {
+  HostTeam& team = team_of_this_thread(threads);
+  return cholesky_panels<NB, TILE>(A, n, n, &team, true);
+}
+
 bool block_ldl_host(double* A, int n, float* L_out, int threads) {
   if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
   HostTeam& team = team_of_this_thread(threads);

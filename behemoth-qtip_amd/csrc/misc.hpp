@@ -12,4 +12,11 @@ void launch_decode_trellis(const uint16_t* trellis, long m, long n, const float*
 // H (n x n fp32) += X^T X for X = rows x n bf16, tiles on or below the diagonal only; then mirror + scale (hessian.hip)
 void launch_hessian_accumulate(const uint16_t* X, long rows, long n, float* H, hipStream_t s);
 void launch_hessian_finish(float* H, long n, float scale, hipStream_t s);
+// NVFP4 fallback quantizer (nvfp4.hip): one 16-column block of the transposed matrices, the feedback of its residual
+// into the columns before it, and a byte transposer for the outputs
+void launch_nvfp4_block(const float* WT, const float* FT, long m, long n, long c0, const float* L, const float* dw,
+                        float global, bool calibrate, bool search, uint8_t* packedT, uint8_t* scalesT, float* E,
+                        hipStream_t s);
+void launch_nvfp4_feedback(float* FT, long m, long n, long c0, const float* E, const float* L, hipStream_t s);
+void launch_transpose_u8(const uint8_t* in, long rows, long cols, uint8_t* out, hipStream_t s);
 }  // namespace qtipmi

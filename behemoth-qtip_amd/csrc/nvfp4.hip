@@ -1,0 +1,219 @@
+// NVFP4 fallback quantizer on the device: scale search and Hessian-calibrated rounding (reference:
+// nvfp4_quantize_group, nv_block_kernel and nv_feedback_kernel, src/nvfp4_gpu.hip:66-243; format src/nvfp4.hpp).
+// Every fp32 operation is the reference kernel's, in its order and without fused multiply-adds, so the bytes equal a
+// CPU evaluation of the same formulas.
+//
+// Layout: the reference walks row-major W with one thread per matrix row, so neighbouring lanes are n floats apart.
+// Here W, the feedback F and the outputs live transposed on the device ([column][row]): a wave's 64 rows are one
+// 256-byte line for every column it touches.  Columns are processed in 16-wide blocks from the last to the first;
+// the residual of a finished block goes to all remaining columns before the next block starts.
+#include "misc.hpp"
+#include "qtip_internal.hpp"
+
+namespace qtipmi {
+namespace {
+
+__device__ __forceinline__ float nv_fp8_dec(unsigned b) {  // non-negative E4M3 code -> value
+  const unsigned e = (b >> 3) & 0xf, m = b & 7;
+  return e == 0 ? ldexpf(float(m), -9) : ldexpf(float(m | 8), int(e) - 10);
+}
+__device__ __forceinline__ unsigned nv_round_even(float v) {
+  const float f = floorf(v), r = v - f;
+  const unsigned n = unsigned(f);
+  return n + unsigned(r > .5f || (r == .5f && (n & 1u)));
+}
+__device__ __forceinline__ unsigned nv_fp8_enc(float x) {  // non-negative finite x, saturating at 448 = code 126
+  x = fminf(fabsf(x), 448.f);
+  if (x < ldexpf(1.f, -6)) return nv_round_even(x * 512.f);
+  int exp;
+  const float frac = frexpf(x, &exp) * 2;
+  unsigned mant = nv_round_even((frac - 1) * 8);
+  int ee = exp + 6;
+  if (mant == 8) {
+    mant = 0;
+    ++ee;
+  }
+  const unsigned c = (unsigned(ee) << 3) | mant;
+  return c < 126u ? c : 126u;
+}
+__device__ __forceinline__ float nv_bf16_round(float f) {
+  uint32_t u = __float_as_uint(f);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return __uint_as_float(u & 0xffff0000u);
+}
+__device__ __forceinline__ float nv_level(int c) {
+  // 0, .5, 1, 1.5, 2, 3, 4, 6
+  return c < 4 ? 0.5f * float(c) : (c < 6 ? float(c - 2) : (c == 6 ? 4.f : 6.f));
+}
+// nearest E2M1 magnitude code of a >= 0, ties to the even code
+__device__ __forceinline__ int nv_fp4_code(float a) {
+  float best = __builtin_inff();
+  int code = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float e = fabsf(a - nv_level(i));
+    if (e < best || (e == best && (i % 2 == 0))) {
+      best = e;
+      code = i;
+    }
+  }
+  return code;
+}
+
+constexpr int kCand = 11;
+
+// One thread per matrix row, one 16-column block (columns c0 .. c0 + 15) per launch.
+//   t_k  = W[k] + F[k] + sum_{j > k in block} d_j Lb[j][k]   target after the feedback
+//   q_k  = bf16(level * dec(s) * global)                       what execution sees
+//   d_k  = W[k] - q_k                                          error fed back
+//   cost = sum_k dw[k] (t_k - q_k)^2                           proxy increment
+// WT, FT: [n][m].  packedT: [n/2][m], scalesT: [n/16][m], E: [16][m].
+__global__ __launch_bounds__(256) void nv_block_kernel(const float* __restrict__ WT, const float* __restrict__ FT, long m,
+                                                       long n, long c0, const float* __restrict__ L,
+                                                       const float* __restrict__ dw, float global, int calibrate,
+                                                       int search, uint8_t* __restrict__ packedT,
+                                                       uint8_t* __restrict__ scalesT, float* __restrict__ E) {
+  __shared__ float Lb[16][16];
+  __shared__ float Dw[16];
+  {
+    const int idx = threadIdx.x;
+    Lb[idx / 16][idx % 16] = calibrate ? L[(c0 + idx / 16) * n + c0 + idx % 16] : 0.f;
+    if (idx < 16) Dw[idx] = dw ? dw[c0 + idx] : 1.f;
+  }
+  __syncthreads();
+  const long r = long(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (r >= m) return;
+  float w[16], base[16];
+  float amax = 0;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    w[k] = WT[(c0 + k) * m + r];
+    base[k] = w[k] + (calibrate ? FT[(c0 + k) * m + r] : 0.f);
+    amax = fmaxf(amax, fabsf(calibrate ? base[k] : w[k]));
+  }
+  unsigned cand[kCand];
+  int nc = 0;
+  const unsigned c1 = nv_fp8_enc(amax / (6.f * global));
+  cand[nc++] = c1;
+  if (search) {
+    const float g[8] = {0.70f, 0.75f, 0.80f, 0.85f, 0.90f, 0.95f, 1.00f, 1.05f};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) cand[nc++] = nv_fp8_enc(amax * g[i] / (6.f * global));
+    cand[nc++] = c1 > 0 ? c1 - 1 : 0;
+    cand[nc++] = c1 < 126 ? c1 + 1 : 126;
+  }
+  float best_cost = __builtin_inff();
+  unsigned best = c1;
+  for (int ci = 0; ci < nc; ++ci) {
+    const unsigned s = cand[ci];
+    const float sd = nv_fp8_dec(s);
+    const float scale = sd * global;
+    float err[16];
+    float cost = 0;
+#pragma unroll
+    for (int k = 15; k >= 0; --k) {
+      float t = base[k];
+      if (calibrate) {
+#pragma unroll
+        for (int j = k + 1; j < 16; ++j) t += err[j] * Lb[j][k];
+      }
+      const float x = scale != 0.f ? t / scale : 0.f;
+      const int code = nv_fp4_code(fabsf(x));
+      const float q = nv_bf16_round((x < 0 ? -1.f : 1.f) * nv_level(code) * sd * global);
+      cost += Dw[k] * (t - q) * (t - q);
+      err[k] = w[k] - q;
+    }
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = s;
+    }
+  }
+  const float sd = nv_fp8_dec(best);
+  const float scale = sd * global;
+  float err[16];
+  unsigned nib[16];
+#pragma unroll
+  for (int k = 15; k >= 0; --k) {
+    float t = base[k];
+    if (calibrate) {
+#pragma unroll
+      for (int j = k + 1; j < 16; ++j) t += err[j] * Lb[j][k];
+    }
+    const float x = scale != 0.f ? t / scale : 0.f;
+    const int code = nv_fp4_code(fabsf(x));
+    const float q = nv_bf16_round((x < 0 ? -1.f : 1.f) * nv_level(code) * sd * global);
+    err[k] = w[k] - q;
+    nib[k] = unsigned(code) | ((__float_as_uint(x) >> 31) ? 8u : 0u);
+  }
+#pragma unroll
+  for (int k = 0; k < 16; k += 2) packedT[((c0 + k) / 2) * m + r] = uint8_t(nib[k] | (nib[k + 1] << 4));
+  scalesT[(c0 / 16) * m + r] = uint8_t(best);
+#pragma unroll
+  for (int k = 0; k < 16; ++k) E[k * m + r] = err[k];
+}
+
+// FT[col][r] += sum_{j < 16} E[j][r] * L[c0 + j][col]  for col < c0 (the sum first, in j order, then one add).
+// A workgroup: 256 rows x 32 columns; the 16 x 32 piece of L sits in LDS.
+__global__ __launch_bounds__(256) void nv_feedback_kernel(float* __restrict__ FT, long m, long n, long c0,
+                                                          const float* __restrict__ E, const float* __restrict__ L) {
+  __shared__ float Ls[16][32];
+  const long col0 = long(blockIdx.y) * 32;
+  for (int idx = threadIdx.x; idx < 512; idx += 256) {
+    const int j = idx >> 5, c = idx & 31;
+    Ls[j][c] = col0 + c < c0 ? L[(c0 + j) * n + col0 + c] : 0.f;
+  }
+  __syncthreads();
+  const long r = long(blockIdx.x) * 256 + threadIdx.x;
+  if (r >= m) return;
+  float e[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) e[j] = E[j * m + r];
+  const int ncol = int(c0 - col0 < 32 ? c0 - col0 : 32);
+  for (int c = 0; c < ncol; ++c) {
+    float acc = 0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc += e[j] * Ls[j][c];
+    FT[(col0 + c) * m + r] += acc;
+  }
+}
+
+// bytes [rows][cols] -> [cols][rows], 32 x 32 patches through LDS
+__global__ __launch_bounds__(256) void transpose_u8_kernel(const uint8_t* __restrict__ in, long rows, long cols,
+                                                           uint8_t* __restrict__ out) {
+  __shared__ uint8_t tile[32][33];
+  const long r0 = long(blockIdx.y) * 32, c0 = long(blockIdx.x) * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const long r = r0 + ty + 8 * k, c = c0 + tx;
+    tile[ty + 8 * k][tx] = r < rows && c < cols ? in[r * cols + c] : uint8_t(0);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const long c = c0 + ty + 8 * k, r = r0 + tx;
+    if (c < cols && r < rows) out[c * rows + r] = tile[tx][ty + 8 * k];
+  }
+}
+
+}  // namespace
+
+void launch_nvfp4_block(const float* WT, const float* FT, long m, long n, long c0, const float* L, const float* dw,
+                        float global, bool calibrate, bool search, uint8_t* packedT, uint8_t* scalesT, float* E,
+                        hipStream_t s) {
+  nv_block_kernel<<<dim3(unsigned((m + 255) / 256)), dim3(256), 0, s>>>(WT, FT, m, n, c0, L, dw, global, calibrate ? 1 : 0,
+                                                                        search ? 1 : 0, packedT, scalesT, E);
+  QTIP_HIP(hipGetLastError());
+}
+void launch_nvfp4_feedback(float* FT, long m, long n, long c0, const float* E, const float* L, hipStream_t s) {
+  if (c0 <= 0) return;
+  nv_feedback_kernel<<<dim3(unsigned((m + 255) / 256), unsigned((c0 + 31) / 32)), dim3(256), 0, s>>>(FT, m, n, c0, E, L);
+  QTIP_HIP(hipGetLastError());
+}
+void launch_transpose_u8(const uint8_t* in, long rows, long cols, uint8_t* out, hipStream_t s) {
+  if (rows <= 0 || cols <= 0) return;
+  transpose_u8_kernel<<<dim3(unsigned((cols + 31) / 32), unsigned((rows + 31) / 32)), dim3(256), 0, s>>>(in, rows, cols, out);
+  QTIP_HIP(hipGetLastError());
+}
+
+}  // namespace qtipmi

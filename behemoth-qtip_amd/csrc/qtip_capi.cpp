@@ -252,6 +252,46 @@ int qtip_hessian_finish_dev(qtip_ctx* ctx, float* dev_H, int n, double scale) {
   });
 }
 
+uint8_t qtip_f32_to_fp8e4m3(float x) { return f32_to_fp8e4m3(x); }
+int qtip_nvfp4_quantize(const float* host_w, int m, int n, uint8_t* host_packed, uint8_t* host_scales, float* global) {
+  return guarded([&] { nvfp4_quantize_host(host_w, m, n, host_packed, host_scales, global); });
+}
+int qtip_nvfp4_dequantize(const uint8_t* host_packed, const uint8_t* host_scales, float global, int m, int n,
+                          float* host_out) {
+  return guarded([&] { nvfp4_dequantize_host(host_packed, host_scales, global, m, n, host_out); });
+}
+int qtip_nvfp4_prepare(const float* host_H, int n, double sigma_reg, int calibrate, int threads, float* host_L,
+                       float* host_dw) {
+  return guarded([&] { nvfp4_prepare_host(host_H, n, sigma_reg, calibrate != 0, threads, host_L, host_dw); });
+}
+int qtip_nvfp4_quantize_prepared(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mats, int n, const float* host_L,
+                                 const float* host_dw, int scale_search) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "nvfp4_quantize_prepared: bad arguments");
+    DeviceGuard g(ctx);
+    nvfp4_quantize_prepared_impl(ctx, nmat, mats, n, host_L, host_dw, scale_search != 0);
+  });
+}
+int qtip_nvfp4_quantize_group(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mats, int n, const float* host_H,
+                              const qtip_nvfp4_opts* opts, int* calibrated) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && n > 0 && n % 16 == 0, "nvfp4_quantize_group: bad arguments");
+    DeviceGuard g(ctx);
+    qtip_nvfp4_opts o{1, 1, 1e-2};
+    if (opts) o = *opts;
+    const bool cal = o.calibrate != 0 && host_H != nullptr;
+    if (calibrated) *calibrated = cal ? 1 : 0;
+    std::vector<float> L, dw;
+    if (host_H) {
+      dw.resize(static_cast<size_t>(n));
+      if (cal) L.resize(size_t(n) * n);
+      nvfp4_prepare_host(host_H, n, o.sigma_reg, cal, 16, cal ? L.data() : nullptr, dw.data());
+    }
+    nvfp4_quantize_prepared_impl(ctx, nmat, mats, n, cal ? L.data() : nullptr, host_H ? dw.data() : nullptr,
+                                 o.scale_search != 0);
+  });
+}
+
 int qtip_run_groups(qtip_ctx* ctx, int ngroups, const qtip_group* groups, const qtip_opts* opts, qtip_timing* timings,
                     double* ldl_wait_s) {
   return guarded([&] {

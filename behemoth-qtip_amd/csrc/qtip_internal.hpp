@@ -131,6 +131,8 @@ struct HostScratch {
 
 // fp64 block LDL on the host (host_ldl.cpp). A: n x n fp64, lower triangle used, destroyed. Returns false if not PD.
 bool block_ldl_host(double* A, int n, float* L_out, int threads);
+// lower Cholesky in place (lower triangle of the n x n fp64 matrix A); false if not positive definite
+bool cholesky_lower_host(double* A, int n, int threads);
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle
 void symmetrize_lower_host(const float* HRr, int n, double* A, int threads);
 

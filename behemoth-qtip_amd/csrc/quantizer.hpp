@@ -252,6 +252,66 @@ inline std::vector<float> dequantize_linear(const LinearOut& lo) {
   return h;
 }
 
+// ---- NVFP4 fallback format (src/nvfp4.hpp:35-60, src/nvfp4_gpu.hpp:17-30): same names, same bytes.
+inline uint8_t f32_to_fp8e4m3(float x) { return qtip_f32_to_fp8e4m3(x); }
+
+struct Nvfp4Tensor {
+  int m = 0, n = 0;             // out x in, n a multiple of 16
+  std::vector<uint8_t> packed;  // [m][n/2], low nibble = first of two values
+  std::vector<uint8_t> scales;  // [m][n/16] E4M3 block scales
+  float global = 1;             // F32 global scale
+  int64_t size_bytes() const { return int64_t(packed.size()) + int64_t(scales.size()) + 4; }
+};
+
+struct Nvfp4Opts {
+  bool scale_search = true;
+  bool calibrate = true;
+  double sigma_reg = 1e-2;
+};
+
+inline Nvfp4Tensor nvfp4_quantize(const float* w, int m, int n) {
+  Nvfp4Tensor t;
+  t.m = m, t.n = n;
+  t.packed.resize(size_t(m) * size_t(n > 0 ? n / 2 : 0));
+  t.scales.resize(size_t(m) * size_t(n > 0 ? n / 16 : 0));
+  detail::check(qtip_nvfp4_quantize(w, m, n, t.packed.data(), t.scales.data(), &t.global), "nvfp4_quantize");
+  return t;
+}
+
+inline std::vector<float> nvfp4_dequantize(const Nvfp4Tensor& t) {
+  std::vector<float> out(size_t(t.m) * size_t(t.n));
+  detail::check(qtip_nvfp4_dequantize(t.packed.data(), t.scales.data(), t.global, t.m, t.n, out.data()), "nvfp4_dequantize");
+  return out;
+}
+
+inline float nvfp4_level(uint8_t code) {
+  constexpr float levels[8] = {0, .5f, 1, 1.5f, 2, 3, 4, 6};
+  return (code & 8 ? -1.f : 1.f) * levels[code & 7];
+}
+
+// The stream argument is accepted for source compatibility; the work runs on the context's own stream and the call
+// returns when the tensors are on the host.
+inline std::vector<Nvfp4Tensor> nvfp4_quantize_group(hipStream_t, const std::vector<const float*>& ws,
+                                                     const std::vector<int>& ms, int n, const float* H,
+                                                     const Nvfp4Opts& opt, bool* calibrated = nullptr) {
+  if (ws.size() != ms.size()) detail::die("nvfp4_quantize_group: ws and ms differ in length");
+  std::vector<Nvfp4Tensor> out(ws.size());
+  std::vector<qtip_nvfp4_matrix> mats(ws.size());
+  for (size_t i = 0; i < ws.size(); ++i) {
+    out[i].m = ms[i], out[i].n = n;
+    out[i].packed.resize(size_t(ms[i] > 0 ? ms[i] : 0) * size_t(n > 0 ? n / 2 : 0));
+    out[i].scales.resize(size_t(ms[i] > 0 ? ms[i] : 0) * size_t(n > 0 ? n / 16 : 0));
+    mats[i] = qtip_nvfp4_matrix{ms[i], ws[i], out[i].packed.data(), out[i].scales.data(), 1.f};
+  }
+  qtip_nvfp4_opts o{opt.scale_search ? 1 : 0, opt.calibrate ? 1 : 0, opt.sigma_reg};
+  int used = 0;
+  detail::check(qtip_nvfp4_quantize_group(detail::context(), int(mats.size()), mats.data(), n, H, &o, &used),
+                "nvfp4_quantize_group");
+  for (size_t i = 0; i < ws.size(); ++i) out[i].global = mats[i].global;
+  if (calibrated) *calibrated = used != 0;
+  return out;
+}
+
 // src/safetensors.hpp:52-70: same calls, same file bytes.
 class SafeTensorsWriter {
  public:
@@ -269,6 +329,12 @@ class SafeTensorsWriter {
     qtip_linear_out o{const_cast<uint16_t*>(r.trellis.data()), const_cast<uint16_t*>(r.su_bf16.data()),
                       const_cast<float*>(r.sv.data()), nullptr, r.wscale, 0.0, 0.0, 0.0};
     detail::check(qtip_st_add_qtip_linear(w_, prefix.c_str(), &o, r.m, r.n, tlut_f16), "SafeTensorsWriter::add_qtip_linear");
+  }
+  // the three tensors write_layer_file stores for an NVFP4 linear (src/pipeline.cpp:342-346)
+  void add_nvfp4_linear(const std::string& prefix, const Nvfp4Tensor& t) {
+    add(prefix + "weight_packed", "U8", {t.m, int64_t(t.n) / 2}, t.packed.data(), t.packed.size());
+    add(prefix + "weight_scale", "F8_E4M3", {t.m, int64_t(t.n) / 16}, t.scales.data(), t.scales.size());
+    add(prefix + "weight_global_scale", "F32", {}, &t.global, 4);
   }
   size_t write(const std::string& path, const std::map<std::string, std::string>& metadata = {{"format", "pt"}}) const {
     std::vector<const char*> kv;

@@ -31,4 +31,10 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
 void reserve_group_ring(qtip_ctx* c, int n, int depth);
 void run_groups_impl(qtip_ctx* c, int ngroups, const qtip_group* groups, const qtip_opts& opt, qtip_timing* timings,
                      double* ldl_wait);
+uint8_t f32_to_fp8e4m3(float x);
+void nvfp4_quantize_host(const float* w, int m, int n, uint8_t* packed, uint8_t* scales, float* global);
+void nvfp4_dequantize_host(const uint8_t* packed, const uint8_t* scales, float global, int m, int n, float* out);
+void nvfp4_prepare_host(const float* H, int n, double sigma_reg, bool calibrate, int threads, float* L, float* dw);
+void nvfp4_quantize_prepared_impl(qtip_ctx* c, int nmat, const qtip_nvfp4_matrix* mats, int n, const float* host_L,
+                                  const float* host_dw, bool search);
 }  // namespace qtipmi

@@ -93,6 +93,43 @@ int main() {
     std::printf("layer file: %zu bytes\n", bytes);
     if (sz != long(bytes) || bytes < out[0].trellis.size() * 2 + out[1].trellis.size() * 2) ++fail;
   }
+  // NVFP4 fallback (the criteria of tests/test_nvfp4.cpp:59-105): upgrades off == the plain quantizer byte for byte,
+  // calibrated rounding lowers the Hessian-weighted error, a group equals single calls
+  {
+    auto proxy = [&](const std::vector<float>& W, const Nvfp4Tensor& t) {
+      std::vector<float> q = nvfp4_dequantize(t);
+      double tot = 0;
+      for (int i = 0; i < t.m; ++i) {
+        std::vector<double> e(static_cast<size_t>(n), 0.0);
+        for (int j = 0; j < n; ++j) e[size_t(j)] = double(W[size_t(i) * n + j]) - q[size_t(i) * n + j];
+        for (int a = 0; a < n; ++a) {
+          double acc = 0;
+          for (int b = 0; b < n; ++b) acc += double(H[size_t(a) * n + b]) * e[size_t(b)];
+          tot += e[size_t(a)] * acc;
+        }
+      }
+      return tot / t.m;
+    };
+    Nvfp4Tensor plain = nvfp4_quantize(W1.data(), 64, n);
+    Nvfp4Opts off;
+    off.scale_search = off.calibrate = false;
+    bool used = true;
+    auto a = nvfp4_quantize_group(S, {W1.data()}, {64}, n, nullptr, off, &used);
+    if (used || a[0].packed != plain.packed || a[0].scales != plain.scales || a[0].global != plain.global) ++fail;
+    auto b = nvfp4_quantize_group(S, {W1.data(), W2.data()}, {64, 32}, n, H.data(), Nvfp4Opts{}, &used);
+    auto c = nvfp4_quantize_group(S, {W2.data()}, {32}, n, H.data(), Nvfp4Opts{});
+    if (!used || b[1].packed != c[0].packed || b[1].scales != c[0].scales) ++fail;
+    const double p0 = proxy(W1, plain), p1 = proxy(W1, b[0]);
+    std::printf("nvfp4: proxy plain %.6g calibrated %.6g (%.1f%%), %lld bytes\n", p0, p1, 100 * p1 / p0,
+                static_cast<long long>(b[0].size_bytes()));
+    if (!(p1 < 0.9 * p0)) ++fail;
+    if (f32_to_fp8e4m3(448.f) != 126 || f32_to_fp8e4m3(-1.f) != (128 | 56) || nvfp4_level(0xf) != -6.f) ++fail;
+    SafeTensorsWriter w;
+    w.add_nvfp4_linear("model.layers.0.a.", b[0]);
+    const char* path = "/tmp/qtip_shim_test_nv.safetensors";
+    if (w.write(path) < b[0].packed.size() + b[0].scales.size() + 4) ++fail;
+    std::remove(path);
+  }
   std::printf(fail ? "SHIM TEST FAILED\n" : "SHIM TEST PASSED\n");
   return fail ? 1 : 0;
 }

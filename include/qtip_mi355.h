@@ -149,6 +149,40 @@ int qtip_quantize_group_h(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, i
 int qtip_hessian_accumulate_dev(qtip_ctx* ctx, const uint16_t* dev_X_bf16, long rows, int n, float* dev_H);
 int qtip_hessian_finish_dev(qtip_ctx* ctx, float* dev_H, int n, double scale);
 
+/* NVFP4 fallback quantizer (src/nvfp4.hpp, src/nvfp4.cpp, src/nvfp4_gpu.hpp, src/nvfp4_gpu.hip): two E2M1 values per
+ * byte (low nibble first), one E4M3 scale per 16 input channels of a row, one fp32 global scale per matrix; the
+ * tensors a layer file stores as weight_packed U8 [m][n/2], weight_scale F8_E4M3 [m][n/16], weight_global_scale F32. */
+uint8_t qtip_f32_to_fp8e4m3(float x); /* src/nvfp4.hpp:15-33 */
+/* nvfp4_quantize, src/nvfp4.cpp:12-55 (host, nearest value): w m x n fp32 -> packed, scales, *global */
+int qtip_nvfp4_quantize(const float* host_w, int m, int n, uint8_t* host_packed, uint8_t* host_scales, float* global);
+/* nvfp4_dequantize, src/nvfp4.cpp:57-70 (host; values rounded to bf16, as execution sees them) */
+int qtip_nvfp4_dequantize(const uint8_t* host_packed, const uint8_t* host_scales, float global, int m, int n,
+                          float* host_out);
+typedef struct { /* Nvfp4Opts, src/nvfp4_gpu.hpp:21-25 */
+  int scale_search; /* 1 */
+  int calibrate;    /* 1 */
+  double sigma_reg; /* 1e-2 */
+} qtip_nvfp4_opts;
+typedef struct { /* one matrix of a group: input and the caller-allocated outputs (Nvfp4Tensor, src/nvfp4.hpp:35-41) */
+  int m;
+  const float* w;  /* host [m][n] fp32 */
+  uint8_t* packed; /* host [m][n/2] */
+  uint8_t* scales; /* host [m][n/16] */
+  float global;    /* out */
+} qtip_nvfp4_matrix;
+/* nvfp4_quantize_group, src/nvfp4_gpu.hip:174-241: the matrices share one input Hessian host_H (n x n fp32; may be
+ * NULL: no calibration, scale search weighted uniformly).  *calibrated (may be NULL) tells whether H was used for the
+ * rounding.  QTIP_E_NOT_PD if the regularised Hessian is not positive definite. */
+int qtip_nvfp4_quantize_group(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mats, int n, const float* host_H,
+                              const qtip_nvfp4_opts* opts, int* calibrated);
+/* The two halves of the call above, for callers that keep the factor: host preparation (src/nvfp4_gpu.hip:181-207:
+ * calibrate -> unit-lower L with H = L D L^T and dw = D, else dw = diag(H) + creg, L untouched) and the device block
+ * loop (:209-241) on a prepared factor (host_L NULL: no calibration; host_dw NULL: uniform weights). */
+int qtip_nvfp4_prepare(const float* host_H, int n, double sigma_reg, int calibrate, int threads, float* host_L,
+                       float* host_dw);
+int qtip_nvfp4_quantize_prepared(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mats, int n, const float* host_L,
+                                 const float* host_dw, int scale_search);
+
 /* Several groups through one context with the overlap of run_qtip_groups, src/pipeline.cpp:229-312: Hessians are
  * rotated on the GPU ahead of use, a side thread runs the host fp64 LDL of the groups in order, and group g is
  * quantized as soon as its factor is ready (the LDL of group g+1 overlaps the GPU work of group g).  HRr and L live

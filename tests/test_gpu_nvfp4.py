@@ -1,0 +1,94 @@
+"""GPU parity of the NVFP4 fallback quantizer through the C ABI: the device block loop (scale search, calibrated
+rounding) against the oracle's CPU restatement of the same formulas, byte for byte, and the criteria of the
+reference's own test (tests/test_nvfp4.cpp:59-105)."""
+import numpy as np
+import pytest
+
+from test_oracle_nvfp4 import _hessian, _weights
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+@pytest.mark.parametrize("name", ["gauss", "heavy"])
+def test_block_loop_bytes_equal_the_cpu_restatement(qz, pkg, oracle, name):
+    say("case: nvfp4 block loop %s" % name)
+    w, _ = _weights(oracle, name)
+    m, n = w.shape
+    H = _hessian(oracle, n, 21)
+    L, D = oracle.nvfp4_prepare(H, 1e-2, True)
+    _, dH = oracle.nvfp4_prepare(H, 1e-2, False)
+    g = oracle.nvfp4_quantize(w)[2]
+    for (Lx, dx, search) in ((None, None, False), (None, None, True), (None, dH, True), (L, D, False), (L, D, True)):
+        t = qz.nvfp4_quantize_prepared([w], n, Lx, dx, search)[0]
+        want = oracle.nvfp4_blocks(w, Lx, dx, g, Lx is not None, search)
+        assert t.global_scale == g
+        assert np.array_equal(t.packed, want[0]) and np.array_equal(t.scales, want[1]), (Lx is not None, dx is not None, search)
+    # upgrades off: the plain host quantizer, byte for byte (tests/test_nvfp4.cpp:64-67)
+    plain = pkg.nvfp4_quantize(w)
+    off = qz.nvfp4_quantize_group([w], n, None, scale_search=False, calibrate=False)[0][0]
+    assert np.array_equal(off.packed, plain.packed) and np.array_equal(off.scales, plain.scales)
+    assert off.global_scale == plain.global_scale
+
+
+@pytest.mark.parametrize("name", ["gauss", "heavy"])
+def test_group_meets_the_reference_test_criteria(qz, pkg, oracle, name):
+    say("case: nvfp4 group %s" % name)
+    w, _ = _weights(oracle, name)
+    m, n = w.shape
+    H = _hessian(oracle, n, 21)
+    naive = pkg.nvfp4_quantize(w)
+    dq = pkg.nvfp4_dequantize
+    (cal,), used = qz.nvfp4_quantize_group([w], n, H)
+    assert used
+    (search_h,), used2 = qz.nvfp4_quantize_group([w], n, H, calibrate=False)
+    assert not used2
+    (search_plain,), _ = qz.nvfp4_quantize_group([w], n, None, calibrate=False)
+    (cal_only,), _ = qz.nvfp4_quantize_group([w], n, H, scale_search=False)
+    pe = oracle.nvfp4_proxy_error
+    p_naive, p_search, p_cal, p_cal_only = pe(w, dq(naive), H), pe(w, dq(search_h), H), pe(w, dq(cal), H), pe(w, dq(cal_only), H)
+    say("  proxy: naive %.4g  search %.4g  calibrated+search %.4g (%.1f%% of naive)  calibrated only %.4g" %
+        (p_naive, p_search, p_cal, 100 * p_cal / p_naive, p_cal_only))
+    assert pe(w, dq(search_plain)) <= pe(w, dq(naive)) * (1 + 1e-9)
+    assert p_search <= p_naive * 1.02 and p_cal < 0.9 * p_naive and p_cal_only <= p_naive
+    for t in (cal, search_h, search_plain, cal_only):
+        assert t.packed.shape == naive.packed.shape and t.global_scale == naive.global_scale
+        assert np.all((t.scales & 0x7f) <= 126) and np.all(np.isfinite(dq(t)))
+    # the library's own factor differs from the oracle's in the last bits at most: nearly all bytes agree
+    L, D = oracle.nvfp4_prepare(H, 1e-2, True)
+    want = oracle.nvfp4_blocks(w, L, D, naive.global_scale, True, True)
+    assert np.mean(cal.packed == want[0]) > 0.98
+    # a group of two matrices equals two single calls
+    grp, _ = qz.nvfp4_quantize_group([w, w[:32]], n, H)
+    (single2,), _ = qz.nvfp4_quantize_group([w[:32]], n, H)
+    assert np.array_equal(grp[0].packed, cal.packed) and np.array_equal(grp[0].scales, cal.scales)
+    assert np.array_equal(grp[1].packed, single2.packed) and np.array_equal(grp[1].scales, single2.scales)
+
+
+def test_nvfp4_layer_shape(qz, pkg, oracle):
+    """A 4096 x 4096 matrix with a dense Hessian: calibrated result beats the plain quantizer in the proxy (fp64 on the
+    device), format valid; prints the time."""
+    import time
+    import torch
+    say("case: nvfp4 4096x4096")
+    m = n = 4096
+    g = torch.Generator(device="cuda").manual_seed(3)
+    w = (torch.randn((m, n), generator=g, device="cuda") * 0.02).cpu().numpy()
+    X = torch.randn((8192, n), generator=g, device="cuda") * torch.exp(0.8 * torch.randn((n,), generator=g, device="cuda"))
+    Hd = (X.T @ X / 8192).double()
+    H = Hd.float().cpu().numpy()
+    t0 = time.time()
+    (cal,), used = qz.nvfp4_quantize_group([w], n, H)
+    dt = time.time() - t0
+    plain = pkg.nvfp4_quantize(w)
+
+    def proxy(t):
+        E = torch.from_numpy(w - pkg.nvfp4_dequantize(t)).cuda().double()
+        return float(((E @ Hd) * E).sum() / m)
+
+    p_cal, p_plain = proxy(cal), proxy(plain)
+    say("  %.2f s; proxy calibrated %.4g, plain %.4g (%.1f%%)" % (dt, p_cal, p_plain, 100 * p_cal / p_plain))
+    assert used and p_cal < 0.9 * p_plain and np.all((cal.scales & 0x7f) <= 126)

@@ -133,3 +133,30 @@ def test_qtip_linear_custom_tlut_and_bad_shapes(pkg, tmp_path):
     bad.m = 24
     with pytest.raises(pkg.QtipError):
         w.add_qtip_linear("r.", bad)
+
+
+def test_nvfp4_layer_file_loads(pkg, tmp_path):
+    """An NVFP4 linear in a layer file (src/pipeline.cpp:342-346): weight_packed U8 [m, n/2], weight_scale F8_E4M3
+    [m, n/16], weight_global_scale F32 scalar; an independent loader reading the scales as E4M3 numbers reproduces the
+    library's dequantizer before its bf16 rounding."""
+    torch = pytest.importorskip("torch")
+    st = pytest.importorskip("safetensors.torch")
+    rng = np.random.default_rng(4)
+    wt = (rng.standard_normal((32, 64)) * 0.03).astype(np.float32)
+    t = pkg.nvfp4_quantize(wt)
+    w = pkg.LayerFileWriter()
+    w.add_nvfp4_linear("model.layers.0.mlp.up_proj.", t)
+    p = str(tmp_path / "nv.safetensors")
+    w.write(p)
+    T = st.load_file(p)
+    b = "model.layers.0.mlp.up_proj."
+    assert T[b + "weight_packed"].dtype == torch.uint8 and tuple(T[b + "weight_packed"].shape) == (32, 32)
+    assert T[b + "weight_scale"].dtype == torch.float8_e4m3fn and tuple(T[b + "weight_scale"].shape) == (32, 4)
+    assert T[b + "weight_global_scale"].shape == () and float(T[b + "weight_global_scale"]) == t.global_scale
+    assert np.array_equal(T[b + "weight_packed"].numpy(), t.packed)
+    levels = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6], np.float32)
+    codes = np.stack([t.packed & 15, t.packed >> 4], axis=-1).reshape(32, 64)
+    sc = T[b + "weight_scale"].float().numpy() * np.float32(t.global_scale)
+    full = levels[codes] * np.repeat(sc, 16, axis=1)
+    bf = torch.from_numpy(full).bfloat16().float().numpy()
+    assert np.array_equal(bf, pkg.nvfp4_dequantize(t))

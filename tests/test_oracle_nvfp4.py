@@ -61,7 +61,8 @@ def test_plain_quantizer_golden(oracle, name):
     assert g == float.fromhex(meta["global"])
     dq = oracle.nvfp4_dequantize(packed, scales, g, m, n)
     assert "%016x" % _fnv1a64(dq.tobytes()) == meta["fnv1a64_dequant"]
-    assert oracle.nvfp4_proxy_error(w, dq) == float.fromhex(meta["mse"])
+    # the sum over rows is an OpenMP reduction in the reference too: its last bits depend on the thread count
+    assert abs(oracle.nvfp4_proxy_error(w, dq) / float.fromhex(meta["mse"]) - 1) < 1e-13
     assert np.all(packed[3, 8:16] & 0x77 == 0) and scales[3, 1] == 0      # the all-zero block
     assert np.all((scales & 0x7f) <= 126)
 
