@@ -1,7 +1,9 @@
 // NVFP4 fallback quantizer on the device: scale search and Hessian-calibrated rounding (reference:
 // nvfp4_quantize_group, nv_block_kernel and nv_feedback_kernel, src/nvfp4_gpu.hip:66-243; format src/nvfp4.hpp).
-// Every fp32 operation is the reference kernel's, in its order and without fused multiply-adds, so the bytes equal a
-// CPU evaluation of the same formulas.
+// Every fp32 operation is the reference kernel's, in its order.  The reference builds with hipcc's default
+// floating-point contraction, which turns its three "sum += a * b" statements (block feedback, cost, column
+// feedback) into fused multiply-adds; this file is built without contraction and writes those three as fmaf, so
+// the bytes equal both the reference's gfx950 build and a CPU evaluation of the same formulas.
 //
 // Layout: the reference walks row-major W with one thread per matrix row, so neighbouring lanes are n floats apart.
 // Here W, the feedback F and the outputs live transposed on the device ([column][row]): a wave's 64 rows are one
@@ -115,12 +117,12 @@ __global__ __launch_bounds__(256) void nv_block_kernel(const float* __restrict__
       float t = base[k];
       if (calibrate) {
 #pragma unroll
-        for (int j = k + 1; j < 16; ++j) t += err[j] * Lb[j][k];
+        for (int j = k + 1; j < 16; ++j) t = fmaf(err[j], Lb[j][k], t);
       }
       const float x = scale != 0.f ? t / scale : 0.f;
       const int code = nv_fp4_code(fabsf(x));
       const float q = nv_bf16_round((x < 0 ? -1.f : 1.f) * nv_level(code) * sd * global);
-      cost += Dw[k] * (t - q) * (t - q);
+      cost = fmaf(Dw[k] * (t - q), t - q, cost);
       err[k] = w[k] - q;
     }
     if (cost < best_cost) {
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(256) void nv_block_kernel(const float* __restrict__
     float t = base[k];
     if (calibrate) {
 #pragma unroll
-      for (int j = k + 1; j < 16; ++j) t += err[j] * Lb[j][k];
+      for (int j = k + 1; j < 16; ++j) t = fmaf(err[j], Lb[j][k], t);
     }
     const float x = scale != 0.f ? t / scale : 0.f;
     const int code = nv_fp4_code(fabsf(x));
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(256) void nv_feedback_kernel(float* __restrict__ FT
   for (int c = 0; c < ncol; ++c) {
     float acc = 0;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) acc += e[j] * Ls[j][c];
+    for (int j = 0; j < 16; ++j) acc = fmaf(e[j], Ls[j][c], acc);
     FT[(col0 + c) * m + r] += acc;
   }
 }

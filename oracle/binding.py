@@ -89,6 +89,114 @@ def lib():
     return L
 
 
+def ref_gpu_lib():
+    """The reference's own device path compiled for gfx950 (None when oracle/_ref was not built).  Its ref_gpu_*
+    functions need a GPU, ref_ldlq does not; in a process that imports torch, import torch first (one HIP runtime per
+    process)."""
+    name = "libqtip_ref_gpu.so"
+    if name in _REF:
+        return _REF[name]
+    path = os.path.join(HERE, "_ref", name)
+    _REF[name] = C.CDLL(path) if os.path.exists(path) else None
+    return _REF[name]
+
+
+def ref_gpu_nvfp4_quantize_group(ws, n, H=None, scale_search=True, calibrate=True, sigma_reg=1e-2):
+    """nvfp4_quantize_group of the reference itself (src/nvfp4_gpu.hip:174-243) -> ([(packed, scales, global)], used)."""
+    R = ref_gpu_lib()
+    ws = [np.ascontiguousarray(w, np.float32) for w in ws]
+    k = len(ws)
+    pk = [np.zeros((w.shape[0], n // 2), np.uint8) for w in ws]
+    sc = [np.zeros((w.shape[0], n // 16), np.uint8) for w in ws]
+    g = np.zeros(k, np.float32)
+    wp = (C.c_void_p * k)(*[w.ctypes.data for w in ws])
+    pp = (C.c_void_p * k)(*[a.ctypes.data for a in pk])
+    sp = (C.c_void_p * k)(*[a.ctypes.data for a in sc])
+    ms = (C.c_int * k)(*[w.shape[0] for w in ws])
+    Hc = None if H is None else np.ascontiguousarray(H, np.float32)
+    R.ref_gpu_nvfp4_quantize_group.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int,
+                                               C.c_double, C.c_void_p, C.c_void_p, C.c_void_p]
+    used = R.ref_gpu_nvfp4_quantize_group(k, wp, ms, n, None if Hc is None else Hc.ctypes.data, int(scale_search),
+                                          int(calibrate), sigma_reg, pp, sp, g.ctypes.data)
+    return [(pk[i], sc[i], float(g[i])) for i in range(k)], bool(used)
+
+
+def ref_ldlq(Wr, L):
+    """ldlq_ref of the reference's GPU test (tests/test_gpu.cpp:180-225; CPU code) -> (hatWr, Q)."""
+    R = ref_gpu_lib()
+    Wr = np.ascontiguousarray(Wr, np.float32)
+    L = np.ascontiguousarray(L, np.float32)
+    m, n = Wr.shape
+    hat = np.zeros((m, n), np.float32)
+    Q = np.zeros(((m // 16) * (n // 16), 128), np.uint16)
+    R.ref_ldlq.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    R.ref_ldlq.restype = None
+    R.ref_ldlq(Wr.ctypes.data, L.ctypes.data, m, n, hat.ctypes.data, Q.ctypes.data)
+    return hat, Q
+
+
+def ref_gpu_quantize_seqs(X):
+    """The reference's device Viterbi, both passes (tests/test_gpu.cpp:67-88) -> (states [B][128], seconds)."""
+    R = ref_gpu_lib()
+    X = np.ascontiguousarray(X, np.float32).reshape(-1, 256)
+    st = np.zeros((X.shape[0], 128), np.uint16)
+    R.ref_gpu_quantize_seqs.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+    R.ref_gpu_quantize_seqs.restype = C.c_double
+    secs = R.ref_gpu_quantize_seqs(X.ctypes.data, X.shape[0], st.ctypes.data)
+    return st, secs
+
+
+def ref_gpu_quantize_group(Ws, H, seed, sigma_reg=1e-2, scale_override=0.9, ldl_threads=16, want_hatW=False):
+    """quantize_group of the reference itself on the GPU (src/quantizer.cpp:340-348): same keys as quantize_group
+    below, per linear, plus its GroupTiming."""
+    R = ref_gpu_lib()
+    Ws = [np.ascontiguousarray(w, np.float32) for w in Ws]
+    H = np.ascontiguousarray(H, np.float32)
+    n = H.shape[0]
+    k = len(Ws)
+    ms = [w.shape[0] for w in Ws]
+    tr = [np.zeros((m // 16) * (n // 16) * 32, np.uint16) for m in ms]
+    su = [np.zeros(n, np.uint16) for _ in ms]
+    sv = [np.zeros(m, np.float32) for m in ms]
+    hw = [np.zeros((m, n), np.float32) for m in ms] if want_hatW else None
+    wscale = np.zeros(k, np.float32)
+    proxy = np.zeros(k)
+    prr = np.zeros(k)
+    tm = np.zeros(8)
+
+    def arr(xs):
+        return (C.c_void_p * k)(*[x.ctypes.data for x in xs])
+
+    R.ref_gpu_quantize_group.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_uint64, C.c_double,
+                                         C.c_double, C.c_int] + [C.c_void_p] * 8
+    R.ref_gpu_quantize_group.restype = None
+    R.ref_gpu_quantize_group(k, arr(Ws), (C.c_int * k)(*ms), n, H.ctypes.data, seed, sigma_reg, scale_override, ldl_threads,
+                             arr(tr), arr(su), arr(sv), arr(hw) if want_hatW else None, wscale.ctypes.data,
+                             proxy.ctypes.data, prr.ctypes.data, tm.ctypes.data)
+    names = ("load", "rht", "ldl_cpu", "ldlq", "viterbi", "proxy", "pack", "total")
+    return dict(trellis=tr, su_bf16=su, sv=sv, hatW=hw, wscale=wscale, proxy=proxy, proxy_rot_reg=prr,
+                timing=dict(zip(names, tm)))
+
+
+def ref_nvfp4_prepare(H, sigma_reg=1e-2):
+    """L (unit lower, fp32) and dw = D of the regularised Hessian as the reference's host code makes them
+    (src/nvfp4_gpu.hip:181-199), with the reference's own compiled cholesky_inplace."""
+    R = ref_lib()
+    H = np.ascontiguousarray(H, np.float32)
+    n = H.shape[0]
+    dsum = 0.0
+    for i in range(n):
+        dsum += float(H[i, i])
+    creg = sigma_reg * dsum / n
+    A = 0.5 * (H.astype(np.float64) + H.T.astype(np.float64))
+    A[np.arange(n), np.arange(n)] += creg
+    A = np.ascontiguousarray(np.tril(A))
+    if R.ref_cholesky(A.reshape(-1), n, 16) != 1:
+        raise ValueError("not positive definite")
+    d = np.diag(A).copy()
+    return np.tril(A / d[None, :], -1).astype(np.float32), (d * d).astype(np.float32)
+
+
 def ref_lib(native=False):
     """The reference's own CPU core compiled in place (None when oracle/_ref was not built)."""
     name = "libqtip_ref_native.so" if native else "libqtip_ref.so"

@@ -927,11 +927,11 @@ static void nv_block_row(const float* w16, const float* f16, const float Lb[16][
     for (int k = 15; k >= 0; --k) {
       float t = base[k];
       if (calibrate)
-        for (int j = k + 1; j < 16; ++j) t += err[j] * Lb[j][k];
+        for (int j = k + 1; j < 16; ++j) t = fmaf(err[j], Lb[j][k], t);
       const float x = scale != 0.f ? t / scale : 0.f;
       const int code = nv_fp4_mag(fabsf(x));
       const float q = qo_bf16_to_f32(qo_f32_to_bf16((x < 0 ? -1.f : 1.f) * kNvLevels[code] * sd * global));
-      cost += Dw[k] * (t - q) * (t - q);
+      cost = fmaf(Dw[k] * (t - q), t - q, cost);
       err[k] = w[k] - q;
     }
     if (cost < best_cost) {
@@ -943,7 +943,7 @@ static void nv_block_row(const float* w16, const float* f16, const float Lb[16][
   for (int k = 15; k >= 0; --k) {
     float t = base[k];
     if (calibrate)
-      for (int j = k + 1; j < 16; ++j) t += err_out[j] * Lb[j][k];
+      for (int j = k + 1; j < 16; ++j) t = fmaf(err_out[j], Lb[j][k], t);
     const float x = scale != 0.f ? t / scale : 0.f;
     const int code = nv_fp4_mag(fabsf(x));
     const float q = qo_bf16_to_f32(qo_f32_to_bf16((x < 0 ? -1.f : 1.f) * kNvLevels[code] * sd * global));
@@ -976,7 +976,7 @@ void qo_nvfp4_blocks(const float* w, int m, int n, const float* L, const float* 
       for (int r = 0; r < m; ++r)
         for (int col = 0; col < c0; ++col) {
           float acc = 0;
-          for (int j = 0; j < 16; ++j) acc += E[(size_t)r * 16 + j] * L[(size_t)(c0 + j) * n + col];
+          for (int j = 0; j < 16; ++j) acc = fmaf(E[(size_t)r * 16 + j], L[(size_t)(c0 + j) * n + col], acc);
           F[(size_t)r * n + col] += acc;
         }
     }

@@ -90,7 +90,9 @@ double qo_proxy(const float* W, const float* hatW, const float* H, int m, int n,
 /* ---- NVFP4 fallback quantizer (two E2M1 values per byte, one E4M3 scale per 16 input channels, one fp32 global
  *      scale per matrix).  Format and the plain quantizer: src/nvfp4.hpp:15-33,54-57, src/nvfp4.cpp:12-87.  Scale
  *      search and Hessian-calibrated rounding: a CPU restatement of the reference's GPU kernels
- *      (src/nvfp4_gpu.hip:66-228) in the same fp32 operation order, no fused multiply-adds. */
+ *      (src/nvfp4_gpu.hip:66-228) in the same fp32 operation order; its three "sum += a * b" statements are fused
+ *      multiply-adds, as hipcc's default contraction compiles them.  Pinned by the bytes the reference's own device
+ *      path returned on a gfx950 GPU (tests/golden/ref_nvfp4_gpu_*) and, on a GPU, by that library itself. */
 uint8_t qo_f32_to_fp8e4m3(float x);
 float qo_fp8e4m3_to_f32(uint8_t b);
 /* nvfp4_quantize, src/nvfp4.cpp:12-55: w m x n fp32 -> packed [m][n/2], scales [m][n/16], *global.  -1 if n % 16. */

@@ -10,6 +10,10 @@ oracle/_ref/libqtip_ref.so exists; the GPU box only reads the committed outputs)
   ref_config1.json        FNV-1a 64 of the packed words of all 4096 config-1 tiles (synthetic tlut)
   ref_config1_packed.bin  those packed words (u16 [4096][32], pack_trellis layout, not swizzled)
   ref_ldl_1024.bin        rows 1000..1007 of L (fp32) from block_ldl_to_L on a seeded n=1024 SPD matrix
+  ref_ldlq_L.bin          a block-LDL factor (f32 [256][256]) and
+  ref_ldlq_Q.bin          the states (u16 [64][128]) ldlq_ref of the reference's GPU test program (CPU code,
+                          tests/test_gpu.cpp:180-225, compiled into oracle/_ref/libqtip_ref_gpu.so) returns for it and
+                          the seeded 64 x 256 Wr of ref_ldlq.json, which also holds the FNV-1a 64 of the returned hatWr
 """
 import json
 import os
@@ -88,6 +92,17 @@ def main():
     L = np.zeros((1024, 1024), np.float32)
     assert R.ref_block_ldl(A.reshape(-1), 1024, L.reshape(-1), 8) == 1
     L[1000:1008].tofile(os.path.join(HERE, "ref_ldl_1024.bin"))
+    # LDLQ with 128-column buffers: the reference's own CPU restatement of ldlq.LDLQ, two buffers, four tile rows
+    if ob.ref_gpu_lib() is not None:
+        m, n = 64, 256
+        Wr = ob.rng_normal(31, m * n).astype(np.float32).reshape(m, n)
+        g = ob.rng_normal(32, n * 2 * n).reshape(n, 2 * n) * (1.0 + (np.arange(2 * n) % 7))
+        Lq = ob.block_ldl(g @ g.T / (2 * n) + 0.05 * np.eye(n))
+        hat, Q = ob.ref_ldlq(Wr, Lq)
+        Lq.tofile(os.path.join(HERE, "ref_ldlq_L.bin"))
+        Q.tofile(os.path.join(HERE, "ref_ldlq_Q.bin"))
+        json.dump({"m": m, "n": n, "w_seed": 31, "fnv1a64_hat": "%016x" % fnv1a64(hat.tobytes())},
+                  open(os.path.join(HERE, "ref_ldlq.json"), "w"))
     # NVFP4: the reference's plain quantizer (src/nvfp4.cpp) on gaussian and heavy-tailed weights (the two cases of
     # tests/test_nvfp4.cpp:47-57, same shapes, this repo's generator), plus the E4M3 encoder on a sweep of values
     nv = {}

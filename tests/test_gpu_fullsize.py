@@ -89,3 +89,36 @@ def test_config5_group_properties(qz, pkg, oracle, synth):
     # states are not degenerate: all 16 new-bit values occur about equally often
     hist = np.bincount((st[::97].reshape(-1) & 15).astype(np.int64), minlength=16) / st[::97].size
     assert hist.min() > 0.04 and hist.max() < 0.09
+
+
+def test_config5_depth_ldlq_rows_against_cpu(qz, pkg, oracle, hyb, synth):
+    """n = 28672, the headline depth: a tile row is a chain of 1792 tiles, each depending on every later column.  Two
+    tile rows (32 weight rows, LDLQ is row-independent) through the GPU LDLQ and through the CPU form with the same L,
+    factored by the library's host LDL from the headline configuration's own Hessian: identical codes (>= 99 % is the
+    bar) down the whole chain."""
+    import torch
+    say("case: config-5 depth LDLQ, 32 rows against the CPU form")
+    qz.set_tlut(None)
+    Ws, H = synth.large_config(5)
+    n, m = H.shape[0], 32
+    H += 0.01 * torch.diagonal(H).mean() * torch.eye(n, device="cuda")
+    W = Ws[0][4000:4000 + m]
+    WT = (W / W.pow(2).mean().sqrt() * 0.9).T.contiguous()        # unit-scale rows at the codebook's working point
+    hp = pkg.HessPrep(n=n, HRr=H.cpu().numpy())
+    del Ws, H
+    pkg.Quantizer.ldl_hessian(hp, threads=16)
+    dL = torch.from_numpy(hp.L).cuda()
+    dH = torch.zeros((n, m), device="cuda")
+    dQ = torch.zeros(((m // 16) * (n // 16), 128), dtype=torch.int16, device="cuda")
+    torch.cuda.synchronize()
+    qz.ldlq_dev(WT, dL, n, m, dH, dQ)
+    qz.synchronize()
+    Q = dQ.cpu().numpy().view(np.uint16)
+    check_trellis_paths(Q)
+    say("  GPU LDLQ done; CPU form on 16 threads ...")
+    hat_o, Q_o = oracle.ldlq(hyb, np.ascontiguousarray(WT.cpu().numpy().T), hp.L, threads=16)
+    same = np.all(Q == Q_o, axis=1)
+    say("  identical trellises: %d of %d" % (int(same.sum()), same.size))
+    assert same.mean() >= 0.99
+    if same.all():
+        assert np.array_equal(dH.cpu().numpy().T, hat_o)

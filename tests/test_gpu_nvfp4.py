@@ -4,7 +4,7 @@ reference's own test (tests/test_nvfp4.cpp:59-105)."""
 import numpy as np
 import pytest
 
-from test_oracle_nvfp4 import _hessian, _weights
+from test_oracle_nvfp4 import _hessian, _weights, device_path_vectors
 
 pytestmark = pytest.mark.gpu
 
@@ -68,6 +68,40 @@ def test_group_meets_the_reference_test_criteria(qz, pkg, oracle, name):
     assert np.array_equal(grp[1].packed, single2.packed) and np.array_equal(grp[1].scales, single2.scales)
 
 
+@pytest.mark.parametrize("name", ["gauss", "heavy"])
+def test_group_bytes_equal_the_golden_device_path_vectors(qz, oracle, name):
+    """The committed bytes of the reference's device path (tests/golden/ref_nvfp4_gpu_*), all option combinations."""
+    say("case: nvfp4 group vs golden device-path vectors, %s" % name)
+    w, _ = _weights(oracle, name)
+    H, cases, g = device_path_vectors(name)
+    for (h, s, c, pk, sc) in cases:
+        (t,), used = qz.nvfp4_quantize_group([w], 256, H if h else None, scale_search=s, calibrate=c)
+        assert used == (h and c) and t.global_scale == g
+        assert np.array_equal(t.packed, pk) and np.array_equal(t.scales, sc), (h, s, c)
+
+
+@pytest.mark.parametrize("name", ["gauss", "heavy"])
+def test_group_bytes_equal_the_reference_device_path(qz, oracle, name):
+    """The reference's own nvfp4_quantize_group, compiled for this GPU from its sources (oracle/_ref), on the same
+    inputs: every packed byte, scale code and global scale of every option combination."""
+    if oracle.ref_gpu_lib() is None:
+        pytest.skip("oracle/_ref/libqtip_ref_gpu.so not built")
+    say("case: nvfp4 group vs the compiled reference, %s" % name)
+    w, _ = _weights(oracle, name)
+    m, n = w.shape
+    H = _hessian(oracle, n, 21)
+    for (Hx, search, cal) in ((None, False, False), (None, True, True), (H, True, False), (H, False, True), (H, True, True)):
+        got, used = qz.nvfp4_quantize_group([w, w[:32]], n, Hx, scale_search=search, calibrate=cal)
+        want, used_ref = oracle.ref_gpu_nvfp4_quantize_group([w, w[:32]], n, Hx, scale_search=search, calibrate=cal)
+        assert used == used_ref
+        for t, (pk, sc, g) in zip(got, want):
+            agree = float(np.mean(t.packed == pk))
+            say("  H %s search %d calibrate %d: packed bytes equal %.4f%%, scales equal %.4f%%" %
+                (Hx is not None, search, cal, 100 * agree, 100 * float(np.mean(t.scales == sc))))
+            assert t.global_scale == g
+            assert np.array_equal(t.scales, sc) and np.array_equal(t.packed, pk)
+
+
 def test_nvfp4_layer_shape(qz, pkg, oracle):
     """A 4096 x 4096 matrix with a dense Hessian: calibrated result beats the plain quantizer in the proxy (fp64 on the
     device), format valid; prints the time."""
@@ -92,3 +126,17 @@ def test_nvfp4_layer_shape(qz, pkg, oracle):
     p_cal, p_plain = proxy(cal), proxy(plain)
     say("  %.2f s; proxy calibrated %.4g, plain %.4g (%.1f%%)" % (dt, p_cal, p_plain, 100 * p_cal / p_plain))
     assert used and p_cal < 0.9 * p_plain and np.all((cal.scales & 0x7f) <= 126)
+    if oracle.ref_gpu_lib() is not None and oracle.ref_lib() is not None:
+        # 16.8 M weights x 11 candidates: a multiply-add rounded differently anywhere in the block loop shows here.
+        # Byte equality is asked with the factor from the reference's own Cholesky; the library's factor differs from
+        # it in the last bit of a few entries, so the group call is held to 99.999 %.
+        t0 = time.time()
+        ((pk, sc, gl),), _ = oracle.ref_gpu_nvfp4_quantize_group([w], n, H)
+        t1 = time.time()
+        L, dw = oracle.ref_nvfp4_prepare(H)
+        same_l = qz.nvfp4_quantize_prepared([w], n, L, dw, True)[0]
+        say("  compiled reference: %.2f s; group call: packed bytes equal %.5f%%, scales %.5f%%; with its factor: %d differ" %
+            (t1 - t0, 100 * float(np.mean(cal.packed == pk)), 100 * float(np.mean(cal.scales == sc)),
+             int((same_l.packed != pk).sum() + (same_l.scales != sc).sum())))
+        assert gl == cal.global_scale and np.array_equal(same_l.scales, sc) and np.array_equal(same_l.packed, pk)
+        assert np.mean(cal.packed == pk) > 0.99999 and np.mean(cal.scales == sc) > 0.99999

@@ -7,7 +7,7 @@ import os
 import numpy as np
 import pytest
 
-from conftest import REFVEC
+from conftest import GOLDEN, REFVEC
 
 
 def load(name, dt):
@@ -372,6 +372,30 @@ def test_ldlq_buffered_equals_naive(oracle, hyb):
             oracle.lib().qo_decode_states(hyb.lut0, hyb.lut1, np.ascontiguousarray(Q[b * (n // 16) + blk]), h)
             tile = hat[16 * b:16 * b + 16, 16 * blk:16 * blk + 16].reshape(-1)
             assert np.array_equal(tile[perm], h)
+
+
+def test_ldlq_equals_the_reference_ldlq(oracle, hyb):
+    """ldlq_ref of the reference's GPU test program (CPU code, tests/test_gpu.cpp:180-225): every state and every
+    reconstructed value of a two-buffer case, from the committed vectors and, where oracle/_ref is built, live."""
+    meta = json.load(open(os.path.join(GOLDEN, "ref_ldlq.json")))
+    m, n = meta["m"], meta["n"]
+    Wr = oracle.rng_normal(meta["w_seed"], m * n).astype(np.float32).reshape(m, n)
+    L = np.fromfile(os.path.join(GOLDEN, "ref_ldlq_L.bin"), np.float32).reshape(n, n)
+    want = np.fromfile(os.path.join(GOLDEN, "ref_ldlq_Q.bin"), np.uint16).reshape(-1, 128)
+    hat, Q = oracle.ldlq(hyb, Wr, L)
+    assert np.array_equal(Q, want)
+    h = 0xcbf29ce484222325
+    for b in hat.tobytes():
+        h = ((h ^ b) * 0x100000001b3) & 0xffffffffffffffff
+    assert "%016x" % h == meta["fnv1a64_hat"]
+    if oracle.ref_gpu_lib() is not None:
+        rng = np.random.default_rng(12)
+        m2, n2 = 32, 384                                  # three buffers
+        W2 = (rng.standard_normal((m2, n2)) * 1.3).astype(np.float32)
+        L2 = oracle.block_ldl(_spd(n2, 13))
+        hat_o, Q_o = oracle.ldlq(hyb, W2, L2)
+        hat_r, Q_r = oracle.ref_ldlq(W2, L2)
+        assert np.array_equal(Q_o, Q_r) and np.array_equal(hat_o, hat_r)
 
 
 def test_ldlq_zero_L_is_tilewise_viterbi(oracle, hyb):

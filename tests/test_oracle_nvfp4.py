@@ -1,7 +1,8 @@
 """Pins the oracle's NVFP4 restatement (no GPU): the plain quantizer and the E4M3 encoder against vectors written by
 the reference's own src/nvfp4.cpp compiled in place (tests/golden/make_ref_vectors.py) and against that library
 directly where it is present; the scale search and the calibrated rounding (a restatement of the reference's GPU
-kernels, src/nvfp4_gpu.hip:66-228) against the criteria of the reference's own test, tests/test_nvfp4.cpp:59-105."""
+kernels, src/nvfp4_gpu.hip:66-228) against the bytes the reference's own device path returned on a gfx950 GPU
+(tests/golden/make_ref_nvfp4_gpu_vectors.py) and the criteria of its test, tests/test_nvfp4.cpp:59-105."""
 import json
 import os
 
@@ -121,3 +122,32 @@ def test_block_loop_meets_the_reference_test_criteria(oracle, name):
     Lu = L.astype(np.float64) + np.eye(n)
     Hr = 0.5 * (H.astype(np.float64) + H.T) + 1e-2 * np.trace(H.astype(np.float64)) / n * np.eye(n)
     assert np.max(np.abs(Lu @ np.diag(D.astype(np.float64)) @ Lu.T - Hr)) < 1e-5 * np.max(np.abs(Hr))
+
+
+def device_path_vectors(name):
+    """(H, [(hessian given, search, calibrate, packed, scales)], global) of tests/golden/ref_nvfp4_gpu_*."""
+    meta = json.load(open(os.path.join(GOLDEN, "ref_nvfp4_gpu.json")))
+    H = np.fromfile(os.path.join(GOLDEN, "ref_nvfp4_gpu_H.bin"), np.float32).reshape(256, 256)
+    blob = np.fromfile(os.path.join(GOLDEN, "ref_nvfp4_gpu_%s.bin" % name), np.uint8)
+    per = 96 * 128 + 96 * 16
+    cases = []
+    for k, (h, s, c) in enumerate(meta["combos"]):
+        b = blob[k * per:(k + 1) * per]
+        cases.append((bool(h), bool(s), bool(c), b[:96 * 128].reshape(96, 128), b[96 * 128:].reshape(96, 16)))
+    return H, cases, float.fromhex(meta["global"][name])
+
+
+@pytest.mark.parametrize("name", ["gauss", "heavy"])
+def test_block_loop_equals_the_reference_device_path(oracle, name):
+    """Every byte nvfp4_quantize_group of the reference returned on the GPU, for all five option combinations."""
+    w, _ = _weights(oracle, name)
+    m, n = w.shape
+    H, cases, g = device_path_vectors(name)
+    assert g == oracle.nvfp4_quantize(w)[2]
+    L, D = oracle.nvfp4_prepare(H, 1e-2, True)
+    _, dH = oracle.nvfp4_prepare(H, 1e-2, False)
+    for (h, s, c, pk, sc) in cases:
+        cal = h and c
+        got = oracle.nvfp4_blocks(w, L if cal else None, (D if cal else dH) if h else None, g, cal, s)
+        assert np.array_equal(got[0], pk) and np.array_equal(got[1], sc), (h, s, c)
+    assert np.allclose(H, _hessian(oracle, n, 21), rtol=1e-5, atol=1e-7)      # the stored Hessian is the seeded one
