@@ -140,3 +140,39 @@ def test_nvfp4_layer_shape(qz, pkg, oracle):
              int((same_l.packed != pk).sum() + (same_l.scales != sc).sum())))
         assert gl == cal.global_scale and np.array_equal(same_l.scales, sc) and np.array_equal(same_l.packed, pk)
         assert np.mean(cal.packed == pk) > 0.99999 and np.mean(cal.scales == sc) > 0.99999
+
+
+def test_nvfp4_config5_shape(qz, pkg):
+    """12288 x 28672 with a dense 28672^2 Hessian (the down-proj shape of the headline configuration): host
+    preparation and device block loop timed apart; format valid, Hessian-weighted error below the plain quantizer's."""
+    import time
+    import torch
+    say("case: nvfp4 12288x28672")
+    m, n = 12288, 28672
+    g = torch.Generator(device="cuda").manual_seed(4)
+    wd = torch.randn((m, n), generator=g, device="cuda") * 0.02
+    X = torch.randn((8192, n), generator=g, device="cuda") * torch.exp(0.8 * torch.randn((n,), generator=g, device="cuda"))
+    Hd = X.T @ X / 8192
+    del X
+    w, H = wd.cpu().numpy(), Hd.cpu().numpy()
+    t0 = time.time()
+    L, dw = pkg.nvfp4_prepare(H, 1e-2, True, 16)
+    t1 = time.time()
+    cal = qz.nvfp4_quantize_prepared([w], n, L, dw, True)[0]
+    t2 = time.time()
+    say("  preparation %.2f s, block loop %.2f s (%.0f Mweights/s)" % (t1 - t0, t2 - t1, m * n / (t2 - t1) / 1e6))
+    del L
+    plain = pkg.nvfp4_quantize(w)
+    assert cal.global_scale == plain.global_scale and np.all((cal.scales & 0x7f) <= 126)
+
+    def proxy(t):
+        E = wd - torch.from_numpy(pkg.nvfp4_dequantize(t)).cuda()
+        tot = 0.0
+        for r0 in range(0, m, 2048):          # fp32 GEMM slabs, fp64 sums: a comparison of two numbers 2.5x apart
+            e = E[r0:r0 + 2048]
+            tot += float(((e @ Hd) * e).double().sum())
+        return tot / m
+
+    p_cal, p_plain = proxy(cal), proxy(plain)
+    say("  proxy calibrated %.4g, plain %.4g (%.1f%%)" % (p_cal, p_plain, 100 * p_cal / p_plain))
+    assert p_cal < 0.9 * p_plain
