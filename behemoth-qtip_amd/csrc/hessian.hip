@@ -96,11 +96,12 @@ __device__ __forceinline__ void store_block_transposed(const Block8x8& b, uint16
 // the MFMAs of slice ks, and the transposes and LDS writes of the next stage between the MFMAs of the last slice.
 template <bool DIAG, int FETCH>
 __device__ __forceinline__ void syrk_stage(floatx16 (&acc)[4][4], const uint16_t* As, const uint16_t* Bs, uint16_t* nxt,
-                                           Block8x8& ga, Block8x8& gb, const uint16_t* __restrict__ X, long rows,
-                                           long n, long r0, long ci, long cj, int offA, int offB, int swr, int sww) {
+                                           Block8x8& ga, Block8x8& gb, const uint16_t* __restrict__ X,
+                                           const uint16_t* __restrict__ XB, long rows, long n, long r0, long ci, long cj,
+                                           int offA, int offB, int swr, int sww) {
   if (FETCH) {
     fetch_block<FETCH == 1>(ga, X, rows, n, r0, ci);
-    if (!DIAG) fetch_block<FETCH == 1>(gb, X, rows, n, r0, cj);
+    if (!DIAG) fetch_block<FETCH == 1>(gb, XB, rows, n, r0, cj);
   }
   bf16x8 fa[2][4], fb[2][4];
 #pragma unroll
@@ -155,14 +156,15 @@ __device__ __forceinline__ void syrk_stage(floatx16 (&acc)[4][4], const uint16_t
 }
 
 template <bool DIAG>
-__device__ __forceinline__ void syrk_tile(floatx16 (&acc)[4][4], uint16_t* lds, const uint16_t* __restrict__ X, long rows,
-                                          long n, long ci, long cj, int ro, int cg, int offA, int offB, int swr) {
+__device__ __forceinline__ void syrk_tile(floatx16 (&acc)[4][4], uint16_t* lds, const uint16_t* __restrict__ X,
+                                          const uint16_t* __restrict__ XB, long rows, long n, long ci, long cj, int ro,
+                                          int cg, int offA, int offB, int swr) {
   const long stages = (rows + kStage - 1) / kStage;
   Block8x8 ga, gb;
   uint16_t* const wr = lds + (8 * cg) * kPitch;  // row of this thread's first column within a slice
   const int sww = ro ^ (cg & 7);
   fetch_block<false>(ga, X, rows, n, 8 * ro, ci);
-  if (!DIAG) fetch_block<false>(gb, X, rows, n, 8 * ro, cj);
+  if (!DIAG) fetch_block<false>(gb, XB, rows, n, 8 * ro, cj);
   store_block_transposed(ga, wr, sww);
   if (!DIAG) store_block_transposed(gb, wr + kSliceU16, sww);
   __syncthreads();
@@ -170,7 +172,7 @@ __device__ __forceinline__ void syrk_tile(floatx16 (&acc)[4][4], uint16_t* lds, 
   long st = 0;
 #define QTIP_SYRK_STAGE(F)                                                                                   \
   syrk_stage<DIAG, F>(acc, lds + (st & 1) * 2 * kSliceU16, lds + (st & 1) * 2 * kSliceU16 + (DIAG ? 0 : kSliceU16), \
-                      wr + ((st + 1) & 1) * 2 * kSliceU16, ga, gb, X, rows, n, (st + 1) * kStage + 8 * ro, ci, cj, offA, offB, swr, sww)
+                      wr + ((st + 1) & 1) * 2 * kSliceU16, ga, gb, X, XB, rows, n, (st + 1) * kStage + 8 * ro, ci, cj, offA, offB, swr, sww)
   for (; (st + 2) * kStage <= rows; ++st) QTIP_SYRK_STAGE(1);
   if (st + 1 < stages) {
     QTIP_SYRK_STAGE(2);
@@ -180,8 +182,14 @@ __device__ __forceinline__ void syrk_tile(floatx16 (&acc)[4][4], uint16_t* lds, 
 #undef QTIP_SYRK_STAGE
 }
 
-__global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __restrict__ X, long rows, long n,
-                                                          float* __restrict__ H, int tiles, int patch_cols) {
+// DOT = false: H += X^T X on the tiles on or below the diagonal (XB == X).
+// DOT = true:  nothing is stored; partial[ti * tiles + tj] = w * sum_ij (X^T XB)_ij H_ij over the tile, w = 2 below the
+//              diagonal and 1 on it: with X^T XB symmetric the partials add up to sum_ij (X^T XB)_ij H_ij of a symmetric
+//              H.  The tiles above the diagonal keep the zero the caller wrote.
+template <bool DOT>
+__global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ XB,
+                                                          long rows, long n, float* __restrict__ H,
+                                                          double* __restrict__ partial, int tiles, int patch_cols) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
   // workgroup -> tile: ids that differ by 8 run on different XCDs; the 32 ids an XCD holds at a time are one patch
   const long b = blockIdx.x;
@@ -219,10 +227,11 @@ __global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __res
 #pragma unroll
       for (int c = 0; c < 4; ++c) acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z, z, acc[a][c], 0, 0, 0);
   }
-  if (ti == tj) syrk_tile<true>(acc, lds, X, rows, n, ci, cj, ro, cg, offA, offB, swr);
-  else syrk_tile<false>(acc, lds, X, rows, n, ci, cj, ro, cg, offA, offB, swr);
+  if (!DOT && ti == tj) syrk_tile<true>(acc, lds, X, XB, rows, n, ci, cj, ro, cg, offA, offB, swr);
+  else syrk_tile<false>(acc, lds, X, XB, rows, n, ci, cj, ro, cg, offA, offB, swr);
 
   // accumulator element v of a lane: row (v % 4) + 8 (v / 4) + 4 (lane / 32), column lane % 32 of the 32 x 32 tile
+  double dot = 0.0;
 #pragma unroll
   for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
@@ -231,8 +240,70 @@ __global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __res
       for (int v = 0; v < 16; ++v) {
         const long gi = ti * kTile + wm * 128 + mi * 32 + (v & 3) + 8 * (v >> 2) + 4 * (lane >> 5);
         const long gj = tj * kTile + wn * 128 + ni * 32 + rl;
-        if (gi < n && gj < n) H[gi * n + gj] += acc[mi][ni][v];
+        if (gi < n && gj < n) {
+          if (DOT) dot += double(acc[mi][ni][v]) * double(H[gi * n + gj]);
+          else H[gi * n + gj] += acc[mi][ni][v];
+        }
       }
+  if (DOT) {
+    // lanes, then waves, in a fixed order (the stage loop ended with a barrier: the staging buffers are free)
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+    double* red = reinterpret_cast<double*>(lds);
+    if (lane == 0) red[wave] = dot;
+    __syncthreads();
+    if (t == 0) partial[ti * tiles + tj] = (ti == tj ? 1.0 : 2.0) * (((red[0] + red[1]) + red[2]) + red[3]);
+  }
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_dev(float f) {  // round to nearest even; the inputs here are finite
+  uint32_t u = __float_as_uint(f);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return uint16_t(u >> 16);
+}
+
+// X[r][c] = A[c][r] - (B ? B[c][r] : 0) for r < m, c < n (A, B: n x m with leading dimension ld), split into bf16 hi + lo
+// and written as the two operand stacks of the three-product form: XA = [hi; hi; lo], XB = [hi; lo; hi] (each 3 m x n),
+// so that XA^T XB = hi^T hi + hi^T lo + lo^T hi.
+__global__ __launch_bounds__(256) void split_transposed_kernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                               long n, long m, long ld, uint16_t* __restrict__ XA,
+                                                               uint16_t* __restrict__ XB) {
+  __shared__ float tile[32][33];
+  const long c0 = long(blockIdx.y) * 32, r0 = long(blockIdx.x) * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const long c = c0 + ty + 8 * k, r = r0 + tx;
+    float v = 0.f;
+    if (c < n && r < m) v = A[c * ld + r] - (B ? B[c * ld + r] : 0.f);
+    tile[ty + 8 * k][tx] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const long r = r0 + ty + 8 * k, c = c0 + tx;
+    if (r < m && c < n) {
+      const float v = tile[tx][ty + 8 * k];
+      const uint16_t hi = f32_to_bf16_dev(v);
+      const uint16_t lo = f32_to_bf16_dev(v - __uint_as_float(uint32_t(hi) << 16));
+      const long o = r * n + c, seg = m * n;
+      XA[o] = hi, XA[seg + o] = hi, XA[2 * seg + o] = lo;
+      XB[o] = hi, XB[seg + o] = lo, XB[2 * seg + o] = hi;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void sum_doubles_kernel(const double* __restrict__ p, long count, double* __restrict__ out) {
+  __shared__ double red[256];
+  double a = 0.0;
+  for (long i = threadIdx.x; i < count; i += 256) a += p[i];
+  red[threadIdx.x] = a;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (int(threadIdx.x) < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *out = red[0];
 }
 
 // H[i][j] for j > i takes H[j][i] (computed tiles hold the lower triangle and the whole diagonal tiles); everything
@@ -262,24 +333,68 @@ __global__ __launch_bounds__(256) void hessian_finish_kernel(float* __restrict__
 
 }  // namespace
 
+namespace {
+// launch geometry shared by the two forms of the kernel; also raises the kernels' dynamic LDS limit once per process
+// (the attribute belongs to the function, not to a device context)
+struct SyrkGrid {
+  int tiles, patch_cols;
+  unsigned grid;
+  explicit SyrkGrid(long n) {
+    static bool configured = false;
+    if (!configured) {
+      QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel<false>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
+      QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel<true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
+      configured = true;
+    }
+    tiles = int((n + kTile - 1) / kTile);
+    const int patch_rows = (tiles + kPatchRows - 1) / kPatchRows;
+    patch_cols = (tiles + kPatchCols - 1) / kPatchCols;
+    const long patches = long(patch_rows) * patch_cols;
+    const long padded = (patches + 7) / 8 * 8;  // whole rounds over the 8 XCDs
+    const long g = padded * kPatchRows * kPatchCols;
+    QTIP_REQUIRE(g < (1l << 31), "symmetric update: n too large (%ld)", n);
+    grid = unsigned(g);
+  }
+};
+}  // namespace
+
 void launch_hessian_accumulate(const uint16_t* X, long rows, long n, float* H, hipStream_t s) {
   QTIP_REQUIRE(X != nullptr && H != nullptr && rows >= 0 && n > 0, "hessian_accumulate: bad arguments");
   QTIP_REQUIRE(n % 8 == 0 && (reinterpret_cast<uintptr_t>(X) & 15) == 0, "hessian_accumulate: rows of X must be 16-byte aligned (n = %ld)", n);
   if (rows == 0) return;
-  static bool configured = false;  // per process; the attribute belongs to the function, not to a device context
-  if (!configured) {
-    QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 int(kLdsBytes)));
-    configured = true;
-  }
-  const int tiles = int((n + kTile - 1) / kTile);
-  const int patch_rows = (tiles + kPatchRows - 1) / kPatchRows, patch_cols = (tiles + kPatchCols - 1) / kPatchCols;
-  const long patches = long(patch_rows) * patch_cols;
-  const long padded = (patches + 7) / 8 * 8;  // whole rounds over the 8 XCDs
-  const long grid = padded * kPatchRows * kPatchCols;
-  QTIP_REQUIRE(grid < (1l << 31), "hessian_accumulate: n too large (%ld)", n);
-  syrk_bf16_kernel<<<dim3(unsigned(grid)), dim3(256), kLdsBytes, s>>>(X, rows, n, H, tiles, patch_cols);
+  SyrkGrid g(n);
+  syrk_bf16_kernel<false><<<dim3(g.grid), dim3(256), kLdsBytes, s>>>(X, X, rows, n, H, nullptr, g.tiles, g.patch_cols);
   QTIP_HIP(hipGetLastError());
+}
+
+// sum_ij H_ij (D^T D)_ij = tr(D H D^T) for D = A^T - B^T (m x n), H symmetric n x n fp32: the quadratic forms of the
+// proxy (src/quantizer.cpp:268-303, which also takes them from bf16 hi/lo products with fp32 accumulation).
+// A, B: n x m fp32 with leading dimension ld (B may be null).  Synchronises the stream.
+double quad_trace_bf16x3(long n, long m, const float* H, const float* A, const float* B, long ld, DBuf<uint16_t>& stack,
+                         DBuf<double>& scratch, hipStream_t s) {
+  if (n <= 0 || m <= 0) return 0.0;
+  QTIP_REQUIRE(n % 8 == 0, "proxy: n must be a multiple of 8 (n = %ld)", n);
+  const size_t seg = size_t(m) * size_t(n);
+  stack.ensure(6 * seg);
+  uint16_t* XA = stack.p;
+  uint16_t* XB = stack.p + 3 * seg;
+  split_transposed_kernel<<<dim3(unsigned((m + 31) / 32), unsigned((n + 31) / 32)), dim3(256), 0, s>>>(A, B, n, m, ld, XA, XB);
+  QTIP_HIP(hipGetLastError());
+  SyrkGrid g(n);
+  const size_t np = size_t(g.tiles) * g.tiles;
+  scratch.ensure(np + 1);
+  QTIP_HIP(hipMemsetAsync(scratch.p, 0, np * sizeof(double), s));
+  syrk_bf16_kernel<true><<<dim3(g.grid), dim3(256), kLdsBytes, s>>>(XA, XB, 3 * m, n, const_cast<float*>(H), scratch.p,
+                                                                    g.tiles, g.patch_cols);
+  QTIP_HIP(hipGetLastError());
+  sum_doubles_kernel<<<dim3(1), dim3(256), 0, s>>>(scratch.p, long(np), scratch.p + np);
+  QTIP_HIP(hipGetLastError());
+  double h = 0;
+  QTIP_HIP(hipMemcpyAsync(&h, scratch.p + np, sizeof(double), hipMemcpyDeviceToHost, s));
+  QTIP_HIP(hipStreamSynchronize(s));
+  return h;
 }
 
 void launch_hessian_finish(float* H, long n, float scale, hipStream_t s) {

@@ -7,8 +7,7 @@
 //    the CPU path and written in trellis sequence order.
 //  * gemm_tn: sum_k A[k][i] * (B1 - B2)[k][j] on the fp64 matrix cores (v_mfma_f64_16x16x4_f64), fp32 operands
 //    widened while staging through LDS.  The cross-buffer feedback ("prod cache") of a 128-column buffer is gathered
-//    from all rows quantized so far by a K-split kernel; a second kernel reduces sum(acc * (B1 - B2)[i][j]) for
-//    tr(X^T H X) (the proxy).
+//    from all rows quantized so far by a K-split kernel.
 //  * gemm_tn_bf16x3: the same prod-cache update with fp32 C and the operands split into bf16 hi + lo
 //    (v_mfma_f32_32x32x16_bf16, three terms), the arithmetic of the reference's GPU path.
 #include <hip/hip_fp16.h>
@@ -57,98 +56,6 @@ __global__ __launch_bounds__(256) void ldlq_prep_kernel(const float* __restrict_
 // ---------------------------------------------------------------- fp64 MFMA GEMM
 typedef double double4_t __attribute__((ext_vector_type(4)));
 constexpr int BM = 128, BN = 128, KC = 16;
-
-// 128 x 128 outputs per workgroup, 4 waves of 64 x 64 (4 x 4 tiles of v_mfma_f64_16x16x4_f64), K in slices of 16
-// staged through LDS as fp64.  M and K are multiples of 16 and of 4 here (multiples of 128 in the LDLQ), N a
-// multiple of 4; rows and columns beyond M / N are masked.
-// MODE 0: C += acc.  MODE 1: partial[block] = sum_ij acc[i][j] * (B1 - B2)[i][j]  (square case: M rows of B)
-template <int MODE>
-__global__ __launch_bounds__(256, 2) void gemm_tn_f64_kernel(int M, int N, int K, const float* __restrict__ A,
-                                                             long lda, const float* __restrict__ B1,
-                                                             const float* __restrict__ B2, long ldb,
-                                                             double* __restrict__ C, long ldc,
-                                                             double* __restrict__ partial) {
-  __shared__ __attribute__((aligned(16))) double As[KC][BM];
-  __shared__ __attribute__((aligned(16))) double Bs[KC][BN];
-  __shared__ double red[4];
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const long i0 = long(blockIdx.y) * BM, j0 = long(blockIdx.x) * BN;
-  double4_t acc[4][4];
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 4; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
-  const int lk = t >> 5, lc = (t & 31) * 4;  // this thread stages rows lk and lk + 8 of a slice, 4 columns at lc
-  const bool a_ok = i0 + lc + 3 < M, b_ok = j0 + lc + 3 < N;
-
-  for (int kc = 0; kc < K; kc += KC) {
-#pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      const int k = lk + 8 * r;
-      float4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
-      if (kc + k < K) {
-        if (a_ok) a = *reinterpret_cast<const float4*>(A + long(kc + k) * lda + i0 + lc);
-        if (b_ok) {
-          b = *reinterpret_cast<const float4*>(B1 + long(kc + k) * ldb + j0 + lc);
-        }
-      }
-      double bx = b.x, by = b.y, bz = b.z, bw = b.w;
-      if (B2 && b_ok && kc + k < K) {
-        const float4 c = *reinterpret_cast<const float4*>(B2 + long(kc + k) * ldb + j0 + lc);
-        bx -= double(c.x), by -= double(c.y), bz -= double(c.z), bw -= double(c.w);
-      }
-      *reinterpret_cast<double2*>(&As[k][lc]) = double2{double(a.x), double(a.y)};
-      *reinterpret_cast<double2*>(&As[k][lc + 2]) = double2{double(a.z), double(a.w)};
-      *reinterpret_cast<double2*>(&Bs[k][lc]) = double2{bx, by};
-      *reinterpret_cast<double2*>(&Bs[k][lc + 2]) = double2{bz, bw};
-    }
-    __syncthreads();
-#pragma unroll
-    for (int kk = 0; kk < KC; kk += 4) {
-      const int kr = kk + (lane >> 4), c = lane & 15;
-      double a[4], b[4];
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) a[mi] = As[kr][wm * 64 + mi * 16 + c];
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni) b[ni] = Bs[kr][wn * 64 + ni * 16 + c];
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni)
-          acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
-    }
-    __syncthreads();
-  }
-  // accumulator element v of a lane: row (lane / 16) + 4 v, column lane % 16 of the 16x16 tile
-  double local = 0.0;
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-    for (int ni = 0; ni < 4; ++ni)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const long gi = i0 + wm * 64 + mi * 16 + (lane >> 4) + 4 * v;
-        const long gj = j0 + wn * 64 + ni * 16 + (lane & 15);
-        if (gi < M && gj < N) {
-          if (MODE == 0) {
-            C[gi * ldc + gj] += acc[mi][ni][v];
-          } else {
-            const long o = gi * ldb + gj;
-            double x = double(B1[o]);
-            if (B2) x -= double(B2[o]);
-            local += acc[mi][ni][v] * x;
-          }
-        }
-      }
-  if (MODE == 1) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off, 64);
-    if (lane == 0) red[wave] = local;
-    __syncthreads();
-    if (t == 0) partial[long(blockIdx.y) * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
-  }
-}
 
 // ---------------------------------------------------------------- fp64 MFMA GEMM, 128 output rows, K split
 // out[y][i][j] = sum over the K slices of split y of A[k][i] * (B1 - B2)[k][j], i < 128: the cross-buffer feedback
@@ -350,20 +257,6 @@ __global__ __launch_bounds__(256) void gemm_tn_bf16x3_kernel(int M, int N, const
       }
 }
 
-__global__ __launch_bounds__(256) void sum_partials_kernel(const double* __restrict__ partial, long count,
-                                                           double* __restrict__ out) {
-  __shared__ double red[256];
-  double acc = 0;
-  for (long i = threadIdx.x; i < count; i += 256) acc += partial[i];
-  red[threadIdx.x] = acc;
-  __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) {
-    if (int(threadIdx.x) < s) red[threadIdx.x] += red[threadIdx.x + s];
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) *out = red[0];
-}
-
 }  // namespace
 
 void launch_ldlq_prep_f64(const float* WT, const float* hatWT, const double* prod, int prod_row0, const float* L, long n,
@@ -412,23 +305,6 @@ void launch_gemm_tn_bf16x3_acc(int M, int N, int K, const float* A, long lda, co
   dim3 grid(unsigned((N + SB - 1) / SB), unsigned((M + SB - 1) / SB));
   gemm_tn_bf16x3_kernel<<<grid, dim3(256), 0, s>>>(M, N, A, lda, B1, B2, ldb, C, ldc);
   QTIP_HIP(hipGetLastError());
-}
-
-double quad_trace_f64(int n, int N, const float* H, const float* B1, const float* B2, long ldb, DBuf<double>& scratch,
-                      hipStream_t s) {
-  if (n <= 0 || N <= 0) return 0.0;
-  QTIP_REQUIRE(n % 4 == 0 && N % 4 == 0 && ldb % 4 == 0, "fp64 GEMM needs 16-byte aligned fp32 rows");
-  dim3 grid(unsigned((N + BN - 1) / BN), unsigned((n + BM - 1) / BM));
-  const long blocks = long(grid.x) * grid.y;
-  scratch.ensure(size_t(blocks) + 1);
-  gemm_tn_f64_kernel<1><<<grid, dim3(256), 0, s>>>(n, N, n, H, n, B1, B2, ldb, nullptr, 0, scratch);
-  QTIP_HIP(hipGetLastError());
-  sum_partials_kernel<<<dim3(1), dim3(256), 0, s>>>(scratch, blocks, scratch + blocks);
-  QTIP_HIP(hipGetLastError());
-  double h = 0;
-  QTIP_HIP(hipMemcpyAsync(&h, scratch + blocks, sizeof(double), hipMemcpyDeviceToHost, s));
-  QTIP_HIP(hipStreamSynchronize(s));
-  return h;
 }
 
 }  // namespace qtipmi

@@ -14,7 +14,4 @@ void launch_gemm_tn_f64_gather(int N, long K, const float* A, long lda, const fl
 // the same product with fp32 C and every operand split into bf16 hi + lo (three MFMA terms, fp32 accumulate); K = 128
 void launch_gemm_tn_bf16x3_acc(int M, int N, int K, const float* A, long lda, const float* B1, const float* B2, long ldb,
                                float* C, long ldc, hipStream_t s);
-// sum over the N columns x of X = B1 - B2 (n x N, stride ldb) of x^T H x, H n x n fp32; synchronises the stream
-double quad_trace_f64(int n, int N, const float* H, const float* B1, const float* B2, long ldb, DBuf<double>& scratch,
-                      hipStream_t s);
 }  // namespace qtipmi

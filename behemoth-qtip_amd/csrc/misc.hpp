@@ -12,6 +12,10 @@ void launch_decode_trellis(const uint16_t* trellis, long m, long n, const float*
 // H (n x n fp32) += X^T X for X = rows x n bf16, tiles on or below the diagonal only; then mirror + scale (hessian.hip)
 void launch_hessian_accumulate(const uint16_t* X, long rows, long n, float* H, hipStream_t s);
 void launch_hessian_finish(float* H, long n, float scale, hipStream_t s);
+// tr(D H D^T) for D = A^T - B^T (m x n; A, B n x m fp32 with leading dimension ld, B may be null), H symmetric n x n
+// fp32, from bf16 hi/lo products on the matrix cores; synchronises the stream
+double quad_trace_bf16x3(long n, long m, const float* H, const float* A, const float* B, long ld, DBuf<uint16_t>& stack,
+                         DBuf<double>& scratch, hipStream_t s);
 // NVFP4 fallback quantizer (nvfp4.hip): one 16-column block of the transposed matrices, the feedback of its residual
 // into the columns before it, and a byte transposer for the outputs
 void launch_nvfp4_block(const float* WT, const float* FT, long m, long n, long c0, const float* L, const float* dw,

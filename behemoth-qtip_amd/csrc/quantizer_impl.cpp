@@ -238,10 +238,11 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
   if (!opt.skip_proxy) {
     DBuf<float> HR(size_t(n) * n);
     QTIP_HIP(hipMemcpyAsync(HR, host_HRr, HR.bytes(), hipMemcpyHostToDevice, s));
+    DBuf<uint16_t> stack;
     for (int li = 0; li < nlin; ++li) {
       const long m = lins[li].m;
-      const double den = quad_trace_f64(n, int(m), HR, WT + off[li], nullptr, mt, c->scratch, s);
-      const double num = quad_trace_f64(n, int(m), HR, WT + off[li], hatWT + off[li], mt, c->scratch, s);
+      const double den = quad_trace_bf16x3(n, m, HR, WT + off[li], nullptr, mt, stack, c->scratch, s);
+      const double num = quad_trace_bf16x3(n, m, HR, WT + off[li], hatWT + off[li], mt, stack, c->scratch, s);
       const double wn2 = c->rht.reduce(WT + off[li], mt, nullptr, 0, n, m, 0);
       const double dn2 = c->rht.reduce(WT + off[li], mt, hatWT + off[li], mt, n, m, 2);
       outs[li].proxy_rot_reg = num / den;

@@ -116,25 +116,23 @@ def run_group(args, pkg):
     n = H.shape[0]
     ms = [int(w.shape[0]) for w in Ws]
     lins = [pkg.LinearIn("w%d" % i, m, w_f32=w) for i, (m, w) in enumerate(zip(ms, Ws))]
-    opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=True, feedback=args.feedback)
+    opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback)
     weights_per_step = sum(ms) * n
 
     stats = {}
 
     def run_steps(K, record):
         """K groups through the library's scheduler: the Hessian of group k+2 is rotated and the one of group k+1 is
-        factored on a side thread while the GPU quantizes group k.  The untimed warm-up groups also evaluate the proxy
-        (the metric's stages are RHT + LDLQ + Viterbi; the proxy's value and cost are reported beside them)."""
-        o = opt if record else pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback)
-        res = q.run_groups([(lins, n, H, 3 + k) for k in range(K)], o)
-        if not record:
-            stats.update(proxy=float(res[-1][0][0].proxy), proxy_s=float(res[-1][1].proxy))
+        factored on a side thread while the GPU quantizes group k.  Every group does all of quantize_group's work,
+        the two proxy errors included."""
+        res = q.run_groups([(lins, n, H, 3 + k) for k in range(K)], opt)
         if record:
             tms = [r[1] for r in res]
             stats.update(rht_s=sum(t.rht for t in tms) / K,      # Hessian rotation + weight RHT + Wscale
                          ldl_s=sum(t.ldl_cpu for t in tms) / K, ldl_wait_s=sum(r[2] for r in res) / K,
                          ldlq_s=sum(t.ldlq for t in tms) / K, viterbi_s=sum(t.viterbi for t in tms) / K,
                          load_s=sum(t.load for t in tms) / K, pack_s=sum(t.pack for t in tms) / K,
+                         proxy_s=sum(t.proxy for t in tms) / K, proxy=float(res[-1][0][0].proxy),
                          wscale=float(res[-1][0][0].wscale))
 
     q.reserve_groups(n)   # page-locked staging ring (3 x (HRr, L)); a worker keeps it for its lifetime
@@ -149,12 +147,12 @@ def run_group(args, pkg):
     wall = time.time() - t0
     ntr = sum(ms) // 16
     launches = n // 16
-    gpu_s = stats["rht_s"] + stats["load_s"] + stats["ldlq_s"] + stats["pack_s"]
+    gpu_s = stats["rht_s"] + stats["load_s"] + stats["ldlq_s"] + stats["proxy_s"] + stats["pack_s"]
     extra = dict(stats)
     extra.update(gpu_only_Mweights_s=weights_per_step / gpu_s / 1e6,
                  serial_Mweights_s=weights_per_step / (gpu_s + stats["ldl_s"]) / 1e6,
                  viterbi_only_Mweights_s=weights_per_step / stats["viterbi_s"] / 1e6,
-                 proxy_in_timed_region=False, ldl_threads=args.ldl_threads, feedback=args.feedback)
+                 proxy_in_timed_region=True, ldl_threads=args.ldl_threads, feedback=args.feedback)
     names = {2: "config2: 1024x1024 group", 3: "config3: 12288x12288 q-proj group",
              4: "config4: gate+up 2x(28672x12288) group", 5: "config5: 12288x28672 down-proj group"}
     return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
