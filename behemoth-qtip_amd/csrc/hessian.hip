@@ -16,6 +16,9 @@
 // XOR-swizzled: conflict-free for the writes and for the lanes' 16-byte fragment reads).  Two LDS stages of 64 rows: the next stage is fetched
 // and written while the matrix cores work on the current one.  Workgroups are numbered so that the 32 that share an
 // XCD (and its L2) at a time form an 8 x 4 patch of tiles, which needs 12 operand slices instead of 33.
+#include <mutex>
+#include <vector>
+
 #include "misc.hpp"
 #include "qtip_internal.hpp"
 
@@ -334,19 +337,26 @@ __global__ __launch_bounds__(256) void hessian_finish_kernel(float* __restrict__
 }  // namespace
 
 namespace {
-// launch geometry shared by the two forms of the kernel; also raises the kernels' dynamic LDS limit once per process
-// (the attribute belongs to the function, not to a device context)
+// launch geometry shared by the two forms of the kernel; also raises the kernels' dynamic LDS limit, once for every
+// device the library is used on (the attribute is kept per device) and safe against concurrent first calls
 struct SyrkGrid {
   int tiles, patch_cols;
   unsigned grid;
   explicit SyrkGrid(long n) {
-    static bool configured = false;
-    if (!configured) {
-      QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel<false>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
-      QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel<true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
-      configured = true;
+    static std::mutex mu;
+    static std::vector<bool> configured;
+    int dev = 0;
+    QTIP_HIP(hipGetDevice(&dev));
+    {
+      std::lock_guard<std::mutex> lk(mu);
+      if (configured.size() <= size_t(dev)) configured.resize(size_t(dev) + 1, false);
+      if (!configured[size_t(dev)]) {
+        QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel<false>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
+        QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel<true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
+        configured[size_t(dev)] = true;
+      }
     }
     tiles = int((n + kTile - 1) / kTile);
     const int patch_rows = (tiles + kPatchRows - 1) / kPatchRows;

@@ -12,7 +12,6 @@
 // the clone is picked at run time so one binary serves any x86-64-v3 host.
 #include <algorithm>
 #include <atomic>
-#include <chrono>
 #include <cmath>
 #include <cstring>
 #include <memory>
@@ -25,7 +24,6 @@
 namespace qtipmi {
 namespace {
 
-double wtime() { return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count(); }
 
 // The team belongs to the calling thread (the factorization may run on a side thread while another thread does
 // other work with a team of its own) and lives until that thread ends or asks for another size.
@@ -186,7 +184,6 @@ static bool factor_diagonal(double* A, long n, int kb) {
 // are factored by this same routine with narrow panels) everything runs on the calling thread.
 template <int NBT, int TILET>
 bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
-  double tdiag = 0, tsolve = 0, tupd = 0, tq;
   const Kernels kn = pick_kernels();
   const int MR = kn.MR, NR = kn.NR;
   std::vector<double> packL;
@@ -198,14 +195,11 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
   double* const packB = packA + capA;
   for (int k = 0; k < n; k += NBT) {
     const int kb = std::min(NBT, n - k);
-    tq = wtime();
     if constexpr (NBT > 64) {
       if (!cholesky_panels<64, 96>(A + long(k) * ld + k, ld, kb, nullptr, false)) return false;
     } else {
       if (!factor_diagonal(A + long(k) * ld + k, ld, kb)) return false;
     }
-    tdiag += wtime() - tq;
-    tq = wtime();
     const int r0 = k + kb, nr = n - r0;
     if (nr <= 0) break;
     for (int j = 0; j < kb; ++j) {
@@ -268,8 +262,6 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
     if (team) team->parallel_for(nPB, 2, solve_chunk);
     else
       for (long gl = 0; gl < nPB; ++gl) solve_chunk(gl);
-    tsolve += wtime() - tq;
-    tq = wtime();
     // trailing update of the lower triangle, tiles (bi, bj <= bi) largest rows first
     const int nT = (nr + TILET - 1) / TILET;
     const long ntask = long(nT) * (nT + 1) / 2;
@@ -296,9 +288,7 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
     if (team) team->parallel_for(ntask, 1, update_tile);
     else
       for (long task = 0; task < ntask; ++task) update_tile(task);
-    tupd += wtime() - tq;
   }
-  if (top && getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "chol: diag %.3f solve+pack %.3f update %.3f\n", tdiag, tsolve, tupd);
   return true;
 }
 
@@ -312,10 +302,7 @@ bool cholesky_lower_host(double* A, int n, int threads) {
 bool block_ldl_host(double* A, int n, float* L_out, int threads) {
   if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
   HostTeam& team = team_of_this_thread(threads);
-  double tq = wtime();
   if (!cholesky_panels<NB, TILE>(A, n, n, &team, true)) return false;
-  const double t_chol = wtime() - tq;
-  tq = wtime();
   const int nb = n / 16;
   // inverse of every 16x16 lower-triangular diagonal block (column by column, forward substitution)
   std::vector<double> inv(size_t(nb) * 256);
@@ -352,7 +339,6 @@ bool block_ldl_host(double* A, int n, float* L_out, int threads) {
     std::memset(lr + long(rb) * 16, 0, sizeof(float) * size_t(n - rb * 16));  // diagonal block and everything right of it
     if (!ok) finite.store(0, std::memory_order_relaxed);
   });
-  if (getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "block_ldl: cholesky %.3f, L assembly %.3f\n", t_chol, wtime() - tq);
   return finite.load() != 0;
 }
 

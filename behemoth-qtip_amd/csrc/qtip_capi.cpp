@@ -26,6 +26,9 @@ static int guarded(F&& f) {
   } catch (const std::exception& e) {
     set_last_error(e.what());
     return QTIP_E_ARG;
+  } catch (...) {
+    set_last_error("unknown exception");
+    return QTIP_E_ARG;
   }
 }
 
@@ -70,17 +73,29 @@ int qtip_create(int device, qtip_ctx** out) {
     QTIP_HIP(hipGetDeviceProperties(&prop, device));
     QTIP_REQUIRE(std::strncmp(prop.gcnArchName, "gfx950", 6) == 0,
                  "qtip_create: device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
-    auto c = std::make_unique<qtip_ctx>();
-    c->device = device;
     int prev = 0;
     QTIP_HIP(hipGetDevice(&prev));
     QTIP_HIP(hipSetDevice(device));
+    // a failure below must not leak the stream or leave another device current
+    struct Cleanup {
+      qtip_ctx* c;
+      int prev;
+      ~Cleanup() {
+        if (c) {
+          if (c->stream) (void)hipStreamDestroy(c->stream);
+          delete c;
+        }
+        (void)hipSetDevice(prev);
+      }
+    } guard{new qtip_ctx(), prev};
+    qtip_ctx* c = guard.c;
+    c->device = device;
     QTIP_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
     c->cb.build(nullptr);
-    upload_codebook(c.get());
+    upload_codebook(c);
     c->rht.init(device, c->stream);
-    (void)hipSetDevice(prev);
-    *out = c.release();
+    *out = c;
+    guard.c = nullptr;
   });
 }
 
@@ -211,6 +226,7 @@ int qtip_dequantize_linear(qtip_ctx* ctx, const uint16_t* host_trellis, const ui
 int qtip_had_K(int n) { return had_K(n); }
 
 void qtip_sign_vector(uint64_t seed, long count, float* host_out) {
+  if (!host_out) return;
   SplitMix r(seed);
   for (long i = 0; i < count; ++i) host_out[i] = r.sign();
 }

@@ -4,7 +4,6 @@
 
 #include <chrono>
 #include <cmath>
-#include <sys/mman.h>
 
 #include <cstdlib>
 #include <cstring>
@@ -27,6 +26,23 @@ double now_s() {
   using namespace std::chrono;
   return duration<double>(steady_clock::now().time_since_epoch()).count();
 }
+
+// Events of one call, destroyed on every way out of it.
+struct Events {
+  std::vector<hipEvent_t> ev;
+  Events() = default;
+  Events(const Events&) = delete;
+  Events& operator=(const Events&) = delete;
+  ~Events() {
+    for (hipEvent_t e : ev) (void)hipEventDestroy(e);
+  }
+  hipEvent_t add(unsigned flags) {
+    hipEvent_t e;
+    QTIP_HIP(hipEventCreateWithFlags(&e, flags));
+    ev.push_back(e);
+    return e;
+  }
+};
 }  // namespace
 
 // ---------------------------------------------------------------- rotate_hessian, src/quantizer.cpp:124-152
@@ -60,9 +76,7 @@ void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L) 
   // pay for mapping and faulting it in again
   HostScratch A(size_t(n) * n * sizeof(double));
   double* a = static_cast<double*>(A.get());
-  const double ts0 = now_s();
   symmetrize_lower_host(host_HRr, n, a, threads);
-  if (getenv("QTIP_LDL_DEBUG")) fprintf(stderr, "ldl_hessian: symmetrize %.3f\n", now_s() - ts0);
   if (!block_ldl_host(a, n, host_L, threads)) throw Error(QTIP_E_NOT_PD, "block LDL failed (H not PD)");
 }
 
@@ -75,25 +89,20 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   hipStream_t s = c->stream;
   ensure_viterbi_workspace(c);
   const long ntr = m / 16, nblk = n / 16;
-  // feedback 0: fp64 feedback sums and fp64 prod cache; feedback 1: fp32 sums, fp32 prod cache updated by the
+  // feedback 0: fp64 feedback sums; the feedback of the rows quantized in earlier buffers is gathered per buffer
+  // into a 128 x m fp64 slab.  feedback 1: fp32 sums, an n x m fp32 prod cache updated after every buffer by the
   // bf16 hi/lo split MFMA product
-  // feedback 0: the feedback of the rows quantized in earlier buffers is gathered per buffer into a 128 x m slab
   DBuf<double> prod(feedback == 0 ? size_t(128) * m : 0), parts(feedback == 0 ? size_t(5) * 128 * m : 0);
   DBuf<float> prod32(feedback == 1 ? size_t(n) * m : 0);
   DBuf<float> X(size_t(ntr) * 256);
   if (feedback == 1) QTIP_HIP(hipMemsetAsync(prod32, 0, prod32.bytes(), s));
   QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
-  std::vector<hipEvent_t> ev;
-  auto mark = [&] {
-    hipEvent_t e;
-    QTIP_HIP(hipEventCreate(&e));
-    QTIP_HIP(hipEventRecord(e, s));
-    ev.push_back(e);
-  };
+  Events timed, pacing;
+  auto mark = [&] { QTIP_HIP(hipEventRecord(timed.add(hipEventDefault), s)); };
   // The queue is kept two buffers (16 launches of ~2 ms) ahead of the GPU and no further: beyond that the
   // submitting thread would spin on a full queue and take a core from the host LDL of the next group.
   hipEvent_t pace[3];
-  for (auto& e : pace) QTIP_HIP(hipEventCreateWithFlags(&e, hipEventBlockingSync | hipEventDisableTiming));
+  for (auto& e : pace) e = pacing.add(hipEventBlockingSync | hipEventDisableTiming);
   long nbuf_done = 0;
   for (long cur = nblk; cur > 0; cur -= 8, ++nbuf_done) {
     const int bufend = int(16 * cur), c0 = bufend - 128;
@@ -128,18 +137,16 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
     }
     QTIP_HIP(hipEventRecord(pace[nbuf_done % 3], s));
   }
-  for (auto& e : pace) (void)hipEventDestroy(e);
   wait_stream_sleeping(s);
   if (vit_seconds) {
     double t = 0;
-    for (size_t i = 0; i + 1 < ev.size(); i += 2) {
+    for (size_t i = 0; i + 1 < timed.ev.size(); i += 2) {
       float ms = 0;
-      QTIP_HIP(hipEventElapsedTime(&ms, ev[i], ev[i + 1]));
+      QTIP_HIP(hipEventElapsedTime(&ms, timed.ev[i], timed.ev[i + 1]));
       t += ms * 1e-3;
     }
     *vit_seconds = t;
   }
-  for (auto e : ev) (void)hipEventDestroy(e);
 }
 
 // ---------------------------------------------------------------- quantize_group, src/quantizer.cpp:176-346

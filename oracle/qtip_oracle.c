@@ -559,8 +559,14 @@ static int ldlq_core(const float* lut0, const float* lut1, const double* WT, con
 
 int qo_ldlq(const float* lut0, const float* lut1, const float* Wr, const float* L, int m, int n, float* hatWr,
             uint16_t* Q, int threads) {
-  double* WT = (double*)malloc(sizeof(double) * (size_t)n * m);
+  if (m <= 0 || n <= 0) return -1;
+  double* WT = (double*)calloc((size_t)n * m, sizeof(double));
   double* hT = (double*)malloc(sizeof(double) * (size_t)n * m);
+  if (!WT || !hT) {
+    free(WT);
+    free(hT);
+    return -1;
+  }
   for (int i = 0; i < m; ++i)
     for (int j = 0; j < n; ++j) WT[(size_t)j * m + i] = Wr[(size_t)i * n + j];
   int rc = ldlq_core(lut0, lut1, WT, L, m, n, hT, Q, threads);
