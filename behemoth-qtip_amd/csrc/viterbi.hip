@@ -14,13 +14,23 @@
 // in opposite order.  A lane therefore owns 8 groups of one metric column c (one for each value m of the low
 // three bits, so that the stride 2m+1 is a compile-time constant) and their mirrors in column 255-c: per step it
 // keeps the two metric columns (2 x 16 fp64) in registers and streams 8 rows of E (16 fp64 each) from LDS, i.e.
-// 160 LDS reads for 256 add-compare-selects.  Which of the two groups 16c+m / 16c+8+m a lane takes, which lanes
-// share a 16-lane quarter-wave, and the padding of the E rows are free parameters; data/viterbi_layout.h holds a
-// choice that minimises LDS bank conflicts (generated by data/gen_viterbi_layout.c).
+// 160 LDS reads for 256 add-compare-selects.
 //
-// LDS per workgroup (~51 KB, three workgroups per CU): E rows stored twice back to back so that the rotation
-// by b4 is a per-lane base address and the stride d*(2m+1) a compile-time offset; metrics single-buffered
-// (columns are read into registers before the step's results are written), padded by one slot per 8 columns.
+// LDS layout: free of bank conflicts.  An 8-byte LDS access is served 16 lanes at a time, and a 16-lane quarter
+// takes as many cycles as the largest number of distinct addresses that fall on one of the 16 bank pairs.
+//   * Lane t runs metric column c = 4u + r + 64b with u = t & 15, r = (t >> 4) & 3, b = (t >> 6) & 1 and owns the
+//     groups j = 16c + 8h + m (h = t >> 7, m = 0..7) and their mirrors.  Bits 6..9 of j(j+1) are then
+//     (u (2t'+1) + const) mod 16 over the 16 lanes of a quarter (t' = 8h + m): 16 different values for every m.
+//   * The error table is stored entry position by row, E[q][row] (q = high 4 bits of the entry, 64 rows of 8 bytes),
+//     so the bank pair of a read is row mod 16 = those bits, whatever the rotation b4; the 16 positions are stored
+//     twice (q = 0..31) so that the rotation is a per-lane base address and the stride d*(2m+1) mod 16 a
+//     compile-time offset.
+//   * The metric of (column c, digit d) sits at c*16 + (pi(d) ^ ((c >> 2) & 15) ^ (c >> 6)) with
+//     pi(d) = 4 (d & 3) + (d >> 2): the 16 lanes of a quarter read 16 different bank pairs for every d, write 16
+//     different ones for every slot, a read address is one XOR of a per-lane base with a constant, and the mirror
+//     group's slot is the group's XOR 0xff3.
+// LDS per workgroup ~50 KB, three workgroups per CU; metrics single-buffered (the columns are read into registers
+// before the step's results are written).
 // Back-pointers (4 bits per group and step) go to HBM as one 64-bit word per thread and step, 2 KB per step,
 // fully coalesced; the first pass only keeps the steps its half-length trace-back needs.
 #include "qtip_internal.hpp"
@@ -28,20 +38,20 @@
 namespace qtipmi {
 namespace {
 
-#include "data/viterbi_layout.h"
-
 constexpr int kThreads = 256;
-constexpr int kRowStride = QTIP_VIT_ROW_STRIDE;  // doubles per E row: 2 x 16 entries + padding
-constexpr int kESlots = 64 * kRowStride + (kRowStride - 32);
-constexpr int kMSlots = 256 * 17;                // metric of (column c, digit d) at c*17 + d
+constexpr int kESlots = 32 * 64;                 // E[q][row]: 16 entry positions stored twice x 64 rows
+constexpr int kMSlots = 4096;                    // metric of (column c, digit d) at m_slot(c, d)
 constexpr int kBpWordsPerTile = 127 * kThreads;  // u64 words
+
+__device__ __forceinline__ constexpr int pi16(int d) { return 4 * (d & 3) + (d >> 2); }
+__device__ __forceinline__ int m_swz(int col) { return ((col >> 2) & 15) ^ (col >> 6); }
+__device__ __forceinline__ int m_slot(int col, int d) { return col * 16 + (pi16(d) ^ m_swz(col)); }
 
 struct Smem {
   double E[kESlots];  // first: its reads use 8-bit immediate offsets from a per-lane base
   double M[kMSlots];
   float x[kSeq];
   uint16_t st[kSteps];
-  uint8_t thread_of_unit[kThreads];  // inverse of kUnitOfLane: back-pointer words are stored in thread order
   double red_c[4];
   uint32_t red_s[4];
   int overlap;
@@ -53,19 +63,18 @@ __device__ __forceinline__ int perm_fwd(int p) {  // sequence position -> tile i
   return a * 128 + b * 16 + c * 8 + d * 2 + e;
 }
 
-// unit (2c + h) that owns group jj < 2048, and the slot m = jj & 7 it sits in
-__device__ __forceinline__ uint32_t owner_unit(uint32_t jj) {
-  const uint32_t c = jj >> 4, m = jj & 7u, half = (jj >> 3) & 1u;
-  return 2u * c + (half ^ ((uint32_t(kHalfSel[c]) >> m) & 1u));
+// thread that owns group jj < 2048 (slot m = jj & 7): column c = jj >> 4 = 4u + r + 64b, half h = bit 3 of jj
+__device__ __forceinline__ uint32_t owner_thread(uint32_t jj) {
+  const uint32_t c = jj >> 4, h = (jj >> 3) & 1u;
+  return ((c & 63u) >> 2) | ((c & 3u) << 4) | ((c >> 6) << 6) | (h << 7);
 }
-// predecessor digit of group j from one step's 256 back-pointer words (word index = thread that runs the owning
-// unit, so that a wave's 64 words are one contiguous 512-byte store; nibble m for the group itself, nibble 8 + m
-// for a mirror group j >= 2048).  Read past the vector L1, which may still hold the previous tile's words.
-__device__ __forceinline__ uint32_t bp_lookup(const Smem& sm, const unsigned long long* step_words, uint32_t j) {
+// predecessor digit of group j from one step's 256 back-pointer words (word index = owning thread, so that a
+// wave's 64 words are one contiguous 512-byte store; nibble m for the group itself, nibble 8 + m for a mirror
+// group j >= 2048).  Read past the vector L1, which may still hold the previous tile's words.
+__device__ __forceinline__ uint32_t bp_lookup(const unsigned long long* step_words, uint32_t j) {
   const uint32_t jj = j < 2048u ? j : 4095u - j;
   const uint32_t shift = (jj & 7u) * 4u + (j < 2048u ? 0u : 32u);
-  const unsigned long long w = __hip_atomic_load(step_words + sm.thread_of_unit[owner_unit(jj)], __ATOMIC_RELAXED,
-                                                 __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long w = __hip_atomic_load(step_words + owner_thread(jj), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return uint32_t(w >> shift) & 15u;
 }
 
@@ -76,33 +85,32 @@ __device__ __forceinline__ uint32_t bp_lookup(const Smem& sm, const unsigned lon
 __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict__ entry_d, int roll, int ov,
                                              unsigned long long* __restrict__ bp, int bp_first) {
   const int tid = threadIdx.x;
-  const int unit = kUnitOfLane[tid];  // 2c + h: which groups of which metric column this lane owns
-  const int colA = unit >> 1, colB = 255 - colA;
-  const uint32_t half_bits = uint32_t(kHalfSel[colA]) ^ ((unit & 1) ? 0xffu : 0u);  // bit m: own 16c+8+m, else 16c+m
+  const int colA = 4 * (tid & 15) + ((tid >> 4) & 3) + 64 * ((tid >> 6) & 1), colB = 255 - colA;
+  const int half = tid >> 7;  // owns 16c + 8 half + m, m = 0..7
   const double INF = __builtin_inf();
 
-  // this thread's 4 codebook entries for the per-step error table: e = tid + 256*q -> row tid & 63, k = (tid >> 6) + 4q
-  // (re-read from the 16 KB global table every step: it stays in the CU's vector L1 and the registers are needed)
+  // this thread's 4 codebook entries for the per-step error table: e = tid + 256*q -> row tid & 63, position
+  // (tid >> 6) + 4q (re-read from the 16 KB global table every step: it stays in the CU's vector L1 and the registers
+  // are needed)
   const double2* __restrict__ entries = reinterpret_cast<const double2*>(entry_d) + tid;
-  const int e_wr = (tid & 63) * kRowStride + kRowPad[tid & 63] + (tid >> 6);
+  const int e_wr = (tid >> 6) * 64 + (tid & 63);
 
-  // per slot: E row base (row * stride + padding + b4) and the metric slot written for the group; the mirror
-  // group's slot is kMirror - that (slot(j) + slot(4095 - j) = 255 * 17 + 15)
+  // per slot: E base (b4 * 64 + row) and the metric slot written for the group; the mirror group's is that ^ kMirror
   int ebase[8], wslot[8];
-  constexpr int kMirror = 255 * 17 + 15;
+  constexpr int kMirror = 0xff3;
 #pragma unroll
   for (int m = 0; m < 8; ++m) {
-    const uint32_t j = 16u * colA + 8u * ((half_bits >> m) & 1u) + m, p = j * (j + 1u);
-    const int row = int((p >> 6) & 63u);
-    ebase[m] = row * kRowStride + kRowPad[row] + int((p >> 12) & 15u);
-    wslot[m] = int(j & 255u) * 17 + int(j >> 8);
+    const uint32_t j = 16u * colA + 8u * uint32_t(half) + m, p = j * (j + 1u);
+    ebase[m] = int((p >> 12) & 15u) * 64 + int((p >> 6) & 63u);
+    wslot[m] = m_slot(int(j & 255u), int(j >> 8));
   }
-  const int rA = colA * 17, rB = colB * 17;
+  // byte offsets of digit pi^-1(0) of the two metric columns; the other digits are XORs with 8 pi(d)
+  int xA = colA * 128 + m_swz(colA) * 8, xB = colB * 128 + m_swz(colB) * 8;
+  const char* const Mb = reinterpret_cast<const char*>(sm.M);
 
   // initial metrics: M_0[g] = 0, or +inf outside group ov
   for (int g = tid; g < kGroups; g += kThreads) {
-    const int col = g & 255, d = g >> 8;
-    sm.M[col * 17 + d] = (ov < 0 || g == ov) ? 0.0 : INF;
+    sm.M[m_slot(g & 255, g >> 8)] = (ov < 0 || g == ov) ? 0.0 : INF;
   }
   __syncthreads();
 
@@ -110,10 +118,13 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
   for (int it = 0; it < kSteps; ++it) {
     // ---- phase R: metric columns -> registers, error table of this step -> LDS
     double MA[16], MB[16];
+    // the 32 read addresses are recomputed in every step (one XOR each): kept across the loop they would take 32
+    // registers the accumulators need
+    asm volatile("" : "+v"(xA), "+v"(xB));
 #pragma unroll
     for (int d = 0; d < 16; ++d) {
-      MA[d] = sm.M[rA + d];
-      MB[d] = sm.M[rB + d];
+      MA[d] = *reinterpret_cast<const double*>(Mb + (xA ^ (8 * pi16(d))));
+      MB[d] = *reinterpret_cast<const double*>(Mb + (xB ^ (8 * pi16(d))));
     }
     {
       const int t = (2 * it + roll) & 255;
@@ -123,8 +134,8 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
         const double2 l = entries[256 * q];
         const double a = l.x - x0, b = l.y - x1;
         const double err = __builtin_fma(a, a, b * b);
-        sm.E[e_wr + 4 * q] = err;
-        sm.E[e_wr + 4 * q + 16] = err;
+        sm.E[e_wr + 256 * q] = err;
+        sm.E[e_wr + 256 * q + 1024] = err;
       }
     }
     __syncthreads();
@@ -133,11 +144,12 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
     // upwards with "<", its mirror scans downwards with "<=" over the same values; both keep the smallest
     // digit among equal minima, as the ascending first-minimum rule of the CPU algorithm does.
     word = 0;
+    const bool digits = it >= bp_first;  // uniform; without them a candidate costs an add and a min
     double cur[8], nxt[8];
     {
       const double* er = sm.E + ebase[0];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) cur[k] = er[k & 15];  // slot 0: stride 1
+      for (int k = 0; k < 8; ++k) cur[k] = er[(k & 15) * 64];  // slot 0: stride 1
     }
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
@@ -145,7 +157,7 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
       {
         const double* er = sm.E + ebase[m];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) nxt[k] = er[((8 + k) * g) & 15];
+        for (int k = 0; k < 8; ++k) nxt[k] = er[(((8 + k) * g) & 15) * 64];
       }
       double ba = cur[0] + MA[0], bb = cur[0] + MB[15], ca, cb;
       uint32_t da = 0, db = 15;
@@ -165,30 +177,61 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
       : [ca] "=&v"(ca), [cb] "=&v"(cb), [ka] "=&s"(mka), [kb] "=&s"(mkb), [ba] "+v"(ba), [bb] "+v"(bb),     \
         [da] "+v"(da), [db] "+v"(db)                                                                        \
       : [e] "v"(EV), [ma] "v"(MAV), [mb] "v"(MBV))
-      QTIP_ACS2(1, 14, cur[1], MA[1], MB[14]);
-      QTIP_ACS2(2, 13, cur[2], MA[2], MB[13]);
-      QTIP_ACS2(3, 12, cur[3], MA[3], MB[12]);
-      QTIP_ACS2(4, 11, cur[4], MA[4], MB[11]);
-      QTIP_ACS2(5, 10, cur[5], MA[5], MB[10]);
-      QTIP_ACS2(6, 9, cur[6], MA[6], MB[9]);
-      QTIP_ACS2(7, 8, cur[7], MA[7], MB[8]);
+      // the same without the digit, for the steps whose back-pointers nobody reads (first half of the first pass)
+#define QTIP_AM2(EV, MAV, MBV)                                       \
+  asm volatile(                                                      \
+      "v_add_f64 %[ca], %[e], %[ma]\n\t"                             \
+      "v_add_f64 %[cb], %[e], %[mb]\n\t"                             \
+      "v_min_f64 %[ba], %[ba], %[ca]\n\t"                            \
+      "v_min_f64 %[bb], %[bb], %[cb]"                                \
+      : [ca] "=&v"(ca), [cb] "=&v"(cb), [ba] "+v"(ba), [bb] "+v"(bb) \
+      : [e] "v"(EV), [ma] "v"(MAV), [mb] "v"(MBV))
+      if (digits) {
+        QTIP_ACS2(1, 14, cur[1], MA[1], MB[14]);
+        QTIP_ACS2(2, 13, cur[2], MA[2], MB[13]);
+        QTIP_ACS2(3, 12, cur[3], MA[3], MB[12]);
+        QTIP_ACS2(4, 11, cur[4], MA[4], MB[11]);
+        QTIP_ACS2(5, 10, cur[5], MA[5], MB[10]);
+        QTIP_ACS2(6, 9, cur[6], MA[6], MB[9]);
+        QTIP_ACS2(7, 8, cur[7], MA[7], MB[8]);
+      } else {
+        QTIP_AM2(cur[1], MA[1], MB[14]);
+        QTIP_AM2(cur[2], MA[2], MB[13]);
+        QTIP_AM2(cur[3], MA[3], MB[12]);
+        QTIP_AM2(cur[4], MA[4], MB[11]);
+        QTIP_AM2(cur[5], MA[5], MB[10]);
+        QTIP_AM2(cur[6], MA[6], MB[9]);
+        QTIP_AM2(cur[7], MA[7], MB[8]);
+      }
       if (m < 7) {
         const int gn = 2 * (m + 1) + 1;
         const double* er = sm.E + ebase[m < 7 ? m + 1 : 7];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) cur[k] = er[(k * gn) & 15];
+        for (int k = 0; k < 8; ++k) cur[k] = er[((k * gn) & 15) * 64];
       }
-      QTIP_ACS2(8, 7, nxt[0], MA[8], MB[7]);
-      QTIP_ACS2(9, 6, nxt[1], MA[9], MB[6]);
-      QTIP_ACS2(10, 5, nxt[2], MA[10], MB[5]);
-      QTIP_ACS2(11, 4, nxt[3], MA[11], MB[4]);
-      QTIP_ACS2(12, 3, nxt[4], MA[12], MB[3]);
-      QTIP_ACS2(13, 2, nxt[5], MA[13], MB[2]);
-      QTIP_ACS2(14, 1, nxt[6], MA[14], MB[1]);
-      QTIP_ACS2(15, 0, nxt[7], MA[15], MB[0]);
+      if (digits) {
+        QTIP_ACS2(8, 7, nxt[0], MA[8], MB[7]);
+        QTIP_ACS2(9, 6, nxt[1], MA[9], MB[6]);
+        QTIP_ACS2(10, 5, nxt[2], MA[10], MB[5]);
+        QTIP_ACS2(11, 4, nxt[3], MA[11], MB[4]);
+        QTIP_ACS2(12, 3, nxt[4], MA[12], MB[3]);
+        QTIP_ACS2(13, 2, nxt[5], MA[13], MB[2]);
+        QTIP_ACS2(14, 1, nxt[6], MA[14], MB[1]);
+        QTIP_ACS2(15, 0, nxt[7], MA[15], MB[0]);
+      } else {
+        QTIP_AM2(nxt[0], MA[8], MB[7]);
+        QTIP_AM2(nxt[1], MA[9], MB[6]);
+        QTIP_AM2(nxt[2], MA[10], MB[5]);
+        QTIP_AM2(nxt[3], MA[11], MB[4]);
+        QTIP_AM2(nxt[4], MA[12], MB[3]);
+        QTIP_AM2(nxt[5], MA[13], MB[2]);
+        QTIP_AM2(nxt[6], MA[14], MB[1]);
+        QTIP_AM2(nxt[7], MA[15], MB[0]);
+      }
 #undef QTIP_ACS2
+#undef QTIP_AM2
       sm.M[wslot[m]] = ba;
-      sm.M[kMirror - wslot[m]] = bb;
+      sm.M[wslot[m] ^ kMirror] = bb;
       word |= (unsigned long long)(da) << (4 * m);
       word |= (unsigned long long)(db) << (32 + 4 * m);
     }
@@ -202,10 +245,10 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
     uint32_t bests = 0xffffffffu;
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
-      const uint32_t ja = 16u * colA + 8u * ((half_bits >> m) & 1u) + m, jb = 4095u - ja;
+      const uint32_t ja = 16u * colA + 8u * uint32_t(half) + m, jb = 4095u - ja;
       const uint32_t sa = (uint32_t(word >> (4 * m)) & 15u) << 12 | ja;
       const uint32_t sb = (uint32_t(word >> (32 + 4 * m)) & 15u) << 12 | jb;
-      const double ca = sm.M[wslot[m]], cb = sm.M[kMirror - wslot[m]];
+      const double ca = sm.M[wslot[m]], cb = sm.M[wslot[m] ^ kMirror];
       if (ca < bestc || (ca == bestc && sa < bests)) bestc = ca, bests = sa;
       if (cb < bestc || (cb == bestc && sb < bests)) bestc = cb, bests = sb;
     }
@@ -226,7 +269,7 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
     }
   } else {
     const uint32_t j = uint32_t(ov), jj = j < 2048u ? j : 4095u - j;
-    if (owner_unit(jj) == uint32_t(unit)) {
+    if (owner_thread(jj) == uint32_t(tid)) {
       const uint32_t shift = (jj & 7u) * 4u + (j < 2048u ? 0u : 32u);
       sm.final_state = (uint32_t(word >> shift) & 15u) << 12 | j;
     }
@@ -240,7 +283,6 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
   __shared__ Smem sm;
   const int u = threadIdx.x;
   unsigned long long* bp = bp_all + size_t(blockIdx.x) * kBpWordsPerTile;
-  sm.thread_of_unit[kUnitOfLane[u]] = uint8_t(u);
   for (long tile = blockIdx.x; tile < job.tiles; tile += gridDim.x) {
     sm.x[u] = job.X[tile * kSeq + u];
     __syncthreads();
@@ -250,7 +292,7 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
       uint32_t s = sm.final_state;  // state of step 127
       for (int i = 127; i > 64; --i) {
         const uint32_t j = s >> 4;
-        s = j | (bp_lookup(sm, bp + size_t(i - 1) * kThreads, j) << 12);
+        s = j | (bp_lookup(bp + size_t(i - 1) * kThreads, j) << 12);
       }
       sm.overlap = int(s >> 4);  // state of step 64, high 12 bits
     }
@@ -263,7 +305,7 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
       sm.st[127] = uint16_t(s);
       for (int i = 127; i > 0; --i) {
         const uint32_t j = s >> 4;
-        s = j | (bp_lookup(sm, bp + size_t(i - 1) * kThreads, j) << 12);
+        s = j | (bp_lookup(bp + size_t(i - 1) * kThreads, j) << 12);
         sm.st[i - 1] = uint16_t(s);
       }
     }
