@@ -11,6 +11,10 @@
 #include <mutex>
 #include <thread>
 
+#include <sys/resource.h>
+#include <sys/syscall.h>
+#include <unistd.h>
+
 #include "quantizer_impl.hpp"
 
 namespace qtipmi {
@@ -92,34 +96,50 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
     }
   });
 
-  try {
-    for (int g = 0; g < ng; ++g) {
-      const double tw = now_s();
-      {
-        std::unique_lock<std::mutex> lk(mu);
-        cv.wait(lk, [&] { return factored > g || ldl_err; });
-        if (factored <= g || (ldl_err && factored == g + 1)) std::rethrow_exception(ldl_err);
+  // The quantize loop runs on a helper thread of lower scheduling priority: the pipeline is bound by the host LDL
+  // whenever n is large, and the LDL team fills every core, so the thread that merely feeds the GPU queue should
+  // lose the core whenever the two compete.  (A thread cannot raise its priority again without privileges, hence
+  // a thread of its own that ends with the call instead of a change to the caller's.)
+  std::exception_ptr feed_err;
+  auto feed = [&] {
+    try {
+      QTIP_HIP(hipSetDevice(c->device));
+      (void)setpriority(PRIO_PROCESS, static_cast<id_t>(syscall(SYS_gettid)), 10);
+      for (int g = 0; g < ng; ++g) {
+        const double tw = now_s();
+        {
+          std::unique_lock<std::mutex> lk(mu);
+          cv.wait(lk, [&] { return factored > g || ldl_err; });
+          if (factored <= g || (ldl_err && factored == g + 1)) std::rethrow_exception(ldl_err);
+        }
+        if (ldl_wait) ldl_wait[g] = now_s() - tw;
+        if (g + 2 < ng) rotate(g + 2);  // into the buffers group g-1 has finished with
+        const int b = g % R;
+        qtip_timing T{};
+        T.rht = t_rot[size_t(g)];
+        T.ldl_cpu = t_ldl[size_t(g)];
+        quantize_group_impl(c, groups[g].nlin, groups[g].lins, groups[g].n, groups[g].seed, su[size_t(b)].data(),
+                            creg[size_t(g)], c->ring_HRr[b].p, c->ring_L[b].p, opt, groups[g].outs, &T);
+        if (tms) tms[g] = T;
       }
-      if (ldl_wait) ldl_wait[g] = now_s() - tw;
-      if (g + 2 < ng) rotate(g + 2);  // into the buffers group g-1 has finished with
-      const int b = g % R;
-      qtip_timing T{};
-      T.rht = t_rot[size_t(g)];
-      T.ldl_cpu = t_ldl[size_t(g)];
-      quantize_group_impl(c, groups[g].nlin, groups[g].lins, groups[g].n, groups[g].seed, su[size_t(b)].data(),
-                          creg[size_t(g)], c->ring_HRr[b].p, c->ring_L[b].p, opt, groups[g].outs, &T);
-      if (tms) tms[g] = T;
-    }
-  } catch (...) {
-    {
+    } catch (...) {
+      feed_err = std::current_exception();
       std::lock_guard<std::mutex> lk(mu);
       stop = true;
       cv.notify_all();
     }
-    ldl_thread.join();
-    throw;
+  };
+  try {
+    std::thread feeder(feed);
+    feeder.join();
+  } catch (...) {  // the helper thread could not be started
+    feed_err = std::current_exception();
+    std::lock_guard<std::mutex> lk(mu);
+    stop = true;
+    cv.notify_all();
   }
   ldl_thread.join();
+  if (feed_err) std::rethrow_exception(feed_err);
 }
 
 }  // namespace qtipmi
