@@ -21,6 +21,8 @@ double quad_trace_bf16x3(long n, long m, const float* H, const float* A, const f
 void launch_nvfp4_block(const float* WT, const float* FT, long m, long n, long c0, const float* L, const float* dw,
                         float global, bool calibrate, bool search, uint8_t* packedT, uint8_t* scalesT, float* E,
                         hipStream_t s);
-void launch_nvfp4_feedback(float* FT, long m, long n, long c0, const float* E, const float* L, hipStream_t s);
+void launch_nvfp4_feedback(float* FT, long m, long n, long c0, long col_lo, const float* E, const float* L,
+                           hipStream_t s);
+void launch_nvfp4_gather(float* FT, long m, long n, long cb, const float* ET, const float* L, hipStream_t s);
 void launch_transpose_u8(const uint8_t* in, long rows, long cols, uint8_t* out, hipStream_t s);
 }  // namespace qtipmi

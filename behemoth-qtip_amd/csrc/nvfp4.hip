@@ -154,12 +154,12 @@ __global__ __launch_bounds__(256) void nv_block_kernel(const float* __restrict__
   for (int k = 0; k < 16; ++k) E[k * m + r] = err[k];
 }
 
-// FT[col][r] += sum_{j < 16} E[j][r] * L[c0 + j][col]  for col < c0 (the sum first, in j order, then one add).
-// A workgroup: 256 rows x 32 columns; the 16 x 32 piece of L sits in LDS.
-__global__ __launch_bounds__(256) void nv_feedback_kernel(float* __restrict__ FT, long m, long n, long c0,
+// FT[col][r] += sum_{j < 16} E[j][r] * L[c0 + j][col]  for col_lo <= col < c0 (the sum first, in j order, then one
+// add).  A workgroup: 256 rows x 32 columns; the 16 x 32 piece of L sits in LDS.
+__global__ __launch_bounds__(256) void nv_feedback_kernel(float* __restrict__ FT, long m, long n, long c0, long col_lo,
                                                           const float* __restrict__ E, const float* __restrict__ L) {
   __shared__ float Ls[16][32];
-  const long col0 = long(blockIdx.y) * 32;
+  const long col0 = col_lo + long(blockIdx.y) * 32;
   for (int idx = threadIdx.x; idx < 512; idx += 256) {
     const int j = idx >> 5, c = idx & 31;
     Ls[j][c] = col0 + c < c0 ? L[(c0 + j) * n + col0 + c] : 0.f;
@@ -177,6 +177,43 @@ __global__ __launch_bounds__(256) void nv_feedback_kernel(float* __restrict__ FT
     for (int j = 0; j < 16; ++j) acc = fmaf(e[j], Ls[j][c], acc);
     FT[(col0 + c) * m + r] += acc;
   }
+}
+
+// The feedback a 128-column buffer [cb, cb + 128) receives from every block behind it, gathered in one pass:
+//   FT[col][r] = ((0 + a_{n-16}) + a_{n-32}) + ... + a_{cb+128},   a_b = sum_{j < 16} E[b + j][r] * L[b + j][col]
+// (each a_b a chain of fused multiply-adds in j order from zero): the values and the order of additions of the
+// block-by-block form, which reads and writes every column left of a block once per block (n^2 m / 4 bytes in all);
+// this form reads the error rows once per buffer (n^2 m / 64 bytes).  ET: the errors of all finished columns, [n][m].
+// A wave: 64 rows x kGatherCols columns (narrow, so that a matrix of 12288 rows still gives every SIMD several waves);
+// the four waves of a workgroup take four neighbouring column pieces of the same 64 rows, so three of them find the
+// error values in the vector L1.  The piece of L of a block is the same for a whole wave and arrives through the
+// scalar cache.
+constexpr int kGatherCols = 8;
+__global__ __launch_bounds__(256) void nv_gather_kernel(float* __restrict__ FT, long m, long n, long cb,
+                                                        const float* __restrict__ ET, const float* __restrict__ L) {
+  const long r = long(blockIdx.x) * 64 + (threadIdx.x & 63);
+  const long col0 = cb + (long(blockIdx.y) * 4 + __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6))) * kGatherCols;
+  if (r >= m) return;
+  float f[kGatherCols];
+#pragma unroll
+  for (int c = 0; c < kGatherCols; ++c) f[c] = 0.f;
+  for (long b = n - 16; b >= cb + 128; b -= 16) {
+    float e[16], acc[kGatherCols];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) e[j] = ET[(b + j) * m + r];
+#pragma unroll
+    for (int c = 0; c < kGatherCols; ++c) acc[c] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float* __restrict__ lrow = L + (b + j) * n + col0;  // uniform over the workgroup
+#pragma unroll
+      for (int c = 0; c < kGatherCols; ++c) acc[c] = fmaf(e[j], lrow[c], acc[c]);
+    }
+#pragma unroll
+    for (int c = 0; c < kGatherCols; ++c) f[c] += acc[c];
+  }
+#pragma unroll
+  for (int c = 0; c < kGatherCols; ++c) FT[(col0 + c) * m + r] = f[c];
 }
 
 // bytes [rows][cols] -> [cols][rows], 32 x 32 patches through LDS
@@ -207,9 +244,18 @@ void launch_nvfp4_block(const float* WT, const float* FT, long m, long n, long c
                                                                         search ? 1 : 0, packedT, scalesT, E);
   QTIP_HIP(hipGetLastError());
 }
-void launch_nvfp4_feedback(float* FT, long m, long n, long c0, const float* E, const float* L, hipStream_t s) {
-  if (c0 <= 0) return;
-  nv_feedback_kernel<<<dim3(unsigned((m + 255) / 256), unsigned((c0 + 31) / 32)), dim3(256), 0, s>>>(FT, m, n, c0, E, L);
+void launch_nvfp4_feedback(float* FT, long m, long n, long c0, long col_lo, const float* E, const float* L,
+                           hipStream_t s) {
+  if (c0 <= col_lo) return;
+  QTIP_REQUIRE(col_lo >= 0 && c0 <= n, "nvfp4 feedback: column window [%ld, %ld) outside [0, %ld)", col_lo, c0, n);
+  nv_feedback_kernel<<<dim3(unsigned((m + 255) / 256), unsigned((c0 - col_lo + 31) / 32)), dim3(256), 0, s>>>(
+      FT, m, n, c0, col_lo, E, L);
+  QTIP_HIP(hipGetLastError());
+}
+void launch_nvfp4_gather(float* FT, long m, long n, long cb, const float* ET, const float* L, hipStream_t s) {
+  QTIP_REQUIRE(cb >= 0 && cb % 16 == 0 && cb + 128 <= n && n % 16 == 0, "nvfp4 gather: buffer [%ld, %ld) outside [0, %ld)",
+               cb, cb + 128, n);
+  nv_gather_kernel<<<dim3(unsigned((m + 63) / 64), 128 / kGatherCols / 4), dim3(256), 0, s>>>(FT, m, n, cb, ET, L);
   QTIP_HIP(hipGetLastError());
 }
 void launch_transpose_u8(const uint8_t* in, long rows, long cols, uint8_t* out, hipStream_t s) {

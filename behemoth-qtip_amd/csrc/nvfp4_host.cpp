@@ -147,19 +147,29 @@ void nvfp4_quantize_prepared_impl(qtip_ctx* c, int nmat, const qtip_nvfp4_matrix
     const long m = M.m;
     const float g = global_scale(M.w, size_t(m) * n);
     const_cast<qtip_nvfp4_matrix&>(M).global = g;
-    DBuf<float> W(size_t(m) * n), WT(size_t(m) * n), FT, E(size_t(16) * m);
+    // E: the residuals W - q of the finished columns, transposed like W; all of them when they are fed back
+    DBuf<float> W(size_t(m) * n), WT(size_t(m) * n), FT, E(cal ? size_t(m) * n : size_t(16) * m);
     DBuf<uint8_t> pT(size_t(m) * n / 2), sT(size_t(m) * n / 16), pk(size_t(m) * n / 2), sc(size_t(m) * n / 16);
     QTIP_HIP(hipMemcpyAsync(W, M.w, W.bytes(), hipMemcpyHostToDevice, s));
     c->rht.transpose(W, m, n, n, WT, m);
     W.release();
+    // Columns go in buffers of 128 from the last to the first.  A buffer first gathers the feedback of every block
+    // behind it in one pass; inside the buffer every block then feeds the columns of the buffer left of it.  Values
+    // and order of the additions are those of the block-by-block form.
+    const long top = (long(n) - 1) / 128 * 128;
     if (cal) {
       FT.alloc(size_t(m) * n);
-      QTIP_HIP(hipMemsetAsync(FT, 0, FT.bytes(), s));
+      QTIP_HIP(hipMemsetAsync(FT.p + size_t(top) * m, 0, size_t(n - top) * m * sizeof(float), s));
     }
-    for (long c0 = n - 16; c0 >= 0; c0 -= 16) {
-      launch_nvfp4_block(WT, cal ? FT.p : nullptr, m, n, c0, cal ? d_L.p : nullptr, host_dw ? d_dw.p : nullptr, g, cal,
-                         search, pT, sT, E, s);
-      if (cal) launch_nvfp4_feedback(FT, m, n, c0, E, d_L, s);
+    for (long cb = top; cb >= 0; cb -= 128) {
+      const long hi = std::min<long>(n, cb + 128);
+      if (cal && hi < n) launch_nvfp4_gather(FT, m, n, cb, E, d_L, s);
+      for (long c0 = hi - 16; c0 >= cb; c0 -= 16) {
+        float* e = cal ? E.p + size_t(c0) * m : E.p;
+        launch_nvfp4_block(WT, cal ? FT.p : nullptr, m, n, c0, cal ? d_L.p : nullptr, host_dw ? d_dw.p : nullptr, g,
+                           cal, search, pT, sT, e, s);
+        if (cal) launch_nvfp4_feedback(FT, m, n, c0, cb, e, d_L, s);
+      }
     }
     launch_transpose_u8(pT, n / 2, m, pk, s);
     launch_transpose_u8(sT, n / 16, m, sc, s);
