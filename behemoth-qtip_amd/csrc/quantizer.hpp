@@ -6,9 +6,11 @@
 #include <hip/hip_runtime.h>
 
 #include <chrono>
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <string>
@@ -32,7 +34,7 @@ struct QuantOpts {  // src/quantizer.hpp:11-19
   int vit_batch = 1024;  // accepted, unused: the tile kernel sizes its own back-pointer workspace
   int ldl_threads = 16;
   bool share_su = true;
-  std::string dump_dir;  // not supported by the shim (must stay empty)
+  std::string dump_dir;  // if set: W (fp32) and, unless want_hatW, the reconstructed hatW (fp32) are written per linear
   bool want_hatW = false;
 };
 
@@ -101,6 +103,48 @@ inline qtip_ctx* context() {
 }
 }  // namespace detail
 
+namespace detail {
+// src/quantizer.cpp:118-121
+inline void write_f32(const std::string& path, const float* p, size_t count) {
+  FILE* f = std::fopen(path.c_str(), "wb");
+  if (!f) return;  // the reference's ofstream write fails as silently
+  std::fwrite(p, 4, count, f);
+  std::fclose(f);
+}
+// The fp32 weight quantize_group works on, as the reference dumps it (src/quantizer.cpp:214-234): the input itself,
+// the bf16 bits widened, or the E4M3 value times its row's bf16 scale (one fp32 product, src/kernels.hip:20-36).
+inline std::vector<float> weight_as_f32(const LinearIn& l, int n) {
+  const size_t count = size_t(l.m) * size_t(n);
+  std::vector<float> w(count);
+  auto bf = [](uint16_t h) {
+    const uint32_t u = uint32_t(h) << 16;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+  };
+  if (l.w_f32) {
+    std::memcpy(w.data(), l.w_f32, count * 4);
+  } else if (l.w_bf16) {
+    for (size_t i = 0; i < count; ++i) w[i] = bf(l.w_bf16[i]);
+  } else if (l.w_fp8) {
+    for (size_t i = 0; i < count; ++i) {
+      const uint8_t b = l.w_fp8[i];
+      const uint32_t e = (b >> 3) & 0xf, m = b & 7;
+      float v = e == 0 ? std::ldexp(float(m), -9) : (e == 15 && m == 7) ? std::nanf("") : std::ldexp(float(m | 8), int(e) - 10);
+      if (b >> 7) v = -v;
+      w[i] = l.scale_bf16 ? v * bf(l.scale_bf16[i / size_t(n)]) : v;
+    }
+  }
+  return w;
+}
+inline void dump_linear(const QuantOpts& opt, const std::string& tag, const LinearIn& l, int n, const float* hatW) {
+  if (opt.dump_dir.empty()) return;
+  const std::vector<float> w = weight_as_f32(l, n);
+  write_f32(opt.dump_dir + "/" + tag + "_" + l.name + ".W.f32", w.data(), w.size());
+  if (!opt.want_hatW && hatW) write_f32(opt.dump_dir + "/" + tag + "_" + l.name + ".hatW.f32", hatW, w.size());
+}
+}  // namespace detail
+
 inline void rotate_hessian(hipStream_t, const float* H, int n, uint64_t seed, const QuantOpts& opt, HessPrep& hp) {
   const double t0 = detail::now_s();
   hp.n = n;
@@ -124,7 +168,7 @@ inline void ldl_hessian(HessPrep& hp, int threads, const std::string& tag) {
 inline std::vector<LinearOut> quantize_group(hipStream_t, Gemm&, const std::vector<LinearIn>& lins, HessPrep& hp,
                                              const QuantOpts& opt, GroupTiming* tm, const std::string& tag) {
   if (!opt.share_su) detail::die("share_su=false not supported (one LDL per group)");
-  if (!opt.dump_dir.empty()) detail::die("dump_dir is not supported by this build (" + tag + ")");
+  const bool need_hat = opt.want_hatW || !opt.dump_dir.empty();
   const int n = hp.n;
   std::vector<qtip_linear_in> cin(lins.size());
   std::vector<qtip_linear_out> cout(lins.size());
@@ -138,8 +182,8 @@ inline std::vector<LinearOut> quantize_group(hipStream_t, Gemm&, const std::vect
     o.trellis.resize(size_t(l.m / 16) * (n / 16) * 32);
     o.su_bf16.resize(size_t(n));
     o.sv.resize(size_t(l.m));
-    if (opt.want_hatW) o.hatW.resize(size_t(l.m) * n);
-    cout[i] = qtip_linear_out{o.trellis.data(), o.su_bf16.data(), o.sv.data(), opt.want_hatW ? o.hatW.data() : nullptr,
+    if (need_hat) o.hatW.resize(size_t(l.m) * n);
+    cout[i] = qtip_linear_out{o.trellis.data(), o.su_bf16.data(), o.sv.data(), need_hat ? o.hatW.data() : nullptr,
                               0.f, 0.0, 0.0, 0.0};
   }
   qtip_opts co;
@@ -155,6 +199,8 @@ inline std::vector<LinearOut> quantize_group(hipStream_t, Gemm&, const std::vect
   for (size_t i = 0; i < lins.size(); ++i) {
     out[i].wscale = cout[i].wscale, out[i].proxy = cout[i].proxy;
     out[i].proxy_rot_reg = cout[i].proxy_rot_reg, out[i].seconds = cout[i].seconds;
+    detail::dump_linear(opt, tag, lins[i], n, out[i].hatW.data());
+    if (!opt.want_hatW) std::vector<float>().swap(out[i].hatW);
   }
   if (tm) *tm = GroupTiming{ct.load, ct.rht, ct.ldl_cpu, ct.ldlq, ct.viterbi, ct.proxy, ct.pack, ct.total};
   return out;
@@ -199,7 +245,7 @@ inline std::vector<std::vector<LinearOut>> run_groups(const std::vector<GroupSpe
                                                       std::vector<GroupTiming>* tms = nullptr,
                                                       std::vector<double>* ldl_wait = nullptr) {
   if (!opt.share_su) detail::die("share_su=false not supported (one LDL per group)");
-  if (!opt.dump_dir.empty()) detail::die("dump_dir is not supported by this build");
+  const bool need_hat = opt.want_hatW || !opt.dump_dir.empty();
   const size_t ng = groups.size();
   std::vector<std::vector<qtip_linear_in>> cin(ng);
   std::vector<std::vector<qtip_linear_out>> cout(ng);
@@ -217,9 +263,9 @@ inline std::vector<std::vector<LinearOut>> run_groups(const std::vector<GroupSpe
       o.trellis.resize(size_t(l.m / 16) * (G.n / 16) * 32);
       o.su_bf16.resize(size_t(G.n));
       o.sv.resize(size_t(l.m));
-      if (opt.want_hatW) o.hatW.resize(size_t(l.m) * G.n);
+      if (need_hat) o.hatW.resize(size_t(l.m) * G.n);
       cout[g][i] = qtip_linear_out{o.trellis.data(), o.su_bf16.data(), o.sv.data(),
-                                   opt.want_hatW ? o.hatW.data() : nullptr, 0.f, 0.0, 0.0, 0.0};
+                                   need_hat ? o.hatW.data() : nullptr, 0.f, 0.0, 0.0, 0.0};
     }
     cg[g] = qtip_group{int(G.lins.size()), cin[g].data(), cout[g].data(), G.n, G.H, 0, G.seed};
   }
@@ -233,6 +279,8 @@ inline std::vector<std::vector<LinearOut>> run_groups(const std::vector<GroupSpe
     for (size_t i = 0; i < out[g].size(); ++i) {
       out[g][i].wscale = cout[g][i].wscale, out[g][i].proxy = cout[g][i].proxy;
       out[g][i].proxy_rot_reg = cout[g][i].proxy_rot_reg, out[g][i].seconds = cout[g][i].seconds;
+      detail::dump_linear(opt, groups[g].tag, groups[g].lins[i], groups[g].n, out[g][i].hatW.data());
+      if (!opt.want_hatW) std::vector<float>().swap(out[g][i].hatW);
     }
   if (tms) {
     tms->clear();

@@ -93,6 +93,47 @@ int main() {
     std::printf("layer file: %zu bytes\n", bytes);
     if (sz != long(bytes) || bytes < out[0].trellis.size() * 2 + out[1].trellis.size() * 2) ++fail;
   }
+  // dump_dir (src/quantizer.cpp:230-234, 321-337): W as fp32 and the reconstruction, one raw file each
+  {
+    QuantOpts od;
+    od.ldl_threads = 4;
+    od.dump_dir = "/tmp";
+    std::vector<uint16_t> wb(size_t(32) * n);  // a bf16 source: the dump holds its widened values
+    for (size_t i = 0; i < wb.size(); ++i) {
+      uint32_t u;
+      std::memcpy(&u, &W2[i], 4);
+      wb[i] = uint16_t(u >> 16);
+    }
+    std::vector<LinearIn> lb(1);
+    lb[0].name = "dump", lb[0].m = 32, lb[0].w_bf16 = wb.data();
+    GroupTiming t2;
+    auto od_out = quantize_group(S, g, lb, n, H.data(), 11, od, &t2, "shimtest");
+    od.dump_dir.clear();
+    od.want_hatW = true;
+    auto od_ref = quantize_group(S, g, lb, n, H.data(), 11, od, &t2, "shimtest");
+    auto slurp = [](const char* path) {
+      std::vector<float> v;
+      if (FILE* f = std::fopen(path, "rb")) {
+        std::fseek(f, 0, SEEK_END);
+        v.resize(size_t(std::ftell(f)) / 4);
+        std::fseek(f, 0, SEEK_SET);
+        if (std::fread(v.data(), 4, v.size(), f) != v.size()) v.clear();
+        std::fclose(f);
+        std::remove(path);
+      }
+      return v;
+    };
+    const std::vector<float> dw = slurp("/tmp/shimtest_dump.W.f32"), dh = slurp("/tmp/shimtest_dump.hatW.f32");
+    bool okw = dw.size() == wb.size();
+    for (size_t i = 0; okw && i < dw.size(); ++i) {
+      const uint32_t u = uint32_t(wb[i]) << 16;
+      float f;
+      std::memcpy(&f, &u, 4);
+      okw = dw[i] == f;
+    }
+    if (!okw || dh != od_ref[0].hatW || !od_out[0].hatW.empty() || od_out[0].trellis != od_ref[0].trellis) ++fail;
+    std::printf("dump_dir: W %zu values, hatW %zu values, mismatches so far %d\n", dw.size(), dh.size(), fail);
+  }
   // NVFP4 fallback (the criteria of tests/test_nvfp4.cpp:59-105): upgrades off == the plain quantizer byte for byte,
   // calibrated rounding lowers the Hessian-weighted error, a group equals single calls
   {
