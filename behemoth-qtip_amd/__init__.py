@@ -107,6 +107,7 @@ def lib():
     L.qtip_f32_to_fp8e4m3.argtypes = [C.c_float]
     L.qtip_nvfp4_quantize.argtypes = [vp, i, i, vp, vp, C.POINTER(C.c_float)]
     L.qtip_nvfp4_dequantize.argtypes = [vp, vp, C.c_float, i, i, vp]
+    L.qtip_nvfp4_proxy_error.argtypes = [vp, vp, i, i, vp, C.POINTER(d)]
     L.qtip_nvfp4_prepare.argtypes = [vp, i, d, i, i, vp, vp]
     L.qtip_nvfp4_quantize_prepared.argtypes = [vp, i, vp, i, vp, vp, i]
     L.qtip_nvfp4_quantize_group.argtypes = [vp, i, vp, i, vp, C.POINTER(_Nvfp4OptsC), C.POINTER(i)]
@@ -503,6 +504,16 @@ def nvfp4_dequantize(t: Nvfp4Tensor):
     _check(lib().qtip_nvfp4_dequantize(_ptr(np.ascontiguousarray(t.packed)), _ptr(np.ascontiguousarray(t.scales)),
                                        t.global_scale, t.m, t.n, _ptr(out)))
     return out
+
+
+def nvfp4_proxy_error(w, what, H=None):
+    """nvfp4_proxy_error, src/nvfp4.cpp:72-87 (host, fp64)."""
+    w = np.ascontiguousarray(w, np.float32)
+    what = np.ascontiguousarray(what, np.float32)
+    Hc = None if H is None else np.ascontiguousarray(H, np.float32)
+    out = C.c_double()
+    _check(lib().qtip_nvfp4_proxy_error(_ptr(w), _ptr(what), w.shape[0], w.shape[1], _ptr(Hc), C.byref(out)))
+    return out.value
 
 
 def nvfp4_prepare(H, sigma_reg=1e-2, calibrate=True, threads=16):

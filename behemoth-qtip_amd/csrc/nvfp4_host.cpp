@@ -97,6 +97,28 @@ void nvfp4_dequantize_host(const uint8_t* packed, const uint8_t* scales, float g
   QTIP_REQUIRE(!bad, "invalid NVFP4 block scale");
 }
 
+double nvfp4_proxy_error_host(const float* w, const float* what, int m, int n, const float* H) {
+  QTIP_REQUIRE(w && what && m > 0 && n > 0, "nvfp4_proxy_error: bad arguments");
+  double total = 0;
+#pragma omp parallel for reduction(+ : total) schedule(static)
+  for (int r = 0; r < m; ++r) {
+    std::vector<double> e(static_cast<size_t>(n), 0.0);
+    for (int j = 0; j < n; ++j) e[size_t(j)] = double(w[size_t(r) * n + j]) - what[size_t(r) * n + j];
+    double row = 0;
+    if (!H) {
+      for (int j = 0; j < n; ++j) row += e[size_t(j)] * e[size_t(j)];
+    } else {
+      for (int i = 0; i < n; ++i) {
+        double acc = 0;
+        for (int j = 0; j < n; ++j) acc += double(H[size_t(i) * n + j]) * e[size_t(j)];
+        row += e[size_t(i)] * acc;
+      }
+    }
+    total += row;
+  }
+  return total / m;
+}
+
 // Regularised Hessian -> what the block loop needs.  calibrate: unit-lower L (H = L D L^T) and dw = D; otherwise
 // dw = diag(H) + creg and L is not touched.
 void nvfp4_prepare_host(const float* H, int n, double sigma_reg, bool calibrate, int threads, float* L, float* dw) {

@@ -276,6 +276,12 @@ int qtip_nvfp4_dequantize(const uint8_t* host_packed, const uint8_t* host_scales
                           float* host_out) {
   return guarded([&] { nvfp4_dequantize_host(host_packed, host_scales, global, m, n, host_out); });
 }
+int qtip_nvfp4_proxy_error(const float* host_w, const float* host_what, int m, int n, const float* host_H, double* out) {
+  return guarded([&] {
+    QTIP_REQUIRE(out != nullptr, "nvfp4_proxy_error: out is null");
+    *out = nvfp4_proxy_error_host(host_w, host_what, m, n, host_H);
+  });
+}
 int qtip_nvfp4_prepare(const float* host_H, int n, double sigma_reg, int calibrate, int threads, float* host_L,
                        float* host_dw) {
   return guarded([&] { nvfp4_prepare_host(host_H, n, sigma_reg, calibrate != 0, threads, host_L, host_dw); });

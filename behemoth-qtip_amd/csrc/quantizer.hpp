@@ -332,6 +332,12 @@ inline std::vector<float> nvfp4_dequantize(const Nvfp4Tensor& t) {
   return out;
 }
 
+inline double nvfp4_proxy_error(const float* w, const float* what, int m, int n, const float* H) {
+  double v = 0;
+  detail::check(qtip_nvfp4_proxy_error(w, what, m, n, H, &v), "nvfp4_proxy_error");
+  return v;
+}
+
 inline float nvfp4_level(uint8_t code) {
   constexpr float levels[8] = {0, .5f, 1, 1.5f, 2, 3, 4, 6};
   return (code & 8 ? -1.f : 1.f) * levels[code & 7];

@@ -34,6 +34,7 @@ void run_groups_impl(qtip_ctx* c, int ngroups, const qtip_group* groups, const q
 uint8_t f32_to_fp8e4m3(float x);
 void nvfp4_quantize_host(const float* w, int m, int n, uint8_t* packed, uint8_t* scales, float* global);
 void nvfp4_dequantize_host(const uint8_t* packed, const uint8_t* scales, float global, int m, int n, float* out);
+double nvfp4_proxy_error_host(const float* w, const float* what, int m, int n, const float* H);
 void nvfp4_prepare_host(const float* H, int n, double sigma_reg, bool calibrate, int threads, float* L, float* dw);
 void nvfp4_quantize_prepared_impl(qtip_ctx* c, int nmat, const qtip_nvfp4_matrix* mats, int n, const float* host_L,
                                   const float* host_dw, bool search);

@@ -158,6 +158,8 @@ int qtip_nvfp4_quantize(const float* host_w, int m, int n, uint8_t* host_packed,
 /* nvfp4_dequantize, src/nvfp4.cpp:57-70 (host; values rounded to bf16, as execution sees them) */
 int qtip_nvfp4_dequantize(const uint8_t* host_packed, const uint8_t* host_scales, float global, int m, int n,
                           float* host_out);
+/* nvfp4_proxy_error, src/nvfp4.cpp:72-87 (host, fp64): tr((W - What) H (W - What)^T) / m; host_H null = identity */
+int qtip_nvfp4_proxy_error(const float* host_w, const float* host_what, int m, int n, const float* host_H, double* out);
 typedef struct { /* Nvfp4Opts, src/nvfp4_gpu.hpp:21-25 */
   int scale_search; /* 1 */
   int calibrate;    /* 1 */

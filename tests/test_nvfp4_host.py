@@ -25,7 +25,12 @@ def test_plain_quantizer_and_dequantizer(pkg, oracle, name):
     want = np.fromfile(os.path.join(GOLDEN, "ref_nvfp4_%s.bin" % name), np.uint8)
     assert np.array_equal(t.packed.reshape(-1), want[:m * n // 2]) and np.array_equal(t.scales.reshape(-1), want[m * n // 2:])
     assert t.global_scale == float.fromhex(meta["global"])
-    assert np.array_equal(pkg.nvfp4_dequantize(t), oracle.nvfp4_dequantize(t.packed, t.scales, t.global_scale, m, n))
+    dq = pkg.nvfp4_dequantize(t)
+    assert np.array_equal(dq, oracle.nvfp4_dequantize(t.packed, t.scales, t.global_scale, m, n))
+    # proxy error: the golden mean squared error of the reference's own code, and a Hessian-weighted case
+    assert abs(pkg.nvfp4_proxy_error(w, dq) / float.fromhex(meta["mse"]) - 1) < 1e-13
+    H = _hessian(oracle, n, 9, samples=40)
+    assert abs(pkg.nvfp4_proxy_error(w, dq, H) / oracle.nvfp4_proxy_error(w, dq, H) - 1) < 1e-12
 
 
 def test_errors(pkg):
