@@ -71,7 +71,6 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
     cv.notify_all();
   };
   rotate(0);
-  if (ng > 1) rotate(1);
 
   std::thread ldl_thread([&] {
     for (int g = 0; g < ng; ++g) {
@@ -105,6 +104,7 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
     try {
       QTIP_HIP(hipSetDevice(c->device));
       (void)setpriority(PRIO_PROCESS, static_cast<id_t>(syscall(SYS_gettid)), 10);
+      if (ng > 1) rotate(1);  // while the first factorisation is already running
       for (int g = 0; g < ng; ++g) {
         const double tw = now_s();
         {
