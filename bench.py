@@ -163,7 +163,7 @@ def run_group(args, pkg):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=8)
+    ap.add_argument("--steps", type=int, default=16)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--config", type=int, default=5, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--ldl-threads", type=int, default=16, help="OpenMP team of the host LDL")
