@@ -159,8 +159,9 @@ struct TileJob {
 };
 size_t viterbi_workspace_bytes(int slots);
 int viterbi_max_slots(int device);
+// start / stop (optional): events stamped at the kernel's own start and end
 void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const float* d_entry_f, void* workspace,
-                          int slots, hipStream_t s);
+                          int slots, hipStream_t s, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 void launch_decode_states(const uint16_t* states, long B, float* hat, const float* d_entry_f, hipStream_t s);
 
 }  // namespace qtipmi

@@ -97,16 +97,17 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   DBuf<float> X(size_t(ntr) * 256);
   if (feedback == 1) QTIP_HIP(hipMemsetAsync(prod32, 0, prod32.bytes(), s));
   QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
-  Events timed, pacing;
-  auto mark = [&] { QTIP_HIP(hipEventRecord(timed.add(hipEventDefault), s)); };
-  // The queue is kept two buffers (16 launches of ~2 ms) ahead of the GPU and no further: beyond that the
-  // submitting thread would spin on a full queue and take a core from the host LDL of the next group.
-  hipEvent_t pace[3];
+  Events timed, pacing;  // timed: a (start, stop) pair per Viterbi launch, stamped by the launch itself
+  // The queue is kept kAhead buffers (8 launches of ~2 ms each) ahead of the GPU and no further: without a bound the
+  // submitting thread would spin on a full queue and take a core from the host LDL of the next group; with less
+  // slack a submitting thread that the scheduler holds back for a few milliseconds leaves the GPU idle.
+  constexpr long kAhead = 4;
+  hipEvent_t pace[kAhead + 1];
   for (auto& e : pace) e = pacing.add(hipEventBlockingSync | hipEventDisableTiming);
   long nbuf_done = 0;
   for (long cur = nblk; cur > 0; cur -= 8, ++nbuf_done) {
     const int bufend = int(16 * cur), c0 = bufend - 128;
-    if (nbuf_done >= 2) QTIP_HIP(hipEventSynchronize(pace[(nbuf_done - 2) % 3]));
+    if (nbuf_done >= kAhead) QTIP_HIP(hipEventSynchronize(pace[(nbuf_done - kAhead) % (kAhead + 1)]));
     if (feedback == 0) {  // prod[r][:] = sum_{k >= bufend} L[k][c0 + r] (WT - hatWT)[k][:], r < 128
       if (bufend < n)
         launch_gemm_tn_f64_gather(int(m), n - bufend, L + long(bufend) * n + c0, n, WT + long(bufend) * m,
@@ -118,7 +119,6 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
       const int col0 = c0 + 16 * i;
       if (feedback == 0) launch_ldlq_prep_f64(WT, hatWT, prod, c0, L, n, m, col0, bufend, X, s);
       else launch_ldlq_prep_f32(WT, hatWT, prod32, L, n, m, col0, bufend, X, s);
-      if (vit_seconds) mark();
       TileJob job;
       job.X = X;
       job.tiles = ntr;
@@ -128,14 +128,15 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
       job.hatWT = hatWT;
       job.ldw = m;
       job.col0 = col0;
-      launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws, c->vit_slots, s);
-      if (vit_seconds) mark();
+      hipEvent_t t0 = nullptr, t1 = nullptr;
+      if (vit_seconds) t0 = timed.add(hipEventDefault), t1 = timed.add(hipEventDefault);
+      launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws, c->vit_slots, s, t0, t1);
     }
     if (c0 > 0 && feedback == 1) {  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
       launch_gemm_tn_bf16x3_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m,
                                 prod32, m, s);
     }
-    QTIP_HIP(hipEventRecord(pace[nbuf_done % 3], s));
+    QTIP_HIP(hipEventRecord(pace[nbuf_done % (kAhead + 1)], s));
   }
   wait_stream_sleeping(s);
   if (vit_seconds) {

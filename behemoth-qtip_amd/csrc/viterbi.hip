@@ -33,6 +33,8 @@
 // before the step's results are written).
 // Back-pointers (4 bits per group and step) go to HBM as one 64-bit word per thread and step, 2 KB per step,
 // fully coalesced; the first pass only keeps the steps its half-length trace-back needs.
+#include <hip/hip_ext.h>
+
 #include "qtip_internal.hpp"
 
 namespace qtipmi {
@@ -356,12 +358,19 @@ int viterbi_max_slots(int device) {
 }
 
 void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const float* d_entry_f, void* workspace,
-                          int slots, hipStream_t s) {
+                          int slots, hipStream_t s, hipEvent_t start, hipEvent_t stop) {
   if (job.tiles <= 0) return;
   QTIP_REQUIRE(job.X != nullptr && slots > 0 && workspace != nullptr, "viterbi: missing operand");
   const unsigned grid = unsigned(job.tiles < slots ? job.tiles : slots);
-  viterbi_tiles_kernel<<<dim3(grid), dim3(kThreads), 0, s>>>(job, d_entry_d, d_entry_f,
-                                                             static_cast<unsigned long long*>(workspace));
+  if (start || stop) {
+    // the runtime stamps the two events at the kernel's own start and end: the time between them is the kernel's,
+    // however late the host got round to queueing it
+    hipExtLaunchKernelGGL(viterbi_tiles_kernel, dim3(grid), dim3(kThreads), 0, s, start, stop, 0, job, d_entry_d,
+                          d_entry_f, static_cast<unsigned long long*>(workspace));
+  } else {
+    viterbi_tiles_kernel<<<dim3(grid), dim3(kThreads), 0, s>>>(job, d_entry_d, d_entry_f,
+                                                               static_cast<unsigned long long*>(workspace));
+  }
   QTIP_HIP(hipGetLastError());
 }
 
