@@ -1,27 +1,37 @@
-// Randomised Hadamard transform pieces for gfx950: sign scaling + natural-order FWHT per power-of-two chunk,
-// the K-point Hadamard-factor mix, tiled transpose, and fixed-order fp64 reductions.
+// Randomised Hadamard transform pieces for gfx950: sign scaling + natural-order FWHT per power-of-two chunk + the
+// K-point Hadamard-factor mix in one kernel, tiled transpose, and fixed-order fp64 reductions.
 //
-// The fp32 operation order is the one of the reference's GPU path (src/kernels.hip:214-254, 293-313:
-// butterflies (a+b, a-b) for h = 1, 2, 4, ...; mix as a signed sum over k ascending from 0; one multiply by
-// 1/sqrt(n) at the end), so results match it bit for bit; only the scheduling differs: the sign scaling is
-// fused into the load, the first three butterfly stages run in registers on 8 consecutive values per lane,
-// and the remaining stages go through LDS.
+// The fp32 operation order is the one of the reference's GPU path (src/kernels.hip:214-254, 293-313: butterflies
+// (a+b, a-b) for h = 1, 2, 4, ...; mix as a signed sum over k ascending from 0; one multiply by 1/sqrt(n) at the
+// end), so results match it bit for bit.  The schedule is built for 64-wide waves and 160 KB of LDS:
+//   * a lane holds up to 16 consecutive values: the butterfly stages below that width run in registers, the next six
+//     stages exchange values between the lanes of the wave (a lane whose index bit is set adds its negated value to
+//     the partner's: a - b as a + (-b)), so a wave finishes a 1024-point transform without LDS or barriers;
+//   * the stages above 1024 (chunks of 2048..8192) run in registers again after one trip through LDS, on values
+//     1024 apart;
+//   * a row of up to 40000 values stays in LDS after its chunks are transformed and the K-point mix reads it from
+//     there, so the row is read from HBM once and written once; the Hadamard factor is a table of sign bits that
+//     flips the sign bit of a value before a plain add.  Longer rows take a second kernel for the mix.
+#include <mutex>
+
 #include "qtip_internal.hpp"
 #include "rht.hpp"
 
 namespace qtipmi {
 namespace {
 
-constexpr int kFwhtThreads = 256;
+constexpr int kRowThreads = 1024;     // 16 waves per row segment
+constexpr int kRowLdsFloats = 40000;  // 160 000 of the 163 840 bytes of LDS
+constexpr int kMixLanes = 64;
 
-// In-place FWHT of one chunk of P values held in LDS buffer v (P <= 8192), all threads of the block.
-// Stages h < 8 run in registers on 8 consecutive values; the rest through LDS.
-template <int EPT>
-__device__ __forceinline__ void fwht_registers(float (&r)[EPT]) {
+__device__ __forceinline__ float flip(float v, uint32_t sign_bit) { return __uint_as_float(__float_as_uint(v) ^ sign_bit); }
+
+template <int N>
+__device__ __forceinline__ void fwht_registers(float (&r)[N]) {
 #pragma unroll
-  for (int h = 1; h < EPT; h <<= 1)
+  for (int h = 1; h < N; h <<= 1)
 #pragma unroll
-    for (int i = 0; i < EPT; i += 2 * h)
+    for (int i = 0; i < N; i += 2 * h)
 #pragma unroll
       for (int j = i; j < i + h; ++j) {
         const float a = r[j], b = r[j + h];
@@ -30,112 +40,143 @@ __device__ __forceinline__ void fwht_registers(float (&r)[EPT]) {
       }
 }
 
-// grid: rows * K blocks; block b handles chunk (b % K) of row (b / K)
-__global__ __launch_bounds__(kFwhtThreads) void fwht_chunks_kernel(float* __restrict__ X, long ld, int P, int K,
-                                                                   float scale, const float* __restrict__ rs,
-                                                                   const float* __restrict__ cs, int vec) {
-  __shared__ float v[8192];
-  const long row = blockIdx.x / K;
-  const int chunk = blockIdx.x % K;
-  float* x = X + row * ld + long(chunk) * P;
+// One wave transforms spans of 64 * EPT consecutive values of the segment (stages h < min(P, 64 * EPT)) and leaves
+// them in v.  seg_len values at x, column sign factors at cs (or null), row factor rsv.
+template <int EPT>
+__device__ __forceinline__ void fwht_spans(const float* __restrict__ x, const float* __restrict__ cs, float rsv,
+                                           bool scaled, bool vec, int seg_len, int P, float* __restrict__ v) {
+  constexpr int S = 64 * EPT;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int hend = P < S ? P : S;
+  for (int base = wave * S + lane * EPT; base - lane * EPT < seg_len; base += (kRowThreads / 64) * S) {
+    float r[EPT];
+    if (EPT >= 4 && vec && base + EPT <= seg_len) {
+#pragma unroll
+      for (int e = 0; e < EPT; e += 4) {
+        const float4 q = *reinterpret_cast<const float4*>(x + base + e);
+        r[e] = q.x, r[e + 1] = q.y, r[e + 2] = q.z, r[e + 3] = q.w;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPT; ++e) r[e] = base + e < seg_len ? x[base + e] : 0.0f;
+    }
+    if (scaled) {
+#pragma unroll
+      for (int e = 0; e < EPT; ++e) {
+        r[e] *= rsv;
+        if (cs && base + e < seg_len) r[e] *= cs[base + e];
+      }
+    }
+    fwht_registers<EPT>(r);
+    for (int h = EPT; h < hend; h <<= 1) {
+      const int mask = h / EPT;
+      const uint32_t neg = (lane & mask) ? 0x80000000u : 0u;
+#pragma unroll
+      for (int e = 0; e < EPT; ++e) r[e] = __shfl_xor(r[e], mask, 64) + flip(r[e], neg);
+    }
+#pragma unroll
+    for (int e = 0; e < EPT; ++e)
+      if (base + e < seg_len) v[base + e] = r[e];
+  }
+}
+
+// Stages h = 1024 .. P/2 of every chunk in v: a thread takes the J = P / 1024 values that lie 1024 apart.
+template <int J>
+__device__ __forceinline__ void fwht_high(float* __restrict__ v, int seg_len) {
+  for (int q = threadIdx.x; q < seg_len / J; q += kRowThreads) {
+    float* p = v + (q >> 10) * (J * 1024) + (q & 1023);
+    float r[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) r[j] = p[j * 1024];
+    fwht_registers<J>(r);
+#pragma unroll
+    for (int j = 0; j < J; ++j) p[j * 1024] = r[j];
+  }
+}
+
+// bit k of row k2 of the table: entry (k2, k) of the mixing matrix is -1
+__device__ __forceinline__ uint32_t neg_bit(const uint32_t* __restrict__ row_bits, int k) {
+  return (row_bits[k >> 5] >> (k & 31)) << 31;
+}
+
+// One workgroup per segment of a row.  mix != 0 (the segment is the whole row, K > 1): out[k2 P + i] =
+// (sum_k +-v[k P + i]) * scale.  Otherwise the transformed values times scale go back in place.
+// KT: the factor size when it is one of the common ones (values in registers), 0 for any K (values re-read from LDS).
+template <int KT>
+__global__ __launch_bounds__(kRowThreads) void rht_rows_kernel(float* __restrict__ X, long ld, int n, int P, int K,
+                                                              int seg, int nseg, float scale,
+                                                              const float* __restrict__ rs,
+                                                              const float* __restrict__ cs,
+                                                              const uint32_t* __restrict__ neg, int mix) {
+  extern __shared__ float v[];
+  const long row = blockIdx.x / nseg;
+  const int col0 = int(blockIdx.x % nseg) * seg;
+  const int seg_len = n - col0 < seg ? n - col0 : seg;
+  float* x = X + row * ld + col0;
+  const bool vec = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0);
+  const bool scaled = rs != nullptr || cs != nullptr;
   const float rsv = rs ? rs[row] : 1.0f;
-  const int t = threadIdx.x;
-  if (vec) {  // P >= 8 and every chunk start is 16-byte aligned
-    // 8 consecutive values per thread and sweep; stages 1, 2, 4 in registers
-    for (int base = 8 * t; base < P; base += 8 * kFwhtThreads) {
-      float r[8];
-      const float4 lo = *reinterpret_cast<const float4*>(x + base);
-      const float4 hi = *reinterpret_cast<const float4*>(x + base + 4);
-      r[0] = lo.x, r[1] = lo.y, r[2] = lo.z, r[3] = lo.w, r[4] = hi.x, r[5] = hi.y, r[6] = hi.z, r[7] = hi.w;
-      if (rs) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) r[e] *= rsv;
-      }
-      if (cs) {
-        const float* c = cs + long(chunk) * P + base;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) r[e] *= c[e];
-      }
-      fwht_registers<8>(r);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[base + e] = r[e];
-    }
-    __syncthreads();
-    for (int h = 8; h < P; h <<= 1) {
-      for (int k = t; k < P / 2; k += kFwhtThreads) {
-        const int i = (k / h) * 2 * h + (k % h);
-        const float a = v[i], b = v[i + h];
-        v[i] = a + b;
-        v[i + h] = a - b;
-      }
-      __syncthreads();
-    }
-  } else {
-    for (int i = t; i < P; i += kFwhtThreads) {
-      float a = x[i];
-      if (rs) a *= rsv;
-      if (cs) a *= cs[long(chunk) * P + i];
-      v[i] = a;
-    }
-    __syncthreads();
-    for (int h = 1; h < P; h <<= 1) {
-      for (int k = t; k < P / 2; k += kFwhtThreads) {
-        const int i = (k / h) * 2 * h + (k % h);
-        const float a = v[i], b = v[i + h];
-        v[i] = a + b;
-        v[i + h] = a - b;
-      }
-      __syncthreads();
-    }
-  }
-  if (scale != 1.0f) {
-    for (int i = t; i < P; i += kFwhtThreads) x[i] = v[i] * scale;
-  } else {
-    for (int i = t; i < P; i += kFwhtThreads) x[i] = v[i];
-  }
-}
-
-// y[k2*P + i] = (sum_k sign[k2][k] * y[k*P + i]) * scale, one thread per (row, i)
-template <int K>
-__global__ __launch_bounds__(256) void had_mix_kernel(float* __restrict__ X, long rows, int P, long ld,
-                                                      const int8_t* __restrict__ had, float scale) {
-  __shared__ int8_t hs[K * K];
-  for (int i = threadIdx.x; i < K * K; i += blockDim.x) hs[i] = had[i];
+  const float* c = cs ? cs + col0 : nullptr;
+  if (P >= 1024) fwht_spans<16>(x, c, rsv, scaled, vec, seg_len, P, v);
+  else if (P == 512) fwht_spans<8>(x, c, rsv, scaled, vec, seg_len, P, v);
+  else if (P == 256) fwht_spans<4>(x, c, rsv, scaled, vec, seg_len, P, v);
+  else if (P == 128) fwht_spans<2>(x, c, rsv, scaled, false, seg_len, P, v);
+  else fwht_spans<1>(x, c, rsv, scaled, false, seg_len, P, v);
   __syncthreads();
-  const long idx = long(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (idx >= rows * P) return;
-  const long row = idx / P;
-  const int i = int(idx % P);
-  float* x = X + row * ld + i;
-  float y[K];
+  if (P > 1024) {
+    if (P == 2048) fwht_high<2>(v, seg_len);
+    else if (P == 4096) fwht_high<4>(v, seg_len);
+    else fwht_high<8>(v, seg_len);
+    __syncthreads();
+  }
+  if (!mix) {
+    for (int i = threadIdx.x; i < seg_len; i += kRowThreads) x[i] = v[i] * scale;
+    return;
+  }
+  // P <= 1024 here would leave threads idle: the outputs k2 of one i are shared out over kRowThreads / P threads
+  const int W = (K + 31) >> 5;
+  const int per = P < kRowThreads ? kRowThreads / P : 1;
+  for (int i = int(threadIdx.x) % (P < kRowThreads ? P : kRowThreads); i < P; i += kRowThreads) {
+    const int first = P < kRowThreads ? int(threadIdx.x) / P : 0;
+    if constexpr (KT > 0) {
+      float y[KT];
 #pragma unroll
-  for (int k = 0; k < K; ++k) y[k] = x[long(k) * P];
+      for (int k = 0; k < KT; ++k) y[k] = v[k * P + i];
+      for (int k2 = first; k2 < KT; k2 += per) {
+        const uint32_t* bits = neg + k2 * W;
+        float s = 0.0f;
 #pragma unroll
-  for (int k2 = 0; k2 < K; ++k2) {
-    float s = 0.0f;
-#pragma unroll
-    for (int k = 0; k < K; ++k) s += hs[k2 * K + k] > 0 ? y[k] : -y[k];
-    x[long(k2) * P] = s * scale;
+        for (int k = 0; k < KT; ++k) s += flip(y[k], neg_bit(bits, k));
+        x[long(k2) * P + i] = s * scale;
+      }
+    } else {
+      for (int k2 = first; k2 < K; k2 += per) {
+        const uint32_t* bits = neg + k2 * W;
+        float s = 0.0f;
+        for (int k = 0; k < K; ++k) s += flip(v[k * P + i], neg_bit(bits, k));
+        x[long(k2) * P + i] = s * scale;
+      }
+    }
   }
 }
 
-// any K: the K inputs of a thread are parked in a global scratch column
-__global__ __launch_bounds__(256) void had_mix_generic_kernel(float* __restrict__ X, long rows, int P, int K, long ld,
-                                                              const int8_t* __restrict__ had, float scale,
-                                                              float* __restrict__ tmp) {
-  const long idx = long(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (idx >= rows * P) return;
-  const long row = idx / P;
-  const int i = int(idx % P);
+// The mix for rows too long for LDS, in place on transformed chunks: one wave per 64 values of i, the K inputs of a
+// lane parked in LDS (ys[k][lane]) because the outputs overwrite them.
+__global__ __launch_bounds__(kMixLanes) void had_mix_long_rows_kernel(float* __restrict__ X, long ld, int P, int K,
+                                                                     float scale, const uint32_t* __restrict__ neg) {
+  extern __shared__ float ys[];
+  const int per_row = (P + kMixLanes - 1) / kMixLanes;
+  const long row = blockIdx.x / per_row;
+  const int i = int(blockIdx.x % per_row) * kMixLanes + int(threadIdx.x);
+  if (i >= P) return;  // the only wave of the workgroup: no barrier is skipped
   float* x = X + row * ld + i;
-  const long total = rows * P;
-  for (int k = 0; k < K; ++k) tmp[long(k) * total + idx] = x[long(k) * P];
+  float* mine = ys + threadIdx.x;
+  for (int k = 0; k < K; ++k) mine[k * kMixLanes] = x[long(k) * P];
+  const int W = (K + 31) >> 5;
   for (int k2 = 0; k2 < K; ++k2) {
+    const uint32_t* bits = neg + k2 * W;
     float s = 0.0f;
-    for (int k = 0; k < K; ++k) {
-      const float t = tmp[long(k) * total + idx];
-      s += had[k2 * K + k] > 0 ? t : -t;
-    }
+    for (int k = 0; k < K; ++k) s += flip(mine[k * kMixLanes], neg_bit(bits, k));
     x[long(k2) * P] = s * scale;
   }
 }
@@ -223,16 +264,50 @@ void Rht::init(int device, hipStream_t stream) {
   partial_.alloc(kRedBlocks + 1);
 }
 
-const int8_t* Rht::device_had(int K, bool transpose) {
+// sign bits of the mixing matrix (hadK, or its transpose), row k2 in (K + 31) / 32 words: bit k set = entry -1
+const uint32_t* Rht::device_had(int K, bool transpose) {
   const int key = K * 2 + (transpose ? 1 : 0);
   for (auto& e : had_) if (e.first == key) return e.second->p;
-  auto m = had_matrix(K, transpose);
-  auto buf = std::make_unique<DBuf<int8_t>>(m.size());
-  QTIP_HIP(hipMemcpyAsync(buf->p, m.data(), m.size(), hipMemcpyHostToDevice, s_));
+  const auto m = had_matrix(K, transpose);
+  const int W = (K + 31) / 32;
+  std::vector<uint32_t> bits(size_t(K) * W, 0u);
+  for (int r = 0; r < K; ++r)
+    for (int k = 0; k < K; ++k)
+      if (m[size_t(r) * K + k] < 0) bits[size_t(r) * W + (k >> 5)] |= 1u << (k & 31);
+  auto buf = std::make_unique<DBuf<uint32_t>>(bits.size());
+  QTIP_HIP(hipMemcpyAsync(buf->p, bits.data(), bits.size() * sizeof(uint32_t), hipMemcpyHostToDevice, s_));
   QTIP_HIP(hipStreamSynchronize(s_));
   had_.emplace_back(key, std::move(buf));
   return had_.back().second->p;
 }
+
+namespace {
+using RowKernel = void (*)(float*, long, int, int, int, int, int, float, const float*, const float*, const uint32_t*,
+                           int);
+RowKernel row_kernel(int K) {
+  switch (K) {
+    case 12: return rht_rows_kernel<12>;
+    case 20: return rht_rows_kernel<20>;
+    case 28: return rht_rows_kernel<28>;
+    case 36: return rht_rows_kernel<36>;
+    default: return rht_rows_kernel<0>;
+  }
+}
+// the row kernels may use all of the LDS; told to the runtime once per device
+void allow_full_lds() {
+  static std::mutex mu;
+  static std::vector<bool> configured;
+  int dev = 0;
+  QTIP_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lk(mu);
+  if (configured.size() <= size_t(dev)) configured.resize(size_t(dev) + 1, false);
+  if (configured[size_t(dev)]) return;
+  for (int K : {0, 12, 20, 28, 36})
+    QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(row_kernel(K)),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, kRowLdsFloats * int(sizeof(float))));
+  configured[size_t(dev)] = true;
+}
+}  // namespace
 
 void Rht::hadamard_rows(float* X, long rows, int n, long ld, bool transpose, const float* rs, const float* cs) {
   const int K = had_K(n);
@@ -241,28 +316,27 @@ void Rht::hadamard_rows(float* X, long rows, int n, long ld, bool transpose, con
   QTIP_REQUIRE(P <= 8192, "hadamard pow2 part %d > 8192 unsupported", P);
   QTIP_REQUIRE(ld >= n, "hadamard: ld %ld < n %d", ld, n);
   if (rows <= 0) return;
+  allow_full_lds();
   const float sc = 1.0f / std::sqrt(float(n));
-  QTIP_REQUIRE(rows * K < (1L << 31), "hadamard: too many chunks");
-  const int vec = (P >= 8 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(X) & 15u) == 0) ? 1 : 0;
-  fwht_chunks_kernel<<<dim3(unsigned(rows * K)), dim3(kFwhtThreads), 0, s_>>>(X, ld, P, K, K == 1 ? sc : 1.0f, rs, cs,
-                                                                               vec);
+  const uint32_t* neg = K > 1 ? device_had(K, transpose) : nullptr;
+  // a row that fits in LDS is transformed and mixed in one pass; a longer one goes chunk group by chunk group and is
+  // mixed by a second kernel
+  const bool whole = n <= kRowLdsFloats;
+  const int seg = whole ? n : kRowLdsFloats / P * P;
+  const int nseg = (n + seg - 1) / seg;
+  QTIP_REQUIRE(rows * nseg < (1L << 31), "hadamard: too many rows");
+  const int mix = whole && K > 1;
+  const float first_scale = (K == 1) ? sc : (mix ? sc : 1.0f);
+  row_kernel(K)<<<dim3(unsigned(rows * nseg)), dim3(kRowThreads), size_t(seg) * sizeof(float), s_>>>(
+      X, ld, n, P, K, seg, nseg, first_scale, rs, cs, neg, mix);
   QTIP_HIP(hipGetLastError());
-  if (K == 1) return;
-  const int8_t* had = device_had(K, transpose);
-  const unsigned nb = unsigned((rows * P + 255) / 256);
-  switch (K) {
-    case 12: had_mix_kernel<12><<<nb, 256, 0, s_>>>(X, rows, P, ld, had, sc); break;
-    case 20: had_mix_kernel<20><<<nb, 256, 0, s_>>>(X, rows, P, ld, had, sc); break;
-    case 28: had_mix_kernel<28><<<nb, 256, 0, s_>>>(X, rows, P, ld, had, sc); break;
-    case 36: had_mix_kernel<36><<<nb, 256, 0, s_>>>(X, rows, P, ld, had, sc); break;
-    default: {
-      DBuf<float> tmp(size_t(rows) * P * K);
-      had_mix_generic_kernel<<<nb, 256, 0, s_>>>(X, rows, P, K, ld, had, sc, tmp);
-      QTIP_HIP(hipGetLastError());
-      QTIP_HIP(hipStreamSynchronize(s_));  // tmp is released on return
-    }
+  if (K > 1 && !mix) {
+    const long per_row = (P + kMixLanes - 1) / kMixLanes;
+    QTIP_REQUIRE(rows * per_row < (1L << 31), "hadamard: too many rows");
+    had_mix_long_rows_kernel<<<dim3(unsigned(rows * per_row)), dim3(kMixLanes), size_t(K) * kMixLanes * sizeof(float),
+                               s_>>>(X, ld, P, K, sc, neg);
+    QTIP_HIP(hipGetLastError());
   }
-  QTIP_HIP(hipGetLastError());
 }
 
 void Rht::transpose(const float* in, long rows, long cols, long ld_in, float* out, long ld_out) {

@@ -22,11 +22,11 @@ class Rht {
   double reduce(const float* A, long lda, const float* B, long ldb, long rows, long cols, int mode);
 
  private:
-  const int8_t* device_had(int K, bool transpose);
+  const uint32_t* device_had(int K, bool transpose);
   int dev_ = 0;
   hipStream_t s_ = nullptr;
   DBuf<double> partial_;
-  std::vector<std::pair<int, std::unique_ptr<DBuf<int8_t>>>> had_;
+  std::vector<std::pair<int, std::unique_ptr<DBuf<uint32_t>>>> had_;
 };
 
 }  // namespace qtipmi

@@ -135,6 +135,17 @@ def ref_ldlq(Wr, L):
     return hat, Q
 
 
+def ref_gpu_hadamard_rows(X, n, transpose):
+    """k_hadamard_rows of the reference on the GPU (src/kernels.hip:293-313); X is rows x ld, returned transformed."""
+    R = ref_gpu_lib()
+    X = np.ascontiguousarray(X, np.float32).copy()
+    rows, ld = X.shape
+    R.ref_gpu_hadamard_rows.argtypes = [C.c_void_p, C.c_long, C.c_int, C.c_long, C.c_int]
+    R.ref_gpu_hadamard_rows.restype = None
+    R.ref_gpu_hadamard_rows(X.ctypes.data, rows, n, ld, int(transpose))
+    return X
+
+
 def ref_gpu_quantize_seqs(X):
     """The reference's device Viterbi, both passes (tests/test_gpu.cpp:67-88) -> (states [B][128], seconds)."""
     R = ref_gpu_lib()

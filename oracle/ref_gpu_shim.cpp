@@ -7,6 +7,7 @@
 //   ref_gpu_quantize_group        quantize_group, src/quantizer.cpp:340-348 (src/quantizer.hpp:72-74)
 //   ref_gpu_quantize_seqs         the two-pass tail-biting Viterbi as the test drives it, tests/test_gpu.cpp:67-88
 //   ref_gpu_nvfp4_quantize_group  nvfp4_quantize_group, src/nvfp4_gpu.hip:174-243
+//   ref_gpu_hadamard_rows         k_hadamard_rows, src/kernels.hip:293-313 (src/gpu.hpp:232)
 #define main ref_test_gpu_main
 #include "test_gpu.cpp"
 #undef main
@@ -27,6 +28,19 @@ void ref_ldlq(const float* Wr, const float* L, int m, int n, float* hatWr, uint1
   ldlq_ref(w, l, m, n, h, q);
   std::memcpy(hatWr, h.data(), h.size() * 4);
   std::memcpy(Q, q.data(), q.size() * 2);
+}
+
+// X: rows x ld fp32 on the host, transformed in place on the device (rows of length n)
+void ref_gpu_hadamard_rows(float* X, long rows, int n, long ld, int transpose) {
+  ensure_stream();
+  float* d = nullptr;
+  const size_t bytes = size_t(rows) * size_t(ld) * sizeof(float);
+  HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d), bytes));
+  HIP_CHECK(hipMemcpy(d, X, bytes, hipMemcpyHostToDevice));
+  k_hadamard_rows(d, rows, n, ld, transpose != 0, S);
+  HIP_CHECK(hipStreamSynchronize(S));
+  HIP_CHECK(hipMemcpy(X, d, bytes, hipMemcpyDeviceToHost));
+  HIP_CHECK(hipFree(d));
 }
 
 // B sequences of 256 fp32 -> states [B][128]; returns the seconds the reference's own timer measured

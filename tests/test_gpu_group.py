@@ -24,7 +24,7 @@ def synth(pkg):
     return mod
 
 
-@pytest.mark.parametrize("n", [64, 96, 80, 448, 1024, 2304, 8192, 12288, 28672])
+@pytest.mark.parametrize("n", [12, 64, 96, 80, 448, 864, 1024, 2304, 3328, 4096, 8192, 12288, 28672, 49152, 53248, 57344])
 def test_hadamard_rows(qz, oracle, n):
     """Bit-identical to the fp32 dataflow of the reference's kernels (restated on the CPU) and within 2e-5 of the
     fp64 definition (tests/test_gpu.cpp:27-50); strided rows keep their padding."""

@@ -33,6 +33,25 @@ def ref(oracle):
     return oracle
 
 
+@pytest.mark.parametrize("n", [96, 448, 1024, 2304, 8192, 12288, 28672, 57344])
+def test_hadamard_equals_reference_device_kernels(qz, ref, n):
+    """k_hadamard_rows of the reference (src/kernels.hip:293-313) on the same strided rows: this library's kernel and
+    the CPU restatement of the fp32 dataflow (qo_hadamard_rows_f32) both equal it bit for bit, padding included."""
+    import torch
+    say("case: hadamard vs reference device kernels n=%d" % n)
+    rows, ld = 5, n + 16
+    x = ref.rng_normal(1000 + n, rows * ld).astype(np.float32).reshape(rows, ld)
+    for tr in (0, 1):
+        want = ref.ref_gpu_hadamard_rows(x, n, tr)
+        d = torch.from_numpy(x.copy()).cuda()
+        qz.hadamard_rows_dev(d, rows, n, ld, tr)
+        qz.synchronize()
+        assert np.array_equal(d.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        cpu = x.copy().reshape(-1)
+        assert ref.lib().qo_hadamard_rows_f32(cpu, rows, n, ld, tr) == 0
+        assert np.array_equal(cpu.reshape(rows, ld).view(np.uint32), want.view(np.uint32))
+
+
 def test_viterbi_equals_reference_device_viterbi(qz, ref):
     """fp16-representable inputs, as LDLQ feeds the Viterbi (the reference's kernel rounds its input to fp16 and scores in
     fp32 with the low mantissa bits reused as a tag; this library scores in fp64 like the reference's CPU code)."""

@@ -101,6 +101,21 @@ def test_hadamard_golden(oracle, n):
         assert np.max(np.abs(y32 - ref)) < 2e-5        # tolerance of tests/test_gpu.cpp:61 for the fp32 dataflow
 
 
+def test_hadamard_f32_equals_the_reference_device_kernels(oracle):
+    """The fp32 dataflow against rows the reference's own device kernels transformed on a gfx950 GPU
+    (k_hadamard_rows, src/kernels.hip:293-313; tests/golden/make_ref_hadamard_gpu_vectors.py): bit for bit."""
+    cases = json.load(open(os.path.join(GOLDEN, "ref_hadamard_gpu.json")))["cases"]
+    blob = np.fromfile(os.path.join(GOLDEN, "ref_hadamard_gpu.bin"), np.uint32)
+    at = 0
+    for n, rows, tr, seed in cases:
+        want = blob[at:at + rows * n]
+        at += rows * n
+        x = oracle.rng_normal(seed, rows * n).astype(np.float32)
+        assert oracle.lib().qo_hadamard_rows_f32(x, rows, n, n, tr) == 0
+        assert np.array_equal(x.view(np.uint32), want), (n, tr)
+    assert at == blob.size
+
+
 def _had_tables():
     import re
     src = open(os.path.join(os.path.dirname(REFVEC), "..", "..", "behemoth-qtip_amd", "csrc", "data",
