@@ -1,57 +1,17 @@
-// LDLQ kernels for gfx950 (reference: ldlq_gpu, src/quantizer.cpp:30-89; ldlq_prep_kernel,
-// src/viterbi.hip:241-267; the CPU form of the algorithm, tests/test_gpu.cpp:180-225).
+// Cross-buffer feedback of LDLQ for gfx950 (reference: ldlq_gpu, src/quantizer.cpp:30-89; the CPU form of the
+// algorithm, tests/test_gpu.cpp:180-225).  The in-buffer feedback of a 16-column block is formed inside the Viterbi
+// kernel (viterbi.hip, tile_targets).
 //
-//  * ldlq_prep: in-buffer error feedback for one 16-column block; one thread per weight row keeps the 16
-//    column targets in registers, the <= 112 rows of L of the open buffer sit in LDS.  fp64 accumulation (the
-//    CPU algorithm's precision: fp64 is full rate on CDNA4 VALUs), result rounded fp64 -> fp32 -> fp16 like
-//    the CPU path and written in trellis sequence order.
 //  * gemm_tn: sum_k A[k][i] * (B1 - B2)[k][j] on the fp64 matrix cores (v_mfma_f64_16x16x4_f64), fp32 operands
 //    widened while staging through LDS.  The cross-buffer feedback ("prod cache") of a 128-column buffer is gathered
 //    from all rows quantized so far by a K-split kernel.
 //  * gemm_tn_bf16x3: the same prod-cache update with fp32 C and the operands split into bf16 hi + lo
 //    (v_mfma_f32_32x32x16_bf16, three terms), the arithmetic of the reference's GPU path.
-#include <hip/hip_fp16.h>
-
 #include "ldlq.hpp"
 #include "qtip_internal.hpp"
 
 namespace qtipmi {
 namespace {
-
-__device__ __forceinline__ int perm_inv(int q) {  // tile index 16*r + c -> sequence position
-  const int a = q >> 7, b = (q >> 4) & 7, c = (q >> 3) & 1, d = (q >> 1) & 3, e = q & 1;
-  return (((b * 4 + d) * 2 + c) * 2 + a) * 2 + e;
-}
-
-template <typename ProdT>
-__global__ __launch_bounds__(256) void ldlq_prep_kernel(const float* __restrict__ WT, const float* __restrict__ hatWT,
-                                                        const ProdT* __restrict__ prod, const float* __restrict__ L,
-                                                        long n, long m, int col0, int bufend, int prod_row0,
-                                                        float* __restrict__ X) {
-  __shared__ ProdT Ls[112][16];
-  const int k0 = col0 + 16, nk = bufend - k0;
-  for (int idx = threadIdx.x; idx < nk * 16; idx += blockDim.x) {
-    const int kk = idx >> 4, c = idx & 15;
-    Ls[kk][c] = ProdT(L[long(k0 + kk) * n + col0 + c]);
-  }
-  __syncthreads();
-  const long j = long(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (j >= m) return;
-  ProdT acc[16];
-#pragma unroll
-  for (int c = 0; c < 16; ++c) acc[c] = ProdT(WT[long(col0 + c) * m + j]) + prod[long(col0 + c - prod_row0) * m + j];
-  for (int kk = 0; kk < nk; ++kk) {
-    const long o = long(k0 + kk) * m + j;
-    const ProdT dk = ProdT(WT[o]) - ProdT(hatWT[o]);
-#pragma unroll
-    for (int c = 0; c < 16; ++c) acc[c] += Ls[kk][c] * dk;
-  }
-  const long bt = j >> 4;
-  const int r = int(j & 15);
-  float* xb = X + bt * 256;
-#pragma unroll
-  for (int c = 0; c < 16; ++c) xb[perm_inv(r * 16 + c)] = __half2float(__float2half_rn(float(acc[c])));
-}
 
 // ---------------------------------------------------------------- fp64 MFMA GEMM
 typedef double double4_t __attribute__((ext_vector_type(4)));
@@ -258,22 +218,6 @@ __global__ __launch_bounds__(256) void gemm_tn_bf16x3_kernel(int M, int N, const
 }
 
 }  // namespace
-
-void launch_ldlq_prep_f64(const float* WT, const float* hatWT, const double* prod, int prod_row0, const float* L, long n,
-                          long m, int col0, int bufend, float* X, hipStream_t s) {
-  QTIP_REQUIRE(bufend - col0 - 16 <= 112 && bufend - col0 - 16 >= 0, "ldlq_prep: block outside its buffer");
-  QTIP_REQUIRE(col0 >= prod_row0, "ldlq_prep: block outside the prod slab");
-  ldlq_prep_kernel<double><<<dim3(unsigned((m + 255) / 256)), dim3(256), 0, s>>>(WT, hatWT, prod, L, n, m, col0,
-                                                                                 bufend, prod_row0, X);
-  QTIP_HIP(hipGetLastError());
-}
-void launch_ldlq_prep_f32(const float* WT, const float* hatWT, const float* prod, const float* L, long n, long m,
-                          int col0, int bufend, float* X, hipStream_t s) {
-  QTIP_REQUIRE(bufend - col0 - 16 <= 112 && bufend - col0 - 16 >= 0, "ldlq_prep: block outside its buffer");
-  ldlq_prep_kernel<float><<<dim3(unsigned((m + 255) / 256)), dim3(256), 0, s>>>(WT, hatWT, prod, L, n, m, col0,
-                                                                                bufend, 0, X);
-  QTIP_HIP(hipGetLastError());
-}
 
 int gemm_splitk_splits(long K) {
   // 96 column tiles x 5 splits keep every CU's two workgroup slots busy at m = 12288; short K ranges are not split

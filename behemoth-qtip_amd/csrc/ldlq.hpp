@@ -1,11 +1,6 @@
 #pragma once
 #include "qtip_internal.hpp"
 namespace qtipmi {
-// prod holds the cross-buffer feedback of rows prod_row0 .. (the whole matrix: 0; one 128-row slab: its first column)
-void launch_ldlq_prep_f64(const float* WT, const float* hatWT, const double* prod, int prod_row0, const float* L, long n,
-                          long m, int col0, int bufend, float* X, hipStream_t s);
-void launch_ldlq_prep_f32(const float* WT, const float* hatWT, const float* prod, const float* L, long n, long m,
-                          int col0, int bufend, float* X, hipStream_t s);
 // P[128][N] = sum_{k < K} A[k][i] * (B1 - B2)[k][j] (fp64 MFMA, K split over workgroups, partial tiles summed in a
 // fixed order); partials: gemm_splitk_splits(K) x 128 x N doubles of scratch
 int gemm_splitk_splits(long K);

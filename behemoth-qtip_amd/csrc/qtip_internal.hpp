@@ -147,9 +147,21 @@ size_t st_write(const qtip_st_writer* w, const char* path, const char* const* me
 
 // ---- GPU launchers (viterbi.hip, rht.hip, ldlq.hip)
 struct TileJob {
-  // inputs: either X (tiles x 256 fp32, sequence order) or the LDLQ feedback operands
+  // inputs: either X (tiles x 256 fp32, sequence order) or the LDLQ feedback operands below
   const float* X = nullptr;
   long tiles = 0;
+  // LDLQ feedback (X null): tile t covers weight rows 16 t .. 16 t + 15 and the columns col0 .. col0 + 15; the
+  // target of (row j, column col0 + c) is
+  //   WT[(col0 + c) * ldw + j] + prod[(col0 + c - prod_row0) * ldw + j]
+  //     + sum over k = col0 + 16 .. bufend - 1 (ascending) of L[k * ldl + col0 + c] * (WT - hatWT)[k * ldw + j],
+  // accumulated in the type of prod (prod64 or prod32, whichever is set) and rounded to fp32, then to fp16.
+  const float* WT = nullptr;
+  const float* L = nullptr;
+  long ldl = 0;
+  int bufend = 0;
+  const double* prod64 = nullptr;
+  const float* prod32 = nullptr;
+  long prod_row0 = 0;
   // outputs (any may be null)
   uint16_t* states = nullptr;  // state words of tile t at states[(t * q_tile_stride + q_offset) * 128]
   long q_tile_stride = 1, q_offset = 0;

@@ -94,7 +94,6 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   // bf16 hi/lo split MFMA product
   DBuf<double> prod(feedback == 0 ? size_t(128) * m : 0), parts(feedback == 0 ? size_t(5) * 128 * m : 0);
   DBuf<float> prod32(feedback == 1 ? size_t(n) * m : 0);
-  DBuf<float> X(size_t(ntr) * 256);
   if (feedback == 1) QTIP_HIP(hipMemsetAsync(prod32, 0, prod32.bytes(), s));
   QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
   Events timed, pacing;  // timed: a (start, stop) pair per Viterbi launch, stamped by the launch itself
@@ -115,13 +114,16 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
       else
         QTIP_HIP(hipMemsetAsync(prod, 0, prod.bytes(), s));
     }
-    for (int i = 7; i >= 0; --i) {
+    for (int i = 7; i >= 0; --i) {  // the kernel forms the block's targets (in-buffer feedback) itself
       const int col0 = c0 + 16 * i;
-      if (feedback == 0) launch_ldlq_prep_f64(WT, hatWT, prod, c0, L, n, m, col0, bufend, X, s);
-      else launch_ldlq_prep_f32(WT, hatWT, prod32, L, n, m, col0, bufend, X, s);
       TileJob job;
-      job.X = X;
       job.tiles = ntr;
+      job.WT = WT;
+      job.L = L;
+      job.ldl = n;
+      job.bufend = bufend;
+      if (feedback == 0) job.prod64 = prod, job.prod_row0 = c0;
+      else job.prod32 = prod32;
       job.states = Q;
       job.q_tile_stride = nblk;
       job.q_offset = col0 / 16;

@@ -279,6 +279,33 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
   __syncthreads();
 }
 
+// The Viterbi input of one tile inside LDLQ: W plus the error feedback of the columns already quantized (the formula
+// at TileJob), which the reference computes in a kernel of its own (ldlq_prep_kernel, src/viterbi.hip:241-267; CPU
+// form tests/test_gpu.cpp:196-207).  The (<= 112) x 16 blocks of L, WT and hatWT the tile needs are staged in the
+// metric array, which is idle between tiles; thread u then owns the sequence position u.
+template <typename Acc>
+__device__ __forceinline__ void tile_targets(Smem& sm, const TileJob& job, long tile, const Acc* __restrict__ prod) {
+  const int u = threadIdx.x;
+  const int k0 = int(job.col0) + 16, nk = job.bufend - k0;
+  float* Ls = reinterpret_cast<float*>(sm.M);
+  float* Ws = Ls + 112 * 16;
+  float* Hs = Ws + 112 * 16;
+  const long row0 = tile * 16;
+  for (int idx = u; idx < nk * 16; idx += kThreads) {
+    const long k = k0 + (idx >> 4);
+    const int e = idx & 15;
+    Ls[idx] = job.L[k * job.ldl + job.col0 + e];
+    Ws[idx] = job.WT[k * job.ldw + row0 + e];
+    Hs[idx] = job.hatWT[k * job.ldw + row0 + e];
+  }
+  __syncthreads();
+  const int q = perm_fwd(u), r = q >> 4, c = q & 15;
+  const long col = job.col0 + c;
+  Acc acc = Acc(job.WT[col * job.ldw + row0 + r]) + prod[(col - job.prod_row0) * job.ldw + row0 + r];
+  for (int kk = 0; kk < nk; ++kk) acc += Acc(Ls[kk * 16 + c]) * (Acc(Ws[kk * 16 + r]) - Acc(Hs[kk * 16 + r]));
+  sm.x[u] = float(_Float16(float(acc)));
+}
+
 __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job, const double* __restrict__ entry_d,
                                                                  const float* __restrict__ entry_f,
                                                                  unsigned long long* __restrict__ bp_all) {
@@ -286,7 +313,9 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
   const int u = threadIdx.x;
   unsigned long long* bp = bp_all + size_t(blockIdx.x) * kBpWordsPerTile;
   for (long tile = blockIdx.x; tile < job.tiles; tile += gridDim.x) {
-    sm.x[u] = job.X[tile * kSeq + u];
+    if (job.X) sm.x[u] = job.X[tile * kSeq + u];
+    else if (job.prod64) tile_targets<double>(sm, job, tile, job.prod64);
+    else tile_targets<float>(sm, job, tile, job.prod32);
     __syncthreads();
     // pass 1 on the sequence rotated by half its length, free ends; only steps 64..126 are traced back
     forward_pass(sm, entry_d, 128, -1, bp, 64);
@@ -360,7 +389,15 @@ int viterbi_max_slots(int device) {
 void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const float* d_entry_f, void* workspace,
                           int slots, hipStream_t s, hipEvent_t start, hipEvent_t stop) {
   if (job.tiles <= 0) return;
-  QTIP_REQUIRE(job.X != nullptr && slots > 0 && workspace != nullptr, "viterbi: missing operand");
+  QTIP_REQUIRE(slots > 0 && workspace != nullptr, "viterbi: missing workspace");
+  if (!job.X) {  // LDLQ block: the targets come from the feedback operands
+    QTIP_REQUIRE(job.WT && job.L && job.hatWT && ((job.prod64 != nullptr) != (job.prod32 != nullptr)),
+                 "viterbi: neither inputs nor complete LDLQ feedback operands");
+    const long nk = job.bufend - job.col0 - 16;
+    QTIP_REQUIRE(job.col0 >= 0 && nk >= 0 && nk <= 112, "viterbi: column block outside its 128-column buffer");
+    QTIP_REQUIRE(job.col0 >= job.prod_row0 && job.ldw >= 16 * job.tiles && job.ldl >= job.bufend,
+                 "viterbi: LDLQ operand geometry");
+  }
   const unsigned grid = unsigned(job.tiles < slots ? job.tiles : slots);
   if (start || stop) {
     // the runtime stamps the two events at the kernel's own start and end: the time between them is the kernel's,
