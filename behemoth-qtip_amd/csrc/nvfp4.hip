@@ -62,81 +62,73 @@ __device__ __forceinline__ int nv_fp4_code(float a) {
   return code;
 }
 
-constexpr int kCand = 11;
+constexpr int kCand = 11;       // scale candidates of the search: the plain one, 8 shrink factors, one code down, one up
+constexpr int kBlockRows = 64;  // matrix rows per workgroup: one per lane
 
-// One thread per matrix row, one 16-column block (columns c0 .. c0 + 15) per launch.
-//   t_k  = W[k] + F[k] + sum_{j > k in block} d_j Lb[j][k]   target after the feedback
+// Block scale candidate number `which` (uniform over a wave) of a row whose 16 targets have the largest magnitude
+// amax; the list and its order are the reference's (src/nvfp4_gpu.hip:97-105).
+__device__ __forceinline__ unsigned nv_candidate(int which, float amax, float global) {
+  if (which >= 1 && which <= 8) {
+    float shrink = 1.05f;
+    switch (which) {
+      case 1: shrink = 0.70f; break;
+      case 2: shrink = 0.75f; break;
+      case 3: shrink = 0.80f; break;
+      case 4: shrink = 0.85f; break;
+      case 5: shrink = 0.90f; break;
+      case 6: shrink = 0.95f; break;
+      case 7: shrink = 1.00f; break;
+      default: break;
+    }
+    return nv_fp8_enc(amax * shrink / (6.f * global));
+  }
+  const unsigned plain = nv_fp8_enc(amax / (6.f * global));
+  if (which == 9) return plain > 0 ? plain - 1 : 0;
+  if (which == 10) return plain < 126 ? plain + 1 : 126;
+  return plain;
+}
+
+// One 16-column block (columns c0 .. c0 + 15) per launch, 64 matrix rows per workgroup, and one wave per scale
+// candidate: the reference's thread walks through its row's candidates one after the other and then rounds once more
+// with the winner (src/nvfp4_gpu.hip:66-158); here the ncand waves of a workgroup round the same 64 rows at the same
+// time, each under its own candidate, leave their costs in LDS, and the wave whose candidate wins a row (smallest cost,
+// the earliest candidate among equals) writes that row's result.  With s the candidate's scale:
+//   t_k  = W[k] + F[k] + sum_{j > k in block} d_j Lb[j][k]   target after the feedback, j ascending
 //   q_k  = bf16(level * dec(s) * global)                       what execution sees
 //   d_k  = W[k] - q_k                                          error fed back
-//   cost = sum_k dw[k] (t_k - q_k)^2                           proxy increment
+//   cost = sum_k dw[k] (t_k - q_k)^2                           proxy increment, k descending
 // WT, FT: [n][m].  packedT: [n/2][m], scalesT: [n/16][m], E: [16][m].
-__global__ __launch_bounds__(256) void nv_block_kernel(const float* __restrict__ WT, const float* __restrict__ FT, long m,
-                                                       long n, long c0, const float* __restrict__ L,
-                                                       const float* __restrict__ dw, float global, int calibrate,
-                                                       int search, uint8_t* __restrict__ packedT,
-                                                       uint8_t* __restrict__ scalesT, float* __restrict__ E) {
+__global__ __launch_bounds__(kBlockRows * kCand) void nv_block_kernel(
+    const float* __restrict__ WT, const float* __restrict__ FT, long m, long n, long c0, const float* __restrict__ L,
+    const float* __restrict__ dw, float global, int calibrate, int ncand, uint8_t* __restrict__ packedT,
+    uint8_t* __restrict__ scalesT, float* __restrict__ E) {
   __shared__ float Lb[16][16];
   __shared__ float Dw[16];
-  {
-    const int idx = threadIdx.x;
-    Lb[idx / 16][idx % 16] = calibrate ? L[(c0 + idx / 16) * n + c0 + idx % 16] : 0.f;
-    if (idx < 16) Dw[idx] = dw ? dw[c0 + idx] : 1.f;
-  }
+  __shared__ float costs[kCand][kBlockRows];
+  const int lane = threadIdx.x & 63;
+  const int which = __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6));
+  for (int idx = threadIdx.x; idx < 256; idx += blockDim.x)
+    Lb[idx >> 4][idx & 15] = calibrate ? L[(c0 + (idx >> 4)) * n + c0 + (idx & 15)] : 0.f;
+  if (threadIdx.x < 16) Dw[threadIdx.x] = dw ? dw[c0 + threadIdx.x] : 1.f;
   __syncthreads();
-  const long r = long(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (r >= m) return;
-  float w[16], base[16];
-  float amax = 0;
+  const long r = long(blockIdx.x) * kBlockRows + lane;
+  const bool live = r < m;
+  float w[16], t0[16], err[16];
+  float amax = 0.f;
 #pragma unroll
   for (int k = 0; k < 16; ++k) {
-    w[k] = WT[(c0 + k) * m + r];
-    base[k] = w[k] + (calibrate ? FT[(c0 + k) * m + r] : 0.f);
-    amax = fmaxf(amax, fabsf(calibrate ? base[k] : w[k]));
+    w[k] = live ? WT[(c0 + k) * m + r] : 0.f;
+    t0[k] = w[k] + (calibrate && live ? FT[(c0 + k) * m + r] : 0.f);
+    amax = fmaxf(amax, fabsf(calibrate ? t0[k] : w[k]));
   }
-  unsigned cand[kCand];
-  int nc = 0;
-  const unsigned c1 = nv_fp8_enc(amax / (6.f * global));
-  cand[nc++] = c1;
-  if (search) {
-    const float g[8] = {0.70f, 0.75f, 0.80f, 0.85f, 0.90f, 0.95f, 1.00f, 1.05f};
-#pragma unroll
-    for (int i = 0; i < 8; ++i) cand[nc++] = nv_fp8_enc(amax * g[i] / (6.f * global));
-    cand[nc++] = c1 > 0 ? c1 - 1 : 0;
-    cand[nc++] = c1 < 126 ? c1 + 1 : 126;
-  }
-  float best_cost = __builtin_inff();
-  unsigned best = c1;
-  for (int ci = 0; ci < nc; ++ci) {
-    const unsigned s = cand[ci];
-    const float sd = nv_fp8_dec(s);
-    const float scale = sd * global;
-    float err[16];
-    float cost = 0;
-#pragma unroll
-    for (int k = 15; k >= 0; --k) {
-      float t = base[k];
-      if (calibrate) {
-#pragma unroll
-        for (int j = k + 1; j < 16; ++j) t = fmaf(err[j], Lb[j][k], t);
-      }
-      const float x = scale != 0.f ? t / scale : 0.f;
-      const int code = nv_fp4_code(fabsf(x));
-      const float q = nv_bf16_round((x < 0 ? -1.f : 1.f) * nv_level(code) * sd * global);
-      cost = fmaf(Dw[k] * (t - q), t - q, cost);
-      err[k] = w[k] - q;
-    }
-    if (cost < best_cost) {
-      best_cost = cost;
-      best = s;
-    }
-  }
-  const float sd = nv_fp8_dec(best);
+  const unsigned code8 = nv_candidate(which, amax, global);
+  const float sd = nv_fp8_dec(code8);
   const float scale = sd * global;
-  float err[16];
-  unsigned nib[16];
+  float cost = 0.f;
+  uint32_t nib_lo = 0, nib_hi = 0;  // E2M1 codes of columns 0..7 and 8..15, 4 bits each
 #pragma unroll
   for (int k = 15; k >= 0; --k) {
-    float t = base[k];
+    float t = t0[k];
     if (calibrate) {
 #pragma unroll
       for (int j = k + 1; j < 16; ++j) t = fmaf(err[j], Lb[j][k], t);
@@ -144,12 +136,25 @@ __global__ __launch_bounds__(256) void nv_block_kernel(const float* __restrict__
     const float x = scale != 0.f ? t / scale : 0.f;
     const int code = nv_fp4_code(fabsf(x));
     const float q = nv_bf16_round((x < 0 ? -1.f : 1.f) * nv_level(code) * sd * global);
+    cost = fmaf(Dw[k] * (t - q), t - q, cost);
     err[k] = w[k] - q;
-    nib[k] = unsigned(code) | ((__float_as_uint(x) >> 31) ? 8u : 0u);
+    const uint32_t nib = uint32_t(code) | ((__float_as_uint(x) >> 31) << 3);
+    if (k < 8) nib_lo |= nib << (4 * k);
+    else nib_hi |= nib << (4 * (k - 8));
   }
+  costs[which][lane] = cost;
+  __syncthreads();
+  int winner = 0;
+  float least = __builtin_inff();
+  for (int i = 0; i < ncand; ++i)
+    if (costs[i][lane] < least) least = costs[i][lane], winner = i;
+  if (!live || winner != which) return;
 #pragma unroll
-  for (int k = 0; k < 16; k += 2) packedT[((c0 + k) / 2) * m + r] = uint8_t(nib[k] | (nib[k + 1] << 4));
-  scalesT[(c0 / 16) * m + r] = uint8_t(best);
+  for (int k = 0; k < 4; ++k) {
+    packedT[(c0 / 2 + k) * m + r] = uint8_t(nib_lo >> (8 * k));
+    packedT[(c0 / 2 + 4 + k) * m + r] = uint8_t(nib_hi >> (8 * k));
+  }
+  scalesT[(c0 / 16) * m + r] = uint8_t(code8);
 #pragma unroll
   for (int k = 0; k < 16; ++k) E[k * m + r] = err[k];
 }
@@ -240,8 +245,9 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(const uint8_t* __rest
 void launch_nvfp4_block(const float* WT, const float* FT, long m, long n, long c0, const float* L, const float* dw,
                         float global, bool calibrate, bool search, uint8_t* packedT, uint8_t* scalesT, float* E,
                         hipStream_t s) {
-  nv_block_kernel<<<dim3(unsigned((m + 255) / 256)), dim3(256), 0, s>>>(WT, FT, m, n, c0, L, dw, global, calibrate ? 1 : 0,
-                                                                        search ? 1 : 0, packedT, scalesT, E);
+  const int ncand = search ? kCand : 1;
+  nv_block_kernel<<<dim3(unsigned((m + kBlockRows - 1) / kBlockRows)), dim3(unsigned(kBlockRows * ncand)), 0, s>>>(
+      WT, FT, m, n, c0, L, dw, global, calibrate ? 1 : 0, ncand, packedT, scalesT, E);
   QTIP_HIP(hipGetLastError());
 }
 void launch_nvfp4_feedback(float* FT, long m, long n, long c0, long col_lo, const float* E, const float* L,
