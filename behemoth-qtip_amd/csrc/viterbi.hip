@@ -35,6 +35,8 @@
 // fully coalesced; the first pass only keeps the steps its half-length trace-back needs.
 #include <hip/hip_ext.h>
 
+#include <type_traits>
+
 #include "qtip_internal.hpp"
 
 namespace qtipmi {
@@ -117,7 +119,9 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
   __syncthreads();
 
   unsigned long long word = 0;
-  for (int it = 0; it < kSteps; ++it) {
+  // one trellis step; DIGITS: the step's back-pointers are wanted (without them a candidate costs an add and a min)
+  auto step = [&](int it, auto digits_tag) __attribute__((always_inline)) {
+    constexpr bool digits = decltype(digits_tag)::value;
     // ---- phase R: metric columns -> registers, error table of this step -> LDS
     double MA[16], MB[16];
     // the 32 read addresses are recomputed in every step (one XOR each): kept across the loop they would take 32
@@ -146,7 +150,6 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
     // upwards with "<", its mirror scans downwards with "<=" over the same values; both keep the smallest
     // digit among equal minima, as the ascending first-minimum rule of the CPU algorithm does.
     word = 0;
-    const bool digits = it >= bp_first;  // uniform; without them a candidate costs an add and a min
     double cur[8], nxt[8];
     {
       const double* er = sm.E + ebase[0];
@@ -188,7 +191,7 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
       "v_min_f64 %[bb], %[bb], %[cb]"                                \
       : [ca] "=&v"(ca), [cb] "=&v"(cb), [ba] "+v"(ba), [bb] "+v"(bb) \
       : [e] "v"(EV), [ma] "v"(MAV), [mb] "v"(MBV))
-      if (digits) {
+      if constexpr (digits) {
         QTIP_ACS2(1, 14, cur[1], MA[1], MB[14]);
         QTIP_ACS2(2, 13, cur[2], MA[2], MB[13]);
         QTIP_ACS2(3, 12, cur[3], MA[3], MB[12]);
@@ -211,7 +214,7 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
 #pragma unroll
         for (int k = 0; k < 8; ++k) cur[k] = er[((k * gn) & 15) * 64];
       }
-      if (digits) {
+      if constexpr (digits) {
         QTIP_ACS2(8, 7, nxt[0], MA[8], MB[7]);
         QTIP_ACS2(9, 6, nxt[1], MA[9], MB[6]);
         QTIP_ACS2(10, 5, nxt[2], MA[10], MB[5]);
@@ -237,9 +240,11 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
       word |= (unsigned long long)(da) << (4 * m);
       word |= (unsigned long long)(db) << (32 + 4 * m);
     }
-    if (it >= bp_first && it < kSteps - 1) bp[size_t(it) * kThreads + tid] = word;
+    if (digits && it < kSteps - 1) bp[size_t(it) * kThreads + tid] = word;
     __syncthreads();
-  }
+  };
+  for (int it = 0; it < bp_first; ++it) step(it, std::false_type{});
+  for (int it = bp_first; it < kSteps; ++it) step(it, std::true_type{});
   // final state: smallest metric, then smallest state, over the metrics of the last step (each lane re-reads the
   // 16 values it has just written; their predecessor digits are the nibbles of the last back-pointer word)
   if (ov < 0) {
