@@ -22,7 +22,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-FLOP_PER_WEIGHT = 393216.0      # 2^16 add-compare-selects per weight, 6 flop each (survey figure for the Viterbi)
+FLOP_PER_WEIGHT = 393216.0      # 2^16 add-compare-selects per weight, counted as 6 flop each
 PEAK_FP64_TFLOPS = 78.6         # MI355X vector fp64
 
 
