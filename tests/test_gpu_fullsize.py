@@ -1,4 +1,4 @@
-"""Full-size checks (benchmark configurations 3 and 5) of the GPU group path: agreement with the CPU form on a row
+"""Full-size checks (benchmark configurations 3, 4 and 5) of the GPU group path: agreement with the CPU form on a row
 subset of the rotated weights (LDLQ is row-independent given L), and size-independent properties of the packed
 output (every trellis tail-biting and link-consistent, decode(states) == hatW on sampled tiles)."""
 import os
@@ -122,3 +122,58 @@ def test_config5_depth_ldlq_rows_against_cpu(qz, pkg, oracle, hyb, synth):
     assert same.mean() >= 0.99
     if same.all():
         assert np.array_equal(dH.cpu().numpy().T, hat_o)
+
+
+def test_config4_two_linears_shared_hessian_rows_against_cpu(qz, pkg, oracle, hyb, synth):
+    """gate + up, two stacked 28672 x 12288 linears sharing one Hessian (one SU, one L, two SV / Wscale): the group
+    call at full size, then two tile rows of each linear recomputed by the CPU form from the same rotated, scaled
+    rows and the same L must give the codes found in that linear's slice of the packed output (>= 99 % is the bar).
+    The rotated rows are formed with the library's own transform, which other tests pin bit for bit."""
+    import torch
+    say("case: config 4 (two linears, shared Hessian) at full size, 64 rows against the CPU form")
+    qz.set_tlut(None)
+    Ws, H = synth.large_config(4)
+    n, m = H.shape[0], Ws[0].shape[0]
+    seed = 4
+    hp = qz.rotate_hessian(H, n, seed)
+    del H
+    pkg.Quantizer.ldl_hessian(hp, threads=16)
+    L = hp.L.copy()                                              # the group call consumes hp.L
+    lins = [pkg.LinearIn("gate", m, w_f32=Ws[0]), pkg.LinearIn("up", m, w_f32=Ws[1])]
+    outs, tm = qz.quantize_group(lins, hp, pkg.QuantOpts(ldl_threads=16))
+    say("  ldlq %.1fs viterbi %.1fs (%.1f Mweights/s) proxy %.5f / %.5f wscale %.6f / %.6f" %
+        (tm.ldlq, tm.viterbi, 2 * m * n / tm.viterbi / 1e6, outs[0].proxy, outs[1].proxy, outs[0].wscale,
+         outs[1].wscale))
+    su = pkg.sign_vector(seed, n)
+    assert np.array_equal(hp.su, su)
+    d_su = torch.from_numpy(su).cuda()
+    rows = np.r_[0:16, 17008:17024]                              # tile rows 0 and 1063 of each linear
+    d_rows = torch.from_numpy(rows).cuda()
+    lut_rms = np.float32(qz.lut_rms)
+    for li, lo in enumerate(outs):
+        assert np.array_equal((lo.su_bf16.astype(np.uint32) << 16).view(np.float32), su)
+        sv = pkg.sign_vector(seed * 1000003 + li + 1, m)
+        assert np.array_equal(lo.sv, sv)
+        assert 0 < lo.proxy < 0.2 and 0 < lo.proxy_rot_reg < 0.2
+        st = pkg.unpack_trellis(pkg.unswizzle_for_kernel(lo.trellis, m, n))
+        check_trellis_paths(st)
+        # Wr^T = U^T_m (U^T_n (diag(SV) W diag(SU)))^T, then the fp32 multiplication by 1 / Wscale
+        A = Ws[li] * torch.from_numpy(sv).cuda()[:, None] * d_su[None, :]
+        torch.cuda.synchronize()                                 # the library works on a stream of its own
+        qz.hadamard_rows_dev(A, m, n, n, True)
+        qz.synchronize()
+        AT = A.T.contiguous()
+        del A
+        torch.cuda.synchronize()
+        qz.hadamard_rows_dev(AT, n, m, m, True)
+        qz.synchronize()
+        rms = float(AT.double().pow(2).mean().sqrt())
+        wscale = rms / (float(lut_rms) * 0.9)
+        assert abs(wscale - lo.wscale) <= 2e-6 * wscale
+        sub = (AT[:, d_rows] * float(np.float32(1.0) / np.float32(lo.wscale))).T.contiguous().cpu().numpy()
+        del AT
+        hat_o, Q_o = oracle.ldlq(hyb, sub, L, threads=16)
+        Q_g = st.reshape(m // 16, n // 16, 128)[[0, 1063]].reshape(-1, 128)
+        same = np.all(Q_g == Q_o, axis=1)
+        say("  linear %d: identical trellises %d of %d" % (li, int(same.sum()), same.size))
+        assert same.mean() >= 0.99
