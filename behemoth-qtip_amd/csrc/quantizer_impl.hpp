@@ -11,7 +11,7 @@ struct qtip_ctx {
   qtipmi::HostCodebook cb;
   qtipmi::DBuf<double> d_entry_d;  // [1024][2] decoded codebook entries, fp64
   qtipmi::DBuf<float> d_entry_f;   // [1024][2] the same as fp32
-  qtipmi::DBuf<unsigned char> vit_ws;  // back-pointer slots of the resident Viterbi workgroups
+  qtipmi::DBuf<unsigned char> vit_ws;  // kept-metrics slots of the resident Viterbi workgroups
   int vit_slots = 0;
   qtipmi::Rht rht;
   qtipmi::DBuf<double> scratch;

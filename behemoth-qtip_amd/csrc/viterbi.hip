@@ -31,8 +31,11 @@
 //     group's slot is the group's XOR 0xff3.
 // LDS per workgroup ~50 KB, three workgroups per CU; metrics single-buffered (the columns are read into registers
 // before the step's results are written).
-// Back-pointers (4 bits per group and step) go to HBM as one 64-bit word per thread and step, 2 KB per step,
-// fully coalesced; the first pass only keeps the steps its half-length trace-back needs.
+// No back-pointers.  A step's 16-way search keeps the minimum only (add + min per candidate); which digit won
+// matters for the 127 groups on the surviving path alone, so the metrics entering every second step (32 KB, written
+// value-major: one contiguous 512-byte store per wave and value) are kept in HBM and the trace-back redoes the
+// add-compare-selects of the path it walks, two steps per round trip, with the forward pass's own fp64 operations
+// and tie rule.  Only the last step tracks its digits (in registers), which the final state needs.
 #include <hip/hip_ext.h>
 
 #include <type_traits>
@@ -45,7 +48,9 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kESlots = 32 * 64;                 // E[q][row]: 16 entry positions stored twice x 64 rows
 constexpr int kMSlots = 4096;                    // metric of (column c, digit d) at m_slot(c, d)
-constexpr int kBpWordsPerTile = 127 * kThreads;  // u64 words
+constexpr int kHistSteps = 63;                           // the metrics entering the odd steps 1, 3 .. 125 are kept
+constexpr int kHistWordsPerTile = kHistSteps * kGroups;  // fp64 words
+enum StepKind { kPlain = 0, kStore = 1, kDigits = 2 };
 
 __device__ __forceinline__ constexpr int pi16(int d) { return 4 * (d & 3) + (d >> 2); }
 __device__ __forceinline__ int m_swz(int col) { return ((col >> 2) & 15) ^ (col >> 6); }
@@ -72,22 +77,19 @@ __device__ __forceinline__ uint32_t owner_thread(uint32_t jj) {
   const uint32_t c = jj >> 4, h = (jj >> 3) & 1u;
   return ((c & 63u) >> 2) | ((c & 3u) << 4) | ((c >> 6) << 6) | (h << 7);
 }
-// predecessor digit of group j from one step's 256 back-pointer words (word index = owning thread, so that a
-// wave's 64 words are one contiguous 512-byte store; nibble m for the group itself, nibble 8 + m for a mirror
-// group j >= 2048).  Read past the vector L1, which may still hold the previous tile's words.
-__device__ __forceinline__ uint32_t bp_lookup(const unsigned long long* step_words, uint32_t j) {
-  const uint32_t jj = j < 2048u ? j : 4095u - j;
-  const uint32_t shift = (jj & 7u) * 4u + (j < 2048u ? 0u : 32u);
-  const unsigned long long w = __hip_atomic_load(step_words + owner_thread(jj), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return uint32_t(w >> shift) & 15u;
+// place of group g in one kept step of metrics: value (jj & 7) (+ 8 for a mirror group) of the owning thread, stored
+// value-major so that a wave's 64 values are one contiguous 512-byte store
+__device__ __forceinline__ uint32_t hist_index(uint32_t g) {
+  const uint32_t jj = g < 2048u ? g : 4095u - g;
+  return ((jj & 7u) + (g < 2048u ? 0u : 8u)) * kThreads + owner_thread(jj);
 }
 
 // One forward pass over the 128 steps.  roll: input rotation (128 for the first pass).  ov < 0: free start and
 // end; otherwise start in states with (s >> 4) == ov and end in the state of group ov.
-// bp: this workgroup's back-pointer words; steps < bp_first are not stored.  Returns nothing; the final state
-// is left in sm.final_state.
+// The even steps first_kept .. 124 also write their results, the metrics entering the next (odd) step, to hist.
+// Returns nothing; the final state is left in sm.final_state.
 __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict__ entry_d, int roll, int ov,
-                                             unsigned long long* __restrict__ bp, int bp_first) {
+                                             double* __restrict__ hist, int first_kept) {
   const int tid = threadIdx.x;
   const int colA = 4 * (tid & 15) + ((tid >> 4) & 3) + 64 * ((tid >> 6) & 1), colB = 255 - colA;
   const int half = tid >> 7;  // owns 16c + 8 half + m, m = 0..7
@@ -119,9 +121,13 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
   __syncthreads();
 
   unsigned long long word = 0;
-  // one trellis step; DIGITS: the step's back-pointers are wanted (without them a candidate costs an add and a min)
-  auto step = [&](int it, auto digits_tag) __attribute__((always_inline)) {
-    constexpr bool digits = decltype(digits_tag)::value;
+  // one trellis step; kDigits: the winning digits are wanted (without them a candidate costs an add and a min);
+  // kStore: the results also go to hist
+  auto step = [&](int it, auto kind_tag) __attribute__((always_inline)) {
+    constexpr int kind = decltype(kind_tag)::value;
+    constexpr bool digits = kind == kDigits;
+    double* hs = nullptr;
+    if constexpr (kind == kStore) hs = hist + size_t(it >> 1) * kGroups + tid;
     // ---- phase R: metric columns -> registers, error table of this step -> LDS
     double MA[16], MB[16];
     // the 32 read addresses are recomputed in every step (one XOR each): kept across the loop they would take 32
@@ -182,7 +188,7 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
       : [ca] "=&v"(ca), [cb] "=&v"(cb), [ka] "=&s"(mka), [kb] "=&s"(mkb), [ba] "+v"(ba), [bb] "+v"(bb),     \
         [da] "+v"(da), [db] "+v"(db)                                                                        \
       : [e] "v"(EV), [ma] "v"(MAV), [mb] "v"(MBV))
-      // the same without the digit, for the steps whose back-pointers nobody reads (first half of the first pass)
+      // the same without the digit
 #define QTIP_AM2(EV, MAV, MBV)                                       \
   asm volatile(                                                      \
       "v_add_f64 %[ca], %[e], %[ma]\n\t"                             \
@@ -237,16 +243,28 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
 #undef QTIP_AM2
       sm.M[wslot[m]] = ba;
       sm.M[wslot[m] ^ kMirror] = bb;
-      word |= (unsigned long long)(da) << (4 * m);
-      word |= (unsigned long long)(db) << (32 + 4 * m);
+      if constexpr (kind == kStore) {
+        hs[m * kThreads] = ba;
+        hs[(8 + m) * kThreads] = bb;
+      }
+      if constexpr (digits) {
+        word |= (unsigned long long)(da) << (4 * m);
+        word |= (unsigned long long)(db) << (32 + 4 * m);
+      }
     }
-    if (digits && it < kSteps - 1) bp[size_t(it) * kThreads + tid] = word;
     __syncthreads();
   };
-  for (int it = 0; it < bp_first; ++it) step(it, std::false_type{});
-  for (int it = bp_first; it < kSteps; ++it) step(it, std::true_type{});
+  using Plain = std::integral_constant<int, kPlain>;
+  using Store = std::integral_constant<int, kStore>;
+  using Digits = std::integral_constant<int, kDigits>;
+#pragma nounroll
+  for (int it = 0; it < kSteps - 1; ++it) {
+    if (!(it & 1) && it >= first_kept && it < kSteps - 2) step(it, Store{});
+    else step(it, Plain{});
+  }
+  step(kSteps - 1, Digits{});
   // final state: smallest metric, then smallest state, over the metrics of the last step (each lane re-reads the
-  // 16 values it has just written; their predecessor digits are the nibbles of the last back-pointer word)
+  // 16 values it has just written; their predecessor digits are the nibbles of the last step's digit word)
   if (ov < 0) {
     double bestc = INF;
     uint32_t bests = 0xffffffffu;
@@ -311,41 +329,103 @@ __device__ __forceinline__ void tile_targets(Smem& sm, const TileJob& job, long 
   sm.x[u] = float(_Float16(float(acc)));
 }
 
+// Trace-back, run by the first wave: walks two steps per round trip to HBM.  s is the state of step it + 1;
+// for every digit d of step it the metric M_it[g_d] of the group g_d = (d << 8) | (j >> 4), j = s >> 4, is rebuilt
+// from the kept metrics of step it - 1 as the forward pass built it (16 lanes, one per digit of step it - 1, same
+// fp64 operations, smallest digit among equal minima), then the 16 candidates of step it are compared the same way.
+// Returns the state of step it_min - 1; record: the states of the steps walked are written to sm.st.
+__device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restrict__ entry_d,
+                                               const double* __restrict__ hist, int roll, uint32_t s, int it_min,
+                                               bool record) {
+  const uint32_t lane = threadIdx.x & 63u, dp = lane & 15u, dq = lane >> 4;
+  const double INF = __builtin_inf();
+#pragma nounroll
+  for (int it = kSteps - 2; it >= it_min; it -= 2) {
+    const uint32_t j = s >> 4;
+    const int ta = (2 * (it - 1) + roll) & 255, tb = (2 * it + roll) & 255;
+    const double xa0 = double(sm.x[ta]), xa1 = double(sm.x[ta + 1]);
+    const double xb0 = double(sm.x[tb]), xb1 = double(sm.x[tb + 1]);
+    const unsigned long long* row =
+        reinterpret_cast<const unsigned long long*>(hist + size_t(it / 2 - 1) * kGroups);
+    double mv[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t d = 4u * q + dq, p = (dp << 8) | (d << 4) | (j >> 8);
+      // past the vector L1, which may hold the previous tile's values
+      mv[q] = __longlong_as_double((long long)__hip_atomic_load(row + hist_index(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    }
+    double best = INF;
+    uint32_t bestd = 0, bestd1 = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t d = 4u * q + dq, g = (d << 8) | (j >> 4);
+      const uint32_t s1 = (dp << 12) | g, e1 = ((s1 * (s1 + 1u)) >> 6) & 1023u;
+      const double a1 = entry_d[2 * e1] - xa0, b1 = entry_d[2 * e1 + 1] - xa1;
+      double c1 = __builtin_fma(a1, a1, b1 * b1) + mv[q];
+      uint32_t k1 = dp;
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) {
+        const double oc = __shfl_xor(c1, off, 64);
+        const uint32_t ok = __shfl_xor(k1, off, 64);
+        if (oc < c1 || (oc == c1 && ok < k1)) c1 = oc, k1 = ok;
+      }
+      const uint32_t s0 = (d << 12) | j, e0 = ((s0 * (s0 + 1u)) >> 6) & 1023u;
+      const double a0 = entry_d[2 * e0] - xb0, b0 = entry_d[2 * e0 + 1] - xb1;
+      const double c0 = __builtin_fma(a0, a0, b0 * b0) + c1;
+      if (q == 0 || c0 < best) best = c0, bestd = d, bestd1 = k1;  // d ascends with q: the first minimum stays
+    }
+#pragma unroll
+    for (int off = 16; off < 64; off <<= 1) {
+      const double oc = __shfl_xor(best, off, 64);
+      const uint32_t od = __shfl_xor(bestd, off, 64), od1 = __shfl_xor(bestd1, off, 64);
+      if (oc < best || (oc == best && od < bestd)) best = oc, bestd = od, bestd1 = od1;
+    }
+    const uint32_t s_it = (bestd << 12) | j;
+    s = (bestd1 << 12) | (s_it >> 4);
+    if (record && lane == 0) {
+      sm.st[it] = uint16_t(s_it);
+      sm.st[it - 1] = uint16_t(s);
+    }
+  }
+  return s;
+}
+
 __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job, const double* __restrict__ entry_d,
                                                                  const float* __restrict__ entry_f,
-                                                                 unsigned long long* __restrict__ bp_all) {
+                                                                 double* __restrict__ hist_all) {
   __shared__ Smem sm;
   const int u = threadIdx.x;
-  unsigned long long* bp = bp_all + size_t(blockIdx.x) * kBpWordsPerTile;
+  double* hist = hist_all + size_t(blockIdx.x) * kHistWordsPerTile;
   for (long tile = blockIdx.x; tile < job.tiles; tile += gridDim.x) {
     if (job.X) sm.x[u] = job.X[tile * kSeq + u];
     else if (job.prod64) tile_targets<double>(sm, job, tile, job.prod64);
     else tile_targets<float>(sm, job, tile, job.prod32);
     __syncthreads();
-    // pass 1 on the sequence rotated by half its length, free ends; only steps 64..126 are traced back
-    forward_pass(sm, entry_d, 128, -1, bp, 64);
-    if (u == 0) {
-      uint32_t s = sm.final_state;  // state of step 127
-      for (int i = 127; i > 64; --i) {
-        const uint32_t j = s >> 4;
-        s = j | (bp_lookup(bp + size_t(i - 1) * kThreads, j) << 12);
+    // pass 1 on the sequence rotated by half its length, free ends, traced back to step 64 for the overlap group;
+    // pass 2 on the sequence itself, tail-biting through that group, traced back in full.  One loop, so that the
+    // step bodies exist once in the instruction cache.
+    int ov = -1;
+#pragma nounroll
+    for (int pass = 0; pass < 2; ++pass) {
+      const int roll = pass == 0 ? kSeq / 2 : 0;
+      forward_pass(sm, entry_d, roll, ov, hist, pass == 0 ? 62 : 0);
+      if (u < 64) {
+        const uint32_t s_last = sm.final_state;  // state of step 127
+        const uint32_t s = trace_back(sm, entry_d, hist, roll, s_last, pass == 0 ? 64 : 2, pass == 1);
+        if (u == 0) {
+          if (pass == 0) {
+            // s is the state of step 63: its low 12 bits are the high 12 bits of the state of step 64
+            sm.overlap = int(s & 0xfffu);
+          } else {
+            // s is the state of step 1; at step 0 the one predecessor group with a finite initial metric is ov
+            sm.st[kSteps - 1] = uint16_t(s_last);
+            sm.st[0] = uint16_t((s >> 4) | ((uint32_t(ov) >> 8) << 12));
+          }
+        }
       }
-      sm.overlap = int(s >> 4);  // state of step 64, high 12 bits
+      __syncthreads();
+      ov = sm.overlap;
     }
-    __syncthreads();
-    const int ov = sm.overlap;
-    // pass 2 on the sequence itself, tail-biting through group ov
-    forward_pass(sm, entry_d, 0, ov, bp, 0);
-    if (u == 0) {
-      uint32_t s = sm.final_state;
-      sm.st[127] = uint16_t(s);
-      for (int i = 127; i > 0; --i) {
-        const uint32_t j = s >> 4;
-        s = j | (bp_lookup(bp + size_t(i - 1) * kThreads, j) << 12);
-        sm.st[i - 1] = uint16_t(s);
-      }
-    }
-    __syncthreads();
     // ---- outputs
     if (job.states && u < kSteps) job.states[(tile * job.q_tile_stride + job.q_offset) * kSteps + u] = sm.st[u];
     if (job.packed && u < kWords) {
@@ -380,7 +460,7 @@ __global__ void decode_states_kernel(const uint16_t* __restrict__ st, long count
 
 }  // namespace
 
-size_t viterbi_workspace_bytes(int slots) { return size_t(slots) * kBpWordsPerTile * sizeof(unsigned long long); }
+size_t viterbi_workspace_bytes(int slots) { return size_t(slots) * kHistWordsPerTile * sizeof(double); }
 
 int viterbi_max_slots(int device) {
   hipDeviceProp_t prop;
@@ -408,10 +488,9 @@ void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const flo
     // the runtime stamps the two events at the kernel's own start and end: the time between them is the kernel's,
     // however late the host got round to queueing it
     hipExtLaunchKernelGGL(viterbi_tiles_kernel, dim3(grid), dim3(kThreads), 0, s, start, stop, 0, job, d_entry_d,
-                          d_entry_f, static_cast<unsigned long long*>(workspace));
+                          d_entry_f, static_cast<double*>(workspace));
   } else {
-    viterbi_tiles_kernel<<<dim3(grid), dim3(kThreads), 0, s>>>(job, d_entry_d, d_entry_f,
-                                                               static_cast<unsigned long long*>(workspace));
+    viterbi_tiles_kernel<<<dim3(grid), dim3(kThreads), 0, s>>>(job, d_entry_d, d_entry_f, static_cast<double*>(workspace));
   }
   QTIP_HIP(hipGetLastError());
 }
