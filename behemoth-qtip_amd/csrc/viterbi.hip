@@ -329,16 +329,39 @@ __device__ __forceinline__ void tile_targets(Smem& sm, const TileJob& job, long 
   sm.x[u] = float(_Float16(float(acc)));
 }
 
+// smallest value over the 16 lanes of a row (lanes 16 r .. 16 r + 15), in each of them: four cross-lane moves inside
+// the vector pipe (neighbour, pair, mirrored half row, mirrored row).  No NaNs reach it.
+__device__ __forceinline__ double row_min16(double c) {
+#define QTIP_ROW_STEP(CTRL)                                                                       \
+  {                                                                                               \
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(c), CTRL, 0xf, 0xf, false);      \
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(c), CTRL, 0xf, 0xf, false);      \
+    const double o = __hiloint2double(hi, lo);                                                    \
+    asm volatile("v_min_f64 %0, %1, %2" : "=v"(c) : "v"(c), "v"(o));                              \
+  }
+  QTIP_ROW_STEP(0xB1)   // quad_perm [1, 0, 3, 2]
+  QTIP_ROW_STEP(0x4E)   // quad_perm [2, 3, 0, 1]
+  QTIP_ROW_STEP(0x141)  // row_half_mirror
+  QTIP_ROW_STEP(0x140)  // row_mirror
+#undef QTIP_ROW_STEP
+  return c;
+}
+
+__device__ __forceinline__ double read_lane_f64(double v, int lane) {
+  return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), lane),
+                          __builtin_amdgcn_readlane(__double2loint(v), lane));
+}
+
 // Trace-back, run by the first wave: walks two steps per round trip to HBM.  s is the state of step it + 1;
 // for every digit d of step it the metric M_it[g_d] of the group g_d = (d << 8) | (j >> 4), j = s >> 4, is rebuilt
-// from the kept metrics of step it - 1 as the forward pass built it (16 lanes, one per digit of step it - 1, same
-// fp64 operations, smallest digit among equal minima), then the 16 candidates of step it are compared the same way.
+// from the kept metrics of step it - 1 as the forward pass built it (the 16 lanes of a row, one per digit of step
+// it - 1, same fp64 operations, smallest digit among equal minima), then the 16 candidates of step it are compared
+// the same way (four per row, then across the four rows).
 // Returns the state of step it_min - 1; record: the states of the steps walked are written to sm.st.
 __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restrict__ entry_d,
                                                const double* __restrict__ hist, int roll, uint32_t s, int it_min,
                                                bool record) {
   const uint32_t lane = threadIdx.x & 63u, dp = lane & 15u, dq = lane >> 4;
-  const double INF = __builtin_inf();
 #pragma nounroll
   for (int it = kSteps - 2; it >= it_min; it -= 2) {
     const uint32_t j = s >> 4;
@@ -354,34 +377,47 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
       // past the vector L1, which may hold the previous tile's values
       mv[q] = __longlong_as_double((long long)__hip_atomic_load(row + hist_index(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     }
-    double best = INF;
-    uint32_t bestd = 0, bestd1 = 0;
+    double e1v[4], e0v[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const uint32_t d = 4u * q + dq, g = (d << 8) | (j >> 4);
       const uint32_t s1 = (dp << 12) | g, e1 = ((s1 * (s1 + 1u)) >> 6) & 1023u;
       const double a1 = entry_d[2 * e1] - xa0, b1 = entry_d[2 * e1 + 1] - xa1;
-      double c1 = __builtin_fma(a1, a1, b1 * b1) + mv[q];
-      uint32_t k1 = dp;
-#pragma unroll
-      for (int off = 1; off < 16; off <<= 1) {
-        const double oc = __shfl_xor(c1, off, 64);
-        const uint32_t ok = __shfl_xor(k1, off, 64);
-        if (oc < c1 || (oc == c1 && ok < k1)) c1 = oc, k1 = ok;
-      }
+      e1v[q] = __builtin_fma(a1, a1, b1 * b1);
       const uint32_t s0 = (d << 12) | j, e0 = ((s0 * (s0 + 1u)) >> 6) & 1023u;
       const double a0 = entry_d[2 * e0] - xb0, b0 = entry_d[2 * e0 + 1] - xb1;
-      const double c0 = __builtin_fma(a0, a0, b0 * b0) + c1;
-      if (q == 0 || c0 < best) best = c0, bestd = d, bestd1 = k1;  // d ascends with q: the first minimum stays
+      e0v[q] = __builtin_fma(a0, a0, b0 * b0);
     }
+    double best = 0;
+    uint32_t bestd = 0, bestd1 = 0;
 #pragma unroll
-    for (int off = 16; off < 64; off <<= 1) {
-      const double oc = __shfl_xor(best, off, 64);
-      const uint32_t od = __shfl_xor(bestd, off, 64), od1 = __shfl_xor(bestd1, off, 64);
-      if (oc < best || (oc == best && od < bestd)) best = oc, bestd = od, bestd1 = od1;
+    for (int q = 0; q < 4; ++q) {
+      const double c1 = e1v[q] + mv[q];
+      const double m1 = row_min16(c1);  // M_it[g_d]
+      // its digit: the first lane of the row that holds the minimum
+      const unsigned long long at_min = __builtin_amdgcn_ballot_w64(c1 == m1);
+      const uint32_t k1 = uint32_t(__builtin_ctz(uint32_t(at_min >> (16u * dq)) & 0xffffu));
+      const double c0 = e0v[q] + m1;
+      const bool take = q == 0 || c0 < best;  // d ascends with q: the first minimum stays
+      best = take ? c0 : best;
+      bestd = take ? 4u * q + dq : bestd;
+      bestd1 = take ? k1 : bestd1;
     }
-    const uint32_t s_it = (bestd << 12) | j;
-    s = (bestd1 << 12) | (s_it >> 4);
+    // every lane of row r now holds that row's best (cost, d, d1); pick across the four rows, smallest d on ties
+    double bc = read_lane_f64(best, 0);
+    uint32_t bd = uint32_t(__builtin_amdgcn_readlane(int(bestd), 0)), bd1 = uint32_t(__builtin_amdgcn_readlane(int(bestd1), 0));
+#pragma unroll
+    for (int r = 1; r < 4; ++r) {
+      const double oc = read_lane_f64(best, 16 * r);
+      const uint32_t od = uint32_t(__builtin_amdgcn_readlane(int(bestd), 16 * r));
+      const uint32_t od1 = uint32_t(__builtin_amdgcn_readlane(int(bestd1), 16 * r));
+      const bool take = oc < bc || (oc == bc && od < bd);
+      bc = take ? oc : bc;
+      bd = take ? od : bd;
+      bd1 = take ? od1 : bd1;
+    }
+    const uint32_t s_it = (bd << 12) | j;
+    s = (bd1 << 12) | (s_it >> 4);
     if (record && lane == 0) {
       sm.st[it] = uint16_t(s_it);
       sm.st[it - 1] = uint16_t(s);
