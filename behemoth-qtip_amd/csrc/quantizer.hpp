@@ -31,7 +31,7 @@ class Gemm {
 struct QuantOpts {  // src/quantizer.hpp:11-19
   double sigma_reg = 1e-2;
   double scale_override = 0.9;
-  int vit_batch = 1024;  // accepted, unused: the tile kernel sizes its own back-pointer workspace
+  int vit_batch = 1024;  // accepted, unused: the tile kernel sizes its own workspace
   int ldl_threads = 16;
   bool share_su = true;
   std::string dump_dir;  // if set: W (fp32) and, unless want_hatW, the reconstructed hatW (fp32) are written per linear
