@@ -159,6 +159,11 @@ def _ptr(a):
         return a.ctypes.data
     if hasattr(a, "data_ptr"):
         assert a.is_contiguous()
+        if a.is_cuda:
+            # the library works on a stream of its own: whatever torch has queued for this tensor (its fill, the
+            # kernel that produced it) must have finished before the library touches it
+            import torch
+            torch.cuda.current_stream(a.device).synchronize()
         return a.data_ptr()
     raise TypeError(type(a))
 

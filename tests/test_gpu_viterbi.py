@@ -133,12 +133,14 @@ def test_ragged_batches_and_device_entry(qz, oracle, hyb):
     assert np.array_equal(pk, oracle.pack_trellis(st))
     # size-independent property at full batch: decode(encode) reproduces hat, cost never above the oracle's on a sample
     dH = torch.zeros((1000, 256), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()                     # the library works on a stream of its own
     qz.decode_states_dev(dS, 1000, dH)
     qz.synchronize()
     l0, l1 = qz.lut()
     assert np.array_equal(dH.cpu().numpy(), np.stack([l0[st], l1[st]], axis=-1).reshape(1000, 256))
     # determinism: a second run gives the same bits
     dS2 = torch.zeros_like(dS)
+    torch.cuda.synchronize()
     qz.viterbi_tiles_dev(dX, 1000, dS2, None)
     qz.synchronize()
     assert torch.equal(dS, dS2)
