@@ -290,7 +290,7 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
       uint32_t s = sm.red_s[0];
       for (int w = 1; w < 4; ++w)
         if (sm.red_c[w] < c || (sm.red_c[w] == c && sm.red_s[w] < s)) c = sm.red_c[w], s = sm.red_s[w];
-      sm.final_state = s;
+      sm.final_state = s & 0xffffu;  // (no comparison succeeds on NaN metrics; the walk needs a 16-bit state anyway)
     }
   } else {
     const uint32_t j = uint32_t(ov), jj = j < 2048u ? j : 4095u - j;
@@ -396,7 +396,9 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
       const double m1 = row_min16(c1);  // M_it[g_d]
       // its digit: the first lane of the row that holds the minimum
       const unsigned long long at_min = __builtin_amdgcn_ballot_w64(c1 == m1);
-      const uint32_t k1 = uint32_t(__builtin_ctz(uint32_t(at_min >> (16u * dq)) & 0xffffu));
+      // (no lane at all if the inputs held a NaN: any digit will do then, but it must stay a digit)
+      const uint32_t row_bits = uint32_t(at_min >> (16u * dq)) & 0xffffu;
+      const uint32_t k1 = row_bits ? uint32_t(__builtin_ctz(row_bits)) : 0u;
       const double c0 = e0v[q] + m1;
       const bool take = q == 0 || c0 < best;  // d ascends with q: the first minimum stays
       best = take ? c0 : best;

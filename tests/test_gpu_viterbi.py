@@ -144,3 +144,20 @@ def test_ragged_batches_and_device_entry(qz, oracle, hyb):
     qz.viterbi_tiles_dev(dX, 1000, dS2, None)
     qz.synchronize()
     assert torch.equal(dS, dS2)
+
+
+def test_non_finite_inputs_leave_other_tiles_alone(qz, oracle, hyb):
+    """Tiles holding NaN or infinite inputs have no meaningful codes, but the launch must complete, write 16-bit
+    states for them and leave every other tile of the same launch exactly as the CPU algorithm has it."""
+    say("case: non-finite inputs")
+    qz.set_tlut(None)
+    X = oracle.rng_normal(123, 64 * 256).astype(np.float32).reshape(64, 256)
+    bad = {3: np.nan, 17: np.inf, 40: -np.inf}
+    for t, v in bad.items():
+        X[t, :] = v
+    X[29, 100] = np.nan                                      # one NaN in the middle of a sequence
+    good = [t for t in range(64) if t not in bad and t != 29]
+    want = oracle.quantize_tiles(hyb, X[good], fast=True)
+    st, pk = qz.viterbi_tiles(X)
+    assert np.array_equal(st[good], want)
+    assert np.array_equal(pk[good], oracle.pack_trellis(want))
