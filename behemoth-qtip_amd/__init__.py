@@ -45,7 +45,7 @@ class _LinearOutC(C.Structure):
 
 class _OptsC(C.Structure):
     _fields_ = [("sigma_reg", C.c_double), ("scale_override", C.c_double), ("ldl_threads", C.c_int),
-                ("feedback", C.c_int), ("skip_proxy", C.c_int)]
+                ("feedback", C.c_int), ("skip_proxy", C.c_int), ("ldl_device_updates", C.c_int)]
 
 
 class _TimingC(C.Structure):
@@ -94,6 +94,7 @@ def lib():
     L.qtip_sign_vector.restype = None
     L.qtip_rotate_hessian.argtypes = [vp, vp, i, i, u64, d, vp, C.POINTER(d), vp]
     L.qtip_ldl_hessian.argtypes = [vp, i, i, vp]
+    L.qtip_ldl_hessian_device_updates.argtypes = [vp, vp, i, i, vp]
     L.qtip_ldlq_dev.argtypes = [vp, vp, vp, l, l, vp, vp, i, C.POINTER(d)]
     L.qtip_default_opts.argtypes = [C.POINTER(_OptsC)]
     L.qtip_default_opts.restype = None
@@ -179,6 +180,7 @@ class QuantOpts:  # src/quantizer.hpp:11-19
     want_hatW: bool = False
     feedback: int = 0          # 0: fp64 feedback (default), 1: fp32 feedback + bf16 hi/lo split MFMA
     skip_proxy: bool = False
+    ldl_device_updates: bool = False   # True: the LDL's trailing updates run on the GPU (same L bit for bit)
 
 
 @dataclass
@@ -337,6 +339,17 @@ class Quantizer:
             _check(rc)
         hp.t_ldl = time.time() - t0
 
+    def ldl_hessian_device_updates(self, hp: HessPrep, threads=16):
+        """ldl_hessian with the trailing updates of the host's panels on the GPU; hp.L equals ldl_hessian's."""
+        import time
+        t0 = time.time()
+        hp.L = np.zeros((hp.n, hp.n), np.float32)
+        rc = lib().qtip_ldl_hessian_device_updates(self._h, _ptr(hp.HRr), hp.n, threads, _ptr(hp.L))
+        if rc != 0:
+            hp.L = None
+            _check(rc)
+        hp.t_ldl = time.time() - t0
+
     def ldlq_dev(self, dWT, dL, n, m, d_hatWT, dQ, time_viterbi=False, feedback=0):
         vs = C.c_double()
         _check(lib().qtip_ldlq_dev(self._h, _ptr(dWT), _ptr(dL), n, m, _ptr(d_hatWT), _ptr(dQ), feedback,
@@ -370,7 +383,8 @@ class Quantizer:
             cout[k].trellis, cout[k].su_bf16, cout[k].sv = _ptr(o.trellis), _ptr(o.su_bf16), _ptr(o.sv)
             cout[k].hatW = _ptr(o.hatW)
             outs.append(o)
-        co = _OptsC(opt.sigma_reg, opt.scale_override, opt.ldl_threads, opt.feedback, 1 if opt.skip_proxy else 0)
+        co = _OptsC(opt.sigma_reg, opt.scale_override, opt.ldl_threads, opt.feedback, 1 if opt.skip_proxy else 0,
+                    1 if opt.ldl_device_updates else 0)
         return cin, cout, outs, co, keep
 
     @staticmethod

@@ -78,7 +78,12 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
       const double t0 = now_s();
       std::exception_ptr err;
       try {
-        ldl_hessian_impl(c->ring_HRr[g % R].p, groups[g].n, opt.ldl_threads, c->ring_L[g % R].p);
+        if (opt.ldl_device_updates) {
+          QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
+          ldl_hessian_assisted_impl(c, c->ring_HRr[g % R].p, groups[g].n, opt.ldl_threads, c->ring_L[g % R].p);
+        } else {
+          ldl_hessian_impl(c->ring_HRr[g % R].p, groups[g].n, opt.ldl_threads, c->ring_L[g % R].p);
+        }
       } catch (...) {
         err = std::current_exception();
       }

@@ -182,8 +182,12 @@ static bool factor_diagonal(double* A, long n, int kb) {
 // Lower Cholesky of the n x n matrix at A (row stride ld) by right-looking panels of width NBT.  With a team the panel
 // solve and the trailing update are shared out; without one (the diagonal blocks of the outer factorization, which
 // are factored by this same routine with narrow panels) everything runs on the calling thread.
+// assist (outer factorization only): the trailing matrix lives elsewhere.  Before a panel is factored its columns,
+// rows k .. n-1, are fetched into a buffer of row stride kb; after the solve the buffer holds the final columns of C
+// and is handed back, and whoever holds the trailing matrix applies the rank-kb update (every element one chain
+// acc = fma(x_ip, x_jp, acc), p ascending from zero, then c -= acc, as the micro-kernels here do).
 template <int NBT, int TILET>
-bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
+bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top, PanelAssist* assist = nullptr) {
   const Kernels kn = pick_kernels();
   const int MR = kn.MR, NR = kn.NR;
   std::vector<double> packL;
@@ -195,15 +199,21 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
   double* const packB = packA + capA;
   for (int k = 0; k < n; k += NBT) {
     const int kb = std::min(NBT, n - k);
+    // the panel: diagonal block at Ap, the rows below follow with stride ldp
+    double* Ap = assist ? assist->fetch(k, kb) : A + long(k) * ld + k;
+    const long ldp = assist ? kb : ld;
     if constexpr (NBT > 64) {
-      if (!cholesky_panels<64, 96>(A + long(k) * ld + k, ld, kb, nullptr, false)) return false;
+      if (!cholesky_panels<64, 96>(Ap, ldp, kb, nullptr, false)) return false;
     } else {
-      if (!factor_diagonal(A + long(k) * ld + k, ld, kb)) return false;
+      if (!factor_diagonal(Ap, ldp, kb)) return false;
     }
     const int r0 = k + kb, nr = n - r0;
-    if (nr <= 0) break;
+    if (nr <= 0) {
+      if (assist) assist->solved(k, kb, Ap);
+      break;
+    }
     for (int j = 0; j < kb; ++j) {
-      for (int p = 0; p < kb; ++p) L11[size_t(j) * kb + p] = p <= j ? A[long(k + j) * ld + k + p] : 0.0;
+      for (int p = 0; p < kb; ++p) L11[size_t(j) * kb + p] = p <= j ? Ap[long(j) * ldp + p] : 0.0;
       rdiag[j] = 1.0 / L11[size_t(j) * kb + j];
     }
     const int nPA = (nr + MR - 1) / MR, nPB = (nr + NR - 1) / NR;
@@ -237,7 +247,7 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
       const int rb = g * NR, rows = std::min(NR, nr - rb);
       double* x = packB + size_t(g) * NR * kb;  // [p][NR], rows beyond `rows` stay zero
       for (int r = 0; r < rows; ++r) {
-        const double* src = A + long(r0 + rb + r) * ld + k;
+        const double* src = Ap + long(kb + rb + r) * ldp;
         for (int p = 0; p < kb; ++p) x[size_t(p) * NR + r] = src[p];
       }
       for (int b = 0; b < nsb; ++b) {
@@ -250,7 +260,7 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
       }
       for (int r = 0; r < rows; ++r) {
         const int i = rb + r;
-        double* dst = A + long(r0 + i) * ld + k;
+        double* dst = Ap + long(kb + i) * ldp;
         double* pa = packA + size_t(i / MR) * MR * kb + (i % MR);
         for (int p = 0; p < kb; ++p) {
           const double v = x[size_t(p) * NR + r];
@@ -262,6 +272,10 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top) {
     if (team) team->parallel_for(nPB, 2, solve_chunk);
     else
       for (long gl = 0; gl < nPB; ++gl) solve_chunk(gl);
+    if (assist) {
+      assist->solved(k, kb, Ap);
+      continue;
+    }
     // trailing update of the lower triangle, tiles (bi, bj <= bi) largest rows first
     const int nT = (nr + TILET - 1) / TILET;
     const long ntask = long(nT) * (nT + 1) / 2;
@@ -299,18 +313,17 @@ bool cholesky_lower_host(double* A, int n, int threads) {
   return cholesky_panels<NB, TILE>(A, n, n, &team, true);
 }
 
-bool block_ldl_host(double* A, int n, float* L_out, int threads) {
-  if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
-  HostTeam& team = team_of_this_thread(threads);
-  if (!cholesky_panels<NB, TILE>(A, n, n, &team, true)) return false;
-  const int nb = n / 16;
+// L columns c0 .. c0 + nc - 1 from the same columns of C: Cp holds rows c0 .. n-1 of those columns (row stride ldc).
+// L = C * blockdiag(C_bb^-1), 16x16 diagonal blocks and everything above them zero.  false if a value is not finite.
+static bool assemble_L_columns(const double* Cp, long ldc, int c0, int nc, int n, float* L_out, HostTeam& team) {
+  const int nbp = nc / 16;
   // inverse of every 16x16 lower-triangular diagonal block (column by column, forward substitution)
-  std::vector<double> inv(size_t(nb) * 256);
-  team.parallel_for(nb, (nb + team.size() - 1) / team.size(), [&](long bl) {
+  std::vector<double> inv(size_t(nbp) * 256);
+  team.parallel_for(nbp, (nbp + team.size() - 1) / team.size(), [&](long bl) {
     const int b = int(bl);
     double D[16][16], V[16][16];
     for (int i = 0; i < 16; ++i)
-      for (int j = 0; j < 16; ++j) D[i][j] = j <= i ? A[long(b * 16 + i) * n + b * 16 + j] : 0.0;
+      for (int j = 0; j < 16; ++j) D[i][j] = j <= i ? Cp[long(b * 16 + i) * ldc + b * 16 + j] : 0.0;
     for (int c = 0; c < 16; ++c)
       for (int i = 0; i < 16; ++i) {
         double s = i == c ? 1.0 : 0.0;
@@ -322,10 +335,14 @@ bool block_ldl_host(double* A, int n, float* L_out, int threads) {
   std::atomic<int> finite{1};
   team.parallel_for(n, 16, [&](long rl) {
     const int r = int(rl);
+    float* lr = L_out + long(r) * n + c0;
+    if (r < c0) {  // above the diagonal blocks of these columns
+      std::memset(lr, 0, sizeof(float) * size_t(nc));
+      return;
+    }
     bool ok = true;
-    const double* ar = A + long(r) * n;
-    float* lr = L_out + long(r) * n;
-    const int rb = r / 16;
+    const double* ar = Cp + long(r - c0) * ldc;
+    const int rb = std::min(nbp, (r - c0) / 16);  // column blocks strictly left of this row's diagonal block
     for (int bj = 0; bj < rb; ++bj) {
       const double* a = ar + bj * 16;
       const double* iv = &inv[size_t(bj) * 256];
@@ -336,10 +353,40 @@ bool block_ldl_host(double* A, int n, float* L_out, int threads) {
         ok = ok && std::isfinite(s);
       }
     }
-    std::memset(lr + long(rb) * 16, 0, sizeof(float) * size_t(n - rb * 16));  // diagonal block and everything right of it
+    if (rb < nbp) std::memset(lr + long(rb) * 16, 0, sizeof(float) * size_t(nc - rb * 16));  // diagonal block and right of it
     if (!ok) finite.store(0, std::memory_order_relaxed);
   });
   return finite.load() != 0;
+}
+
+bool block_ldl_host(double* A, int n, float* L_out, int threads) {
+  if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
+  HostTeam& team = team_of_this_thread(threads);
+  if (!cholesky_panels<NB, TILE>(A, n, n, &team, true)) return false;
+  return assemble_L_columns(A, n, 0, n, n, L_out, team);
+}
+
+int ldl_panel_width() { return NB; }
+
+bool block_ldl_assisted(int n, float* L_out, int threads, PanelAssist& assist) {
+  if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
+  HostTeam& team = team_of_this_thread(threads);
+  // L is assembled panel by panel from the solved columns as they pass through the host
+  struct Wrap : PanelAssist {
+    PanelAssist& inner;
+    int n;
+    float* L;
+    HostTeam& team;
+    bool finite = true;
+    Wrap(PanelAssist& i, int n_, float* L_, HostTeam& t) : inner(i), n(n_), L(L_), team(t) {}
+    double* fetch(int k, int kb) override { return inner.fetch(k, kb); }
+    void solved(int k, int kb, const double* panel) override {
+      inner.solved(k, kb, panel);  // the update is queued first and runs while L is assembled
+      finite = assemble_L_columns(panel, kb, k, kb, n, L, team) && finite;
+    }
+  } wrap(assist, n, L_out, team);
+  if (!cholesky_panels<NB, TILE>(nullptr, 0, n, &team, true, &wrap)) return false;
+  return wrap.finite;
 }
 
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle (tiled so both reads stay in cache)

@@ -1,0 +1,124 @@
+// Host fp64 block LDL with the trailing updates on the GPU (host_ldl.cpp, block_ldl_assisted): the host factors and
+// solves one 512-column panel at a time in its own arithmetic, the device holds the symmetric fp64 work matrix and
+// applies the rank-512 updates.  v_mfma_f64_16x16x4_f64 accumulates its four products like a chain of fused
+// multiply-adds in ascending k (checked bit for bit against std::fma chains), and the host's micro-kernels form every
+// element of an update as exactly such a chain over the panel depth from zero followed by one subtraction, so the
+// factor is the host's bit for bit.
+#include <algorithm>
+
+#include "quantizer_impl.hpp"
+
+namespace qtipmi {
+namespace {
+
+typedef double double4_t __attribute__((ext_vector_type(4)));
+
+// A[i][j] = (H[i][j] + H[j][i]) / 2 in fp64, lower triangle (symmetrize_lower_host)
+__global__ void symmetrize_lower_kernel(const float* __restrict__ H, long n, double* __restrict__ A) {
+  const long j = long(blockIdx.x) * blockDim.x + threadIdx.x, i = blockIdx.y;
+  if (j > i || j >= n) return;
+  A[i * n + j] = 0.5 * (double(H[i * n + j]) + double(H[j * n + i]));
+}
+
+// C[i][j] -= sum_p X[i][p] * X[j][p] for the 128 x 128 tile (bi, bj <= bi) of the nr x nr lower triangle.
+// X: nr x kb (row stride kb), C: row stride ldc.  256 threads, 2 x 2 waves of 64 x 64, K staged 16 at a time.
+constexpr int UT = 128, UK = 16;
+__global__ __launch_bounds__(256) void rank_update_lower_kernel(const double* __restrict__ X, int nr, int kb,
+                                                              double* __restrict__ C, long ldc) {
+  // tile index -> (bi, bj), rows of the triangle enumerated from the top
+  int bi = 0, rem = blockIdx.x;
+  while (rem > bi) {
+    rem -= bi + 1;
+    ++bi;
+  }
+  const int bj = rem, i0 = bi * UT, j0 = bj * UT;
+  __shared__ double Xi[UK][UT + 4], Xj[UK][UT + 4];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
+  double4_t acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
+  const int lrow = t & 127, lk = (t >> 7) * 8;
+  for (int k0 = 0; k0 < kb; k0 += UK) {
+    {
+      const int ri = i0 + lrow, rj = j0 + lrow;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const int kk = k0 + lk + q;
+        Xi[lk + q][lrow] = (ri < nr && kk < kb) ? X[long(ri) * kb + kk] : 0.0;
+        Xj[lk + q][lrow] = (rj < nr && kk < kb) ? X[long(rj) * kb + kk] : 0.0;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < UK; kk += 4) {
+      const int kr = kk + (lane >> 4), c = lane & 15;
+      double a[4], b[4];
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) a[mi] = Xi[kr][wm * 64 + mi * 16 + c];
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) b[ni] = Xj[kr][wn * 64 + ni * 16 + c];
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int gi = i0 + wm * 64 + mi * 16 + (lane >> 4) + 4 * v, gj = j0 + wn * 64 + ni * 16 + (lane & 15);
+        if (gi < nr && gj <= gi) C[long(gi) * ldc + gj] -= acc[mi][ni][v];
+      }
+}
+
+struct DeviceTrailing final : PanelAssist {
+  qtip_ctx* c;
+  long n;
+  hipStream_t s;
+  DeviceTrailing(qtip_ctx* c_, long n_) : c(c_), n(n_), s(c_->ldl_stream) {}
+  double* fetch(int k, int kb) override {
+    const long rows = n - k;
+    QTIP_HIP(hipMemcpy2DAsync(c->ldl_panel.p, size_t(kb) * 8, c->ldl_A.p + long(k) * n + k, size_t(n) * 8,
+                              size_t(kb) * 8, size_t(rows), hipMemcpyDeviceToHost, s));
+    QTIP_HIP(hipStreamSynchronize(s));
+    return c->ldl_panel.p;
+  }
+  void solved(int k, int kb, const double* panel) override {
+    const long r0 = k + kb, nr = n - r0;
+    if (nr <= 0) return;
+    // the stream orders this copy before the next fetch into the same page-locked buffer
+    QTIP_HIP(hipMemcpyAsync(c->ldl_X.p, panel + long(kb) * kb, size_t(nr) * kb * 8, hipMemcpyHostToDevice, s));
+    const long nt = (nr + UT - 1) / UT, tiles = nt * (nt + 1) / 2;
+    rank_update_lower_kernel<<<dim3(unsigned(tiles)), dim3(256), 0, s>>>(c->ldl_X.p, int(nr), kb,
+                                                                        c->ldl_A.p + r0 * n + r0, n);
+    QTIP_HIP(hipGetLastError());
+  }
+};
+
+}  // namespace
+
+void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int threads, float* host_L) {
+  QTIP_REQUIRE(c && n > 0 && n % 16 == 0 && host_HRr && host_L, "ldl_hessian (device updates): bad arguments (n = %d)", n);
+  if (!c->ldl_stream) QTIP_HIP(hipStreamCreateWithFlags(&c->ldl_stream, hipStreamNonBlocking));
+  hipStream_t s = c->ldl_stream;
+  const size_t nn = size_t(n) * n, nb = size_t(ldl_panel_width());
+  c->ldl_A.ensure(nn);
+  c->ldl_H.ensure(nn);
+  c->ldl_X.ensure(size_t(n) * nb);
+  if (c->ldl_panel.n < size_t(n) * nb) c->ldl_panel.alloc(size_t(n) * nb);
+  QTIP_HIP(hipMemcpyAsync(c->ldl_H.p, host_HRr, nn * 4, hipMemcpyHostToDevice, s));
+  symmetrize_lower_kernel<<<dim3(unsigned((n + 255) / 256), unsigned(n)), dim3(256), 0, s>>>(c->ldl_H.p, n, c->ldl_A.p);
+  QTIP_HIP(hipGetLastError());
+  DeviceTrailing dev(c, n);
+  const bool ok = block_ldl_assisted(n, host_L, threads, dev);
+  QTIP_HIP(hipStreamSynchronize(s));
+  if (!ok) throw Error(QTIP_E_NOT_PD, "block LDL failed (H not PD)");
+}
+
+}  // namespace qtipmi

@@ -104,6 +104,10 @@ void qtip_destroy(qtip_ctx* ctx) {
   int prev = 0;
   (void)hipGetDevice(&prev);
   (void)hipSetDevice(ctx->device);
+  if (ctx->ldl_stream) {
+    (void)hipStreamSynchronize(ctx->ldl_stream);
+    (void)hipStreamDestroy(ctx->ldl_stream);
+  }
   if (ctx->stream) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipStreamDestroy(ctx->stream);
@@ -238,6 +242,7 @@ void qtip_default_opts(qtip_opts* o) {
   o->ldl_threads = 16;
   o->feedback = 0;
   o->skip_proxy = 0;
+  o->ldl_device_updates = 0;
 }
 
 void qtip_pack_trellis(const uint16_t* states, long B, uint16_t* packed) { pack_trellis_host(states, B, packed); }
@@ -398,6 +403,14 @@ int qtip_ldl_hessian(const float* host_HRr, int n, int threads, float* host_L) {
   return guarded([&] { ldl_hessian_impl(host_HRr, n, threads, host_L); });
 }
 
+int qtip_ldl_hessian_device_updates(qtip_ctx* ctx, const float* host_HRr, int n, int threads, float* host_L) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "null context");
+    DeviceGuard g(ctx);
+    ldl_hessian_assisted_impl(ctx, host_HRr, n, threads, host_L);
+  });
+}
+
 int qtip_ldlq_dev(qtip_ctx* ctx, const float* dev_WT, const float* dev_L, long n, long m, float* dev_hatWT,
                   uint16_t* dev_Q, int feedback, double* vit_seconds) {
   return guarded([&] {
@@ -434,7 +447,8 @@ int qtip_quantize_group_h(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, i
     auto t0 = std::chrono::steady_clock::now();
     rotate_hessian_impl(ctx, H, h_on_device != 0, n, seed, o.sigma_reg, su.data(), &creg, HRr.data());
     auto t1 = std::chrono::steady_clock::now();
-    ldl_hessian_impl(HRr.data(), n, o.ldl_threads, L.data());
+    if (o.ldl_device_updates) ldl_hessian_assisted_impl(ctx, HRr.data(), n, o.ldl_threads, L.data());
+    else ldl_hessian_impl(HRr.data(), n, o.ldl_threads, L.data());
     auto t2 = std::chrono::steady_clock::now();
     T.rht = std::chrono::duration<double>(t1 - t0).count();
     T.ldl_cpu = std::chrono::duration<double>(t2 - t1).count();

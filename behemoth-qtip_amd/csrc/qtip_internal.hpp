@@ -131,6 +131,19 @@ struct HostScratch {
 
 // fp64 block LDL on the host (host_ldl.cpp). A: n x n fp64, lower triangle used, destroyed. Returns false if not PD.
 bool block_ldl_host(double* A, int n, float* L_out, int threads);
+// The same factorization with the trailing matrix kept by someone else (the GPU): the host factors and solves one
+// panel of ldl_panel_width() columns at a time.  fetch(k, kb) returns a buffer of row stride kb holding rows k .. n-1
+// of the columns k .. k+kb-1 as updated so far; solved(k, kb, panel) receives it back with the final columns of the
+// Cholesky factor: the rows kb .. n-k-1 of it are the operand of the rank-kb update of the trailing matrix, which
+// must form every element as one chain acc = fma(x_ip, x_jp, acc), p = 0 .. kb-1 from zero, then c -= acc, for L to
+// equal block_ldl_host's bit for bit.
+struct PanelAssist {
+  virtual double* fetch(int k, int kb) = 0;
+  virtual void solved(int k, int kb, const double* panel) = 0;
+  virtual ~PanelAssist() = default;
+};
+int ldl_panel_width();
+bool block_ldl_assisted(int n, float* L_out, int threads, PanelAssist& assist);
 // lower Cholesky in place (lower triangle of the n x n fp64 matrix A); false if not positive definite
 bool cholesky_lower_host(double* A, int n, int threads);
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle

@@ -16,6 +16,12 @@ struct qtip_ctx {
   qtipmi::Rht rht;
   qtipmi::DBuf<double> scratch;
   qtipmi::HBuf<float> ring_HRr[3], ring_L[3];  // page-locked staging of run_groups, kept between calls
+  // LDL with the trailing updates on the device (ldl_assist.hip): own stream, fp64 work matrix, fp32 upload of HRr,
+  // solved panel rows, page-locked panel buffer; allocated on first use
+  hipStream_t ldl_stream = nullptr;
+  qtipmi::DBuf<double> ldl_A, ldl_X;
+  qtipmi::DBuf<float> ldl_H;
+  qtipmi::HBuf<double> ldl_panel;
 };
 
 namespace qtipmi {
@@ -23,6 +29,7 @@ void ensure_viterbi_workspace(qtip_ctx* c);
 void rotate_hessian_impl(qtip_ctx* c, const float* H, bool on_device, int n, uint64_t seed, double sigma_reg,
                          float* host_su, double* creg, float* host_HRr);
 void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L);
+void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int threads, float* host_L);
 void ldlq_impl(qtip_ctx* c, const float* dWT, const float* dL, long n, long m, float* d_hatWT, uint16_t* dQ,
                int feedback, double* vit_seconds);
 void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,

@@ -87,6 +87,13 @@ int qtip_rotate_hessian(qtip_ctx* ctx, const float* H, int h_on_device, int n, u
  * HRr n x n fp32 in, L n x n fp32 out (strictly block-lower). */
 int qtip_ldl_hessian(const float* host_HRr, int n, int threads, float* host_L);
 
+/* The same factorization with the trailing updates of the host's panels on the GPU.  No counterpart in the
+ * reference (its ldl_hessian is host only, src/quantizer.cpp:154-165): the host still factors and solves every
+ * panel in fp64 with its own code, the device keeps the fp64 work matrix and applies the rank-512 updates on the
+ * matrix cores in the host's own order of operations, so host_L is qtip_ldl_hessian's bit for bit.  Works on a
+ * stream of its own inside ctx; may run on a side thread while another thread quantizes through the same ctx. */
+int qtip_ldl_hessian_device_updates(qtip_ctx* ctx, const float* host_HRr, int n, int threads, float* host_L);
+
 /* ldlq_gpu, src/quantizer.cpp:30-89.  WT n x m fp32 (scaled), L n x n fp32, both on the device;
  * outputs hatWT n x m fp32 and Q[(m/16)*(n/16)][128] u16 on the device.  feedback as in qtip_opts;
  * vit_seconds may be NULL. */
@@ -122,6 +129,8 @@ typedef struct { /* QuantOpts, src/quantizer.hpp:11-19 */
   int feedback;          /* 0: fp64 feedback sums + fp64 MFMA prod cache (default, tracks the fp64 CPU form);
                             1: fp32 feedback sums + bf16 hi/lo split MFMA prod cache (the reference GPU's arithmetic) */
   int skip_proxy;        /* 1: leave proxy fields 0 */
+  int ldl_device_updates;/* 0 (default): block LDL on the host as in the reference; 1: qtip_run_groups and
+                            qtip_quantize_group_h factor through qtip_ldl_hessian_device_updates (same L) */
 } qtip_opts;
 void qtip_default_opts(qtip_opts* o);
 
