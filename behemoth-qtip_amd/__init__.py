@@ -180,7 +180,7 @@ class QuantOpts:  # src/quantizer.hpp:11-19
     want_hatW: bool = False
     feedback: int = 0          # 0: fp64 feedback (default), 1: fp32 feedback + bf16 hi/lo split MFMA
     skip_proxy: bool = False
-    ldl_device_updates: bool = False   # True: the LDL's trailing updates run on the GPU (same L bit for bit)
+    ldl_device_updates: bool = True    # the LDL's trailing updates run on the GPU (same L bit for bit); False: host alone
 
 
 @dataclass

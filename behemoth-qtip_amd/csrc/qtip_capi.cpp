@@ -242,7 +242,7 @@ void qtip_default_opts(qtip_opts* o) {
   o->ldl_threads = 16;
   o->feedback = 0;
   o->skip_proxy = 0;
-  o->ldl_device_updates = 0;
+  o->ldl_device_updates = 1;
 }
 
 void qtip_pack_trellis(const uint16_t* states, long B, uint16_t* packed) { pack_trellis_host(states, B, packed); }

@@ -36,6 +36,9 @@ struct QuantOpts {  // src/quantizer.hpp:11-19
   bool share_su = true;
   std::string dump_dir;  // if set: W (fp32) and, unless want_hatW, the reconstructed hatW (fp32) are written per linear
   bool want_hatW = false;
+  // not in the reference: the group calls hand the trailing updates of the host LDL to the GPU (the factor is the
+  // host's bit for bit); false keeps the factorization on the host alone
+  bool ldl_device_updates = true;
 };
 
 struct LinearIn {  // src/quantizer.hpp:21-28
@@ -189,6 +192,7 @@ inline std::vector<LinearOut> quantize_group(hipStream_t, Gemm&, const std::vect
   qtip_opts co;
   qtip_default_opts(&co);
   co.sigma_reg = opt.sigma_reg, co.scale_override = opt.scale_override, co.ldl_threads = opt.ldl_threads;
+  co.ldl_device_updates = opt.ldl_device_updates ? 1 : 0;
   qtip_timing ct{};
   ct.rht = hp.t_rot, ct.ldl_cpu = hp.t_ldl;
   detail::check(qtip_quantize_group(detail::context(), int(lins.size()), cin.data(), n, hp.seed, hp.su.data(), hp.creg,
@@ -272,6 +276,7 @@ inline std::vector<std::vector<LinearOut>> run_groups(const std::vector<GroupSpe
   qtip_opts co;
   qtip_default_opts(&co);
   co.sigma_reg = opt.sigma_reg, co.scale_override = opt.scale_override, co.ldl_threads = opt.ldl_threads;
+  co.ldl_device_updates = opt.ldl_device_updates ? 1 : 0;
   std::vector<qtip_timing> ct(ng);
   std::vector<double> waits(ng, 0.0);
   detail::check(qtip_run_groups(detail::context(), int(ng), cg.data(), &co, ct.data(), waits.data()), "run_groups");

@@ -116,7 +116,8 @@ def run_group(args, pkg):
     n = H.shape[0]
     ms = [int(w.shape[0]) for w in Ws]
     lins = [pkg.LinearIn("w%d" % i, m, w_f32=w) for i, (m, w) in enumerate(zip(ms, Ws))]
-    opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback)
+    opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback,
+                        ldl_device_updates=not args.host_ldl)
     weights_per_step = sum(ms) * n
 
     stats = {}
@@ -152,11 +153,13 @@ def run_group(args, pkg):
     extra.update(gpu_only_Mweights_s=weights_per_step / gpu_s / 1e6,
                  serial_Mweights_s=weights_per_step / (gpu_s + stats["ldl_s"]) / 1e6,
                  viterbi_only_Mweights_s=weights_per_step / stats["viterbi_s"] / 1e6,
-                 proxy_in_timed_region=True, ldl_threads=args.ldl_threads, feedback=args.feedback)
+                 proxy_in_timed_region=True, ldl_threads=args.ldl_threads, feedback=args.feedback,
+                 ldl_device_updates=not args.host_ldl)
     names = {2: "config2: 1024x1024 group", 3: "config3: 12288x12288 q-proj group",
              4: "config4: gate+up 2x(28672x12288) group", 5: "config5: 12288x28672 down-proj group"}
     return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
-                vit_launch_weights=ntr * 256, workload=names[cfg] + " (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)",
+                vit_launch_weights=ntr * 256, workload=names[cfg] + (" (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)" if args.host_ldl else
+                                       " (RHT + fp64 LDL: host panels, GPU trailing updates + LDLQ + 2-pass Viterbi + pack)"),
                 extra=extra)
 
 
@@ -168,6 +171,9 @@ def main():
     ap.add_argument("--config", type=int, default=5, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--ldl-threads", type=int, default=16, help="OpenMP team of the host LDL")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--host-ldl", action="store_true",
+                    help="keep the fp64 block LDL on the host alone, as the reference does (default: the host factors and "
+                         "solves the panels and hands the trailing updates to the GPU; the factor is the same bit for bit)")
     ap.add_argument("--feedback", type=int, default=0, choices=[0, 1],
                     help="0: fp64 LDLQ feedback (default); 1: fp32 feedback + bf16 hi/lo split MFMA prod cache")
     ap.add_argument("--pmc-calibration", action="store_true",

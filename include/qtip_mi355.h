@@ -129,8 +129,9 @@ typedef struct { /* QuantOpts, src/quantizer.hpp:11-19 */
   int feedback;          /* 0: fp64 feedback sums + fp64 MFMA prod cache (default, tracks the fp64 CPU form);
                             1: fp32 feedback sums + bf16 hi/lo split MFMA prod cache (the reference GPU's arithmetic) */
   int skip_proxy;        /* 1: leave proxy fields 0 */
-  int ldl_device_updates;/* 0 (default): block LDL on the host as in the reference; 1: qtip_run_groups and
-                            qtip_quantize_group_h factor through qtip_ldl_hessian_device_updates (same L) */
+  int ldl_device_updates;/* 1 (default): qtip_run_groups and qtip_quantize_group_h factor through
+                            qtip_ldl_hessian_device_updates (panels on the host, trailing updates on the GPU, same L
+                            bit for bit); 0: block LDL on the host alone, as in the reference */
 } qtip_opts;
 void qtip_default_opts(qtip_opts* o);
 
