@@ -23,7 +23,7 @@ __global__ void symmetrize_lower_kernel(const float* __restrict__ H, long n, dou
 // C[i][j] -= sum_p X[i][p] * X[j][p] for the 128 x 128 tile (bi, bj <= bi) of the nr x nr lower triangle.
 // X: nr x kb (row stride kb), C: row stride ldc.  256 threads, 2 x 2 waves of 64 x 64, K staged 16 at a time.
 constexpr int UT = 128, UK = 16;
-__global__ __launch_bounds__(256) void rank_update_lower_kernel(const double* __restrict__ X, int nr, int kb,
+__global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double* __restrict__ X, int nr, int kb,
                                                               double* __restrict__ C, long ldc) {
   // tile index -> (bi, bj), rows of the triangle enumerated from the top
   int bi = 0, rem = blockIdx.x;
@@ -40,17 +40,26 @@ __global__ __launch_bounds__(256) void rank_update_lower_kernel(const double* __
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
   const int lrow = t & 127, lk = (t >> 7) * 8;
-  for (int k0 = 0; k0 < kb; k0 += UK) {
-    {
-      const int ri = i0 + lrow, rj = j0 + lrow;
+  const int ri = i0 + lrow, rj = j0 + lrow;
+  // the next 16 columns of the two row blocks travel from HBM while the matrix cores work on the present ones
+  double pi[8], pj[8];
+  auto fetch = [&](int k0) {
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const int kk = k0 + lk + q;
-        Xi[lk + q][lrow] = (ri < nr && kk < kb) ? X[long(ri) * kb + kk] : 0.0;
-        Xj[lk + q][lrow] = (rj < nr && kk < kb) ? X[long(rj) * kb + kk] : 0.0;
-      }
+    for (int q = 0; q < 8; ++q) {
+      const int kk = k0 + lk + q;
+      pi[q] = (ri < nr && kk < kb) ? X[long(ri) * kb + kk] : 0.0;
+      pj[q] = (rj < nr && kk < kb) ? X[long(rj) * kb + kk] : 0.0;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < kb; k0 += UK) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      Xi[lk + q][lrow] = pi[q];
+      Xj[lk + q][lrow] = pj[q];
     }
     __syncthreads();
+    if (k0 + UK < kb) fetch(k0 + UK);
 #pragma unroll
     for (int kk = 0; kk < UK; kk += 4) {
       const int kr = kk + (lane >> 4), c = lane & 15;
