@@ -112,17 +112,21 @@ struct DeviceTrailing final : PanelAssist {
 
 }  // namespace
 
-void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int threads, float* host_L) {
-  QTIP_REQUIRE(c && n > 0 && n % 16 == 0 && host_HRr && host_L, "ldl_hessian (device updates): bad arguments (n = %d)", n);
+// dev_HRr (optional): the rotated Hessian already on the device (then host_HRr is not read)
+void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int threads, float* host_L,
+                               const float* dev_HRr) {
+  QTIP_REQUIRE(c && n > 0 && n % 16 == 0 && (host_HRr || dev_HRr) && host_L,
+               "ldl_hessian (device updates): bad arguments (n = %d)", n);
   if (!c->ldl_stream) QTIP_HIP(hipStreamCreateWithFlags(&c->ldl_stream, hipStreamNonBlocking));
   hipStream_t s = c->ldl_stream;
   const size_t nn = size_t(n) * n, nb = size_t(ldl_panel_width());
   c->ldl_A.ensure(nn);
-  c->ldl_H.ensure(nn);
+  if (!dev_HRr) c->ldl_H.ensure(nn);
   c->ldl_X.ensure(size_t(n) * nb);
   if (c->ldl_panel.n < size_t(n) * nb) c->ldl_panel.alloc(size_t(n) * nb);
-  QTIP_HIP(hipMemcpyAsync(c->ldl_H.p, host_HRr, nn * 4, hipMemcpyHostToDevice, s));
-  symmetrize_lower_kernel<<<dim3(unsigned((n + 255) / 256), unsigned(n)), dim3(256), 0, s>>>(c->ldl_H.p, n, c->ldl_A.p);
+  if (!dev_HRr) QTIP_HIP(hipMemcpyAsync(c->ldl_H.p, host_HRr, nn * 4, hipMemcpyHostToDevice, s));
+  symmetrize_lower_kernel<<<dim3(unsigned((n + 255) / 256), unsigned(n)), dim3(256), 0, s>>>(dev_HRr ? dev_HRr : c->ldl_H.p, n,
+                                                                                              c->ldl_A.p);
   QTIP_HIP(hipGetLastError());
   DeviceTrailing dev(c, n);
   const bool ok = block_ldl_assisted(n, host_L, threads, dev);

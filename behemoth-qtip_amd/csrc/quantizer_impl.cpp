@@ -47,15 +47,18 @@ struct Events {
 
 // ---------------------------------------------------------------- rotate_hessian, src/quantizer.cpp:124-152
 void rotate_hessian_impl(qtip_ctx* c, const float* H, bool on_device, int n, uint64_t seed, double sigma_reg,
-                         float* host_su, double* creg, float* host_HRr) {
-  QTIP_REQUIRE(n > 0 && H && host_su && creg && host_HRr, "rotate_hessian: bad arguments");
+                         float* host_su, double* creg, float* host_HRr, float* dev_HRr) {
+  // dev_HRr (optional): n x n device buffer of the caller in which the rotated Hessian is left; host_HRr may then be
+  // null (no copy to the host)
+  QTIP_REQUIRE(n > 0 && H && host_su && creg && (host_HRr || dev_HRr), "rotate_hessian: bad arguments");
   QTIP_REQUIRE(had_K(n) > 0, "unsupported hadamard dim %d", n);
   hipStream_t s = c->stream;
   SplitMix rng(seed);
   for (int i = 0; i < n; ++i) host_su[i] = rng.sign();
   DBuf<float> d_su{size_t(n)};
   QTIP_HIP(hipMemcpyAsync(d_su, host_su, size_t(n) * 4, hipMemcpyHostToDevice, s));
-  DBuf<float> Ht(size_t(n) * n), HR(size_t(n) * n);
+  DBuf<float> Ht(size_t(n) * n), HR_own(dev_HRr ? 0 : size_t(n) * n);
+  float* const HR = dev_HRr ? dev_HRr : HR_own.p;
   QTIP_HIP(hipMemcpyAsync(Ht, H, size_t(n) * n * 4, on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, s));
   // regularize_H: H += sigma_reg * mean(diag(H)) * I, before the rotation
   const double dsum = c->rht.reduce(Ht, n, nullptr, 0, n, n, 3);
@@ -65,7 +68,7 @@ void rotate_hessian_impl(qtip_ctx* c, const float* H, bool on_device, int n, uin
   c->rht.hadamard_rows(Ht, n, n, n, true, d_su, d_su);
   c->rht.transpose(Ht, n, n, n, HR, n);
   c->rht.hadamard_rows(HR, n, n, n, true);
-  QTIP_HIP(hipMemcpyAsync(host_HRr, HR, size_t(n) * n * 4, hipMemcpyDeviceToHost, s));
+  if (host_HRr) QTIP_HIP(hipMemcpyAsync(host_HRr, HR, size_t(n) * n * 4, hipMemcpyDeviceToHost, s));
   QTIP_HIP(hipStreamSynchronize(s));
 }
 
@@ -155,11 +158,11 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
 // ---------------------------------------------------------------- quantize_group, src/quantizer.cpp:176-346
 void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
                          double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
-                         qtip_linear_out* outs, qtip_timing* tm) {
+                         qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr) {
   QTIP_REQUIRE(nlin > 0 && lins && outs && host_su && host_L, "quantize_group: bad arguments");
   QTIP_REQUIRE(n % 128 == 0, "LDLQ needs n %% 128 == 0 (n = %d)", n);
   QTIP_REQUIRE(had_K(n) > 0 && n / had_K(n) <= 8192, "unsupported hadamard dim %d", n);
-  QTIP_REQUIRE(opt.skip_proxy || host_HRr, "quantize_group: HRr is needed for the proxy");
+  QTIP_REQUIRE(opt.skip_proxy || host_HRr || dev_HRr, "quantize_group: HRr is needed for the proxy");
   hipStream_t s = c->stream;
   qtip_timing T{};
   if (tm) T.rht = tm->rht, T.ldl_cpu = tm->ldl_cpu;
@@ -246,8 +249,10 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
 
   // ---- proxy (rotated, scaled domain; Wscale cancels), src/quantizer.cpp:268-303
   if (!opt.skip_proxy) {
-    DBuf<float> HR(size_t(n) * n);
-    QTIP_HIP(hipMemcpyAsync(HR, host_HRr, HR.bytes(), hipMemcpyHostToDevice, s));
+    // the rotated Hessian: the caller's device copy if it kept one, else uploaded
+    DBuf<float> HR_own(dev_HRr ? 0 : size_t(n) * n);
+    if (!dev_HRr) QTIP_HIP(hipMemcpyAsync(HR_own, host_HRr, HR_own.bytes(), hipMemcpyHostToDevice, s));
+    const float* const HR = dev_HRr ? dev_HRr : HR_own.p;
     DBuf<uint16_t> stack;
     for (int li = 0; li < nlin; ++li) {
       const long m = lins[li].m;
