@@ -46,10 +46,14 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
   const int R = std::min(3, ng);
   reserve_group_ring(c, nmax, R);
   // with the LDL's updates on the device the rotated Hessian never leaves it: the factorization reads it there and so
-  // does the proxy, which saves one copy down and two up per group (HRr in the host ring is then unused)
+  // does the proxy, and the factor goes up column block by column block as it is assembled: one copy down and three up
+  // fewer per group on the quantizing stream (HRr in the host ring is then unused)
   const bool keep_dev = opt.ldl_device_updates != 0;
   if (keep_dev)
-    for (int b = 0; b < R; ++b) c->ring_dHRr[b].ensure(size_t(nmax) * nmax);
+    for (int b = 0; b < R; ++b) {
+      c->ring_dHRr[b].ensure(size_t(nmax) * nmax);
+      c->ring_dL[b].ensure(size_t(nmax) * nmax);
+    }
   const size_t ngz = size_t(ng);
   std::vector<std::vector<float>> su;
   for (int b = 0; b < R; ++b) su.emplace_back(std::vector<float>(static_cast<size_t>(nmax), 0.0f));
@@ -86,7 +90,8 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
       try {
         if (opt.ldl_device_updates) {
           QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
-          ldl_hessian_assisted_impl(c, nullptr, groups[g].n, opt.ldl_threads, c->ring_L[g % R].p, c->ring_dHRr[g % R].p);
+          ldl_hessian_assisted_impl(c, nullptr, groups[g].n, opt.ldl_threads, c->ring_L[g % R].p, c->ring_dHRr[g % R].p,
+                                    c->ring_dL[g % R].p);
         } else {
           ldl_hessian_impl(c->ring_HRr[g % R].p, groups[g].n, opt.ldl_threads, c->ring_L[g % R].p);
         }
@@ -124,7 +129,7 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
         T.ldl_cpu = t_ldl[size_t(g)];
         quantize_group_impl(c, groups[g].nlin, groups[g].lins, groups[g].n, groups[g].seed, su[size_t(b)].data(),
                             creg[size_t(g)], keep_dev ? nullptr : c->ring_HRr[b].p, c->ring_L[b].p, opt, groups[g].outs, &T,
-                            keep_dev ? c->ring_dHRr[b].p : nullptr);
+                            keep_dev ? c->ring_dHRr[b].p : nullptr, keep_dev ? c->ring_dL[b].p : nullptr);
         if (tms) tms[g] = T;
       }
     } catch (...) {

@@ -383,6 +383,7 @@ bool block_ldl_assisted(int n, float* L_out, int threads, PanelAssist& assist) {
     void solved(int k, int kb, const double* panel) override {
       inner.solved(k, kb, panel);  // the update is queued first and runs while L is assembled
       finite = assemble_L_columns(panel, kb, k, kb, n, L, team) && finite;
+      inner.assembled(k, kb);
     }
   } wrap(assist, n, L_out, team);
   if (!cholesky_panels<NB, TILE>(nullptr, 0, n, &team, true, &wrap)) return false;

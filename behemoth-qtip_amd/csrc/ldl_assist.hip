@@ -90,7 +90,14 @@ struct DeviceTrailing final : PanelAssist {
   qtip_ctx* c;
   long n;
   hipStream_t s;
-  DeviceTrailing(qtip_ctx* c_, long n_) : c(c_), n(n_), s(c_->ldl_stream) {}
+  const float* host_L;
+  float* dev_L;  // optional: L is also left on the device, column block by column block as it is assembled
+  DeviceTrailing(qtip_ctx* c_, long n_, const float* hL, float* dL) : c(c_), n(n_), s(c_->ldl_stream), host_L(hL), dev_L(dL) {}
+  void assembled(int k, int kb) override {
+    if (!dev_L) return;
+    QTIP_HIP(hipMemcpy2DAsync(dev_L + k, size_t(n) * 4, host_L + k, size_t(n) * 4, size_t(kb) * 4, size_t(n),
+                              hipMemcpyHostToDevice, s));
+  }
   double* fetch(int k, int kb) override {
     const long rows = n - k;
     QTIP_HIP(hipMemcpy2DAsync(c->ldl_panel.p, size_t(kb) * 8, c->ldl_A.p + long(k) * n + k, size_t(n) * 8,
@@ -113,8 +120,9 @@ struct DeviceTrailing final : PanelAssist {
 }  // namespace
 
 // dev_HRr (optional): the rotated Hessian already on the device (then host_HRr is not read)
+// dev_L (optional): n x n device buffer that receives L as well
 void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int threads, float* host_L,
-                               const float* dev_HRr) {
+                               const float* dev_HRr, float* dev_L) {
   QTIP_REQUIRE(c && n > 0 && n % 16 == 0 && (host_HRr || dev_HRr) && host_L,
                "ldl_hessian (device updates): bad arguments (n = %d)", n);
   if (!c->ldl_stream) QTIP_HIP(hipStreamCreateWithFlags(&c->ldl_stream, hipStreamNonBlocking));
@@ -128,7 +136,7 @@ void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int th
   symmetrize_lower_kernel<<<dim3(unsigned((n + 255) / 256), unsigned(n)), dim3(256), 0, s>>>(dev_HRr ? dev_HRr : c->ldl_H.p, n,
                                                                                               c->ldl_A.p);
   QTIP_HIP(hipGetLastError());
-  DeviceTrailing dev(c, n);
+  DeviceTrailing dev(c, n, host_L, dev_L);
   const bool ok = block_ldl_assisted(n, host_L, threads, dev);
   QTIP_HIP(hipStreamSynchronize(s));
   if (!ok) throw Error(QTIP_E_NOT_PD, "block LDL failed (H not PD)");

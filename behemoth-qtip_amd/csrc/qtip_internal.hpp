@@ -140,6 +140,8 @@ bool block_ldl_host(double* A, int n, float* L_out, int threads);
 struct PanelAssist {
   virtual double* fetch(int k, int kb) = 0;
   virtual void solved(int k, int kb, const double* panel) = 0;
+  // the columns k .. k+kb-1 of L_out are final (all n rows)
+  virtual void assembled(int k, int kb) {}
   virtual ~PanelAssist() = default;
 };
 int ldl_panel_width();

@@ -158,7 +158,7 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
 // ---------------------------------------------------------------- quantize_group, src/quantizer.cpp:176-346
 void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
                          double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
-                         qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr) {
+                         qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr, const float* dev_L) {
   QTIP_REQUIRE(nlin > 0 && lins && outs && host_su && host_L, "quantize_group: bad arguments");
   QTIP_REQUIRE(n % 128 == 0, "LDLQ needs n %% 128 == 0 (n = %d)", n);
   QTIP_REQUIRE(had_K(n) > 0 && n / had_K(n) <= 8192, "unsupported hadamard dim %d", n);
@@ -231,8 +231,9 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
     }
   }
 
-  DBuf<float> Ld(size_t(n) * n);
-  QTIP_HIP(hipMemcpyAsync(Ld, host_L, size_t(n) * n * 4, hipMemcpyHostToDevice, s));
+  // the factor: the caller's device copy if it kept one, else uploaded
+  DBuf<float> Ld(dev_L ? 0 : size_t(n) * n);
+  if (!dev_L) QTIP_HIP(hipMemcpyAsync(Ld, host_L, size_t(n) * n * 4, hipMemcpyHostToDevice, s));
   QTIP_HIP(hipStreamSynchronize(s));
   T.load += now_s() - t0;
   t0 = now_s();
@@ -241,7 +242,7 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
   DBuf<float> hatWT(size_t(n) * mt);
   DBuf<uint16_t> Q(size_t(mt / 16) * (n / 16) * 128);
   double vit = 0;
-  ldlq_impl(c, WT, Ld, n, mt, hatWT, Q, opt.feedback, &vit);
+  ldlq_impl(c, WT, dev_L ? dev_L : Ld.p, n, mt, hatWT, Q, opt.feedback, &vit);
   T.ldlq += now_s() - t0;
   T.viterbi += vit;
   t0 = now_s();

@@ -16,7 +16,7 @@ struct qtip_ctx {
   qtipmi::Rht rht;
   qtipmi::DBuf<double> scratch;
   qtipmi::HBuf<float> ring_HRr[3], ring_L[3];  // page-locked staging of run_groups, kept between calls
-  qtipmi::DBuf<float> ring_dHRr[3];            // run_groups with device-updated LDL: the rotated Hessians stay here
+  qtipmi::DBuf<float> ring_dHRr[3], ring_dL[3];  // run_groups with device-updated LDL: rotated Hessians and factors stay here
   // LDL with the trailing updates on the device (ldl_assist.hip): own stream, fp64 work matrix, fp32 upload of HRr,
   // solved panel rows, page-locked panel buffer; allocated on first use
   hipStream_t ldl_stream = nullptr;
@@ -31,12 +31,13 @@ void rotate_hessian_impl(qtip_ctx* c, const float* H, bool on_device, int n, uin
                          float* host_su, double* creg, float* host_HRr, float* dev_HRr = nullptr);
 void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L);
 void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int threads, float* host_L,
-                               const float* dev_HRr = nullptr);
+                               const float* dev_HRr = nullptr, float* dev_L = nullptr);
 void ldlq_impl(qtip_ctx* c, const float* dWT, const float* dL, long n, long m, float* d_hatWT, uint16_t* dQ,
                int feedback, double* vit_seconds);
 void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
                          double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
-                         qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr = nullptr);
+                         qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr = nullptr,
+                         const float* dev_L = nullptr);
 void reserve_group_ring(qtip_ctx* c, int n, int depth);
 void run_groups_impl(qtip_ctx* c, int ngroups, const qtip_group* groups, const qtip_opts& opt, qtip_timing* timings,
                      double* ldl_wait);
