@@ -322,13 +322,21 @@ def test_run_groups_equals_group_by_group(qz, oracle, pkg, synth):
             assert a.wscale == b.wscale and a.proxy == b.proxy and a.proxy_rot_reg == b.proxy_rot_reg
         assert tm.total > 0 and tm.ldl_cpu > 0 and tm.rht > 0 and wait >= 0
     assert qz.run_groups([], opt) == []
+    # the same with the factorization on the host alone (the reference's form): identical outputs
+    host = qz.run_groups(cases, pkg.QuantOpts(ldl_threads=8, ldl_device_updates=False))
+    for (outs, _, _), (houts, htm, _) in zip(res, host):
+        for a, b in zip(outs, houts):
+            assert np.array_equal(a.trellis, b.trellis) and a.wscale == b.wscale
+            assert a.proxy == b.proxy and a.proxy_rot_reg == b.proxy_rot_reg
+        assert htm.ldl_cpu > 0
     # failure in the third of four groups
     rng = np.random.default_rng(1)
     G = rng.standard_normal((256, 8)).astype(np.float32)
     bad = list(cases[:2]) + [(cases[2][0], 256, G @ G.T, 5), cases[3]]
-    with pytest.raises(pkg.QtipError) as e:
-        qz.run_groups(bad, pkg.QuantOpts(ldl_threads=8, sigma_reg=0.0))
-    assert e.value.code == pkg.QTIP_E_NOT_PD
+    for dev in (True, False):
+        with pytest.raises(pkg.QtipError) as e:
+            qz.run_groups(bad, pkg.QuantOpts(ldl_threads=8, sigma_reg=0.0, ldl_device_updates=dev))
+        assert e.value.code == pkg.QTIP_E_NOT_PD
     # the context is still usable
     again = qz.run_groups(cases[:1], opt)
     assert np.array_equal(again[0][0][0].trellis, res[0][0][0].trellis)
