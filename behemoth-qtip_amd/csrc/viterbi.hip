@@ -63,6 +63,8 @@ struct Smem {
   uint16_t st[kSteps];
   double red_c[4];
   uint32_t red_s[4];
+  double tr_c[2][4];    // trace-back: the four waves' best candidates of a round (cost; d | d1 << 8), two sets
+  uint32_t tr_d[2][4];
   int overlap;
   uint32_t final_state;
 };
@@ -352,75 +354,72 @@ __device__ __forceinline__ double read_lane_f64(double v, int lane) {
                           __builtin_amdgcn_readlane(__double2loint(v), lane));
 }
 
-// Trace-back, run by the first wave: walks two steps per round trip to HBM.  s is the state of step it + 1;
+// Trace-back, run by all four waves: walks two steps per round trip to HBM.  s is the state of step it + 1;
 // for every digit d of step it the metric M_it[g_d] of the group g_d = (d << 8) | (j >> 4), j = s >> 4, is rebuilt
 // from the kept metrics of step it - 1 as the forward pass built it (the 16 lanes of a row, one per digit of step
 // it - 1, same fp64 operations, smallest digit among equal minima), then the 16 candidates of step it are compared
-// the same way (four per row, then across the four rows).
+// the same way: wave w takes the digits 4w .. 4w+3 (one per row), picks among its four, and the four waves' picks
+// meet in LDS (two alternating sets of slots, one barrier per round).
 // Returns the state of step it_min - 1; record: the states of the steps walked are written to sm.st.
 __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restrict__ entry_d,
                                                const double* __restrict__ hist, int roll, uint32_t s, int it_min,
                                                bool record) {
-  const uint32_t lane = threadIdx.x & 63u, dp = lane & 15u, dq = lane >> 4;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, dp = lane & 15u, d = 4u * wave + (lane >> 4);
+  int set = 0;
 #pragma nounroll
-  for (int it = kSteps - 2; it >= it_min; it -= 2) {
+  for (int it = kSteps - 2; it >= it_min; it -= 2, set ^= 1) {
     const uint32_t j = s >> 4;
     const int ta = (2 * (it - 1) + roll) & 255, tb = (2 * it + roll) & 255;
     const double xa0 = double(sm.x[ta]), xa1 = double(sm.x[ta + 1]);
     const double xb0 = double(sm.x[tb]), xb1 = double(sm.x[tb + 1]);
     const unsigned long long* row =
         reinterpret_cast<const unsigned long long*>(hist + size_t(it / 2 - 1) * kGroups);
-    double mv[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint32_t d = 4u * q + dq, p = (dp << 8) | (d << 4) | (j >> 8);
-      // past the vector L1, which may hold the previous tile's values
-      mv[q] = __longlong_as_double((long long)__hip_atomic_load(row + hist_index(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    }
-    double e1v[4], e0v[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const uint32_t d = 4u * q + dq, g = (d << 8) | (j >> 4);
-      const uint32_t s1 = (dp << 12) | g, e1 = ((s1 * (s1 + 1u)) >> 6) & 1023u;
-      const double a1 = entry_d[2 * e1] - xa0, b1 = entry_d[2 * e1 + 1] - xa1;
-      e1v[q] = __builtin_fma(a1, a1, b1 * b1);
-      const uint32_t s0 = (d << 12) | j, e0 = ((s0 * (s0 + 1u)) >> 6) & 1023u;
-      const double a0 = entry_d[2 * e0] - xb0, b0 = entry_d[2 * e0 + 1] - xb1;
-      e0v[q] = __builtin_fma(a0, a0, b0 * b0);
-    }
-    double best = 0;
-    uint32_t bestd = 0, bestd1 = 0;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const double c1 = e1v[q] + mv[q];
-      const double m1 = row_min16(c1);  // M_it[g_d]
-      // its digit: the first lane of the row that holds the minimum
-      const unsigned long long at_min = __builtin_amdgcn_ballot_w64(c1 == m1);
-      // (no lane at all if the inputs held a NaN: any digit will do then, but it must stay a digit)
-      const uint32_t row_bits = uint32_t(at_min >> (16u * dq)) & 0xffffu;
-      const uint32_t k1 = row_bits ? uint32_t(__builtin_ctz(row_bits)) : 0u;
-      const double c0 = e0v[q] + m1;
-      const bool take = q == 0 || c0 < best;  // d ascends with q: the first minimum stays
-      best = take ? c0 : best;
-      bestd = take ? 4u * q + dq : bestd;
-      bestd1 = take ? k1 : bestd1;
-    }
-    // every lane of row r now holds that row's best (cost, d, d1); pick across the four rows, smallest d on ties
-    double bc = read_lane_f64(best, 0);
-    uint32_t bd = uint32_t(__builtin_amdgcn_readlane(int(bestd), 0)), bd1 = uint32_t(__builtin_amdgcn_readlane(int(bestd1), 0));
+    const uint32_t p = (dp << 8) | (d << 4) | (j >> 8);
+    // past the vector L1, which may hold the previous tile's values
+    const double mv = __longlong_as_double((long long)__hip_atomic_load(row + hist_index(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    const uint32_t g = (d << 8) | (j >> 4);
+    const uint32_t s1 = (dp << 12) | g, e1 = ((s1 * (s1 + 1u)) >> 6) & 1023u;
+    const double a1 = entry_d[2 * e1] - xa0, b1 = entry_d[2 * e1 + 1] - xa1;
+    const uint32_t s0 = (d << 12) | j, e0 = ((s0 * (s0 + 1u)) >> 6) & 1023u;
+    const double a0 = entry_d[2 * e0] - xb0, b0 = entry_d[2 * e0 + 1] - xb1;
+    const double c1 = __builtin_fma(a1, a1, b1 * b1) + mv;
+    const double m1 = row_min16(c1);  // M_it[g_d]
+    // its digit: the first lane of the row that holds the minimum (no lane at all if the inputs held a NaN: any
+    // digit will do then, but it must stay a digit)
+    const unsigned long long at_min = __builtin_amdgcn_ballot_w64(c1 == m1);
+    const uint32_t row_bits = uint32_t(at_min >> (lane & 48u)) & 0xffffu;
+    const uint32_t k1 = row_bits ? uint32_t(__builtin_ctz(row_bits)) : 0u;
+    const double c0 = __builtin_fma(a0, a0, b0 * b0) + m1;
+    // every lane of row r holds that row's (cost, d1) for d = 4 wave + r; pick across the four rows, smallest d on ties
+    double bc = read_lane_f64(c0, 0);
+    uint32_t bd = 4u * wave, bd1 = uint32_t(__builtin_amdgcn_readlane(int(k1), 0));
 #pragma unroll
     for (int r = 1; r < 4; ++r) {
-      const double oc = read_lane_f64(best, 16 * r);
-      const uint32_t od = uint32_t(__builtin_amdgcn_readlane(int(bestd), 16 * r));
-      const uint32_t od1 = uint32_t(__builtin_amdgcn_readlane(int(bestd1), 16 * r));
-      const bool take = oc < bc || (oc == bc && od < bd);
+      const double oc = read_lane_f64(c0, 16 * r);
+      const uint32_t od1 = uint32_t(__builtin_amdgcn_readlane(int(k1), 16 * r));
+      const bool take = oc < bc;  // rows ascend in d: the first minimum stays
       bc = take ? oc : bc;
-      bd = take ? od : bd;
+      bd = take ? 4u * wave + uint32_t(r) : bd;
       bd1 = take ? od1 : bd1;
     }
-    const uint32_t s_it = (bd << 12) | j;
-    s = (bd1 << 12) | (s_it >> 4);
-    if (record && lane == 0) {
+    if (lane == 0) {
+      sm.tr_c[set][wave] = bc;
+      sm.tr_d[set][wave] = bd | (bd1 << 8);
+    }
+    __syncthreads();
+    bc = sm.tr_c[set][0];
+    uint32_t bdd = sm.tr_d[set][0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const double oc = sm.tr_c[set][w];
+      const uint32_t od = sm.tr_d[set][w];
+      const bool take = oc < bc;  // waves ascend in d
+      bc = take ? oc : bc;
+      bdd = take ? od : bdd;
+    }
+    const uint32_t s_it = ((bdd & 15u) << 12) | j;
+    s = (((bdd >> 8) & 15u) << 12) | (s_it >> 4);
+    if (record && threadIdx.x == 0) {
       sm.st[it] = uint16_t(s_it);
       sm.st[it - 1] = uint16_t(s);
     }
@@ -447,7 +446,7 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
     for (int pass = 0; pass < 2; ++pass) {
       const int roll = pass == 0 ? kSeq / 2 : 0;
       forward_pass(sm, entry_d, roll, ov, hist, pass == 0 ? 62 : 0);
-      if (u < 64) {
+      {
         const uint32_t s_last = sm.final_state;  // state of step 127
         const uint32_t s = trace_back(sm, entry_d, hist, roll, s_last, pass == 0 ? 64 : 2, pass == 1);
         if (u == 0) {
