@@ -375,8 +375,8 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
     const unsigned long long* row =
         reinterpret_cast<const unsigned long long*>(hist + size_t(it / 2 - 1) * kGroups);
     const uint32_t p = (dp << 8) | (d << 4) | (j >> 8);
-    // past the vector L1, which may hold the previous tile's values
-    const double mv = __longlong_as_double((long long)__hip_atomic_load(row + hist_index(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    // written by this workgroup's own waves before the barrier that ended the forward pass: workgroup scope suffices
+    const double mv = __longlong_as_double((long long)__hip_atomic_load(row + hist_index(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
     const uint32_t g = (d << 8) | (j >> 4);
     const uint32_t s1 = (dp << 12) | g, e1 = ((s1 * (s1 + 1u)) >> 6) & 1023u;
     const double a1 = entry_d[2 * e1] - xa0, b1 = entry_d[2 * e1 + 1] - xa1;
