@@ -20,11 +20,25 @@ __global__ void symmetrize_lower_kernel(const float* __restrict__ H, long n, dou
   A[i * n + j] = 0.5 * (double(H[i * n + j]) + double(H[j * n + i]));
 }
 
-// C[i][j] -= sum_p X[i][p] * X[j][p] for the 128 x 128 tile (bi, bj <= bi) of the nr x nr lower triangle.
-// X: nr x kb (row stride kb), C: row stride ldc.  256 threads, 2 x 2 waves of 64 x 64, K staged 16 at a time.
+// Xt[p][i] = X[i][p]: the solved rows arrive row by row (nr x kb); the update reads them column by column
+__global__ __launch_bounds__(256) void transpose_panel_kernel(const double* __restrict__ X, int nr, int kb,
+                                                            double* __restrict__ Xt) {
+  __shared__ double tile[32][33];
+  const int i0 = blockIdx.x * 32, p0 = blockIdx.y * 32, tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int r = ty; r < 32; r += 8)
+    if (i0 + r < nr && p0 + tx < kb) tile[r][tx] = X[long(i0 + r) * kb + p0 + tx];
+  __syncthreads();
+  for (int r = ty; r < 32; r += 8)
+    if (p0 + r < kb && i0 + tx < nr) Xt[long(p0 + r) * nr + i0 + tx] = tile[tx][r];
+}
+
+// C[i][j] -= sum_p X[i][p] * X[j][p] for the 128 x 128 tile (bi, bj <= bi) of the nr x nr lower triangle, every
+// element one chain over p = 0 .. kb-1 from zero.  Xt: kb x nr (the transposed solved rows, row stride nr, nr a
+// multiple of 4), C: row stride ldc.  256 threads, 2 x 2 waves of 64 x 64, K staged 16 at a time; the next 16 columns
+// travel from HBM while the matrix cores work on the present ones.
 constexpr int UT = 128, UK = 16;
-__global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double* __restrict__ X, int nr, int kb,
-                                                              double* __restrict__ C, long ldc) {
+__global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double* __restrict__ Xt, int nr, int kb,
+                                                                 double* __restrict__ C, long ldc) {
   // tile index -> (bi, bj), rows of the triangle enumerated from the top
   int bi = 0, rem = blockIdx.x;
   while (rem > bi) {
@@ -32,31 +46,33 @@ __global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double*
     ++bi;
   }
   const int bj = rem, i0 = bi * UT, j0 = bj * UT;
-  __shared__ double Xi[UK][UT + 4], Xj[UK][UT + 4];
+  __shared__ __attribute__((aligned(16))) double Xi[UK][UT], Xj[UK][UT];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
   double4_t acc[4][4];
 #pragma unroll
   for (int a = 0; a < 4; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
-  const int lrow = t & 127, lk = (t >> 7) * 8;
-  const int ri = i0 + lrow, rj = j0 + lrow;
-  // the next 16 columns of the two row blocks travel from HBM while the matrix cores work on the present ones
-  double pi[8], pj[8];
+  const int lk = t >> 5, lc = (t & 31) * 4;  // this thread stages rows lk and lk + 8 of a slice, 4 columns at lc
+  const bool i_ok = i0 + lc + 3 < nr, j_ok = j0 + lc + 3 < nr;  // nr is a multiple of 4: a group of 4 is in or out
+  double4_t pi[2], pj[2];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const int kk = k0 + lk + q;
-      pi[q] = (ri < nr && kk < kb) ? X[long(ri) * kb + kk] : 0.0;
-      pj[q] = (rj < nr && kk < kb) ? X[long(rj) * kb + kk] : 0.0;
+    for (int r = 0; r < 2; ++r) {
+      const int k = k0 + lk + 8 * r;
+      pi[r] = pj[r] = double4_t{0, 0, 0, 0};
+      if (k < kb) {
+        if (i_ok) pi[r] = *reinterpret_cast<const double4_t*>(Xt + long(k) * nr + i0 + lc);
+        if (j_ok) pj[r] = *reinterpret_cast<const double4_t*>(Xt + long(k) * nr + j0 + lc);
+      }
     }
   };
   fetch(0);
   for (int k0 = 0; k0 < kb; k0 += UK) {
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      Xi[lk + q][lrow] = pi[q];
-      Xj[lk + q][lrow] = pj[q];
+    for (int r = 0; r < 2; ++r) {
+      *reinterpret_cast<double4_t*>(&Xi[lk + 8 * r][lc]) = pi[r];
+      *reinterpret_cast<double4_t*>(&Xj[lk + 8 * r][lc]) = pj[r];
     }
     __syncthreads();
     if (k0 + UK < kb) fetch(k0 + UK);
@@ -111,7 +127,10 @@ struct DeviceTrailing final : PanelAssist {
     // the stream orders this copy before the next fetch into the same page-locked buffer
     QTIP_HIP(hipMemcpyAsync(c->ldl_X.p, panel + long(kb) * kb, size_t(nr) * kb * 8, hipMemcpyHostToDevice, s));
     const long nt = (nr + UT - 1) / UT, tiles = nt * (nt + 1) / 2;
-    rank_update_lower_kernel<<<dim3(unsigned(tiles)), dim3(256), 0, s>>>(c->ldl_X.p, int(nr), kb,
+    transpose_panel_kernel<<<dim3(unsigned((nr + 31) / 32), unsigned((kb + 31) / 32)), dim3(256), 0, s>>>(
+        c->ldl_X.p, int(nr), kb, c->ldl_Xt.p);
+    QTIP_HIP(hipGetLastError());
+    rank_update_lower_kernel<<<dim3(unsigned(tiles)), dim3(256), 0, s>>>(c->ldl_Xt.p, int(nr), kb,
                                                                         c->ldl_A.p + r0 * n + r0, n);
     QTIP_HIP(hipGetLastError());
   }
@@ -131,6 +150,7 @@ void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int th
   c->ldl_A.ensure(nn);
   if (!dev_HRr) c->ldl_H.ensure(nn);
   c->ldl_X.ensure(size_t(n) * nb);
+  c->ldl_Xt.ensure(size_t(n) * nb);
   if (c->ldl_panel.n < size_t(n) * nb) c->ldl_panel.alloc(size_t(n) * nb);
   if (!dev_HRr) QTIP_HIP(hipMemcpyAsync(c->ldl_H.p, host_HRr, nn * 4, hipMemcpyHostToDevice, s));
   symmetrize_lower_kernel<<<dim3(unsigned((n + 255) / 256), unsigned(n)), dim3(256), 0, s>>>(dev_HRr ? dev_HRr : c->ldl_H.p, n,

@@ -20,7 +20,7 @@ struct qtip_ctx {
   // LDL with the trailing updates on the device (ldl_assist.hip): own stream, fp64 work matrix, fp32 upload of HRr,
   // solved panel rows, page-locked panel buffer; allocated on first use
   hipStream_t ldl_stream = nullptr;
-  qtipmi::DBuf<double> ldl_A, ldl_X;
+  qtipmi::DBuf<double> ldl_A, ldl_X, ldl_Xt;
   qtipmi::DBuf<float> ldl_H;
   qtipmi::HBuf<double> ldl_panel;
 };
