@@ -144,6 +144,7 @@ void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int th
                                const float* dev_HRr, float* dev_L) {
   QTIP_REQUIRE(c && n > 0 && n % 16 == 0 && (host_HRr || dev_HRr) && host_L,
                "ldl_hessian (device updates): bad arguments (n = %d)", n);
+  QTIP_REQUIRE(n <= 65535, "ldl_hessian (device updates): n = %d is beyond one grid dimension", n);
   if (!c->ldl_stream) QTIP_HIP(hipStreamCreateWithFlags(&c->ldl_stream, hipStreamNonBlocking));
   hipStream_t s = c->ldl_stream;
   const size_t nn = size_t(n) * n, nb = size_t(ldl_panel_width());
@@ -157,7 +158,13 @@ void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int th
                                                                                               c->ldl_A.p);
   QTIP_HIP(hipGetLastError());
   DeviceTrailing dev(c, n, host_L, dev_L);
-  const bool ok = block_ldl_assisted(n, host_L, threads, dev);
+  bool ok = false;
+  try {
+    ok = block_ldl_assisted(n, host_L, threads, dev);
+  } catch (...) {
+    (void)hipStreamSynchronize(s);  // copies that read the caller's L must not outlive the call
+    throw;
+  }
   QTIP_HIP(hipStreamSynchronize(s));
   if (!ok) throw Error(QTIP_E_NOT_PD, "block LDL failed (H not PD)");
 }
