@@ -134,7 +134,7 @@ def run_group(args, pkg):
                          ldlq_s=sum(t.ldlq for t in tms) / K, viterbi_s=sum(t.viterbi for t in tms) / K,
                          load_s=sum(t.load for t in tms) / K, pack_s=sum(t.pack for t in tms) / K,
                          proxy_s=sum(t.proxy for t in tms) / K, proxy=float(res[-1][0][0].proxy),
-                         wscale=float(res[-1][0][0].wscale))
+                         wscale=float(res[-1][0][0].wscale), cmp_outs=res[min(K, 6) - 1][0])
 
     q.reserve_groups(n)   # page-locked staging ring (3 x (HRr, L)); a worker keeps it for its lifetime
     if args.warmup > 0:
@@ -146,6 +146,23 @@ def run_group(args, pkg):
     q.synchronize()
     torch.cuda.synchronize()
     wall = time.time() - t0
+    host_only = {}
+    if not args.host_ldl and not args.no_host_ldl_leg:
+        # beside it (outside the timed region): the same groups with the block LDL on the host alone, as the
+        # reference factors; fewer groups, so the one exposed factorization at the start weighs more
+        kh = min(args.steps, 6)
+        hopt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback,
+                             ldl_device_updates=False)
+        q.synchronize()
+        th = time.time()
+        hres = q.run_groups([(lins, n, H, 3 + k) for k in range(kh)], hopt)
+        q.synchronize()
+        th = time.time() - th
+        host_only = dict(host_ldl_Mweights_s=weights_per_step * kh / th / 1e6, host_ldl_groups=kh,
+                         host_ldl_s=sum(r[1].ldl_cpu for r in hres) / kh,
+                         host_ldl_same_codes=bool(all(np.array_equal(a.trellis, b.trellis) and a.proxy == b.proxy
+                                                      for a, b in zip(hres[-1][0], stats["cmp_outs"]))))
+    stats.pop("cmp_outs", None)
     ntr = sum(ms) // 16
     launches = n // 16
     gpu_s = stats["rht_s"] + stats["load_s"] + stats["ldlq_s"] + stats["proxy_s"] + stats["pack_s"]
@@ -155,12 +172,42 @@ def run_group(args, pkg):
                  viterbi_only_Mweights_s=weights_per_step / stats["viterbi_s"] / 1e6,
                  proxy_in_timed_region=True, ldl_threads=args.ldl_threads, feedback=args.feedback,
                  ldl_device_updates=not args.host_ldl)
+    extra.update(host_only)
     names = {2: "config2: 1024x1024 group", 3: "config3: 12288x12288 q-proj group",
              4: "config4: gate+up 2x(28672x12288) group", 5: "config5: 12288x28672 down-proj group"}
     return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
                 vit_launch_weights=ntr * 256, workload=names[cfg] + (" (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)" if args.host_ldl else
                                        " (RHT + fp64 LDL: host panels, GPU trailing updates + LDLQ + 2-pass Viterbi + pack)"),
                 extra=extra)
+
+
+def run_ldl_only(args, pkg):
+    """The factorization alone (nothing else on the GPU): seconds per call for both forms, and whether the two
+    factors are the same bits."""
+    import numpy as np
+    synth = load_synth()
+    q = pkg.Quantizer(0)
+    if args.config == 2:
+        _, H_h = synth.config2()
+        import torch
+        H = torch.from_numpy(H_h).cuda()
+    else:
+        _, H = synth.large_config(args.config if args.config != 1 else 5)
+    n = H.shape[0]
+    hp = q.rotate_hessian(H, n, 3)
+    del H
+    dev, host = [], []
+    for _ in range(3):
+        q.ldl_hessian_device_updates(hp, threads=args.ldl_threads)
+        dev.append(hp.t_ldl)
+    L_dev = hp.L
+    reps = 1 if args.host_ldl_once else 3
+    for _ in range(reps):
+        pkg.Quantizer.ldl_hessian(hp, threads=args.ldl_threads)
+        host.append(hp.t_ldl)
+    same = bool(np.array_equal(L_dev.view(np.uint32), hp.L.view(np.uint32)))
+    print(json.dumps({"workload": "block LDL alone, n = %d" % n, "device_updates_s": dev, "host_only_s": host,
+                      "same_factor_bits": same, "ldl_threads": args.ldl_threads}), flush=True)
 
 
 def main():
@@ -174,6 +221,12 @@ def main():
     ap.add_argument("--host-ldl", action="store_true",
                     help="keep the fp64 block LDL on the host alone, as the reference does (default: the host factors and "
                          "solves the panels and hands the trailing updates to the GPU; the factor is the same bit for bit)")
+    ap.add_argument("--ldl-only", action="store_true",
+                    help="time the block LDL of the configuration's rotated Hessian by itself, three times each: host panels "
+                         "with GPU trailing updates, and host alone (not the contract's metric; one line of JSON)")
+    ap.add_argument("--host-ldl-once", action="store_true", help="with --ldl-only: one host-only factorization instead of three")
+    ap.add_argument("--no-host-ldl-leg", action="store_true",
+                    help="skip the extra host-only-LDL groups reported beside the default run")
     ap.add_argument("--feedback", type=int, default=0, choices=[0, 1],
                     help="0: fp64 LDLQ feedback (default); 1: fp32 feedback + bf16 hi/lo split MFMA prod cache")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -196,6 +249,8 @@ def main():
         b.copy_(a)          # 1 GiB read + 1 GiB written by one elementwise kernel
         torch.cuda.synchronize()
         del a, b
+    if args.ldl_only:
+        return run_ldl_only(args, pkg)
     res = run_viterbi_only(args, pkg) if args.config == 1 else run_group(args, pkg)
     value = res["weights"] / res["wall"] / 1e6
     achieved = res["vit_launch_weights"] * FLOP_PER_WEIGHT / res["vit_launch_s"] / 1e12
