@@ -51,8 +51,9 @@ void upload_codebook(qtip_ctx* c) {
 
 void ensure_viterbi_workspace(qtip_ctx* c) {
   if (c->vit_slots > 0) return;
-  c->vit_slots = viterbi_max_slots(c->device);
-  c->vit_ws.alloc(viterbi_workspace_bytes(c->vit_slots));
+  const int slots = viterbi_max_slots(c->device);
+  c->vit_ws.alloc(viterbi_workspace_bytes(slots));
+  c->vit_slots = slots;  // only once the workspace exists
 }
 }  // namespace qtipmi
 
@@ -336,6 +337,29 @@ int qtip_reserve_groups(qtip_ctx* ctx, int n) {
     QTIP_REQUIRE(ctx != nullptr && n > 0, "reserve_groups: bad arguments");
     DeviceGuard g(ctx);
     reserve_group_ring(ctx, n, 3);
+  });
+}
+
+int qtip_selftest_failed_alloc_is_retried(void) {
+  // host only: the next two device allocations are made to fail; a buffer whose allocation failed must stay empty,
+  // so that the next ensure() allocates again instead of handing a null pointer to a kernel
+  return guarded([&] {
+    DBuf<double> b;
+    test_fail_next_device_allocs(2);
+    for (int attempt = 0; attempt < 2; ++attempt) {
+      const long calls = test_device_alloc_calls();
+      bool threw = false;
+      try {
+        b.ensure(1024);
+      } catch (const Error& e) {
+        threw = e.code == QTIP_E_HIP;
+      }
+      test_fail_next_device_allocs(1 - attempt);
+      QTIP_REQUIRE(threw, "attempt %d: a failed allocation did not raise", attempt);
+      QTIP_REQUIRE(test_device_alloc_calls() == calls + 1, "attempt %d: ensure() did not try to allocate", attempt);
+      QTIP_REQUIRE(b.p == nullptr && b.n == 0, "attempt %d: a failed allocation left n = %zu", attempt, b.n);
+    }
+    test_fail_next_device_allocs(0);
   });
 }
 

@@ -2,6 +2,7 @@
 // selection, trellis packing.  Semantics follow the reference files named at each function.
 #include <sys/mman.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -23,6 +24,19 @@ void fail(int code, const char* fmt, ...) {
   va_end(ap);
   throw Error(code, buf);
 }
+
+// hipMalloc behind one door, so that a host-only test can see an allocation fail and be retried without a GPU
+static std::atomic<int> g_fail_allocs{0};
+static std::atomic<long> g_alloc_calls{0};
+hipError_t device_malloc(void** p, size_t bytes) {
+  g_alloc_calls.fetch_add(1);
+  int left = g_fail_allocs.load();
+  while (left > 0 && !g_fail_allocs.compare_exchange_weak(left, left - 1)) {}
+  if (left > 0) return hipErrorOutOfMemory;
+  return hipMalloc(p, bytes);
+}
+void test_fail_next_device_allocs(int count) { g_fail_allocs.store(count); }
+long test_device_alloc_calls() { return g_alloc_calls.load(); }
 
 // IEEE binary16 <-> binary32, round to nearest even (src/common.hpp:49-78 of the reference)
 uint16_t f32_to_fp16(float f) {

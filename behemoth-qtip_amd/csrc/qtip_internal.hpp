@@ -38,6 +38,11 @@ void set_last_error(const std::string& m);
     if (!(cond)) ::qtipmi::fail(QTIP_E_ARG, __VA_ARGS__);    \
   } while (0)
 
+// hipMalloc; a host-only test can make the next calls fail (test_fail_next_device_allocs) without touching a GPU
+hipError_t device_malloc(void** p, size_t bytes);
+void test_fail_next_device_allocs(int count);
+long test_device_alloc_calls();
+
 // Device buffer released on scope exit.
 template <class T>
 struct DBuf {
@@ -50,8 +55,8 @@ struct DBuf {
   ~DBuf() { release(); }
   void alloc(size_t count) {
     release();
-    n = count;
-    if (count) QTIP_HIP(hipMalloc(reinterpret_cast<void**>(&p), count * sizeof(T)));
+    if (count) QTIP_HIP(device_malloc(reinterpret_cast<void**>(&p), count * sizeof(T)));
+    n = count;  // only after the allocation succeeded: a failed one leaves an empty buffer that ensure() retries
   }
   void ensure(size_t count) {
     if (count > n) alloc(count);

@@ -236,6 +236,10 @@ int qtip_st_write(qtip_st_writer* w, const char* path, const char* const* metada
 /* fp16 bits of the context's codebook table [512][2] (Codebook::tlut_h, src/qtip_core.hpp:24-31) */
 int qtip_get_tlut_f16(qtip_ctx* ctx, uint16_t* host_tlut_f16);
 
+/* Host-only self test (no GPU needed, no counterpart in the reference): a device buffer of the context whose
+ * allocation failed stays empty, so the next call allocates again instead of launching on a null pointer.  0 = ok. */
+int qtip_selftest_failed_alloc_is_retried(void);
+
 /* Host packers (pack_trellis / unpack_trellis / swizzle_for_kernel / unswizzle_for_kernel,
  * src/qtip_core.cpp:194-253) */
 void qtip_pack_trellis(const uint16_t* states, long B, uint16_t* packed);

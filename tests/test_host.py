@@ -22,6 +22,14 @@ def test_abi_exports_every_declared_symbol(pkg):
     assert not missing, missing
 
 
+def test_failed_device_allocation_is_retried(pkg):
+    """A context buffer whose hipMalloc failed must stay empty (n = 0), so that the next ensure() allocates again;
+    the failure is simulated on the host, no GPU involved."""
+    L = C.CDLL(pkg.LIB_PATH)
+    L.qtip_last_error.restype = C.c_char_p
+    assert L.qtip_selftest_failed_alloc_is_retried() == 0, L.qtip_last_error()
+
+
 def test_missing_library_fails_loudly(pkg, monkeypatch):
     monkeypatch.setattr(pkg, "LIB_PATH", os.path.join(ROOT, "nowhere", "libqtip_mi355.so"))
     monkeypatch.setattr(pkg, "_lib", None)
