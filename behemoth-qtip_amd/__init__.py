@@ -21,6 +21,9 @@ LIB_PATH = os.path.join(CSRC, "libqtip_mi355.so")
 QTIP_OK, QTIP_E_ARG, QTIP_E_HIP, QTIP_E_NOT_PD, QTIP_E_NOMEM = 0, -1, -2, -3, -4
 
 
+NOALLOC_MAX_TILES = 4096  # QTIP_NOALLOC_MAX_TILES
+
+
 class QtipError(RuntimeError):
     def __init__(self, code, msg):
         super().__init__("qtip error %d: %s" % (code, msg))
@@ -85,6 +88,7 @@ def lib():
     L.qtip_get_lut.argtypes = [vp, vp, vp]
     L.qtip_viterbi_tiles.argtypes = [vp, vp, l, vp, vp]
     L.qtip_viterbi_tiles_dev.argtypes = [vp, vp, l, vp, vp]
+    L.qtip_viterbi_tiles_dev_noalloc.argtypes = [vp, vp, l, vp, vp]
     L.qtip_decode_states_dev.argtypes = [vp, vp, l, vp]
     L.qtip_hadamard_rows_dev.argtypes = [vp, vp, l, i, l, i]
     L.qtip_decode_trellis_dev.argtypes = [vp, vp, i, i, vp]
@@ -288,6 +292,10 @@ class Quantizer:
 
     def viterbi_tiles_dev(self, dX, B, d_states=None, d_packed=None):
         _check(lib().qtip_viterbi_tiles_dev(self._h, _ptr(dX), B, _ptr(d_states), _ptr(d_packed)))
+
+    def viterbi_tiles_dev_noalloc(self, dX, B, d_states=None, d_packed=None):
+        """viterbi_tiles_dev on the library's fixed workspace: allocates nothing, B <= NOALLOC_MAX_TILES."""
+        _check(lib().qtip_viterbi_tiles_dev_noalloc(self._h, _ptr(dX), B, _ptr(d_states), _ptr(d_packed)))
 
     def decode_states_dev(self, d_states, B, d_hat):
         _check(lib().qtip_decode_states_dev(self._h, _ptr(d_states), B, _ptr(d_hat)))

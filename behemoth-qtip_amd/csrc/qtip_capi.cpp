@@ -95,6 +95,7 @@ int qtip_create(int device, qtip_ctx** out) {
     c->cb.build(nullptr);
     upload_codebook(c);
     c->rht.init(device, c->stream);
+    viterbi_static_scratch_init(device);
     *out = c;
     guard.c = nullptr;
   });
@@ -162,6 +163,26 @@ int qtip_viterbi_tiles_dev(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* 
     job.states = dev_states;
     job.packed = dev_packed;
     launch_viterbi_tiles(job, ctx->d_entry_d, ctx->d_entry_f, ctx->vit_ws, ctx->vit_slots, ctx->stream);
+  });
+}
+
+int qtip_viterbi_tiles_dev_noalloc(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* dev_states,
+                                   uint16_t* dev_packed) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && B >= 0, "viterbi_tiles_noalloc: bad arguments");
+    QTIP_REQUIRE(B <= QTIP_NOALLOC_MAX_TILES, "viterbi_tiles_noalloc: B = %ld exceeds the maximum of %d tiles per call",
+                 B, QTIP_NOALLOC_MAX_TILES);
+    if (B == 0) return;
+    QTIP_REQUIRE(dev_X != nullptr, "viterbi_tiles_noalloc: X is null");
+    DeviceGuard g(ctx);
+    void* ws = viterbi_static_scratch(ctx->device);
+    QTIP_REQUIRE(ws != nullptr, "viterbi_tiles_noalloc: no static scratch on device %d", ctx->device);
+    TileJob job;
+    job.X = dev_X;
+    job.tiles = B;
+    job.states = dev_states;
+    job.packed = dev_packed;
+    launch_viterbi_tiles(job, ctx->d_entry_d, ctx->d_entry_f, ws, viterbi_static_slots(), ctx->stream);
   });
 }
 

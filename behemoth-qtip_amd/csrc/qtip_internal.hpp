@@ -194,6 +194,11 @@ int viterbi_max_slots(int device);
 // start / stop (optional): events stamped at the kernel's own start and end
 void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const float* d_entry_f, void* workspace,
                           int slots, hipStream_t s, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
+// Kept-metrics slots that are part of the code object (no allocation): viterbi_static_scratch_init looks up the
+// array's address on `device`, which must be current, once; viterbi_static_scratch returns it (null before that).
+int viterbi_static_slots();
+void viterbi_static_scratch_init(int device);
+void* viterbi_static_scratch(int device);
 void launch_decode_states(const uint16_t* states, long B, float* hat, const float* d_entry_f, hipStream_t s);
 
 }  // namespace qtipmi

@@ -38,6 +38,7 @@
 // and tie rule.  Only the last step tracks its digits (in registers), which the final state needs.
 #include <hip/hip_ext.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "qtip_internal.hpp"
@@ -51,6 +52,15 @@ constexpr int kMSlots = 4096;                    // metric of (column c, digit d
 constexpr int kHistSteps = 63;                           // the metrics entering the odd steps 1, 3 .. 125 are kept
 constexpr int kHistWordsPerTile = kHistSteps * kGroups;  // fp64 words
 enum StepKind { kPlain = 0, kStore = 1, kDigits = 2 };
+
+// Kept-metrics slots for callers that may not allocate (qtip_viterbi_tiles_dev_noalloc): part of the code object, so
+// every device that loads the library holds its own copy (63 MiB) until the process ends.  Host code must not use
+// this name as an address; the per-device address comes from hipGetSymbolAddress (static_scratch_of below).
+constexpr int kStaticSlots = 32;
+static __device__ __align__(256) double scratch[size_t(kStaticSlots) * kHistWordsPerTile];
+constexpr int kMaxDevices = 64;
+double* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
 
 __device__ __forceinline__ constexpr int pi16(int d) { return 4 * (d & 3) + (d >> 2); }
 __device__ __forceinline__ int m_swz(int col) { return ((col >> 2) & 15) ^ (col >> 6); }
@@ -530,6 +540,28 @@ void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const flo
     viterbi_tiles_kernel<<<dim3(grid), dim3(kThreads), 0, s>>>(job, d_entry_d, d_entry_f, static_cast<double*>(workspace));
   }
   QTIP_HIP(hipGetLastError());
+}
+
+int viterbi_static_slots() { return kStaticSlots; }
+
+void viterbi_static_scratch_init(int device) {
+  QTIP_REQUIRE(device >= 0 && device < kMaxDevices, "device %d: the static Viterbi scratch is tracked for devices 0..%d",
+               device, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device]) return;
+  int cur = -1;
+  QTIP_HIP(hipGetDevice(&cur));
+  QTIP_REQUIRE(cur == device, "static scratch: device %d must be current (current: %d)", device, cur);
+  void* p = nullptr;
+  QTIP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+  QTIP_REQUIRE(p != nullptr, "static scratch: no device address on device %d", device);
+  g_scratch_ptr[device] = static_cast<double*>(p);
+}
+
+void* viterbi_static_scratch(int device) {
+  if (device < 0 || device >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  return g_scratch_ptr[device];
 }
 
 void launch_decode_states(const uint16_t* states, long B, float* hat, const float* d_entry_f, hipStream_t s) {

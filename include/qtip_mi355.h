@@ -54,6 +54,19 @@ int qtip_viterbi_tiles(qtip_ctx* ctx, const float* host_X, long B, uint16_t* hos
 /* Same with device pointers; asynchronous on the context's stream. */
 int qtip_viterbi_tiles_dev(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* dev_states, uint16_t* dev_packed);
 
+/* qtip_viterbi_tiles_dev without any allocation.  No counterpart in the reference (its launch chain allocates its
+ * back-pointer buffer per call, src/quantizer.cpp:38); it is for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The kept-metrics workspace, which
+ * qtip_viterbi_tiles_dev allocates on its first call (2 MiB per resident workgroup, 768 of them), is here a fixed
+ * array inside the library's code object: 32 slots, 63 MiB per device, held until the process ends; its address is
+ * looked up once per device in qtip_create.  B <= QTIP_NOALLOC_MAX_TILES, else QTIP_E_ARG; 32 tiles run at a time.
+ * Results equal qtip_viterbi_tiles_dev's bit for bit.  Asynchronous on the context's stream.  All calls on one device
+ * share the array: calls that overlap on one device (two contexts, two streams) race.  Nothing in it needs clearing
+ * between calls: a workgroup writes every kept metric before it reads it. */
+#define QTIP_NOALLOC_MAX_TILES 4096
+int qtip_viterbi_tiles_dev_noalloc(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* dev_states,
+                                   uint16_t* dev_packed);
+
 /* hat[i] = lut[state[i]] (k_decode_states, src/viterbi.hip:231-238): B x 128 states -> B x 256 fp32 */
 int qtip_decode_states_dev(qtip_ctx* ctx, const uint16_t* dev_states, long B, float* dev_hat);
 
