@@ -4,12 +4,22 @@
 //   A = C C^T (lower Cholesky, fp64)  ->  L = C * blockdiag(C_bb^-1) with the 16x16 diagonal blocks and the
 //   upper triangle zeroed, stored as fp32.
 //
-// Own layout of the work: right-looking panels of width NB; the diagonal block is factored in place, the rows
-// below are solved in chunks of NR rows held transposed (64-column sub-blocks: rank update through the micro-kernel
-// plus a small triangular substitution), and the trailing symmetric update runs as a packed
-// register-blocked rank-NB kernel over lower-triangular tiles handed out dynamically to a team of host threads (host_team.hpp).  The
-// micro-kernels are written with GCC vector extensions and compiled twice (AVX2 baseline, AVX-512 clone);
-// the clone is picked at run time so one binary serves any x86-64-v3 host.
+// The factor is the reference's bit for bit, which fixes the order of operations of every element (the schedule,
+// the register blocking and the data layout are this file's own):
+//   * right-looking panels of width NB = 256;
+//   * diagonal block: left-looking, s = a_ij, then s = fma(-l_ip, l_jp, s) for p ascending inside the block, the
+//     diagonal element the same chain with i = j, sqrt, division by the square root (src/qtip_core.cpp:331-347);
+//   * rows below the block: x_j = ((s0 + s1) + (s2 + s3)) * (1 / l_jj), where s0 starts at the element, s1..s3 at zero,
+//     s_(p mod 4) = fma(-l_jp, x_p, s_(p mod 4)) over the full groups of four p < j and the leftover p go to s0
+//     (src/qtip_core.cpp:376-394);
+//   * trailing update: c -= acc with acc one chain fma(x_ip, x_jp, acc), p ascending over the panel from zero
+//     (src/qtip_core.cpp:267-317).
+// Here the diagonal block is factored on a transposed copy so that the chains of 8 rows run in one vector, the rows
+// below are solved in chunks of NR rows held transposed, and the trailing symmetric update runs as a packed
+// register-blocked rank-NB kernel over lower-triangular tiles handed out dynamically to a team of host threads
+// (host_team.hpp).  The kernels are written with GCC vector extensions and compiled twice (AVX2 baseline, AVX-512
+// clone); the clone is picked at run time so one binary serves any x86-64-v3 host.  Built with -ffp-contract=fast:
+// every a * b + c below is one fused operation.
 #include <algorithm>
 #include <atomic>
 #include <cmath>
@@ -39,7 +49,7 @@ typedef double v8d __attribute__((vector_size(64), aligned(8)));
 typedef double v4d __attribute__((vector_size(32), aligned(8)));
 
 #ifndef QTIP_LDL_NB
-#define QTIP_LDL_NB 512
+#define QTIP_LDL_NB 256  // the reference's panel width: part of the factor's bits
 #endif
 #ifndef QTIP_LDL_TILE
 #define QTIP_LDL_TILE 384
@@ -118,80 +128,107 @@ static void micro_4x12(int kc, const double* __restrict__ a, const double* __res
     for (int j = 0; j < nr; ++j) C[i * ldc + j] -= t[i][j >> 2][j & 3];
 }
 
-// ---- panel solve  X * L11^T = A21 on a chunk of NR rows held transposed, x[p][NR] (the layout of one packed
-// B micro-panel).  The panel depth is cut into sub-blocks of SUB columns: the contribution of the columns already
-// solved goes through the rank-update micro-kernel, only the SUB x SUB triangle is substituted here.
-constexpr int SUB = 64;
-#define QTIP_TRI_SOLVE(NAME, NRC)                                                                              \
-  static void NAME(int nb, const double* __restrict__ Lbb, int ldl, const double* __restrict__ rdiag,          \
+// ---- panel solve  X * L11^T = A21 on a chunk of NRC rows held transposed, x[p][NRC] (the layout of one packed
+// B micro-panel), in the order given at the top of the file: four partial sums per element, the lanes are rows.
+#define QTIP_TRI_SOLVE(NAME, VT, VW, NRC)                                                                      \
+  static void NAME(int nb, const double* __restrict__ L11, int ldl, const double* __restrict__ rdiag,          \
                    double* __restrict__ x) {                                                                   \
+    constexpr int NV = NRC / VW;                                                                               \
     for (int j = 0; j < nb; ++j) {                                                                             \
-      double acc[NRC];                                                                                         \
-      double* xj = x + size_t(j) * NRC;                                                                        \
-      for (int c = 0; c < NRC; ++c) acc[c] = xj[c];                                                            \
-      const double* lj = Lbb + size_t(j) * ldl;                                                                \
-      for (int q = 0; q < j; ++q) {                                                                            \
-        const double l = lj[q];                                                                                \
-        const double* xq = x + size_t(q) * NRC;                                                                \
-        for (int c = 0; c < NRC; ++c) acc[c] -= l * xq[c];                                                     \
+      VT s0[NV], s1[NV], s2[NV], s3[NV];                                                                       \
+      VT* xj = reinterpret_cast<VT*>(x + size_t(j) * NRC);                                                     \
+      for (int v = 0; v < NV; ++v) s0[v] = xj[v], s1[v] = s2[v] = s3[v] = VT{};                                \
+      const double* lj = L11 + size_t(j) * ldl;                                                                \
+      int p = 0;                                                                                               \
+      for (; p + 4 <= j; p += 4) {                                                                             \
+        const VT* xp = reinterpret_cast<const VT*>(x + size_t(p) * NRC);                                       \
+        const double l0 = lj[p], l1 = lj[p + 1], l2 = lj[p + 2], l3 = lj[p + 3];                               \
+        for (int v = 0; v < NV; ++v) {                                                                         \
+          s0[v] -= l0 * xp[v];                                                                                 \
+          s1[v] -= l1 * xp[NV + v];                                                                            \
+          s2[v] -= l2 * xp[2 * NV + v];                                                                        \
+          s3[v] -= l3 * xp[3 * NV + v];                                                                        \
+        }                                                                                                      \
+      }                                                                                                        \
+      for (; p < j; ++p) {                                                                                     \
+        const VT* xp = reinterpret_cast<const VT*>(x + size_t(p) * NRC);                                       \
+        const double l0 = lj[p];                                                                               \
+        for (int v = 0; v < NV; ++v) s0[v] -= l0 * xp[v];                                                      \
       }                                                                                                        \
       const double rd = rdiag[j];                                                                              \
-      for (int c = 0; c < NRC; ++c) xj[c] = acc[c] * rd;                                                       \
+      for (int v = 0; v < NV; ++v) xj[v] = ((s0[v] + s1[v]) + (s2[v] + s3[v])) * rd;                           \
     }                                                                                                          \
   }
-__attribute__((target("avx512f"))) QTIP_TRI_SOLVE(tri_solve_24, 24)
-QTIP_TRI_SOLVE(tri_solve_12, 12)
+__attribute__((target("avx512f"))) QTIP_TRI_SOLVE(tri_solve_24, v8d, 8, 24)
+QTIP_TRI_SOLVE(tri_solve_12, v4d, 4, 12)
 #undef QTIP_TRI_SOLVE
+
+// ---- lower Cholesky of the kb x kb diagonal block at A (row stride ld), in the order given at the top of the file.
+// T: scratch of kb * ldt doubles, ldt = kb rounded up to 32; T[p * ldt + i] = l_ip, so that column j is finished by
+// running the chains of the rows i >= j, 8 (or 4) rows to a vector, four vectors in flight.  The lanes of rows i < j
+// carry meaningless values that no later column reads.  false if the block is not positive definite.
+#define QTIP_FACTOR_DIAG(NAME, VT, VW)                                                                         \
+  static bool NAME(double* __restrict__ A, long ld, int kb, double* __restrict__ T, int ldt) {                 \
+    for (int p = 0; p < kb; ++p) {                                                                             \
+      for (int i = 0; i < p; ++i) T[size_t(p) * ldt + i] = 0.0;                                                \
+      for (int i = p; i < kb; ++i) T[size_t(p) * ldt + i] = A[long(i) * ld + p];                               \
+      for (int i = kb; i < ldt; ++i) T[size_t(p) * ldt + i] = 0.0;                                             \
+    }                                                                                                          \
+    for (int j = 0; j < kb; ++j) {                                                                             \
+      double* tj = T + size_t(j) * ldt;                                                                        \
+      for (int i0 = (j / (4 * VW)) * (4 * VW); i0 < kb; i0 += 4 * VW) {                                        \
+        VT a0 = *reinterpret_cast<VT*>(tj + i0), a1 = *reinterpret_cast<VT*>(tj + i0 + VW),                    \
+           a2 = *reinterpret_cast<VT*>(tj + i0 + 2 * VW), a3 = *reinterpret_cast<VT*>(tj + i0 + 3 * VW);       \
+        for (int p = 0; p < j; ++p) {                                                                          \
+          const double* tp = T + size_t(p) * ldt;                                                              \
+          const double l = tp[j];                                                                              \
+          a0 -= l * *reinterpret_cast<const VT*>(tp + i0);                                                     \
+          a1 -= l * *reinterpret_cast<const VT*>(tp + i0 + VW);                                                \
+          a2 -= l * *reinterpret_cast<const VT*>(tp + i0 + 2 * VW);                                            \
+          a3 -= l * *reinterpret_cast<const VT*>(tp + i0 + 3 * VW);                                            \
+        }                                                                                                      \
+        *reinterpret_cast<VT*>(tj + i0) = a0, *reinterpret_cast<VT*>(tj + i0 + VW) = a1;                       \
+        *reinterpret_cast<VT*>(tj + i0 + 2 * VW) = a2, *reinterpret_cast<VT*>(tj + i0 + 3 * VW) = a3;          \
+      }                                                                                                        \
+      double d = tj[j];                                                                                        \
+      if (!(d > 0) || !std::isfinite(d)) return false;                                                         \
+      d = std::sqrt(d);                                                                                        \
+      tj[j] = d;                                                                                               \
+      for (int i = j + 1; i < kb; ++i) tj[i] = tj[i] / d;                                                      \
+    }                                                                                                          \
+    for (int p = 0; p < kb; ++p)                                                                               \
+      for (int i = p; i < kb; ++i) A[long(i) * ld + p] = T[size_t(p) * ldt + i];                               \
+    return true;                                                                                               \
+  }
+__attribute__((target("avx512f"))) QTIP_FACTOR_DIAG(factor_diag_8, v8d, 8)
+QTIP_FACTOR_DIAG(factor_diag_4, v4d, 4)
+#undef QTIP_FACTOR_DIAG
 
 struct Kernels {
   int MR, NR;
   void (*micro)(int, const double*, const double*, double*, long, int, int);
   void (*tri_solve)(int, const double*, int, const double*, double*);
+  bool (*factor_diag)(double*, long, int, double*, int);
 };
 static Kernels pick_kernels() {
   __builtin_cpu_init();
-  if (__builtin_cpu_supports("avx512f")) return Kernels{8, 24, micro_8x24, tri_solve_24};
-  return Kernels{4, 12, micro_4x12, tri_solve_12};
+  if (__builtin_cpu_supports("avx512f")) return Kernels{8, 24, micro_8x24, tri_solve_24, factor_diag_8};
+  return Kernels{4, 12, micro_4x12, tri_solve_12, factor_diag_4};
 }
 
-// unblocked lower Cholesky of the kb x kb diagonal block at A (row stride n); false if not positive definite
-static bool factor_diagonal(double* A, long n, int kb) {
-  for (int j = 0; j < kb; ++j) {
-    double* aj = A + long(j) * n;
-    double d = aj[j];
-    for (int p = 0; p < j; ++p) d -= aj[p] * aj[p];
-    if (!(d > 0) || !std::isfinite(d)) return false;
-    d = std::sqrt(d);
-    aj[j] = d;
-    const double rd = 1.0 / d;
-    for (int i = j + 1; i < kb; ++i) {
-      double* ai = A + long(i) * n;
-      double s0 = ai[j], s1 = 0;
-      int p = 0;
-      for (; p + 2 <= j; p += 2) {
-        s0 -= ai[p] * aj[p];
-        s1 -= ai[p + 1] * aj[p + 1];
-      }
-      if (p < j) s0 -= ai[p] * aj[p];
-      ai[j] = (s0 + s1) * rd;
-    }
-  }
-  return true;
-}
-
-// Lower Cholesky of the n x n matrix at A (row stride ld) by right-looking panels of width NBT.  With a team the panel
-// solve and the trailing update are shared out; without one (the diagonal blocks of the outer factorization, which
-// are factored by this same routine with narrow panels) everything runs on the calling thread.
-// assist (outer factorization only): the trailing matrix lives elsewhere.  Before a panel is factored its columns,
-// rows k .. n-1, are fetched into a buffer of row stride kb; after the solve the buffer holds the final columns of C
-// and is handed back, and whoever holds the trailing matrix applies the rank-kb update (every element one chain
+// Lower Cholesky of the n x n matrix at A (row stride ld) by right-looking panels of width NBT, shared out over the
+// team.
+// assist: the trailing matrix lives elsewhere.  Before a panel is factored its columns, rows k .. n-1, are fetched
+// into a buffer of row stride kb; after the solve the buffer holds the final columns of C and is handed back, and
+// whoever holds the trailing matrix applies the rank-kb update (every element one chain
 // acc = fma(x_ip, x_jp, acc), p ascending from zero, then c -= acc, as the micro-kernels here do).
 template <int NBT, int TILET>
-bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top, PanelAssist* assist = nullptr) {
+bool cholesky_panels(double* A, long ld, int n, HostTeam* team, PanelAssist* assist = nullptr) {
   const Kernels kn = pick_kernels();
   const int MR = kn.MR, NR = kn.NR;
-  std::vector<double> packL;
-  std::vector<double> L11(static_cast<size_t>(NBT) * NBT, 0.0), rdiag(static_cast<size_t>(NBT), 0.0);
+  constexpr int LDT = (NBT + 31) / 32 * 32;
+  std::vector<double> L11(static_cast<size_t>(NBT) * NBT, 0.0), rdiag(static_cast<size_t>(NBT), 0.0),
+      diagT(static_cast<size_t>(NBT) * LDT);
   // packed copies of the solved panel (A side: MR-row micro-panels, B side: NR-row micro-panels), first panel largest
   const size_t capA = size_t((n + MR - 1) / MR) * MR * NBT, capB = size_t((n + NR - 1) / NR) * NR * NBT;
   HostScratch packs((capA + capB) * sizeof(double));
@@ -202,11 +239,7 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top, PanelA
     // the panel: diagonal block at Ap, the rows below follow with stride ldp
     double* Ap = assist ? assist->fetch(k, kb) : A + long(k) * ld + k;
     const long ldp = assist ? kb : ld;
-    if constexpr (NBT > 64) {
-      if (!cholesky_panels<64, 96>(Ap, ldp, kb, nullptr, false)) return false;
-    } else {
-      if (!factor_diagonal(Ap, ldp, kb)) return false;
-    }
+    if (!kn.factor_diag(Ap, ldp, kb, diagT.data(), LDT)) return false;
     const int r0 = k + kb, nr = n - r0;
     if (nr <= 0) {
       if (assist) assist->solved(k, kb, Ap);
@@ -222,25 +255,6 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top, PanelA
       for (int p = 0; p < kb; ++p) packA[size_t(i / MR) * MR * kb + size_t(p) * MR + (i % MR)] = 0.0;
     for (int i = nr; i < nPB * NR; ++i)
       for (int p = 0; p < kb; ++p) packB[size_t(i / NR) * NR * kb + size_t(p) * NR + (i % NR)] = 0.0;
-    // L11 sub-block rows packed for the micro-kernel's A side: for sub-block b, tile it: [q < 64 b][MR] holding
-    // L11[64 b + MR it + i][q]
-    const int nsb = (kb + SUB - 1) / SUB;
-    size_t offL[NBT / SUB + 1];
-    {
-      size_t o = 0;
-      for (int b = 0; b < nsb; ++b) {
-        offL[b] = o;
-        const int p0 = b * SUB, pb = std::min(SUB, kb - p0);
-        o += size_t((pb + MR - 1) / MR) * MR * p0;
-      }
-      packL.assign(o, 0.0);
-      for (int b = 1; b < nsb; ++b) {
-        const int p0 = b * SUB, pb = std::min(SUB, kb - p0);
-        for (int i = 0; i < pb; ++i)
-          for (int q = 0; q < p0; ++q)
-            packL[offL[b] + size_t(i / MR) * MR * p0 + size_t(q) * MR + (i % MR)] = L11[size_t(p0 + i) * kb + q];
-      }
-    }
     // panel solve in place in the packed B micro-panels (one chunk = NR rows), then write back and pack the A side
     auto solve_chunk = [&](long gl) {
       const int g = int(gl);
@@ -250,14 +264,7 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top, PanelA
         const double* src = Ap + long(kb + rb + r) * ldp;
         for (int p = 0; p < kb; ++p) x[size_t(p) * NR + r] = src[p];
       }
-      for (int b = 0; b < nsb; ++b) {
-        const int p0 = b * SUB, pb = std::min(SUB, kb - p0);
-        if (b > 0)
-          for (int it = 0; it * MR < pb; ++it)
-            kn.micro(p0, packL.data() + offL[b] + size_t(it) * MR * p0, x, x + size_t(p0 + it * MR) * NR, NR,
-                     std::min(MR, pb - it * MR), NR);
-        kn.tri_solve(pb, L11.data() + size_t(p0) * kb + p0, kb, rdiag.data() + p0, x + size_t(p0) * NR);
-      }
+      kn.tri_solve(kb, L11.data(), kb, rdiag.data(), x);
       for (int r = 0; r < rows; ++r) {
         const int i = rb + r;
         double* dst = Ap + long(kb + i) * ldp;
@@ -310,7 +317,7 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, bool top, PanelA
 
 bool cholesky_lower_host(double* A, int n, int threads) {
   HostTeam& team = team_of_this_thread(threads);
-  return cholesky_panels<NB, TILE>(A, n, n, &team, true);
+  return cholesky_panels<NB, TILE>(A, n, n, &team);
 }
 
 // L columns c0 .. c0 + nc - 1 from the same columns of C: Cp holds rows c0 .. n-1 of those columns (row stride ldc).
@@ -362,7 +369,7 @@ static bool assemble_L_columns(const double* Cp, long ldc, int c0, int nc, int n
 bool block_ldl_host(double* A, int n, float* L_out, int threads) {
   if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
   HostTeam& team = team_of_this_thread(threads);
-  if (!cholesky_panels<NB, TILE>(A, n, n, &team, true)) return false;
+  if (!cholesky_panels<NB, TILE>(A, n, n, &team)) return false;
   return assemble_L_columns(A, n, 0, n, n, L_out, team);
 }
 
@@ -386,7 +393,7 @@ bool block_ldl_assisted(int n, float* L_out, int threads, PanelAssist& assist) {
       inner.assembled(k, kb);
     }
   } wrap(assist, n, L_out, team);
-  if (!cholesky_panels<NB, TILE>(nullptr, 0, n, &team, true, &wrap)) return false;
+  if (!cholesky_panels<NB, TILE>(nullptr, 0, n, &team, &wrap)) return false;
   return wrap.finite;
 }
 

@@ -23,7 +23,8 @@ i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
 
 def build(force=False):
     so = os.path.join(HERE, "liboracle.so")
-    if force or not os.path.exists(so):
+    src = [os.path.join(HERE, f) for f in ("qtip_oracle.c", "qtip_oracle.h")]
+    if force or not os.path.exists(so) or os.path.getmtime(so) < max(os.path.getmtime(f) for f in src):
         subprocess.check_call(["make", "-C", HERE, "-B" if force else "-s", os.path.join(HERE, "liboracle.so")])
     return so
 

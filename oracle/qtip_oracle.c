@@ -432,31 +432,79 @@ int qo_unswizzle_for_kernel(const uint16_t* in, int m, int n, uint16_t* packed) 
 }
 
 /* ------------------------------------------------------------------ Cholesky / block LDL */
-/* Textbook row-by-row lower Cholesky in fp64 (the reference's blocked code, src/qtip_core.cpp:321-442,
- * computes the same factor with a different summation order). Lower triangle in, lower triangle out. */
+/* Right-looking blocked lower Cholesky in fp64, src/qtip_core.cpp:321-442, with every element formed by the
+ * reference's own sequence of operations (its build contracts a * b + c into one fused operation), so that the
+ * factor equals the compiled reference's bit for bit; checked against it live and through committed rows of L.
+ * Per 256-column panel:
+ *   diagonal block, unblocked (:331-347): s = a_ij; s = fma(-l_ip, l_jp, s) for p ascending inside the block;
+ *     l_jj = sqrt(s_jj); l_ij = s_ij / l_jj;
+ *   rows below (:376-394): four partial sums, s0 from the element and s1..s3 from zero; the full groups of four
+ *     p < j feed s_(p mod 4) = fma(-l_jp, x_p, s_(p mod 4)), leftover p feed s0;
+ *     x_j = ((s0 + s1) + (s2 + s3)) * (1 / l_jj);
+ *   trailing update (:267-317, :409-427): acc = fma(x_ip, x_jp, acc) for p ascending over the panel from zero, then
+ *     c_ij -= acc.
+ * Lower triangle in, lower triangle out. */
 int qo_cholesky(double* A, int n) {
-  for (int j = 0; j < n; ++j) {
-    double* aj = A + (long)j * n;
-    double d = aj[j];
-    for (int p = 0; p < j; ++p) d -= aj[p] * aj[p];
-    if (!(d > 0)) return 0;
-    d = sqrt(d);
-    aj[j] = d;
-    int fail = 0;
-#pragma omp parallel for schedule(static) if (n - j > 256)
-    for (int i = j + 1; i < n; ++i) {
-      double* ai = A + (long)i * n;
-      double s = ai[j];
-      for (int p = 0; p < j; ++p) s -= ai[p] * aj[p];
-      ai[j] = s / d;
+  enum { NB = 256 };
+  double* Lkk = (double*)malloc(sizeof(double) * NB * NB);
+  for (int k = 0; k < n; k += NB) {
+    const int kb = n - k < NB ? n - k : NB;
+    for (int j = k; j < k + kb; ++j) {
+      double* aj = A + (long)j * n;
+      double d = aj[j];
+      for (int p = k; p < j; ++p) d = fma(-aj[p], aj[p], d);
+      if (!(d > 0)) {
+        free(Lkk);
+        return 0;
+      }
+      d = sqrt(d);
+      aj[j] = d;
+      for (int i = j + 1; i < k + kb; ++i) {
+        double* ai = A + (long)i * n;
+        double s = ai[j];
+        for (int p = k; p < j; ++p) s = fma(-ai[p], aj[p], s);
+        ai[j] = s / d;
+      }
     }
-    if (fail) return 0;
+    const int r0 = k + kb;
+    if (r0 >= n) break;
+    for (int j = 0; j < kb; ++j)
+      for (int p = 0; p <= j; ++p) Lkk[j * NB + p] = A[(long)(k + j) * n + k + p];
+#pragma omp parallel for schedule(dynamic, 8)
+    for (int i = r0; i < n; ++i) {
+      double* x = A + (long)i * n + k;
+      for (int j = 0; j < kb; ++j) {
+        const double* lj = Lkk + j * NB;
+        double s0 = x[j], s1 = 0, s2 = 0, s3 = 0;
+        int p = 0;
+        for (; p + 4 <= j; p += 4) {
+          s0 = fma(-lj[p], x[p], s0);
+          s1 = fma(-lj[p + 1], x[p + 1], s1);
+          s2 = fma(-lj[p + 2], x[p + 2], s2);
+          s3 = fma(-lj[p + 3], x[p + 3], s3);
+        }
+        for (; p < j; ++p) s0 = fma(-lj[p], x[p], s0);
+        x[j] = ((s0 + s1) + (s2 + s3)) * (1.0 / lj[j]);
+      }
+    }
+#pragma omp parallel for schedule(dynamic, 8)
+    for (int i = n - 1; i >= r0; --i) {
+      const double* xi = A + (long)i * n + k;
+      for (int j = r0; j <= i; ++j) {
+        const double* xj = A + (long)j * n + k;
+        double acc = 0;
+        for (int p = 0; p < kb; ++p) acc = fma(xi[p], xj[p], acc);
+        A[(long)i * n + j] -= acc;
+      }
+    }
   }
+  free(Lkk);
   return 1;
 }
 
 /* block_LDL(H, 16) followed by zeroing the diagonal blocks, src/qtip_core.cpp:444-487:
- * L = C * blockdiag(C_bb^-1), strictly block-lower, fp32. A (fp64, lower triangle used) is destroyed. */
+ * L = C * blockdiag(C_bb^-1), strictly block-lower, fp32. A (fp64, lower triangle used) is destroyed.
+ * The sums are chains of fused multiply-adds, as the reference's build makes them. */
 int qo_block_ldl_to_L(double* A, int n, float* L) {
   if (n % 16) return 0;
   if (!qo_cholesky(A, n)) return 0;
@@ -469,7 +517,7 @@ int qo_block_ldl_to_L(double* A, int n, float* L) {
     for (int c = 0; c < 16; ++c)
       for (int i = 0; i < 16; ++i) {
         double s = (i == c) ? 1.0 : 0.0;
-        for (int p = 0; p < i; ++p) s -= D[i][p] * Iv[p][c];
+        for (int p = 0; p < i; ++p) s = fma(-D[i][p], Iv[p][c], s);
         Iv[i][c] = s / D[i][i];
       }
     for (int i = 0; i < 16; ++i)
@@ -490,7 +538,7 @@ int qo_block_ldl_to_L(double* A, int n, float* L) {
       const double* iv = inv + (size_t)bj * 256;
       for (int j = 0; j < 16; ++j) {
         double s = 0;
-        for (int p = j; p < 16; ++p) s += a[p] * iv[p * 16 + j];
+        for (int p = j; p < 16; ++p) s = fma(a[p], iv[p * 16 + j], s);
         o[j] = (float)s;
         if (!isfinite(s)) finite = 0;
       }

@@ -10,6 +10,10 @@ oracle/_ref/libqtip_ref.so exists; the GPU box only reads the committed outputs)
   ref_config1.json        FNV-1a 64 of the packed words of all 4096 config-1 tiles (synthetic tlut)
   ref_config1_packed.bin  those packed words (u16 [4096][32], pack_trellis layout, not swizzled)
   ref_ldl_1024.bin        rows 1000..1007 of L (fp32) from block_ldl_to_L on a seeded n=1024 SPD matrix
+  ref_ldl_2560_f32.bin    rows 255, 256, 257, 1279, 1280, 2558, 2559 of L (fp32) from block_ldl_to_L on a seeded
+                          n=2560 SPD matrix rounded to fp32 first (the input type of ldl_hessian): ten 256-column
+                          panels deep, so the rows carry the blocked code's order of operations
+                          (`python make_ref_vectors.py ldl` writes the two LDL files only)
   ref_ldlq_L.bin          a block-LDL factor (f32 [256][256]) and
   ref_ldlq_Q.bin          the states (u16 [64][128]) ldlq_ref of the reference's GPU test program (CPU code,
                           tests/test_gpu.cpp:180-225, compiled into oracle/_ref/libqtip_ref_gpu.so) returns for it and
@@ -48,9 +52,29 @@ def ldl_case(n=1024, seed=3):
     return H
 
 
+LDL_2560_ROWS = (255, 256, 257, 1279, 1280, 2558, 2559)
+
+
+def ldl_vectors(R):
+    H = ldl_case()
+    A = H.copy()
+    L = np.zeros((1024, 1024), np.float32)
+    assert R.ref_block_ldl(A.reshape(-1), 1024, L.reshape(-1), 8) == 1
+    L[1000:1008].tofile(os.path.join(HERE, "ref_ldl_1024.bin"))
+    n = 2560
+    H32 = ldl_case(n, 5).astype(np.float32)
+    A = np.tril(0.5 * (H32.astype(np.float64) + H32.astype(np.float64).T))
+    L = np.zeros((n, n), np.float32)
+    assert R.ref_block_ldl(A.reshape(-1), n, L.reshape(-1), 8) == 1
+    L[list(LDL_2560_ROWS)].tofile(os.path.join(HERE, "ref_ldl_2560_f32.bin"))
+
+
 def main():
     R = ob.ref_lib()
     assert R is not None, "build oracle/_ref first (make -C oracle ref)"
+    if sys.argv[1:] == ["ldl"]:
+        ldl_vectors(R)
+        return
     out = {}
     for seed in (0, 7):
         u = np.zeros(64, np.uint64)
@@ -87,11 +111,7 @@ def main():
                "fnv1a64_states": "%016x" % fnv1a64(st_all.tobytes())},
               open(os.path.join(HERE, "ref_config1.json"), "w"))
 
-    H = ldl_case()
-    A = H.copy()
-    L = np.zeros((1024, 1024), np.float32)
-    assert R.ref_block_ldl(A.reshape(-1), 1024, L.reshape(-1), 8) == 1
-    L[1000:1008].tofile(os.path.join(HERE, "ref_ldl_1024.bin"))
+    ldl_vectors(R)
     # LDLQ with 128-column buffers: the reference's own CPU restatement of ldlq.LDLQ, two buffers, four tile rows
     if ob.ref_gpu_lib() is not None:
         m, n = 64, 256
