@@ -7,14 +7,15 @@
 // The factor is the reference's bit for bit, which fixes the order of operations of every element (the schedule,
 // the register blocking and the data layout are this file's own):
 //   * right-looking panels of width NB = 256;
-//   * diagonal block: left-looking, s = a_ij, then s = fma(-l_ip, l_jp, s) for p ascending inside the block, the
-//     diagonal element the same chain with i = j, sqrt, division by the square root (src/qtip_core.cpp:331-347);
+//   * diagonal block: left-looking, s = a_ij minus the products l_ip * l_jp for p ascending inside the block, fused
+//     or not as the reference's build has them (host_ldl_diag.cpp), sqrt, division by the square root
+//     (src/qtip_core.cpp:329-343);
 //   * rows below the block: x_j = ((s0 + s1) + (s2 + s3)) * (1 / l_jj), where s0 starts at the element, s1..s3 at zero,
 //     s_(p mod 4) = fma(-l_jp, x_p, s_(p mod 4)) over the full groups of four p < j and the leftover p go to s0
 //     (src/qtip_core.cpp:376-394);
 //   * trailing update: c -= acc with acc one chain fma(x_ip, x_jp, acc), p ascending over the panel from zero
 //     (src/qtip_core.cpp:267-317).
-// Here the diagonal block is factored on a transposed copy so that the chains of 8 rows run in one vector, the rows
+// Here the rows
 // below are solved in chunks of NR rows held transposed, and the trailing symmetric update runs as a packed
 // register-blocked rank-NB kernel over lower-triangular tiles handed out dynamically to a team of host threads
 // (host_team.hpp).  The kernels are written with GCC vector extensions and compiled twice (AVX2 baseline, AVX-512
@@ -163,46 +164,12 @@ __attribute__((target("avx512f"))) QTIP_TRI_SOLVE(tri_solve_24, v8d, 8, 24)
 QTIP_TRI_SOLVE(tri_solve_12, v4d, 4, 12)
 #undef QTIP_TRI_SOLVE
 
-// ---- lower Cholesky of the kb x kb diagonal block at A (row stride ld), in the order given at the top of the file.
-// T: scratch of kb * ldt doubles, ldt = kb rounded up to 32; T[p * ldt + i] = l_ip, so that column j is finished by
-// running the chains of the rows i >= j, 8 (or 4) rows to a vector, four vectors in flight.  The lanes of rows i < j
-// carry meaningless values that no later column reads.  false if the block is not positive definite.
-#define QTIP_FACTOR_DIAG(NAME, VT, VW)                                                                         \
-  static bool NAME(double* __restrict__ A, long ld, int kb, double* __restrict__ T, int ldt) {                 \
-    for (int p = 0; p < kb; ++p) {                                                                             \
-      for (int i = 0; i < p; ++i) T[size_t(p) * ldt + i] = 0.0;                                                \
-      for (int i = p; i < kb; ++i) T[size_t(p) * ldt + i] = A[long(i) * ld + p];                               \
-      for (int i = kb; i < ldt; ++i) T[size_t(p) * ldt + i] = 0.0;                                             \
-    }                                                                                                          \
-    for (int j = 0; j < kb; ++j) {                                                                             \
-      double* tj = T + size_t(j) * ldt;                                                                        \
-      for (int i0 = (j / (4 * VW)) * (4 * VW); i0 < kb; i0 += 4 * VW) {                                        \
-        VT a0 = *reinterpret_cast<VT*>(tj + i0), a1 = *reinterpret_cast<VT*>(tj + i0 + VW),                    \
-           a2 = *reinterpret_cast<VT*>(tj + i0 + 2 * VW), a3 = *reinterpret_cast<VT*>(tj + i0 + 3 * VW);       \
-        for (int p = 0; p < j; ++p) {                                                                          \
-          const double* tp = T + size_t(p) * ldt;                                                              \
-          const double l = tp[j];                                                                              \
-          a0 -= l * *reinterpret_cast<const VT*>(tp + i0);                                                     \
-          a1 -= l * *reinterpret_cast<const VT*>(tp + i0 + VW);                                                \
-          a2 -= l * *reinterpret_cast<const VT*>(tp + i0 + 2 * VW);                                            \
-          a3 -= l * *reinterpret_cast<const VT*>(tp + i0 + 3 * VW);                                            \
-        }                                                                                                      \
-        *reinterpret_cast<VT*>(tj + i0) = a0, *reinterpret_cast<VT*>(tj + i0 + VW) = a1;                       \
-        *reinterpret_cast<VT*>(tj + i0 + 2 * VW) = a2, *reinterpret_cast<VT*>(tj + i0 + 3 * VW) = a3;          \
-      }                                                                                                        \
-      double d = tj[j];                                                                                        \
-      if (!(d > 0) || !std::isfinite(d)) return false;                                                         \
-      d = std::sqrt(d);                                                                                        \
-      tj[j] = d;                                                                                               \
-      for (int i = j + 1; i < kb; ++i) tj[i] = tj[i] / d;                                                      \
-    }                                                                                                          \
-    for (int p = 0; p < kb; ++p)                                                                               \
-      for (int i = p; i < kb; ++i) A[long(i) * ld + p] = T[size_t(p) * ldt + i];                               \
-    return true;                                                                                               \
-  }
-__attribute__((target("avx512f"))) QTIP_FACTOR_DIAG(factor_diag_8, v8d, 8)
-QTIP_FACTOR_DIAG(factor_diag_4, v4d, 4)
-#undef QTIP_FACTOR_DIAG
+}  // namespace
+// lower Cholesky of the kb x kb diagonal block at A (row stride ld) (host_ldl_diag.cpp, built without contraction: it
+// has to say which of its operations are fused); T: scratch of kb * ldt doubles, ldt >= kb rounded up to 32
+bool factor_diag_avx512(double* A, long ld, int kb, double* T, int ldt);
+bool factor_diag_avx2(double* A, long ld, int kb, double* T, int ldt);
+namespace {
 
 struct Kernels {
   int MR, NR;
@@ -212,8 +179,8 @@ struct Kernels {
 };
 static Kernels pick_kernels() {
   __builtin_cpu_init();
-  if (__builtin_cpu_supports("avx512f")) return Kernels{8, 24, micro_8x24, tri_solve_24, factor_diag_8};
-  return Kernels{4, 12, micro_4x12, tri_solve_12, factor_diag_4};
+  if (__builtin_cpu_supports("avx512f")) return Kernels{8, 24, micro_8x24, tri_solve_24, factor_diag_avx512};
+  return Kernels{4, 12, micro_4x12, tri_solve_12, factor_diag_avx2};
 }
 
 // Lower Cholesky of the n x n matrix at A (row stride ld) by right-looking panels of width NBT, shared out over the

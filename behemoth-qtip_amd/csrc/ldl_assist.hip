@@ -1,6 +1,6 @@
 // Host fp64 block LDL with the trailing updates on the GPU (host_ldl.cpp, block_ldl_assisted): the host factors and
-// solves one 512-column panel at a time in its own arithmetic, the device holds the symmetric fp64 work matrix and
-// applies the rank-512 updates.  v_mfma_f64_16x16x4_f64 accumulates its four products like a chain of fused
+// solves one 256-column panel at a time in its own arithmetic, the device holds the symmetric fp64 work matrix and
+// applies the rank-256 updates.  v_mfma_f64_16x16x4_f64 accumulates its four products like a chain of fused
 // multiply-adds in ascending k (checked bit for bit against std::fma chains), and the host's micro-kernels form every
 // element of an update as exactly such a chain over the panel depth from zero followed by one subtraction, so the
 // factor is the host's bit for bit.

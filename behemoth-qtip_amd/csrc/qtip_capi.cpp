@@ -448,6 +448,13 @@ int qtip_ldl_hessian(const float* host_HRr, int n, int threads, float* host_L) {
   return guarded([&] { ldl_hessian_impl(host_HRr, n, threads, host_L); });
 }
 
+int qtip_cholesky_inplace(double* host_A, int n, int threads) {
+  return guarded([&] {
+    QTIP_REQUIRE(host_A != nullptr && n > 0, "cholesky_inplace: bad arguments (n = %d)", n);
+    if (!cholesky_lower_host(host_A, n, threads)) throw Error(QTIP_E_NOT_PD, "Cholesky failed (matrix not PD)");
+  });
+}
+
 int qtip_ldl_hessian_device_updates(qtip_ctx* ctx, const float* host_HRr, int n, int threads, float* host_L) {
   return guarded([&] {
     QTIP_REQUIRE(ctx != nullptr, "null context");

@@ -100,9 +100,14 @@ int qtip_rotate_hessian(qtip_ctx* ctx, const float* H, int h_on_device, int n, u
  * HRr n x n fp32 in, L n x n fp32 out (strictly block-lower). */
 int qtip_ldl_hessian(const float* host_HRr, int n, int threads, float* host_L);
 
+/* cholesky_inplace, src/qtip_core.hpp:24-67 / src/qtip_core.cpp:321-442: lower Cholesky factor of the n x n fp64
+ * matrix host_A (row-major, lower triangle read and overwritten, the rest untouched or scratch), the reference's
+ * order of operations, hence its bits.  Host only.  QTIP_E_NOT_PD if the matrix is not positive definite. */
+int qtip_cholesky_inplace(double* host_A, int n, int threads);
+
 /* The same factorization with the trailing updates of the host's panels on the GPU.  No counterpart in the
  * reference (its ldl_hessian is host only, src/quantizer.cpp:154-165): the host still factors and solves every
- * panel in fp64 with its own code, the device keeps the fp64 work matrix and applies the rank-512 updates on the
+ * panel in fp64 with its own code, the device keeps the fp64 work matrix and applies the rank-256 updates on the
  * matrix cores in the host's own order of operations, so host_L is qtip_ldl_hessian's bit for bit.  Works on a
  * stream of its own inside ctx; may run on a side thread while another thread quantizes through the same ctx. */
 int qtip_ldl_hessian_device_updates(qtip_ctx* ctx, const float* host_HRr, int n, int threads, float* host_L);

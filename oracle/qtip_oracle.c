@@ -436,8 +436,12 @@ int qo_unswizzle_for_kernel(const uint16_t* in, int m, int n, uint16_t* packed) 
  * reference's own sequence of operations (its build contracts a * b + c into one fused operation), so that the
  * factor equals the compiled reference's bit for bit; checked against it live and through committed rows of L.
  * Per 256-column panel:
- *   diagonal block, unblocked (:331-347): s = a_ij; s = fma(-l_ip, l_jp, s) for p ascending inside the block;
- *     l_jj = sqrt(s_jj); l_ij = s_ij / l_jj;
+ *   diagonal block, unblocked (:329-343): s = a_ij minus the products l_ip * l_jp, p ascending inside the block;
+ *     l_jj = sqrt(s_jj); l_ij = s_ij / l_jj.  The reference's build (GCC -O3) vectorizes these two sums as
+ *     in-order reductions, which decides what is fused: over the full groups of four p the products are rounded
+ *     on their own and subtracted one after the other; of the len mod 4 terms left, an element below the
+ *     diagonal subtracts two as rounded products (if there are two or three) and the last odd one as a fused
+ *     multiply-add, the diagonal element takes all of them as fused multiply-adds;
  *   rows below (:376-394): four partial sums, s0 from the element and s1..s3 from zero; the full groups of four
  *     p < j feed s_(p mod 4) = fma(-l_jp, x_p, s_(p mod 4)), leftover p feed s0;
  *     x_j = ((s0 + s1) + (s2 + s3)) * (1 / l_jj);
@@ -451,8 +455,14 @@ int qo_cholesky(double* A, int n) {
     const int kb = n - k < NB ? n - k : NB;
     for (int j = k; j < k + kb; ++j) {
       double* aj = A + (long)j * n;
+      const int full = k + ((j - k) & ~3), rem = (j - k) & 3;
       double d = aj[j];
-      for (int p = k; p < j; ++p) d = fma(-aj[p], aj[p], d);
+      for (int p = k; p < full; p += 4) {
+        const double t0 = aj[p] * aj[p], t1 = aj[p + 1] * aj[p + 1], t2 = aj[p + 2] * aj[p + 2],
+                     t3 = aj[p + 3] * aj[p + 3];
+        d = (((d - t0) - t1) - t2) - t3;
+      }
+      for (int p = full; p < j; ++p) d = fma(-aj[p], aj[p], d);
       if (!(d > 0)) {
         free(Lkk);
         return 0;
@@ -462,7 +472,12 @@ int qo_cholesky(double* A, int n) {
       for (int i = j + 1; i < k + kb; ++i) {
         double* ai = A + (long)i * n;
         double s = ai[j];
-        for (int p = k; p < j; ++p) s = fma(-ai[p], aj[p], s);
+        const int unfused = full + (rem >= 2 ? 2 : 0);
+        for (int p = k; p < unfused; ++p) {
+          const double t = ai[p] * aj[p];
+          s -= t;
+        }
+        if (rem & 1) s = fma(-ai[j - 1], aj[j - 1], s);
         ai[j] = s / d;
       }
     }

@@ -13,7 +13,9 @@ oracle/_ref/libqtip_ref.so exists; the GPU box only reads the committed outputs)
   ref_ldl_2560_f32.bin    rows 255, 256, 257, 1279, 1280, 2558, 2559 of L (fp32) from block_ldl_to_L on a seeded
                           n=2560 SPD matrix rounded to fp32 first (the input type of ldl_hessian): ten 256-column
                           panels deep, so the rows carry the blocked code's order of operations
-                          (`python make_ref_vectors.py ldl` writes the two LDL files only)
+  ref_chol_528_rows.bin   rows 255, 256, 300, 511, 512, 527 of the fp64 Cholesky factor (cholesky_inplace) of a seeded
+                          n=528 SPD matrix: every bit of the factor, not only what survives the rounding to fp32
+                          (`python make_ref_vectors.py ldl` writes the three LDL files only)
   ref_ldlq_L.bin          a block-LDL factor (f32 [256][256]) and
   ref_ldlq_Q.bin          the states (u16 [64][128]) ldlq_ref of the reference's GPU test program (CPU code,
                           tests/test_gpu.cpp:180-225, compiled into oracle/_ref/libqtip_ref_gpu.so) returns for it and
@@ -53,6 +55,7 @@ def ldl_case(n=1024, seed=3):
 
 
 LDL_2560_ROWS = (255, 256, 257, 1279, 1280, 2558, 2559)
+CHOL_528_ROWS = (255, 256, 300, 511, 512, 527)
 
 
 def ldl_vectors(R):
@@ -67,6 +70,10 @@ def ldl_vectors(R):
     L = np.zeros((n, n), np.float32)
     assert R.ref_block_ldl(A.reshape(-1), n, L.reshape(-1), 8) == 1
     L[list(LDL_2560_ROWS)].tofile(os.path.join(HERE, "ref_ldl_2560_f32.bin"))
+    n = 528
+    A = np.tril(ldl_case(n, 6))
+    assert R.ref_cholesky(A.reshape(-1), n, 4) == 1
+    np.tril(A)[list(CHOL_528_ROWS)].tofile(os.path.join(HERE, "ref_chol_528_rows.bin"))
 
 
 def main():

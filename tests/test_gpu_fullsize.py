@@ -29,41 +29,81 @@ def check_trellis_paths(st):
     assert np.all(((st[:, :-1] << 4) & 0xffff) == (st[:, 1:] & 0xfff0)), "trellis links"
 
 
-def test_config3_shape_ldlq_row_subset(qz, pkg, oracle, hyb):
-    """n = m = 12288: GPU LDLQ over all 768 tile rows; tile rows 0-1 and 400-401 recomputed by the CPU form from the
-    same WT rows and the same L must give identical codes (>= 99 % is the bar)."""
+def reference_factor(oracle, HRr, threads=16):
+    """L of the rotated Hessian from the REFERENCE's own block_ldl_to_L (its CPU core compiled into oracle/_ref),
+    after the symmetrization of its ldl_hessian (src/quantizer.cpp:154-165).  A missing library is a failure here,
+    not a skip: these tests are what ties the full-depth chains to the reference's factor."""
+    R = oracle.ref_lib()
+    assert R is not None, "oracle/_ref/libqtip_ref.so is missing: build it with make -C oracle ref"
+    n = HRr.shape[0]
+    A = np.empty((n, n), np.float64)
+    blk = 2048
+    for i in range(0, n, blk):                                   # 0.5 * (H + H^T), a row block at a time
+        A[i:i + blk] = 0.5 * (HRr[i:i + blk].astype(np.float64) + HRr[:, i:i + blk].T.astype(np.float64))
+    L = np.zeros((n, n), np.float32)
+    assert R.ref_block_ldl(A.reshape(-1), n, L.reshape(-1), threads) == 1
+    return L
+
+
+def agreement_by_depth(same, nblk, label):
+    """same: (tile rows, n / 16) booleans, column block 0 first.  LDLQ walks from the last column block to the first,
+    so depth octile 0 is the right-most eighth of the columns.  Prints the share of identical trellises per octile."""
+    by_depth = same[:, ::-1]
+    parts = np.array_split(np.arange(nblk), 8)
+    shares = [float(by_depth[:, p].mean()) for p in parts]
+    say("  %s: identical trellises per depth octile (first quantized -> last): %s"
+        % (label, " ".join("%.4f" % v for v in shares)))
+    return shares
+
+
+def test_config3_group_rows_against_reference_chain(qz, pkg, oracle, hyb, synth):
+    """Configuration 3 on its own inputs (12288 x 12288, 1 % of the weights x 10, 32 outlier channels) through the group
+    call, whose factor comes from the library's default LDL (host panels, trailing updates on the GPU).  The reference
+    chain beside it: block_ldl_to_L of the compiled reference on the same rotated Hessian, then the CPU LDLQ on two
+    tile rows.  The two factors must be the same 32-bit words and the codes of those rows identical (>= 99 % is the
+    bar) over all 768 column blocks."""
     import torch
-    say("case: config-3 shape LDLQ, 64-row subset against the CPU form")
+    say("case: config 3 through the group call, 32 rows against reference LDL + CPU LDLQ")
     qz.set_tlut(None)
-    n = m = 12288
-    gen = torch.Generator(device="cuda").manual_seed(5)
-    # SPD Hessian with a decaying spectrum and correlated channels, factored by the library's own host LDL
-    X = torch.randn((4096, n), generator=gen, device="cuda") * torch.linspace(0.3, 2.0, n, device="cuda")
-    X[:, 1:] += 0.7 * X[:, :-1]
-    H = (X.T @ X / 4096.0)
-    H += 0.01 * torch.diagonal(H).mean() * torch.eye(n, device="cuda")
-    hp = pkg.HessPrep(n=n, HRr=H.cpu().numpy())
-    del X, H
-    pkg.Quantizer.ldl_hessian(hp, threads=16)
-    WT = torch.randn((n, m), generator=gen, device="cuda")
-    dL = torch.from_numpy(hp.L).cuda()
-    dH = torch.zeros((n, m), device="cuda")
-    dQ = torch.zeros(((m // 16) * (n // 16), 128), dtype=torch.int16, device="cuda")
+    Ws, H = synth.large_config(3)
+    n, m = H.shape[0], Ws[0].shape[0]
+    seed = 11
+    hp = qz.rotate_hessian(H, n, seed)
+    del H
+    L_ref = reference_factor(oracle, hp.HRr)
+    qz.ldl_hessian_device_updates(hp, threads=16)
+    diff = int(np.count_nonzero(hp.L.view(np.uint32) != L_ref.view(np.uint32)))
+    say("  words of L differing from the reference's factor: %d of %d" % (diff, L_ref.size))
+    assert diff == 0
+    outs, tm = qz.quantize_group([pkg.LinearIn("q", m, w_f32=Ws[0])], hp, pkg.QuantOpts(ldl_threads=16))
+    lo = outs[0]
+    say("  ldlq %.1fs viterbi %.1fs (%.1f Mweights/s) proxy %.5f wscale %.6f"
+        % (tm.ldlq, tm.viterbi, m * n / tm.viterbi / 1e6, lo.proxy, lo.wscale))
+    assert 0 < lo.proxy < 0.2 and 0 < lo.proxy_rot_reg < 0.2
+    st = pkg.unpack_trellis(pkg.unswizzle_for_kernel(lo.trellis, m, n))
+    check_trellis_paths(st)
+    su, sv = pkg.sign_vector(seed, n), pkg.sign_vector(seed * 1000003 + 1, m)
+    assert np.array_equal(hp.su, su) and np.array_equal(lo.sv, sv)
+    # Wr^T = U^T_m (U^T_n (diag(SV) W diag(SU)))^T with the library's transform (pinned bit for bit elsewhere), then
+    # the fp32 multiplication by 1 / Wscale
+    A = Ws[0] * torch.from_numpy(sv).cuda()[:, None] * torch.from_numpy(su).cuda()[None, :]
     torch.cuda.synchronize()
-    vs = qz.ldlq_dev(WT, dL, n, m, dH, dQ, time_viterbi=True)
-    say("  GPU LDLQ done, viterbi %.2fs (%.1f Mweights/s)" % (vs, n * m / vs / 1e6))
-    Q = dQ.cpu().numpy().view(np.uint16).reshape(m // 16, n // 16, 128)
-    check_trellis_paths(Q.reshape(-1, 128))
-    rows = np.r_[0:32, 6400:6432]
-    Wr_sub = np.ascontiguousarray(WT[:, torch.from_numpy(rows).cuda()].cpu().numpy().T)
-    hat_o, Q_o = oracle.ldlq(hyb, Wr_sub, hp.L, threads=16)
-    Q_g = np.concatenate([Q[0:2], Q[400:402]]).reshape(-1, 128)
-    same = np.all(Q_g == Q_o, axis=1).mean()
-    say("  identical trellises on the subset: %.4f of %d" % (same, Q_o.shape[0]))
-    assert same >= 0.99
-    hat_g = dH[:, torch.from_numpy(rows).cuda()].cpu().numpy().T
-    if same == 1.0:
-        assert np.array_equal(hat_g, hat_o)
+    qz.hadamard_rows_dev(A, m, n, n, True)
+    qz.synchronize()
+    AT = A.T.contiguous()
+    del A
+    torch.cuda.synchronize()
+    qz.hadamard_rows_dev(AT, n, m, m, True)
+    qz.synchronize()
+    rows = np.r_[0:16, 6400:6416]
+    sub = (AT[:, torch.from_numpy(rows).cuda()] * float(np.float32(1.0) / np.float32(lo.wscale))).T.contiguous().cpu().numpy()
+    del AT
+    hat_o, Q_o = oracle.ldlq(hyb, sub, L_ref, threads=16)
+    Q_g = st.reshape(m // 16, n // 16, 128)[[0, 400]].reshape(-1, 128)
+    same = np.all(Q_g == Q_o, axis=1).reshape(2, n // 16)
+    agreement_by_depth(same, n // 16, "config 3")
+    say("  identical trellises: %d of %d" % (int(same.sum()), same.size))
+    assert same.mean() >= 0.99
 
 
 def test_config5_group_properties(qz, pkg, oracle, synth):
@@ -91,22 +131,26 @@ def test_config5_group_properties(qz, pkg, oracle, synth):
     assert hist.min() > 0.04 and hist.max() < 0.09
 
 
-def test_config5_depth_ldlq_rows_against_cpu(qz, pkg, oracle, hyb, synth):
-    """n = 28672, the headline depth: a tile row is a chain of 1792 tiles, each depending on every later column.  Two
-    tile rows (32 weight rows, LDLQ is row-independent) through the GPU LDLQ and through the CPU form with the same L,
-    factored by the library's host LDL from the headline configuration's own Hessian: identical codes (>= 99 % is the
-    bar) down the whole chain."""
+def test_config5_depth_rows_against_reference_chain(qz, pkg, oracle, hyb, synth):
+    """n = 28672, the headline depth: a tile row is a chain of 1792 tiles, each depending on every later column.
+    Product chain: the library's default LDL (host panels, trailing updates on the GPU) of the headline
+    configuration's rotated Hessian, then the GPU LDLQ on two tile rows (LDLQ is row-independent).  Reference chain:
+    block_ldl_to_L of the compiled reference on the same rotated Hessian, then the CPU LDLQ on the same rows.  The
+    factors must be the same 32-bit words and the codes identical (>= 99 % is the bar) down the whole chain."""
     import torch
-    say("case: config-5 depth LDLQ, 32 rows against the CPU form")
+    say("case: config-5 depth, own LDL + GPU LDLQ against reference LDL + CPU LDLQ on 32 rows")
     qz.set_tlut(None)
     Ws, H = synth.large_config(5)
     n, m = H.shape[0], 32
-    H += 0.01 * torch.diagonal(H).mean() * torch.eye(n, device="cuda")
     W = Ws[0][4000:4000 + m]
     WT = (W / W.pow(2).mean().sqrt() * 0.9).T.contiguous()        # unit-scale rows at the codebook's working point
-    hp = pkg.HessPrep(n=n, HRr=H.cpu().numpy())
+    hp = qz.rotate_hessian(H, n, 3)
     del Ws, H
-    pkg.Quantizer.ldl_hessian(hp, threads=16)
+    qz.ldl_hessian_device_updates(hp, threads=16)
+    say("  own factor done; reference block_ldl_to_L on 16 threads ...")
+    L_ref = reference_factor(oracle, hp.HRr)
+    diff = int(np.count_nonzero(hp.L.view(np.uint32) != L_ref.view(np.uint32)))
+    say("  words of L differing from the reference's factor: %d of %d" % (diff, L_ref.size))
     dL = torch.from_numpy(hp.L).cuda()
     dH = torch.zeros((n, m), device="cuda")
     dQ = torch.zeros(((m // 16) * (n // 16), 128), dtype=torch.int16, device="cuda")
@@ -116,9 +160,11 @@ def test_config5_depth_ldlq_rows_against_cpu(qz, pkg, oracle, hyb, synth):
     Q = dQ.cpu().numpy().view(np.uint16)
     check_trellis_paths(Q)
     say("  GPU LDLQ done; CPU form on 16 threads ...")
-    hat_o, Q_o = oracle.ldlq(hyb, np.ascontiguousarray(WT.cpu().numpy().T), hp.L, threads=16)
-    same = np.all(Q == Q_o, axis=1)
+    hat_o, Q_o = oracle.ldlq(hyb, np.ascontiguousarray(WT.cpu().numpy().T), L_ref, threads=16)
+    same = np.all(Q == Q_o, axis=1).reshape(m // 16, n // 16)
+    agreement_by_depth(same, n // 16, "config 5")
     say("  identical trellises: %d of %d" % (int(same.sum()), same.size))
+    assert diff == 0
     assert same.mean() >= 0.99
     if same.all():
         assert np.array_equal(dH.cpu().numpy().T, hat_o)
@@ -127,7 +173,8 @@ def test_config5_depth_ldlq_rows_against_cpu(qz, pkg, oracle, hyb, synth):
 def test_config4_two_linears_shared_hessian_rows_against_cpu(qz, pkg, oracle, hyb, synth):
     """gate + up, two stacked 28672 x 12288 linears sharing one Hessian (one SU, one L, two SV / Wscale): the group
     call at full size, then two tile rows of each linear recomputed by the CPU form from the same rotated, scaled
-    rows and the same L must give the codes found in that linear's slice of the packed output (>= 99 % is the bar).
+    rows and the reference's own factor of the same rotated Hessian (which the library's host LDL must equal word for
+    word) must give the codes found in that linear's slice of the packed output (>= 99 % is the bar).
     The rotated rows are formed with the library's own transform, which other tests pin bit for bit."""
     import torch
     say("case: config 4 (two linears, shared Hessian) at full size, 64 rows against the CPU form")
@@ -138,7 +185,8 @@ def test_config4_two_linears_shared_hessian_rows_against_cpu(qz, pkg, oracle, hy
     hp = qz.rotate_hessian(H, n, seed)
     del H
     pkg.Quantizer.ldl_hessian(hp, threads=16)
-    L = hp.L.copy()                                              # the group call consumes hp.L
+    L = reference_factor(oracle, hp.HRr)                         # the reference's own factor of the same matrix
+    assert np.array_equal(hp.L.view(np.uint32), L.view(np.uint32)), "host LDL differs from the reference's factor"
     lins = [pkg.LinearIn("gate", m, w_f32=Ws[0]), pkg.LinearIn("up", m, w_f32=Ws[1])]
     outs, tm = qz.quantize_group(lins, hp, pkg.QuantOpts(ldl_threads=16))
     say("  ldlq %.1fs viterbi %.1fs (%.1f Mweights/s) proxy %.5f / %.5f wscale %.6f / %.6f" %
@@ -175,5 +223,6 @@ def test_config4_two_linears_shared_hessian_rows_against_cpu(qz, pkg, oracle, hy
         hat_o, Q_o = oracle.ldlq(hyb, sub, L, threads=16)
         Q_g = st.reshape(m // 16, n // 16, 128)[[0, 1063]].reshape(-1, 128)
         same = np.all(Q_g == Q_o, axis=1)
+        agreement_by_depth(same.reshape(2, n // 16), n // 16, "config 4 linear %d" % li)
         say("  linear %d: identical trellises %d of %d" % (li, int(same.sum()), same.size))
         assert same.mean() >= 0.99

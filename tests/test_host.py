@@ -101,6 +101,32 @@ def test_host_ldl_matches_oracle(pkg, oracle, n, threads):
         assert np.all(hp.L[16 * b:16 * b + 16, 16 * b:] == 0)
 
 
+def test_cholesky_inplace_fp64_bits(pkg, oracle):
+    """qtip_cholesky_inplace: every bit of the fp64 factor equals the compiled reference's committed rows (n = 528) and
+    the oracle's factor of a matrix with correlated, badly scaled channels (n = 784)."""
+    L = pkg.lib()
+    L.qtip_cholesky_inplace.argtypes = [C.c_void_p, C.c_int, C.c_int]
+    n = 528
+    gm = oracle.rng_normal(6, n * 64).reshape(n, 64)
+    A = np.tril(gm @ gm.T / 64 + 0.05 * np.eye(n))
+    assert L.qtip_cholesky_inplace(A.ctypes.data, n, 3) == 0
+    rows = [255, 256, 300, 511, 512, 527]
+    want = np.fromfile(os.path.join(GOLDEN, "ref_chol_528_rows.bin"), np.uint64).reshape(len(rows), n)
+    assert np.array_equal(np.tril(A)[rows].view(np.uint64), want)
+    n = 784
+    rng = np.random.default_rng(4)
+    G = rng.normal(size=(n, n + 100))
+    G[:, 1:] += 0.8 * G[:, :-1]
+    G[rng.choice(n, 16, replace=False)] *= 20
+    H = np.tril(G @ G.T / (n + 100) + 0.02 * np.eye(n))
+    A, B = H.copy(), H.copy()
+    assert L.qtip_cholesky_inplace(A.ctypes.data, n, 8) == 0
+    assert oracle.lib().qo_cholesky(B.reshape(-1), n) == 1
+    assert np.array_equal(np.tril(A).view(np.uint64), np.tril(B).view(np.uint64))
+    bad = -np.eye(16)
+    assert L.qtip_cholesky_inplace(bad.ctypes.data, 16, 1) == pkg.QTIP_E_NOT_PD
+
+
 def test_host_ldl_golden_1024(pkg, oracle):
     n = 1024
     gm = oracle.rng_normal(3, n * 64).reshape(n, 64)

@@ -51,6 +51,18 @@ def test_ldl_1024_golden(oracle):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_cholesky_528_fp64_golden(oracle):
+    """Every bit of the fp64 factor (two 256-column panels and a ragged third): rows written by the compiled
+    reference's cholesky_inplace."""
+    n = 528
+    gm = oracle.rng_normal(6, n * 64).reshape(n, 64)
+    A = np.tril(gm @ gm.T / 64 + 0.05 * np.eye(n))
+    assert oracle.lib().qo_cholesky(A.reshape(-1), n) == 1
+    rows = [255, 256, 300, 511, 512, 527]
+    want = g("ref_chol_528_rows.bin", np.uint64).reshape(len(rows), n)
+    assert np.array_equal(np.tril(A)[rows].view(np.uint64), want)
+
+
 def test_ldl_2560_f32_golden(oracle):
     n = 2560
     gm = oracle.rng_normal(5, n * 64).reshape(n, 64)
@@ -134,7 +146,13 @@ def test_ref_hadamard_pack_ldl_live(oracle, ref):
     assert np.array_equal(un, oracle.unpack_trellis(a))
     for n in (272, 1024, 1296):
         G = rng.normal(size=(n, n + 128))
+        if n == 1296:        # correlated channels and a few of large scale: the fp32 rounding of L hides less here
+            G[:, 1:] += 0.8 * G[:, :-1]
+            G[rng.choice(n, 16, replace=False)] *= 20
         H = G @ G.T / (n + 128) + 0.02 * np.eye(n)
+        C1, C2 = np.tril(H), np.tril(H)
+        assert ref.ref_cholesky(C1.reshape(-1), n, 4) == 1 and L.qo_cholesky(C2.reshape(-1), n) == 1
+        assert np.array_equal(np.tril(C1).view(np.uint64), np.tril(C2).view(np.uint64)), "fp64 Cholesky factors differ"
         A = H.copy()
         Lr = np.zeros((n, n), np.float32)
         assert ref.ref_block_ldl(A.reshape(-1), n, Lr.reshape(-1), 4) == 1
