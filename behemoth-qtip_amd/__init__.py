@@ -36,6 +36,17 @@ def build(jobs=8):
     return LIB_PATH
 
 
+def _stream_handle(stream):
+    if stream is None:
+        import sys
+        torch = sys.modules.get("torch")
+        if torch is None or not torch.cuda.is_available():
+            return None
+        stream = torch.cuda.current_stream()
+    h = getattr(stream, "cuda_stream", stream)
+    return C.c_void_p(int(h)) if h else None
+
+
 class _LinearInC(C.Structure):
     _fields_ = [("m", C.c_int), ("w_f32", C.c_void_p), ("w_bf16", C.c_void_p), ("w_fp8", C.c_void_p),
                 ("scale_bf16", C.c_void_p), ("on_device", C.c_int)]
@@ -48,7 +59,8 @@ class _LinearOutC(C.Structure):
 
 class _OptsC(C.Structure):
     _fields_ = [("sigma_reg", C.c_double), ("scale_override", C.c_double), ("ldl_threads", C.c_int),
-                ("feedback", C.c_int), ("skip_proxy", C.c_int), ("ldl_device_updates", C.c_int)]
+                ("feedback", C.c_int), ("skip_proxy", C.c_int), ("ldl_device_updates", C.c_int),
+                ("ldlq_chains", C.c_int)]
 
 
 class _TimingC(C.Structure):
@@ -89,6 +101,9 @@ def lib():
     L.qtip_viterbi_tiles.argtypes = [vp, vp, l, vp, vp]
     L.qtip_viterbi_tiles_dev.argtypes = [vp, vp, l, vp, vp]
     L.qtip_viterbi_tiles_dev_noalloc.argtypes = [vp, vp, l, vp, vp]
+    L.qtip_stream_wait.argtypes = [vp, vp]
+    L.qtip_stream_signal.argtypes = [vp, vp]
+    L.qtip_device_lut.argtypes = [vp, C.POINTER(vp)]
     L.qtip_decode_states_dev.argtypes = [vp, vp, l, vp]
     L.qtip_hadamard_rows_dev.argtypes = [vp, vp, l, i, l, i]
     L.qtip_decode_trellis_dev.argtypes = [vp, vp, i, i, vp]
@@ -185,6 +200,7 @@ class QuantOpts:  # src/quantizer.hpp:11-19
     feedback: int = 0          # 0: fp64 feedback (default), 1: fp32 feedback + bf16 hi/lo split MFMA
     skip_proxy: bool = False
     ldl_device_updates: bool = True    # the LDL's trailing updates run on the GPU (same L bit for bit); False: host alone
+    ldlq_chains: int = 0       # independent chains of launches the tile rows are dealt to (0: the library's default, 2)
 
 
 @dataclass
@@ -266,6 +282,21 @@ class Quantizer:
 
     def synchronize(self):
         _check(lib().qtip_synchronize(self._h))
+
+    def stream_wait(self, stream=None):
+        """The context's stream waits for everything queued so far on `stream` (a hipStream_t as an integer, a
+        torch.cuda.Stream, or None: torch's current stream if torch is loaded, else the null stream)."""
+        _check(lib().qtip_stream_wait(self._h, _stream_handle(stream)))
+
+    def stream_signal(self, stream=None):
+        """`stream` waits for everything queued so far on the context's stream."""
+        _check(lib().qtip_stream_signal(self._h, _stream_handle(stream)))
+
+    def device_lut(self):
+        """Device address of the 65536-entry fp16-pair table (device_lut(), src/quantizer.cpp:14-28)."""
+        p = C.c_void_p()
+        _check(lib().qtip_device_lut(self._h, C.byref(p)))
+        return p.value
 
     def set_tlut(self, tlut):
         t = None if tlut is None else np.ascontiguousarray(tlut, np.float32).reshape(1024)
@@ -392,7 +423,7 @@ class Quantizer:
             cout[k].hatW = _ptr(o.hatW)
             outs.append(o)
         co = _OptsC(opt.sigma_reg, opt.scale_override, opt.ldl_threads, opt.feedback, 1 if opt.skip_proxy else 0,
-                    1 if opt.ldl_device_updates else 0)
+                    1 if opt.ldl_device_updates else 0, opt.ldlq_chains)
         return cin, cout, outs, co, keep
 
     @staticmethod

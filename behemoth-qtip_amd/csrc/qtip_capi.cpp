@@ -1,6 +1,8 @@
 // extern "C" surface of libqtip_mi355.so (declared in include/qtip_mi355.h).  Exceptions thrown by the
 // implementation stop here and become return codes plus a thread-local message.
+#include <algorithm>
 #include <chrono>
+#include <cstdlib>
 #include <cstring>
 #include <exception>
 #include <vector>
@@ -47,6 +49,16 @@ void upload_codebook(qtip_ctx* c) {
   QTIP_HIP(hipMemcpyAsync(c->d_entry_d, c->cb.entry_d, sizeof(c->cb.entry_d), hipMemcpyHostToDevice, c->stream));
   QTIP_HIP(hipMemcpyAsync(c->d_entry_f, c->cb.entry_f, sizeof(c->cb.entry_f), hipMemcpyHostToDevice, c->stream));
   QTIP_HIP(hipStreamSynchronize(c->stream));
+}
+
+// the context's stream waits for `other` (or the reverse): an event recorded on one, waited for on the other
+static void order_streams(hipStream_t first, hipStream_t then) {
+  hipEvent_t e;
+  QTIP_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  hipError_t rc = hipEventRecord(e, first);
+  if (rc == hipSuccess) rc = hipStreamWaitEvent(then, e, 0);
+  (void)hipEventDestroy(e);  // released once the recorded work has completed
+  QTIP_HIP(rc);
 }
 
 void ensure_viterbi_workspace(qtip_ctx* c) {
@@ -110,6 +122,11 @@ void qtip_destroy(qtip_ctx* ctx) {
     (void)hipStreamSynchronize(ctx->ldl_stream);
     (void)hipStreamDestroy(ctx->ldl_stream);
   }
+  for (hipStream_t cs : ctx->chain_stream)
+    if (cs) {
+      (void)hipStreamSynchronize(cs);
+      (void)hipStreamDestroy(cs);
+    }
   if (ctx->stream) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipStreamDestroy(ctx->stream);
@@ -134,6 +151,43 @@ int qtip_set_tlut(qtip_ctx* ctx, const float* host_tlut) {
     QTIP_HIP(hipStreamSynchronize(ctx->stream));
     ctx->cb.build(host_tlut);
     upload_codebook(ctx);
+    ctx->lut_h2_valid = false;
+  });
+}
+
+int qtip_stream_wait(qtip_ctx* ctx, void* caller_stream) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "null context");
+    DeviceGuard g(ctx);
+    order_streams(static_cast<hipStream_t>(caller_stream), ctx->stream);
+  });
+}
+
+int qtip_stream_signal(qtip_ctx* ctx, void* caller_stream) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "null context");
+    DeviceGuard g(ctx);
+    order_streams(ctx->stream, static_cast<hipStream_t>(caller_stream));
+  });
+}
+
+int qtip_device_lut(qtip_ctx* ctx, const uint32_t** dev_lut_h2) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && dev_lut_h2 != nullptr, "device_lut: bad arguments");
+    DeviceGuard g(ctx);
+    if (!ctx->lut_h2_valid) {
+      std::vector<uint32_t> h2(static_cast<size_t>(kStates));
+      for (uint32_t s = 0; s < uint32_t(kStates); ++s) {
+        const uint32_t e = HostCodebook::entry_of_state(s);
+        const uint32_t h0 = uint32_t(ctx->cb.tlut_h[e & 511u][0]) ^ ((e >> 9) ? 0x8000u : 0u);
+        h2[s] = h0 | (uint32_t(ctx->cb.tlut_h[e & 511u][1]) << 16);
+      }
+      ctx->d_lut_h2.ensure(h2.size());
+      QTIP_HIP(hipMemcpyAsync(ctx->d_lut_h2, h2.data(), h2.size() * 4, hipMemcpyHostToDevice, ctx->stream));
+      QTIP_HIP(hipStreamSynchronize(ctx->stream));
+      ctx->lut_h2_valid = true;
+    }
+    *dev_lut_h2 = ctx->d_lut_h2.p;
   });
 }
 
@@ -265,6 +319,7 @@ void qtip_default_opts(qtip_opts* o) {
   o->feedback = 0;
   o->skip_proxy = 0;
   o->ldl_device_updates = 1;
+  o->ldlq_chains = 0;
 }
 
 void qtip_pack_trellis(const uint16_t* states, long B, uint16_t* packed) { pack_trellis_host(states, B, packed); }
@@ -468,7 +523,7 @@ int qtip_ldlq_dev(qtip_ctx* ctx, const float* dev_WT, const float* dev_L, long n
   return guarded([&] {
     QTIP_REQUIRE(ctx != nullptr && dev_WT && dev_L && dev_hatWT && dev_Q, "ldlq: bad arguments");
     DeviceGuard g(ctx);
-    ldlq_impl(ctx, dev_WT, dev_L, n, m, dev_hatWT, dev_Q, feedback, vit_seconds);
+    ldlq_impl(ctx, dev_WT, dev_L, n, m, dev_hatWT, dev_Q, feedback, vit_seconds, 0);
   });
 }
 

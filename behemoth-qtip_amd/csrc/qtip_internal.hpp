@@ -172,7 +172,7 @@ struct TileJob {
   long tiles = 0;
   // LDLQ feedback (X null): tile t covers weight rows 16 t .. 16 t + 15 and the columns col0 .. col0 + 15; the
   // target of (row j, column col0 + c) is
-  //   WT[(col0 + c) * ldw + j] + prod[(col0 + c - prod_row0) * ldw + j]
+  //   WT[(col0 + c) * ldw + j] + prod[(col0 + c - prod_row0) * ldp + j]
   //     + sum over k = col0 + 16 .. bufend - 1 (ascending) of L[k * ldl + col0 + c] * (WT - hatWT)[k * ldw + j],
   // accumulated in the type of prod (prod64 or prod32, whichever is set) and rounded to fp32, then to fp16.
   const float* WT = nullptr;
@@ -182,6 +182,7 @@ struct TileJob {
   const double* prod64 = nullptr;
   const float* prod32 = nullptr;
   long prod_row0 = 0;
+  long ldp = 0;  // row stride of prod (0: ldw)
   // outputs (any may be null)
   uint16_t* states = nullptr;  // state words of tile t at states[(t * q_tile_stride + q_offset) * 128]
   long q_tile_stride = 1, q_offset = 0;
@@ -200,6 +201,8 @@ int viterbi_static_slots();
 void viterbi_static_scratch_init(int device);
 void* viterbi_static_scratch(int device);
 void launch_decode_states(const uint16_t* states, long B, float* hat, const float* d_entry_f, hipStream_t s);
+// keeps the stream busy for about `microseconds` (one wave watching the clock, with a bound on its turns)
+void launch_delay(double microseconds, hipStream_t s);
 
 }  // namespace qtipmi
 

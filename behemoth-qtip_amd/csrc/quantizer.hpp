@@ -148,8 +148,12 @@ inline void dump_linear(const QuantOpts& opt, const std::string& tag, const Line
 }
 }  // namespace detail
 
-inline void rotate_hessian(hipStream_t, const float* H, int n, uint64_t seed, const QuantOpts& opt, HessPrep& hp) {
+// The reference queues its work on the caller's stream s.  Here the context's stream first waits for what s holds so
+// far (device memory or host buffers that s is still filling are complete before they are read); every call below is
+// complete on the host when it returns, as the reference's is.
+inline void rotate_hessian(hipStream_t s, const float* H, int n, uint64_t seed, const QuantOpts& opt, HessPrep& hp) {
   const double t0 = detail::now_s();
+  detail::check(qtip_stream_wait(detail::context(), s), "rotate_hessian");
   hp.n = n;
   hp.seed = seed;
   hp.su.resize(size_t(n));
@@ -168,9 +172,10 @@ inline void ldl_hessian(HessPrep& hp, int threads, const std::string& tag) {
   hp.t_ldl = detail::now_s() - t0;
 }
 
-inline std::vector<LinearOut> quantize_group(hipStream_t, Gemm&, const std::vector<LinearIn>& lins, HessPrep& hp,
+inline std::vector<LinearOut> quantize_group(hipStream_t s, Gemm&, const std::vector<LinearIn>& lins, HessPrep& hp,
                                              const QuantOpts& opt, GroupTiming* tm, const std::string& tag) {
   if (!opt.share_su) detail::die("share_su=false not supported (one LDL per group)");
+  detail::check(qtip_stream_wait(detail::context(), s), "quantize_group");
   const bool need_hat = opt.want_hatW || !opt.dump_dir.empty();
   const int n = hp.n;
   std::vector<qtip_linear_in> cin(lins.size());
@@ -221,16 +226,20 @@ inline std::vector<LinearOut> quantize_group(hipStream_t s, Gemm& gemm, const st
 
 // WT n x m, L n x n, hatWT n x m, Q on the device (src/quantizer.hpp:70-73); vit_batch and the LUT pointer are
 // accepted for source compatibility (the library holds its own codebook tables).
-inline void ldlq_gpu(hipStream_t, Gemm&, const float* WT, const float* L, long n, long m, float* hatWT, uint16_t* Q,
+inline void ldlq_gpu(hipStream_t s, Gemm&, const float* WT, const float* L, long n, long m, float* hatWT, uint16_t* Q,
                      int /*vit_batch*/, const uint32_t* /*lut_h2_dev*/, double* vit_s) {
+  // WT and L may still be in the making on s (the reference's quantize_group forms them there and calls this without
+  // a synchronization in between, src/quantizer.cpp:239-265); the call returns with hatWT and Q complete
+  detail::check(qtip_stream_wait(detail::context(), s), "ldlq_gpu");
   detail::check(qtip_ldlq_dev(detail::context(), WT, L, n, m, hatWT, Q, 0, vit_s), "ldlq_gpu");
 }
 
-// The reference returns its device half2 LUT; the library keeps its tables private, so this only makes sure the
-// context (and with it the tables) exists on the current device.
+// src/quantizer.cpp:14-28: the decoded table on the current device, one fp16 pair per state.  (The library's own
+// kernels read tables of the 1024 distinct entries; this one exists for callers that hand it to kernels of theirs.)
 inline const uint32_t* device_lut() {
-  (void)detail::context();
-  return nullptr;
+  const uint32_t* p = nullptr;
+  detail::check(qtip_device_lut(detail::context(), &p), "device_lut");
+  return p;
 }
 
 // ---------------------------------------------------------------- callers either side of quantize_group

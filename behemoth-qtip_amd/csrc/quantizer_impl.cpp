@@ -2,6 +2,7 @@
 // Operation order, seeds and formulas follow the reference's src/quantizer.cpp:30-346 (cited per step).
 #include "quantizer_impl.hpp"
 
+#include <algorithm>
 #include <chrono>
 #include <cmath>
 
@@ -84,74 +85,136 @@ void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L) 
 }
 
 // ---------------------------------------------------------------- ldlq_gpu, src/quantizer.cpp:30-89
+// Given L, the tile rows of a group are independent of each other (the feedback of a weight row comes from its own
+// residuals only), so the tile rows are dealt to up to three chains, each with its own stream, feedback slab and share
+// of the kept-metrics slots, which walk the column blocks by themselves.  The chains start a third of a tile's time
+// apart and keep that distance: while the workgroups of one chain walk their trace-backs (a chain of HBM round
+// trips during which they issue next to nothing), those of the other two, resident on the same compute units, run
+// their forward passes.  One chain alone leaves the chip idle for the length of every trace-back.
 void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, float* hatWT, uint16_t* Q, int feedback,
-               double* vit_seconds) {
+               double* vit_seconds, int chains) {
   QTIP_REQUIRE(n % 128 == 0, "LDLQ needs n %% 128 == 0 (n = %ld)", n);
+  QTIP_REQUIRE(chains >= 0 && chains <= 3, "LDLQ runs as 1 to 3 chains (0: default), not %d", chains);
   QTIP_REQUIRE(m % 16 == 0 && m > 0, "LDLQ needs m %% 16 == 0 (m = %ld)", m);
   QTIP_REQUIRE(feedback == 0 || feedback == 1, "unknown feedback mode %d", feedback);
   hipStream_t s = c->stream;
   ensure_viterbi_workspace(c);
   const long ntr = m / 16, nblk = n / 16;
+  // chains: only where every chain still fills its share of the chip
+  int nch = chains == 0 ? 2 : chains;
+  while (nch > 1 && ntr < long(nch) * (c->vit_slots / nch)) --nch;
+  struct Chain {
+    hipStream_t s;
+    long tile0, tiles;   // tile rows tile0 .. tile0 + tiles - 1
+    long r0, rows;       // weight rows (columns of WT) 16 tile0 .., 16 tiles of them
+    int slot0, slots;    // share of the kept-metrics workspace
+    double* prod;        // feedback 0: 128 x rows slab
+    double* parts;
+  } ch[3];
+  for (int k = 0; k < nch; ++k) {
+    if (k > 0 && !c->chain_stream[k - 1]) QTIP_HIP(hipStreamCreateWithFlags(&c->chain_stream[k - 1], hipStreamNonBlocking));
+    ch[k].s = k == 0 ? s : c->chain_stream[k - 1];
+    ch[k].tile0 = ntr * k / nch;
+    ch[k].tiles = ntr * (k + 1) / nch - ch[k].tile0;
+    ch[k].r0 = 16 * ch[k].tile0;
+    ch[k].rows = 16 * ch[k].tiles;
+    ch[k].slot0 = c->vit_slots * k / nch;
+    ch[k].slots = c->vit_slots * (k + 1) / nch - ch[k].slot0;
+  }
   // feedback 0: fp64 feedback sums; the feedback of the rows quantized in earlier buffers is gathered per buffer
-  // into a 128 x m fp64 slab.  feedback 1: fp32 sums, an n x m fp32 prod cache updated after every buffer by the
-  // bf16 hi/lo split MFMA product
-  DBuf<double> prod(feedback == 0 ? size_t(128) * m : 0), parts(feedback == 0 ? size_t(5) * 128 * m : 0);
+  // into a 128 x rows fp64 slab per chain.  feedback 1: fp32 sums, an n x m fp32 prod cache updated after every
+  // buffer by the bf16 hi/lo split MFMA product
+  const int max_splits = gemm_splitk_splits(n);
+  DBuf<double> prod(feedback == 0 ? size_t(128) * m : 0), parts(feedback == 0 ? size_t(max_splits) * 128 * m : 0);
+  for (int k = 0; k < nch && feedback == 0; ++k) {
+    ch[k].prod = prod.p + size_t(128) * ch[k].r0;
+    ch[k].parts = parts.p + size_t(max_splits) * 128 * ch[k].r0;
+  }
   DBuf<float> prod32(feedback == 1 ? size_t(n) * m : 0);
   if (feedback == 1) QTIP_HIP(hipMemsetAsync(prod32, 0, prod32.bytes(), s));
   QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
-  Events timed, pacing;  // timed: a (start, stop) pair per Viterbi launch, stamped by the launch itself
+  Events timed, pacing, joins;  // timed: a (start, stop) pair per Viterbi launch, stamped by the launch itself
+  // the other chains start once the caller's inputs and the cleared outputs are there, a third (two thirds) of a
+  // tile's time later; a resident workgroup takes about 1.25 ms for a tile, and a launch walks tiles / slots of them
+  if (nch > 1) {
+    hipEvent_t ready = joins.add(hipEventDisableTiming);
+    QTIP_HIP(hipEventRecord(ready, s));
+    for (int k = 1; k < nch; ++k) {
+      QTIP_HIP(hipStreamWaitEvent(ch[k].s, ready, 0));
+      const double launch_us = 1250.0 * double((ch[k].tiles + ch[k].slots - 1) / ch[k].slots);
+      launch_delay(launch_us * k / nch, ch[k].s);
+    }
+  }
   // The queue is kept kAhead buffers (8 launches of ~2 ms each) ahead of the GPU and no further: without a bound the
   // submitting thread would spin on a full queue and take a core from the host LDL of the next group; with less
   // slack a submitting thread that the scheduler holds back for a few milliseconds leaves the GPU idle.
   constexpr long kAhead = 4;
-  hipEvent_t pace[kAhead + 1];
-  for (auto& e : pace) e = pacing.add(hipEventBlockingSync | hipEventDisableTiming);
-  long nbuf_done = 0;
-  for (long cur = nblk; cur > 0; cur -= 8, ++nbuf_done) {
-    const int bufend = int(16 * cur), c0 = bufend - 128;
-    if (nbuf_done >= kAhead) QTIP_HIP(hipEventSynchronize(pace[(nbuf_done - kAhead) % (kAhead + 1)]));
-    if (feedback == 0) {  // prod[r][:] = sum_{k >= bufend} L[k][c0 + r] (WT - hatWT)[k][:], r < 128
-      if (bufend < n)
-        launch_gemm_tn_f64_gather(int(m), n - bufend, L + long(bufend) * n + c0, n, WT + long(bufend) * m,
-                                  hatWT + long(bufend) * m, m, prod, parts, s);
-      else
-        QTIP_HIP(hipMemsetAsync(prod, 0, prod.bytes(), s));
+  hipEvent_t pace[3][kAhead + 1];
+  for (int k = 0; k < nch; ++k)
+    for (auto& e : pace[k]) e = pacing.add(hipEventBlockingSync | hipEventDisableTiming);
+  try {
+    long nbuf_done = 0;
+    for (long cur = nblk; cur > 0; cur -= 8, ++nbuf_done) {
+      const int bufend = int(16 * cur), c0 = bufend - 128;
+      for (int k = 0; k < nch; ++k) {
+        const Chain& C = ch[k];
+        if (nbuf_done >= kAhead) QTIP_HIP(hipEventSynchronize(pace[k][(nbuf_done - kAhead) % (kAhead + 1)]));
+        if (feedback == 0) {  // prod[r][:] = sum_{k >= bufend} L[k][c0 + r] (WT - hatWT)[k][:], r < 128
+          if (bufend < n)
+            launch_gemm_tn_f64_gather(int(C.rows), n - bufend, L + long(bufend) * n + c0, n, WT + long(bufend) * m + C.r0,
+                                      hatWT + long(bufend) * m + C.r0, m, C.prod, C.parts, C.s);
+          else
+            QTIP_HIP(hipMemsetAsync(C.prod, 0, size_t(128) * C.rows * sizeof(double), C.s));
+        }
+        for (int i = 7; i >= 0; --i) {  // the kernel forms the block's targets (in-buffer feedback) itself
+          const int col0 = c0 + 16 * i;
+          TileJob job;
+          job.tiles = C.tiles;
+          job.WT = WT + C.r0;
+          job.L = L;
+          job.ldl = n;
+          job.bufend = bufend;
+          if (feedback == 0) job.prod64 = C.prod, job.prod_row0 = c0, job.ldp = C.rows;
+          else job.prod32 = prod32 + C.r0;
+          job.states = Q + size_t(C.tile0) * nblk * 128;
+          job.q_tile_stride = nblk;
+          job.q_offset = col0 / 16;
+          job.hatWT = hatWT + C.r0;
+          job.ldw = m;
+          job.col0 = col0;
+          hipEvent_t t0 = nullptr, t1 = nullptr;
+          if (vit_seconds) t0 = timed.add(hipEventDefault), t1 = timed.add(hipEventDefault);
+          launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws.p + viterbi_workspace_bytes(C.slot0), C.slots,
+                               C.s, t0, t1);
+        }
+        if (c0 > 0 && feedback == 1) {  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
+          launch_gemm_tn_bf16x3_acc(c0, int(C.rows), 128, L + long(c0) * n, n, WT + long(c0) * m + C.r0,
+                                    hatWT + long(c0) * m + C.r0, m, prod32 + C.r0, m, C.s);
+        }
+        QTIP_HIP(hipEventRecord(pace[k][nbuf_done % (kAhead + 1)], C.s));
+      }
     }
-    for (int i = 7; i >= 0; --i) {  // the kernel forms the block's targets (in-buffer feedback) itself
-      const int col0 = c0 + 16 * i;
-      TileJob job;
-      job.tiles = ntr;
-      job.WT = WT;
-      job.L = L;
-      job.ldl = n;
-      job.bufend = bufend;
-      if (feedback == 0) job.prod64 = prod, job.prod_row0 = c0;
-      else job.prod32 = prod32;
-      job.states = Q;
-      job.q_tile_stride = nblk;
-      job.q_offset = col0 / 16;
-      job.hatWT = hatWT;
-      job.ldw = m;
-      job.col0 = col0;
-      hipEvent_t t0 = nullptr, t1 = nullptr;
-      if (vit_seconds) t0 = timed.add(hipEventDefault), t1 = timed.add(hipEventDefault);
-      launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws, c->vit_slots, s, t0, t1);
+    // the caller's stream continues when every chain is through
+    for (int k = 1; k < nch; ++k) {
+      hipEvent_t done = joins.add(hipEventDisableTiming);
+      QTIP_HIP(hipEventRecord(done, ch[k].s));
+      QTIP_HIP(hipStreamWaitEvent(s, done, 0));
     }
-    if (c0 > 0 && feedback == 1) {  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
-      launch_gemm_tn_bf16x3_acc(c0, int(m), 128, L + long(c0) * n, n, WT + long(c0) * m, hatWT + long(c0) * m, m,
-                                prod32, m, s);
-    }
-    QTIP_HIP(hipEventRecord(pace[nbuf_done % (kAhead + 1)], s));
+  } catch (...) {
+    // nothing queued on a chain may outlive the buffers of this call
+    for (int k = 0; k < nch; ++k) (void)hipStreamSynchronize(ch[k].s);
+    throw;
   }
   wait_stream_sleeping(s);
   if (vit_seconds) {
+    // the chains' launches overlap: the time the column blocks take is the launches' total over the chains
     double t = 0;
     for (size_t i = 0; i + 1 < timed.ev.size(); i += 2) {
       float ms = 0;
       QTIP_HIP(hipEventElapsedTime(&ms, timed.ev[i], timed.ev[i + 1]));
       t += ms * 1e-3;
     }
-    *vit_seconds = t;
+    *vit_seconds = t / nch;
   }
 }
 
@@ -242,7 +305,7 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
   DBuf<float> hatWT(size_t(n) * mt);
   DBuf<uint16_t> Q(size_t(mt / 16) * (n / 16) * 128);
   double vit = 0;
-  ldlq_impl(c, WT, dev_L ? dev_L : Ld.p, n, mt, hatWT, Q, opt.feedback, &vit);
+  ldlq_impl(c, WT, dev_L ? dev_L : Ld.p, n, mt, hatWT, Q, opt.feedback, &vit, opt.ldlq_chains);
   T.ldlq += now_s() - t0;
   T.viterbi += vit;
   t0 = now_s();

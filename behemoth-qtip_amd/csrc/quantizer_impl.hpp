@@ -11,8 +11,13 @@ struct qtip_ctx {
   qtipmi::HostCodebook cb;
   qtipmi::DBuf<double> d_entry_d;  // [1024][2] decoded codebook entries, fp64
   qtipmi::DBuf<float> d_entry_f;   // [1024][2] the same as fp32
+  qtipmi::DBuf<uint32_t> d_lut_h2; // [65536] fp16 pairs per state, built when a caller asks for it
+  bool lut_h2_valid = false;
   qtipmi::DBuf<unsigned char> vit_ws;  // kept-metrics slots of the resident Viterbi workgroups
   int vit_slots = 0;
+  // LDLQ runs its tile rows as up to three independent chains of launches, on the context's stream and these two,
+  // a third of a tile's time apart, so that one chain's trace-backs run under the others' forward passes
+  hipStream_t chain_stream[2] = {nullptr, nullptr};
   qtipmi::Rht rht;
   qtipmi::DBuf<double> scratch;
   qtipmi::HBuf<float> ring_HRr[3], ring_L[3];  // page-locked staging of run_groups, kept between calls
@@ -33,7 +38,7 @@ void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L);
 void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int threads, float* host_L,
                                const float* dev_HRr = nullptr, float* dev_L = nullptr);
 void ldlq_impl(qtip_ctx* c, const float* dWT, const float* dL, long n, long m, float* d_hatWT, uint16_t* dQ,
-               int feedback, double* vit_seconds);
+               int feedback, double* vit_seconds, int chains);
 void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
                          double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
                          qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr = nullptr,

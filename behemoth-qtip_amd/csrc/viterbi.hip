@@ -336,7 +336,7 @@ __device__ __forceinline__ void tile_targets(Smem& sm, const TileJob& job, long 
   __syncthreads();
   const int q = perm_fwd(u), r = q >> 4, c = q & 15;
   const long col = job.col0 + c;
-  Acc acc = Acc(job.WT[col * job.ldw + row0 + r]) + prod[(col - job.prod_row0) * job.ldw + row0 + r];
+  Acc acc = Acc(job.WT[col * job.ldw + row0 + r]) + prod[(col - job.prod_row0) * (job.ldp ? job.ldp : job.ldw) + row0 + r];
   for (int kk = 0; kk < nk; ++kk) acc += Acc(Ls[kk * 16 + c]) * (Acc(Ws[kk * 16 + r]) - Acc(Hs[kk * 16 + r]));
   sm.x[u] = float(_Float16(float(acc)));
 }
@@ -495,6 +495,12 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
   }
 }
 
+// One wave that returns after `ticks` of the constant-rate clock (100 MHz), or after a bounded number of looks at it.
+__global__ void delay_kernel(unsigned long long ticks) {
+  const unsigned long long t0 = wall_clock64();
+  for (int i = 0; i < (1 << 22) && wall_clock64() - t0 < ticks; ++i) __builtin_amdgcn_s_sleep(32);
+}
+
 __global__ void decode_states_kernel(const uint16_t* __restrict__ st, long count, float* __restrict__ hat,
                                      const float* __restrict__ entry_f) {
   const long i = long(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -562,6 +568,12 @@ void* viterbi_static_scratch(int device) {
   if (device < 0 || device >= kMaxDevices) return nullptr;
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   return g_scratch_ptr[device];
+}
+
+void launch_delay(double microseconds, hipStream_t s) {
+  if (microseconds <= 0) return;
+  delay_kernel<<<dim3(1), dim3(64), 0, s>>>((unsigned long long)(microseconds * 100.0));
+  QTIP_HIP(hipGetLastError());
 }
 
 void launch_decode_states(const uint16_t* states, long B, float* hat, const float* d_entry_f, hipStream_t s) {

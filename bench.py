@@ -117,7 +117,7 @@ def run_group(args, pkg):
     ms = [int(w.shape[0]) for w in Ws]
     lins = [pkg.LinearIn("w%d" % i, m, w_f32=w) for i, (m, w) in enumerate(zip(ms, Ws))]
     opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback,
-                        ldl_device_updates=not args.host_ldl)
+                        ldl_device_updates=not args.host_ldl, ldlq_chains=args.chains)
     weights_per_step = sum(ms) * n
 
     stats = {}
@@ -152,7 +152,7 @@ def run_group(args, pkg):
         # reference factors; fewer groups, so the one exposed factorization at the start weighs more
         kh = min(args.steps, 6)
         hopt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback,
-                             ldl_device_updates=False)
+                             ldl_device_updates=False, ldlq_chains=args.chains)
         q.synchronize()
         th = time.time()
         hres = q.run_groups([(lins, n, H, 3 + k) for k in range(kh)], hopt)
@@ -229,6 +229,8 @@ def main():
                     help="skip the extra host-only-LDL groups reported beside the default run")
     ap.add_argument("--feedback", type=int, default=0, choices=[0, 1],
                     help="0: fp64 LDLQ feedback (default); 1: fp32 feedback + bf16 hi/lo split MFMA prod cache")
+    ap.add_argument("--chains", type=int, default=0, choices=[0, 1, 2, 3],
+                    help="independent chains of launches LDLQ deals the tile rows to (0: the library's default, 2)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="first run one plain 1 GiB device copy kernel (known traffic, scales the rocprof byte counters)")
     args = ap.parse_args()

@@ -36,6 +36,16 @@ const char* qtip_last_error(void);
 void* qtip_stream(qtip_ctx* ctx);
 int qtip_synchronize(qtip_ctx* ctx);
 
+/* The reference's entry points take the caller's hipStream_t and queue their work on it (src/quantizer.hpp:60-78);
+ * this library works on the context's own stream.  These two calls carry the ordering across: after
+ * qtip_stream_wait the context's stream starts nothing before everything queued on caller_stream so far is done
+ * (call it before an entry point that reads device memory the caller produced asynchronously); after
+ * qtip_stream_signal the caller's stream starts nothing before the context's work queued so far is done (call it
+ * after an asynchronous *_dev entry point whose results the caller's stream will read).  caller_stream: a
+ * hipStream_t as an opaque pointer, NULL for the null stream.  Neither call blocks the host. */
+int qtip_stream_wait(qtip_ctx* ctx, void* caller_stream);
+int qtip_stream_signal(qtip_ctx* ctx, void* caller_stream);
+
 /* Codebook (replaces the hard-wired codebook(), src/qtip_core.cpp:18-50, and device_lut(),
  * src/quantizer.cpp:14-28).  tlut: 512 x 2 fp32, NULL selects the built-in HYB table.  The table is
  * rounded to fp16 (RNE) and expanded by quantlut_sym as the reference does. */
@@ -43,6 +53,12 @@ int qtip_set_tlut(qtip_ctx* ctx, const float* host_tlut);
 double qtip_lut_rms(qtip_ctx* ctx);
 /* decoded 65536-entry LUT (fp16 values as fp32), either pointer may be NULL */
 int qtip_get_lut(qtip_ctx* ctx, float* host_lut0, float* host_lut1);
+
+/* device_lut(), src/quantizer.cpp:14-28: the decoded 65536-entry table on the context's device as the reference's
+ * kernels read it, one word per state, fp16 bits of component 0 in the low half and of component 1 in the high half
+ * (Codebook::lut_h2, src/qtip_core.cpp:41).  Built on first use and after every qtip_set_tlut; owned by the context,
+ * valid until the next qtip_set_tlut or qtip_destroy. */
+int qtip_device_lut(qtip_ctx* ctx, const uint32_t** dev_lut_h2);
 
 /* Two-pass tail-biting Viterbi of B independent 256-value sequences (replaces the launch chain
  * k_viterbi_fwd(roll) -> k_viterbi_overlap -> k_viterbi_fwd(overlap) -> k_viterbi_finish of
@@ -150,6 +166,10 @@ typedef struct { /* QuantOpts, src/quantizer.hpp:11-19 */
   int ldl_device_updates;/* 1 (default): qtip_run_groups and qtip_quantize_group_h factor through
                             qtip_ldl_hessian_device_updates (panels on the host, trailing updates on the GPU, same L
                             bit for bit); 0: block LDL on the host alone, as in the reference */
+  int ldlq_chains;       /* LDLQ deals the tile rows of a group to this many independent chains of launches (each on
+                            a stream of its own inside ctx), so that the trace-backs of one run under the forward
+                            passes of the others; same codes whatever the number.  0 (default): 2; at most 3, which
+                            pays only with more than HIP's default of four hardware queues per process */
 } qtip_opts;
 void qtip_default_opts(qtip_opts* o);
 

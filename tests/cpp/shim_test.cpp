@@ -93,6 +93,64 @@ int main() {
     std::printf("layer file: %zu bytes\n", bytes);
     if (sz != long(bytes) || bytes < out[0].trellis.size() * 2 + out[1].trellis.size() * 2) ++fail;
   }
+  // ldlq_gpu on operands still in the making on the caller's stream (the reference's quantize_group forms WT there and
+  // calls ldlq_gpu without a synchronization in between, src/quantizer.cpp:239-265): a long run of fills is queued
+  // on S ahead of the copies that bring WT and L to the device, so a library that did not wait for S would read
+  // zeros; the states must equal those of the same call on settled operands.  device_lut() is the decoded table.
+  {
+    const long m = 64, nn = n;
+    std::vector<float> hWT(size_t(nn) * m), hL(size_t(nn) * nn, 0.f);
+    for (auto& v : hWT) v = float(N01(rng));
+    for (int i = 0; i < nn; ++i)
+      for (int j = 0; j < (i / 16) * 16; ++j) hL[size_t(i) * nn + j] = float(0.05 * N01(rng));
+    float *pWT = nullptr, *pL = nullptr, *dWT = nullptr, *dL = nullptr, *dHat = nullptr, *big = nullptr;
+    uint16_t *dQ1 = nullptr, *dQ2 = nullptr;
+    const size_t bigBytes = size_t(1) << 31, qn = size_t(m / 16) * (nn / 16) * 128;
+    bool ok = hipHostMalloc(reinterpret_cast<void**>(&pWT), hWT.size() * 4, hipHostMallocDefault) == hipSuccess &&
+              hipHostMalloc(reinterpret_cast<void**>(&pL), hL.size() * 4, hipHostMallocDefault) == hipSuccess &&
+              hipMalloc(reinterpret_cast<void**>(&dWT), hWT.size() * 4) == hipSuccess &&
+              hipMalloc(reinterpret_cast<void**>(&dL), hL.size() * 4) == hipSuccess &&
+              hipMalloc(reinterpret_cast<void**>(&dHat), hWT.size() * 4) == hipSuccess &&
+              hipMalloc(reinterpret_cast<void**>(&dQ1), qn * 2) == hipSuccess &&
+              hipMalloc(reinterpret_cast<void**>(&dQ2), qn * 2) == hipSuccess &&
+              hipMalloc(reinterpret_cast<void**>(&big), bigBytes) == hipSuccess;
+    if (ok) {
+      std::memcpy(pWT, hWT.data(), hWT.size() * 4);
+      std::memcpy(pL, hL.data(), hL.size() * 4);
+      ok = hipMemset(dWT, 0, hWT.size() * 4) == hipSuccess && hipMemset(dL, 0, hL.size() * 4) == hipSuccess &&
+           hipDeviceSynchronize() == hipSuccess;
+      for (int rep = 0; ok && rep < 16; ++rep) ok = hipMemsetAsync(big, rep, bigBytes, S) == hipSuccess;  // ~10 ms of fills
+      ok = ok && hipMemcpyAsync(dWT, pWT, hWT.size() * 4, hipMemcpyHostToDevice, S) == hipSuccess &&
+           hipMemcpyAsync(dL, pL, hL.size() * 4, hipMemcpyHostToDevice, S) == hipSuccess;
+      if (ok) ldlq_gpu(S, g, dWT, dL, nn, m, dHat, dQ1, 1024, device_lut(), nullptr);
+      ok = ok && hipStreamSynchronize(S) == hipSuccess;
+      if (ok) ldlq_gpu(S, g, dWT, dL, nn, m, dHat, dQ2, 1024, device_lut(), nullptr);
+      std::vector<uint16_t> q1(qn), q2(qn);
+      ok = ok && hipMemcpy(q1.data(), dQ1, qn * 2, hipMemcpyDeviceToHost) == hipSuccess &&
+           hipMemcpy(q2.data(), dQ2, qn * 2, hipMemcpyDeviceToHost) == hipSuccess;
+      size_t same = 0, zero = 0;
+      for (size_t i = 0; i < qn; ++i) same += q1[i] == q2[i], zero += q2[i] == 0;
+      std::printf("ldlq_gpu on operands still being copied on the caller's stream: %zu of %zu state words equal\n", same, qn);
+      if (same != qn || zero > qn / 2) ++fail;
+      // device_lut(): fp16 pair per state; against the host's decoded table at a few states
+      std::vector<uint32_t> h2(65536);
+      std::vector<float> l0(65536), l1(65536);
+      const uint32_t* dl = device_lut();
+      ok = ok && dl != nullptr && hipMemcpy(h2.data(), dl, h2.size() * 4, hipMemcpyDeviceToHost) == hipSuccess &&
+           qtip_get_lut(detail::context(), l0.data(), l1.data()) == QTIP_OK;
+      auto half = [](uint16_t h) {
+        const int e = (h >> 10) & 31, mnt = h & 1023;
+        const float v = e == 0 ? std::ldexp(float(mnt), -24) : std::ldexp(float(mnt | 1024), e - 25);
+        return (h >> 15) ? -v : v;
+      };
+      for (uint32_t st = 0; ok && st < 65536; st += 97)
+        if (half(uint16_t(h2[st])) != l0[st] || half(uint16_t(h2[st] >> 16)) != l1[st]) ok = false;
+    }
+    if (!ok) ++fail;
+    std::printf("caller-stream ordering and device_lut: mismatches so far %d\n", fail);
+    (void)hipFree(big), (void)hipFree(dQ2), (void)hipFree(dQ1), (void)hipFree(dHat), (void)hipFree(dL), (void)hipFree(dWT);
+    (void)hipHostFree(pL), (void)hipHostFree(pWT);
+  }
   // dump_dir (src/quantizer.cpp:230-234, 321-337): W as fp32 and the reconstruction, one raw file each
   {
     QuantOpts od;

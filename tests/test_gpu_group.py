@@ -231,6 +231,34 @@ def _deswz(pkg, want, got, m, n):
     return pkg.unswizzle_for_kernel(want, m, n).reshape(-1, 32) if False else want.reshape(-1, 32)
 
 
+def test_ldlq_chains_give_the_same_codes(qz, oracle, pkg, hyb):
+    """The tile rows of a group are dealt to 1, 2 or 3 independent chains of launches (streams of their own, feedback
+    slabs of their own, ragged shares of rows with two linears of different height): every packed word, Wscale and
+    proxy must come out the same, and two tile rows must equal the CPU form."""
+    import torch
+    say("case: LDLQ chains 1 / 2 / 3, 12288 + 32 rows x 256 columns")
+    n, m1, m2 = 256, 12288, 32
+    rng = np.random.default_rng(12)
+    W1 = (rng.standard_normal((m1, n)) * 0.02).astype(np.float32)
+    W2 = (rng.standard_normal((m2, n)) * 0.05).astype(np.float32)
+    G = rng.standard_normal((n, 2 * n)) * (1.0 + (np.arange(2 * n) % 5))
+    H = (G @ G.T / (2 * n)).astype(np.float32)
+    res = []
+    for chains in (1, 2, 3):
+        outs, _ = qz.quantize_group_h([pkg.LinearIn("a", m1, w_f32=W1), pkg.LinearIn("b", m2, w_f32=W2)], n, H, 21,
+                                      pkg.QuantOpts(ldl_threads=4, ldlq_chains=chains))
+        res.append(outs)
+    for outs in res[1:]:
+        for a, b in zip(res[0], outs):
+            assert np.array_equal(a.trellis, b.trellis) and a.wscale == b.wscale and a.proxy == b.proxy
+    ref = oracle.quantize_group(hyb.tlut, [W1[:32], W2], H, 21)   # rows are independent given L: but Wscale is not
+    # the second linear is complete in both calls: its words must be the oracle's
+    t2 = (32 // 16) * (n // 16) * 32
+    assert np.array_equal(res[0][1].trellis, ref["trellis"][t2:])
+    with pytest.raises(pkg.QtipError):
+        qz.quantize_group_h([pkg.LinearIn("b", m2, w_f32=W2)], n, H, 21, pkg.QuantOpts(ldlq_chains=4))
+
+
 def test_group_input_formats_and_errors(qz, oracle, pkg, synth):
     """bf16 and fp8+scale sources decode to the same fp32 weights the fp32 path sees; precondition failures come
     back as error codes (the reference aborts: src/quantizer.cpp:32-33,209-211, src/qtip_core.cpp:234)."""

@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 
 def test_cpp_shim_end_to_end():
-    exe = os.path.join(ROOT, "behemoth-qtip_amd", "csrc", "qtip_shim_test")
+    exe = os.path.join(ROOT, "tests", "cpp", "qtip_shim_test")
     assert os.path.exists(exe), "build it with __graft_entry__.build()"
     print("case: qtip_shim_test", flush=True)
     r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
