@@ -84,8 +84,7 @@ def test_group_bytes_equal_the_golden_device_path_vectors(qz, oracle, name):
 def test_group_bytes_equal_the_reference_device_path(qz, oracle, name):
     """The reference's own nvfp4_quantize_group, compiled for this GPU from its sources (oracle/_ref), on the same
     inputs: every packed byte, scale code and global scale of every option combination."""
-    if oracle.ref_gpu_lib() is None:
-        pytest.skip("oracle/_ref/libqtip_ref_gpu.so not built")
+    assert oracle.ref_gpu_lib() is not None, "oracle/_ref/libqtip_ref_gpu.so is missing: build it with make -C oracle ref"
     say("case: nvfp4 group vs the compiled reference, %s" % name)
     w, _ = _weights(oracle, name)
     m, n = w.shape

@@ -28,8 +28,9 @@ def synth():
 @pytest.fixture(scope="module")
 def ref(oracle):
     import torch  # noqa: F401  (one HIP runtime per process: torch's first)
-    if oracle.ref_gpu_lib() is None:
-        pytest.skip("oracle/_ref/libqtip_ref_gpu.so not built")
+    # a GPU test without the reference's device path is a failure, not a skip: these tests are the live pin of the
+    # whole call against the reference (the committed group vectors pin the CPU restatement only)
+    assert oracle.ref_gpu_lib() is not None, "oracle/_ref/libqtip_ref_gpu.so is missing: build it with make -C oracle ref"
     return oracle
 
 
