@@ -1,9 +1,43 @@
 """Seeded synthetic layers for the benchmark configurations (the five benchmark configurations: tiles only, 1024 x 1024, q-proj, gate+up, down-proj).
 
-Small configurations are generated with numpy on the host (bit-stable across machines); the large ones with
-torch on the GPU so that set-up takes seconds, not minutes.  Input synthesis is never timed.
+Small configurations are generated with numpy on the host (bit-stable across machines); the large ones on the GPU so
+that set-up takes seconds, not minutes, from the reference's own splitmix64 stream (Rng, src/common.hpp:91-107): the
+k-th output of a stream is a function of (seed, k) alone, so a tensor is filled in parallel and depends on no
+library's generator, only on fp64 log / cos / sqrt of the device.  Input synthesis is never timed.
 """
 import numpy as np
+
+_M64 = (1 << 64) - 1
+_GAMMA = 0x9E3779B97F4A7C15
+
+
+def splitmix_u64(seed, count, start=0):
+    """Outputs start .. start + count - 1 of Rng(seed).next() (src/common.hpp:91-100) as a uint64 array."""
+    s0 = (int(seed) * _GAMMA + 0x1234567) & _M64
+    k = np.arange(start + 1, start + count + 1, dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        z = np.uint64(s0) + k * np.uint64(_GAMMA)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    return z ^ (z >> np.uint64(31))
+
+
+def splitmix_uniform(seed, count, start=0):
+    """Rng::uniform: the top 53 bits of next() as a double in [0, 1)."""
+    return (splitmix_u64(seed, count, start) >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)
+
+
+def splitmix_normal(seed, count):
+    """Rng::normal (Box-Muller on two consecutive uniforms, src/common.hpp:101-105), numpy on the host."""
+    u = splitmix_uniform(seed, 2 * count).reshape(count, 2)
+    u1 = np.maximum(u[:, 0], 1e-300)
+    return np.sqrt(-2.0 * np.log(u1)) * np.cos(6.283185307179586 * u[:, 1])
+
+
+def synthetic_tlut(seed=1):
+    """Benchmark configuration 1's codebook: 512 x 2 fp32 drawn N(0, 1) from the splitmix stream, rescaled to unit rms."""
+    v = splitmix_normal(seed, 1024).astype(np.float32).reshape(512, 2)
+    return (v / np.float32(np.sqrt(np.mean(v.astype(np.float64) ** 2)))).astype(np.float32)
 
 
 def _bf16_round(x):
@@ -47,22 +81,71 @@ def small_group(seed=33, n=256, ms=(64, 32)):
     return Ws, H
 
 
-# ---------------------------------------------------------------- large configurations (torch, on the GPU)
-def _ar1_torch(gen, rows, n, rho, n_outliers, outlier_scale, device):
+# ---------------------------------------------------------------- large configurations (on the GPU)
+class DeviceStream:
+    """The splitmix stream of one seed on a torch device; every draw continues where the last one ended."""
+
+    def __init__(self, seed, device="cuda"):
+        self.s0 = (int(seed) * _GAMMA + 0x1234567) & _M64
+        self.pos = 0
+        self.device = device
+
+    @staticmethod
+    def _i64(v):      # a 64-bit pattern as the int64 torch computes with (wrapping arithmetic)
+        v &= _M64
+        return v - (1 << 64) if v >= (1 << 63) else v
+
+    @staticmethod
+    def _srl(z, k):   # logical shift right of an int64 tensor
+        return (z >> k) & ((1 << (64 - k)) - 1)
+
+    def _uniform_flat(self, count):
+        import torch
+        k = torch.arange(self.pos + 1, self.pos + count + 1, dtype=torch.int64, device=self.device)
+        self.pos += count
+        z = k * self._i64(_GAMMA) + self._i64(self.s0)
+        z = (z ^ self._srl(z, 30)) * self._i64(0xBF58476D1CE4E5B9)
+        z = (z ^ self._srl(z, 27)) * self._i64(0x94D049BB133111EB)
+        z = z ^ self._srl(z, 31)
+        return self._srl(z, 11).to(torch.float64) * (1.0 / 9007199254740992.0)
+
+    def uniform(self, shape, chunk=1 << 25):
+        import torch
+        count = int(np.prod(shape))
+        out = torch.empty(count, dtype=torch.float32, device=self.device)
+        for a in range(0, count, chunk):
+            b = min(count, a + chunk)
+            out[a:b] = self._uniform_flat(b - a).to(torch.float32)
+        return out.reshape(shape)
+
+    def normal(self, shape, chunk=1 << 24):
+        """fp32 N(0, 1): Box-Muller on two consecutive uniforms per value, in fp64, as Rng::normal."""
+        import torch
+        count = int(np.prod(shape))
+        out = torch.empty(count, dtype=torch.float32, device=self.device)
+        for a in range(0, count, chunk):
+            b = min(count, a + chunk)
+            u = self._uniform_flat(2 * (b - a)).reshape(b - a, 2)
+            u1 = torch.clamp(u[:, 0], min=1e-300)
+            out[a:b] = (torch.sqrt(-2.0 * torch.log(u1)) * torch.cos(6.283185307179586 * u[:, 1])).to(torch.float32)
+        return out.reshape(shape)
+
+
+def _ar1_device(st, rows, n, rho, n_outliers, outlier_scale):
     import torch
-    # stationary AR(1) across channels, built blockwise with the closed form x_j = sum_k rho^(j-k) s e_k via a
-    # scan in chunks (exact recurrence inside a chunk, carried state between chunks)
-    e = torch.randn((rows, n), generator=gen, device=device, dtype=torch.float32)
+    device = st.device
+    # stationary AR(1) across channels, x_j = rho x_(j-1) + s e_j, as a scan in chunks of 256 channels (a cumulative
+    # sum in a domain scaled by rho^k, which stays in range over 256 channels), the state carried between chunks
+    e = st.normal((rows, n))
     s = float(np.sqrt(1.0 - rho * rho))
     x = torch.empty_like(e)
-    # recurrence as a causal filter: cumulative sum in a scaled domain, 256 channels at a time for range safety
     carry = torch.zeros((rows,), device=device)
     step = 256
     for j0 in range(0, n, step):
         j1 = min(n, j0 + step)
         w = j1 - j0
         k = torch.arange(w, device=device, dtype=torch.float32)
-        scale = rho ** k                     # rho^k
+        scale = rho ** k
         blk = e[:, j0:j1] * s
         if j0 == 0:
             blk[:, 0] = e[:, 0]
@@ -70,7 +153,7 @@ def _ar1_torch(gen, rows, n, rho, n_outliers, outlier_scale, device):
         y = y + carry[:, None] * (rho ** (k + 1))
         x[:, j0:j1] = y
         carry = y[:, -1]
-    ch = torch.randperm(n, generator=gen, device=device)[:n_outliers]
+    ch = torch.argsort(st.uniform((n,)))[:n_outliers]      # the channels scaled up: the n_outliers smallest draws
     x[:, ch] *= outlier_scale
     return x.to(torch.bfloat16)
 
@@ -86,36 +169,35 @@ def large_config(cfg, device="cuda", seed=None):
     """Configurations 3, 4 and 5 as device tensors: (list of W, H).  fp32 GEMM accumulation for H."""
     import torch
     torch.backends.cuda.matmul.allow_tf32 = False
-    gen = torch.Generator(device=device)
-    gen.manual_seed(1000 + cfg if seed is None else seed)
+    st = DeviceStream(1000 + cfg if seed is None else seed, device)
     if cfg == 3:     # q-proj: W 12288x12288 Gaussian*0.015 with 1% entries x10
         n, ms = 12288, [12288]
         Ws = []
         for m in ms:
-            w = torch.randn((m, n), generator=gen, device=device) * 0.015
-            mask = torch.rand((m, n), generator=gen, device=device) < 0.01
+            w = st.normal((m, n)) * 0.015
+            mask = st.uniform((m, n)) < 0.01
             Ws.append(torch.where(mask, w * 10.0, w).contiguous())
-        H = _hessian_from(_ar1_torch(gen, 16384, n, 0.8, 32, 20.0, device))
+        H = _hessian_from(_ar1_device(st, 16384, n, 0.8, 32, 20.0))
     elif cfg == 4:   # gate+up: two stacked 28672x12288, Gaussian*0.012 with 0.5% x8, shared Hessian
         n, ms = 12288, [28672, 28672]
         Ws = []
         for m in ms:
-            w = torch.randn((m, n), generator=gen, device=device) * 0.012
-            mask = torch.rand((m, n), generator=gen, device=device) < 0.005
+            w = st.normal((m, n)) * 0.012
+            mask = st.uniform((m, n)) < 0.005
             Ws.append(torch.where(mask, w * 8.0, w).contiguous())
-        H = _hessian_from(_ar1_torch(gen, 16384, n, 0.8, 32, 20.0, device))
+        H = _hessian_from(_ar1_device(st, 16384, n, 0.8, 32, 20.0))
     elif cfg == 5:   # down-proj: W 12288x28672 Student-t(4)*0.01; X = g1 * silu(g2), 8192 rows: rank-deficient H
         n, m = 28672, 12288
-        z = torch.randn((m, n), generator=gen, device=device)
+        z = st.normal((m, n))
         chi = torch.zeros((m, n), device=device)
         for _ in range(4):
-            g = torch.randn((m, n), generator=gen, device=device)
+            g = st.normal((m, n))
             chi += g * g
             del g
         Ws = [(0.01 * z / torch.sqrt(chi / 4.0)).contiguous()]
         del z, chi
-        g1 = torch.randn((8192, n), generator=gen, device=device)
-        g2 = torch.randn((8192, n), generator=gen, device=device)
+        g1 = st.normal((8192, n))
+        g2 = st.normal((8192, n))
         xb = (g1 * torch.nn.functional.silu(g2)).to(torch.bfloat16)
         del g1, g2
         H = _hessian_from(xb)

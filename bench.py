@@ -39,7 +39,7 @@ def load_synth():
     return mod
 
 
-def cpu_baseline(seconds_budget=15.0, threads=16):
+def cpu_viterbi_sample(seconds_budget, threads):
     """Reference CPU Viterbi (oracle/_ref when present, else the oracle port) on a bounded sample of tiles."""
     import concurrent.futures as cf
     import numpy as np
@@ -76,13 +76,58 @@ def cpu_baseline(seconds_budget=15.0, threads=16):
                       "%.1f s on %d threads" % (done[0], dt, threads)}
 
 
+def cpu_baseline(threads=16, group=None):
+    """The CPU path timed on this host.  Always: the reference's CPU Viterbi on a sample of tiles.  With `group`
+    (n, weights, HRr, L of the benchmark's group, host arrays): the group path as the reference's CPU code would run
+    it, from two bounded samples: the CPU LDLQ (oracle port of tests/test_gpu.cpp:180-225: fp64 feedback, fp16
+    rounding, two-pass Viterbi per tile) on 256 weight rows over the last 2048 columns of the group (its own factor),
+    and the reference's compiled block_ldl_to_L on the group's rotated Hessian in full.  `value` extrapolates the
+    LDLQ sample's rate to the group's weights and adds the factorization."""
+    import numpy as np
+    from oracle import binding as ob
+    vit = cpu_viterbi_sample(10.0 if group else 15.0, threads)
+    if not group:
+        return vit
+    n, weights, HRr, L = group
+    ncol = min(n, 2048)
+    rows = 16 * threads
+    Lsub = np.ascontiguousarray(L[n - ncol:, n - ncol:])
+    Wr = (ob.rng_normal(78, rows * ncol).reshape(rows, ncol) * (0.9 * ob.Codebook().lut_rms)).astype(np.float32)
+    t0 = time.time()
+    ob.ldlq(ob.Codebook(), Wr, Lsub, threads=threads)
+    t_ldlq = time.time() - t0
+    ldlq_rate = rows * ncol / t_ldlq
+    out = {"unit": "Mweights/s", "cores": threads, "kind": "port", "viterbi_only": vit,
+           "ldlq_sample_Mweights_s": ldlq_rate / 1e6,
+           "sample": "CPU LDLQ (port) on %d rows x the last %d columns of the group with the group's own factor, rows "
+                     "drawn at the rotated weights' scale, %.1f s on %d threads; extrapolated to %d weights"
+                     % (rows, ncol, t_ldlq, threads, weights)}
+    R = ob.ref_lib()
+    t_ldl = None
+    if R is not None:
+        A = np.empty((n, n), np.float64)
+        for i in range(0, n, 2048):       # 0.5 (H + H^T) as the reference's ldl_hessian forms it, not timed
+            A[i:i + 2048] = 0.5 * (HRr[i:i + 2048].astype(np.float64) + HRr[:, i:i + 2048].T.astype(np.float64))
+        Lr = np.zeros((n, n), np.float32)
+        t0 = time.time()
+        ok = R.ref_block_ldl(A.reshape(-1), n, Lr.reshape(-1), threads)
+        t_ldl = time.time() - t0
+        out["block_ldl_reference_s"] = t_ldl
+        out["block_ldl_reference_same_factor_bits"] = bool(ok == 1 and np.array_equal(Lr.view(np.uint32), L.view(np.uint32)))
+        out["sample"] += "; block_ldl_to_L of the compiled reference on the group's rotated Hessian (n = %d) in full, " \
+                         "%.1f s on %d threads" % (n, t_ldl, threads)
+        del A, Lr
+    out["value"] = weights / (weights / ldlq_rate + (t_ldl or 0.0)) / 1e6
+    return out
+
+
 def run_viterbi_only(args, pkg):
     """Configuration 1: 4096 independent tiles, Viterbi only."""
     import numpy as np
     import torch
-    from oracle import binding as ob
-    q = pkg.Quantizer(0, tlut=ob.synthetic_tlut(1))
-    X = torch.from_numpy(ob.rng_normal(1234, 4096 * 256).astype(np.float32).reshape(4096, 256)).cuda()
+    synth = load_synth()
+    q = pkg.Quantizer(0, tlut=synth.synthetic_tlut(1))
+    X = torch.from_numpy(synth.splitmix_normal(1234, 4096 * 256).astype(np.float32).reshape(4096, 256)).cuda()
     S = torch.zeros((4096, 128), dtype=torch.int16, device="cuda")
     P = torch.zeros((4096, 32), dtype=torch.int16, device="cuda")
     for _ in range(args.warmup):
@@ -134,7 +179,8 @@ def run_group(args, pkg):
                          ldlq_s=sum(t.ldlq for t in tms) / K, viterbi_s=sum(t.viterbi for t in tms) / K,
                          load_s=sum(t.load for t in tms) / K, pack_s=sum(t.pack for t in tms) / K,
                          proxy_s=sum(t.proxy for t in tms) / K, proxy=float(res[-1][0][0].proxy),
-                         wscale=float(res[-1][0][0].wscale), cmp_outs=res[min(K, 6) - 1][0])
+                         wscale=float(res[-1][0][0].wscale), cmp_outs=res[min(K, 6) - 1][0],
+                         cmp_outs3=res[min(K, 3) - 1][0])
 
     q.reserve_groups(n)   # page-locked staging ring (3 x (HRr, L)); a worker keeps it for its lifetime
     if args.warmup > 0:
@@ -162,9 +208,35 @@ def run_group(args, pkg):
                          host_ldl_s=sum(r[1].ldl_cpu for r in hres) / kh,
                          host_ldl_same_codes=bool(all(np.array_equal(a.trellis, b.trellis) and a.proxy == b.proxy
                                                       for a, b in zip(hres[-1][0], stats["cmp_outs"]))))
+    host_inputs = {}
+    if not args.no_host_input_leg:
+        # beside it (outside the timed region): the same groups with W and H handed over as host pointers, as the
+        # reference's entry point takes them (src/quantizer.hpp:21-28,75-77): pageable host memory, PCIe inside
+        kq = min(args.steps, 3)
+        lins_h = [pkg.LinearIn("w%d" % i, m, w_f32=w.cpu().numpy()) for i, (m, w) in enumerate(zip(ms, Ws))]
+        H_host = H.cpu().numpy()
+        q.synchronize()
+        th = time.time()
+        hres = q.run_groups([(lins_h, n, H_host, 3 + k) for k in range(kq)], opt)
+        q.synchronize()
+        th = time.time() - th
+        host_inputs = dict(host_inputs_Mweights_s=weights_per_step * kq / th / 1e6, host_inputs_groups=kq,
+                           host_inputs_load_s=sum(r[1].load for r in hres) / kq,
+                           host_inputs_same_codes=bool(all(np.array_equal(a.trellis, b.trellis) and a.proxy == b.proxy
+                                                           for a, b in zip(hres[-1][0], stats["cmp_outs3"]))))
+        del lins_h, H_host, hres
+    cpu_group = None
+    if not args.no_cpu_baseline:
+        hp = q.rotate_hessian(H, n, 3)
+        q.ldl_hessian_device_updates(hp, threads=args.ldl_threads)
+        cpu_group = (n, weights_per_step, hp.HRr, hp.L)
     stats.pop("cmp_outs", None)
+    stats.pop("cmp_outs3", None)
     ntr = sum(ms) // 16
     launches = n // 16
+    nch = args.chains or 2        # the library's rule: a chain must fill its share of the 768 resident workgroups
+    while nch > 1 and ntr < 768:
+        nch -= 1
     gpu_s = stats["rht_s"] + stats["load_s"] + stats["ldlq_s"] + stats["proxy_s"] + stats["pack_s"]
     extra = dict(stats)
     extra.update(gpu_only_Mweights_s=weights_per_step / gpu_s / 1e6,
@@ -173,12 +245,13 @@ def run_group(args, pkg):
                  proxy_in_timed_region=True, ldl_threads=args.ldl_threads, feedback=args.feedback,
                  ldl_device_updates=not args.host_ldl)
     extra.update(host_only)
+    extra.update(host_inputs)
     names = {2: "config2: 1024x1024 group", 3: "config3: 12288x12288 q-proj group",
              4: "config4: gate+up 2x(28672x12288) group", 5: "config5: 12288x28672 down-proj group"}
     return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
                 vit_launch_weights=ntr * 256, workload=names[cfg] + (" (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)" if args.host_ldl else
                                        " (RHT + fp64 LDL: host panels, GPU trailing updates + LDLQ + 2-pass Viterbi + pack)"),
-                extra=extra)
+                extra=extra, cpu_group=cpu_group, concurrent=nch)
 
 
 def run_ldl_only(args, pkg):
@@ -225,6 +298,8 @@ def main():
                     help="time the block LDL of the configuration's rotated Hessian by itself, three times each: host panels "
                          "with GPU trailing updates, and host alone (not the contract's metric; one line of JSON)")
     ap.add_argument("--host-ldl-once", action="store_true", help="with --ldl-only: one host-only factorization instead of three")
+    ap.add_argument("--no-host-input-leg", action="store_true",
+                    help="skip the extra groups with W and H passed as host pointers reported beside the default run")
     ap.add_argument("--no-host-ldl-leg", action="store_true",
                     help="skip the extra host-only-LDL groups reported beside the default run")
     ap.add_argument("--feedback", type=int, default=0, choices=[0, 1],
@@ -256,26 +331,39 @@ def main():
     res = run_viterbi_only(args, pkg) if args.config == 1 else run_group(args, pkg)
     value = res["weights"] / res["wall"] / 1e6
     achieved = res["vit_launch_weights"] * FLOP_PER_WEIGHT / res["vit_launch_s"] / 1e12
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "viterbi_traffic.json")
-    if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("config%d_bytes_per_launch" % args.config)
-        except Exception:
-            traffic = None
+    # counters of the same launch, collected offline with rocprofv3 --pmc (a profiler cannot run inside this process):
+    # HBM bytes per launch and the share of cycles the LDS pipe is busy; the files name the commands that made them
+    traffic, counters = None, {}
+    try:
+        traffic = json.load(open(os.path.join(ROOT, "profiles", "viterbi_traffic.json"))).get(
+            "config%d_bytes_per_launch" % args.config)
+    except Exception:
+        traffic = None
+    try:
+        counters = json.load(open(os.path.join(ROOT, "profiles", "viterbi_counters.json"))).get("config%d" % args.config, {})
+    except Exception:
+        counters = {}
     out = {
         "metric": "Mweights/s quantized (RHT+LDLQ+2-pass Viterbi) 12288x28672; % VALU/LDS peak",
         "value": value, "unit": "Mweights/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": res["wall"] / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": dict({"workload": res["workload"]}, **res["extra"]),
+        # launch_ms: the average duration of one Viterbi launch (a start and a stop event stamped by every launch of
+        # the timed region itself); concurrent_launches of them run side by side, each on tiles_per_launch tiles, so
+        # weights_per_launch weights pass in that time
         "roofline": {"bound": "valu", "kernel": "viterbi_tiles_kernel", "achieved": achieved, "peak": PEAK_FP64_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP64_TFLOPS, "traffic": traffic,
+                     "traffic_source": "profiles/viterbi_traffic.json (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; offline)",
                      "launch_ms": res["vit_launch_s"] * 1e3, "weights_per_launch": res["vit_launch_weights"],
-                     "flop_per_weight": FLOP_PER_WEIGHT},
+                     "concurrent_launches": res.get("concurrent", 1),
+                     "tiles_per_launch": res["vit_launch_weights"] // 256 // res.get("concurrent", 1),
+                     "flop_per_weight": FLOP_PER_WEIGHT,
+                     "lds_frac": counters.get("lds_active_frac"), "valu_frac": counters.get("valu_busy_frac"),
+                     "counters_source": "profiles/viterbi_counters.json (rocprofv3 --pmc SQ_*; offline)"},
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(threads=min(16, os.cpu_count() or 1))
+        out["cpu_baseline"] = cpu_baseline(threads=min(16, os.cpu_count() or 1), group=res.get("cpu_group"))
     print(json.dumps(out), flush=True)
 
 
