@@ -5,8 +5,8 @@
 //  * gemm_tn: sum_k A[k][i] * (B1 - B2)[k][j] on the fp64 matrix cores (v_mfma_f64_16x16x4_f64), fp32 operands
 //    widened while staging through LDS.  The cross-buffer feedback ("prod cache") of a 128-column buffer is gathered
 //    from all rows quantized so far by a K-split kernel.
-//  * gemm_tn_bf16x3: the same prod-cache update with fp32 C and the operands split into bf16 hi + lo
-//    (v_mfma_f32_32x32x16_bf16, three terms), the arithmetic of the reference's GPU path.
+//  * gemm_tn_bf16x3_gather: the same gathered product in the arithmetic of the reference's GPU path: every fp32
+//    operand split into bf16 hi + lo, three v_mfma_f32_32x32x16_bf16 terms, fp32 accumulation.
 #include "ldlq.hpp"
 #include "qtip_internal.hpp"
 
@@ -106,15 +106,10 @@ __global__ void sum_splits_kernel(const double* __restrict__ part, int splits, l
   P[i] = s;
 }
 
-// ---------------------------------------------------------------- bf16 hi/lo split MFMA GEMM (fp32 accumulate)
-// C[M][N] += sum_k A[k][i] * (B1 - B2)[k][j] for K = 128, with every fp32 operand x split as hi = bf16(x),
-// lo = bf16(x - hi) and the product taken as hi*hi + hi*lo + lo*hi on v_mfma_f32_32x32x16_bf16 (the reference's
-// K-concatenated three-term form, src/quantizer.cpp:66-76, without materialising the concatenated operands).
-// One workgroup = 128 x 128 outputs; the whole K = 128 panel of both operands is split once into LDS
-// ([row][k] with k contiguous: a lane's 8 consecutive k are one 16-byte read), 4 waves of 64 x 64.
+// ---------------------------------------------------------------- bf16 hi/lo split operands
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-constexpr int SB = 128, SK = 128, SLD = SK + 8;  // row stride in bf16 elements (272 bytes: 16-byte reads conflict-free)
+constexpr int SB = 128;  // rows and columns of a workgroup's output tile
 
 __device__ __forceinline__ uint32_t bf16_rne_bits(float f) {
   uint32_t u = __float_as_uint(f);
@@ -123,42 +118,62 @@ __device__ __forceinline__ uint32_t bf16_rne_bits(float f) {
   return u >> 16;
 }
 
-__global__ __launch_bounds__(256) void gemm_tn_bf16x3_kernel(int M, int N, const float* __restrict__ A, long lda,
-                                                             const float* __restrict__ B1,
-                                                             const float* __restrict__ B2, long ldb,
-                                                             float* __restrict__ C, long ldc) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ah[SB][SLD], Al[SB][SLD], Bh[SB][SLD], Bl[SB][SLD];
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const long i0 = long(blockIdx.y) * SB, j0 = long(blockIdx.x) * SB;
-  // ---- split both panels into LDS: a task is 4 rows (i or j) x 8 consecutive k
-  for (int task = t; task < 2 * 512; task += 256) {
-    const bool isB = task >= 512;
-    const int q = task & 511, rg = q & 31, kg = q >> 5;
-    const long r0 = (isB ? j0 : i0) + rg * 4;
-    float v[8][4];
+// ---------------------------------------------------------------- bf16 hi/lo split MFMA GEMM, gathered (fp32 accumulate)
+// out[y][i][j] = sum over the K slices of split y of A[k][i] * (B1 - B2)[k][j], i < 128, in the arithmetic of the
+// reference's prod-cache update (src/quantizer.cpp:66-76: x = hi + lo in bf16, product = hi*hi + hi*lo + lo*hi, fp32
+// accumulate) but gathered like the fp64 kernel above: K is everything quantized so far, nothing is
+// read-modified-written.  128 x 128 outputs per workgroup, 4 waves of 64 x 64 (2 x 2 tiles of 32 x 32); K goes
+// through LDS 32 rows at a time, split on the way ([row][k] with k contiguous: a lane's 8 consecutive k are one
+// 16-byte read; the row stride of 80 bytes keeps those reads free of bank conflicts); a thread stages 4 rows x 8 k of
+// one operand per slice and fetches the next slice's while the matrix cores work.  Bound by HBM, not by the matrix
+// cores: a row k of the operands is (128 + 2 N) fp32 for 768 N flop.
+constexpr int GK = 32, GLD = GK + 8;
+__global__ __launch_bounds__(256, 2) void gemm_tn_bf16x3_gather_kernel(int N, long K, const float* __restrict__ A,
+                                                                       long lda, const float* __restrict__ B1,
+                                                                       const float* __restrict__ B2, long ldb,
+                                                                       float* __restrict__ out, long ldo) {
+  __shared__ __attribute__((aligned(16))) uint16_t Ah[SB][GLD], Al[SB][GLD], Bh[SB][GLD], Bl[SB][GLD];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
+  const long j0 = long(blockIdx.x) * SB;
+  const long slices = (K + GK - 1) / GK;
+  const long s0 = slices * blockIdx.y / gridDim.y, s1 = slices * (blockIdx.y + 1) / gridDim.y;
+  // staging task of this thread: operand, 4 rows at rg * 4, 8 k at kg * 8 of the slice
+  const bool isB = t >= 128;
+  const int rg = t & 31, kg = (t >> 5) & 3;
+  const long r0 = (isB ? j0 : 0) + rg * 4;
+  const bool in_range = isB ? r0 + 3 < N : true;
+  float4 g1[8], g2[8];
+  auto fetch = [&](long slice) {
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) {
-      const long k = kg * 8 + kk;
-      float4 x = {0.f, 0.f, 0.f, 0.f};
-      if (r0 + 3 < (isB ? N : M)) {
+      const long k = slice * GK + kg * 8 + kk;
+      g1[kk] = g2[kk] = float4{0.f, 0.f, 0.f, 0.f};
+      if (k < K && in_range) {
         if (!isB) {
-          x = *reinterpret_cast<const float4*>(A + k * lda + r0);
+          g1[kk] = *reinterpret_cast<const float4*>(A + k * lda + r0);
         } else {
-          x = *reinterpret_cast<const float4*>(B1 + k * ldb + r0);
-          if (B2) {
-            const float4 y = *reinterpret_cast<const float4*>(B2 + k * ldb + r0);
-            x.x -= y.x, x.y -= y.y, x.z -= y.z, x.w -= y.w;
-          }
+          g1[kk] = *reinterpret_cast<const float4*>(B1 + k * ldb + r0);
+          g2[kk] = *reinterpret_cast<const float4*>(B2 + k * ldb + r0);
         }
       }
-      v[kk][0] = x.x, v[kk][1] = x.y, v[kk][2] = x.z, v[kk][3] = x.w;
     }
+  };
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+  const int kq = 8 * (lane >> 5), rl = lane & 31;
+  if (s0 < s1) fetch(s0);
+  for (long sl = s0; sl < s1; ++sl) {
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii) {
       uint32_t hi[4], lo[4];
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
-        const float a = v[2 * p][ii], b = v[2 * p + 1][ii];
+        const float a = (&g1[2 * p].x)[ii] - (&g2[2 * p].x)[ii], b = (&g1[2 * p + 1].x)[ii] - (&g2[2 * p + 1].x)[ii];
         const uint32_t ha = bf16_rne_bits(a), hb = bf16_rne_bits(b);
         const uint32_t la = bf16_rne_bits(a - __uint_as_float(ha << 16)), lb = bf16_rne_bits(b - __uint_as_float(hb << 16));
         hi[p] = ha | (hb << 16);
@@ -169,52 +184,54 @@ __global__ __launch_bounds__(256) void gemm_tn_bf16x3_kernel(int M, int N, const
       *reinterpret_cast<uint4*>(dh) = uint4{hi[0], hi[1], hi[2], hi[3]};
       *reinterpret_cast<uint4*>(dl) = uint4{lo[0], lo[1], lo[2], lo[3]};
     }
-  }
-  __syncthreads();
-  const int wm = wave >> 1, wn = wave & 1;
-  floatx16 acc[2][2];
+    __syncthreads();
+    if (sl + 1 < s1) fetch(sl + 1);
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+    for (int ks = 0; ks < GK / 16; ++ks) {
+      bf16x8 ah[2], al[2], bh[2], bl[2];
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
-  const int kq = 8 * (lane >> 5), rl = lane & 31;
-#pragma unroll
-  for (int ks = 0; ks < SK / 16; ++ks) {
-    bf16x8 ah[2], al[2], bh[2], bl[2];
-#pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
-      const int r = wm * 64 + mi * 32 + rl;
-      ah[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Ah[r][ks * 16 + kq]));
-      al[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Al[r][ks * 16 + kq]));
-    }
-#pragma unroll
-    for (int ni = 0; ni < 2; ++ni) {
-      const int r = wn * 64 + ni * 32 + rl;
-      bh[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Bh[r][ks * 16 + kq]));
-      bl[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Bl[r][ks * 16 + kq]));
-    }
-#pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+      for (int mi = 0; mi < 2; ++mi) {
+        const int r = wm * 64 + mi * 32 + rl;
+        ah[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Ah[r][ks * 16 + kq]));
+        al[mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Al[r][ks * 16 + kq]));
+      }
 #pragma unroll
       for (int ni = 0; ni < 2; ++ni) {
-        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mi], bh[ni], acc[mi][ni], 0, 0, 0);
-        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mi], bl[ni], acc[mi][ni], 0, 0, 0);
-        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mi], bh[ni], acc[mi][ni], 0, 0, 0);
+        const int r = wn * 64 + ni * 32 + rl;
+        bh[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Bh[r][ks * 16 + kq]));
+        bl[ni] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Bl[r][ks * 16 + kq]));
       }
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) {
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mi], bh[ni], acc[mi][ni], 0, 0, 0);
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mi], bl[ni], acc[mi][ni], 0, 0, 0);
+          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mi], bh[ni], acc[mi][ni], 0, 0, 0);
+        }
+    }
+    __syncthreads();
   }
   // accumulator element v of a lane: row (v % 4) + 8 (v / 4) + 4 (lane / 32), column lane % 32 of the 32x32 tile
+  float* o = out + long(blockIdx.y) * SB * ldo;
 #pragma unroll
   for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
     for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const long gi = i0 + wm * 64 + mi * 32 + (v & 3) + 8 * (v >> 2) + 4 * (lane >> 5);
+        const long gi = wm * 64 + mi * 32 + (v & 3) + 8 * (v >> 2) + 4 * (lane >> 5);
         const long gj = j0 + wn * 64 + ni * 32 + rl;
-        if (gi < M && gj < N) C[gi * ldc + gj] += acc[mi][ni][v];
+        if (gj < N) o[gi * ldo + gj] = acc[mi][ni][v];
       }
+}
+
+__global__ void sum_splits_f32_kernel(const float* __restrict__ part, int splits, long count, float* __restrict__ P) {
+  const long i = long(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float s = part[i];
+  for (int k = 1; k < splits; ++k) s += part[long(k) * count + i];
+  P[i] = s;
 }
 
 }  // namespace
@@ -241,14 +258,19 @@ void launch_gemm_tn_f64_gather(int N, long K, const float* A, long lda, const fl
   }
 }
 
-void launch_gemm_tn_bf16x3_acc(int M, int N, int K, const float* A, long lda, const float* B1, const float* B2, long ldb,
-                               float* C, long ldc, hipStream_t s) {
-  if (M <= 0 || N <= 0) return;
-  QTIP_REQUIRE(K == SK, "split-bf16 GEMM is built for K = %d (got %d)", SK, K);
-  QTIP_REQUIRE(lda % 4 == 0 && ldb % 4 == 0 && N % 4 == 0 && M % 4 == 0, "split-bf16 GEMM needs 16-byte aligned rows");
-  dim3 grid(unsigned((N + SB - 1) / SB), unsigned((M + SB - 1) / SB));
-  gemm_tn_bf16x3_kernel<<<grid, dim3(256), 0, s>>>(M, N, A, lda, B1, B2, ldb, C, ldc);
+void launch_gemm_tn_bf16x3_gather(int N, long K, const float* A, long lda, const float* B1, const float* B2, long ldb,
+                                  float* P, float* partials, hipStream_t s) {
+  QTIP_REQUIRE(N > 0 && K > 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 && B2 != nullptr,
+               "split-bf16 gather GEMM needs 16-byte aligned fp32 rows");
+  const int S = gemm_splitk_splits(K);
+  dim3 grid(unsigned((N + SB - 1) / SB), unsigned(S));
+  gemm_tn_bf16x3_gather_kernel<<<grid, dim3(256), 0, s>>>(N, K, A, lda, B1, B2, ldb, S == 1 ? P : partials, N);
   QTIP_HIP(hipGetLastError());
+  if (S > 1) {
+    const long count = long(SB) * N;
+    sum_splits_f32_kernel<<<dim3(unsigned((count + 255) / 256)), dim3(256), 0, s>>>(partials, S, count, P);
+    QTIP_HIP(hipGetLastError());
+  }
 }
 
 }  // namespace qtipmi

@@ -108,8 +108,8 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
     long tile0, tiles;   // tile rows tile0 .. tile0 + tiles - 1
     long r0, rows;       // weight rows (columns of WT) 16 tile0 .., 16 tiles of them
     int slot0, slots;    // share of the kept-metrics workspace
-    double* prod;        // feedback 0: 128 x rows slab
-    double* parts;
+    double *prod, *parts;     // feedback 0: 128 x rows slab and the split-K partial slabs
+    float *prod32, *parts32;  // feedback 1: the same in fp32
   } ch[3];
   for (int k = 0; k < nch; ++k) {
     if (k > 0 && !c->chain_stream[k - 1]) QTIP_HIP(hipStreamCreateWithFlags(&c->chain_stream[k - 1], hipStreamNonBlocking));
@@ -121,17 +121,17 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
     ch[k].slot0 = c->vit_slots * k / nch;
     ch[k].slots = c->vit_slots * (k + 1) / nch - ch[k].slot0;
   }
-  // feedback 0: fp64 feedback sums; the feedback of the rows quantized in earlier buffers is gathered per buffer
-  // into a 128 x rows fp64 slab per chain.  feedback 1: fp32 sums, an n x m fp32 prod cache updated after every
-  // buffer by the bf16 hi/lo split MFMA product
+  // The feedback of the rows quantized in earlier buffers is gathered per buffer into a 128 x rows slab per chain:
+  // feedback 0 in fp64 (fp64 MFMA), feedback 1 in fp32 from bf16 hi/lo split operands (the reference GPU's arithmetic)
   const int max_splits = gemm_splitk_splits(n);
   DBuf<double> prod(feedback == 0 ? size_t(128) * m : 0), parts(feedback == 0 ? size_t(max_splits) * 128 * m : 0);
-  for (int k = 0; k < nch && feedback == 0; ++k) {
-    ch[k].prod = prod.p + size_t(128) * ch[k].r0;
-    ch[k].parts = parts.p + size_t(max_splits) * 128 * ch[k].r0;
+  DBuf<float> prod32(feedback == 1 ? size_t(128) * m : 0), parts32(feedback == 1 ? size_t(max_splits) * 128 * m : 0);
+  for (int k = 0; k < nch; ++k) {
+    ch[k].prod = feedback == 0 ? prod.p + size_t(128) * ch[k].r0 : nullptr;
+    ch[k].parts = feedback == 0 ? parts.p + size_t(max_splits) * 128 * ch[k].r0 : nullptr;
+    ch[k].prod32 = feedback == 1 ? prod32.p + size_t(128) * ch[k].r0 : nullptr;
+    ch[k].parts32 = feedback == 1 ? parts32.p + size_t(max_splits) * 128 * ch[k].r0 : nullptr;
   }
-  DBuf<float> prod32(feedback == 1 ? size_t(n) * m : 0);
-  if (feedback == 1) QTIP_HIP(hipMemsetAsync(prod32, 0, prod32.bytes(), s));
   QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
   Events timed, pacing, joins;  // timed: a (start, stop) pair per Viterbi launch, stamped by the launch itself
   // the other chains start once the caller's inputs and the cleared outputs are there, a third (two thirds) of a
@@ -159,12 +159,16 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
       for (int k = 0; k < nch; ++k) {
         const Chain& C = ch[k];
         if (nbuf_done >= kAhead) QTIP_HIP(hipEventSynchronize(pace[k][(nbuf_done - kAhead) % (kAhead + 1)]));
-        if (feedback == 0) {  // prod[r][:] = sum_{k >= bufend} L[k][c0 + r] (WT - hatWT)[k][:], r < 128
-          if (bufend < n)
-            launch_gemm_tn_f64_gather(int(C.rows), n - bufend, L + long(bufend) * n + c0, n, WT + long(bufend) * m + C.r0,
-                                      hatWT + long(bufend) * m + C.r0, m, C.prod, C.parts, C.s);
-          else
-            QTIP_HIP(hipMemsetAsync(C.prod, 0, size_t(128) * C.rows * sizeof(double), C.s));
+        // prod[r][:] = sum_{k >= bufend} L[k][c0 + r] (WT - hatWT)[k][:], r < 128
+        const float* Lp = L + long(bufend) * n + c0;
+        const float *Wp = WT + long(bufend) * m + C.r0, *Hp = hatWT + long(bufend) * m + C.r0;
+        if (bufend == n) {
+          if (feedback == 0) QTIP_HIP(hipMemsetAsync(C.prod, 0, size_t(128) * C.rows * sizeof(double), C.s));
+          else QTIP_HIP(hipMemsetAsync(C.prod32, 0, size_t(128) * C.rows * sizeof(float), C.s));
+        } else if (feedback == 0) {
+          launch_gemm_tn_f64_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod, C.parts, C.s);
+        } else {
+          launch_gemm_tn_bf16x3_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod32, C.parts32, C.s);
         }
         for (int i = 7; i >= 0; --i) {  // the kernel forms the block's targets (in-buffer feedback) itself
           const int col0 = c0 + 16 * i;
@@ -174,8 +178,9 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
           job.L = L;
           job.ldl = n;
           job.bufend = bufend;
-          if (feedback == 0) job.prod64 = C.prod, job.prod_row0 = c0, job.ldp = C.rows;
-          else job.prod32 = prod32 + C.r0;
+          if (feedback == 0) job.prod64 = C.prod;
+          else job.prod32 = C.prod32;
+          job.prod_row0 = c0, job.ldp = C.rows;
           job.states = Q + size_t(C.tile0) * nblk * 128;
           job.q_tile_stride = nblk;
           job.q_offset = col0 / 16;
@@ -186,10 +191,6 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
           if (vit_seconds) t0 = timed.add(hipEventDefault), t1 = timed.add(hipEventDefault);
           launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws.p + viterbi_workspace_bytes(C.slot0), C.slots,
                                C.s, t0, t1);
-        }
-        if (c0 > 0 && feedback == 1) {  // prod[0:c0, :] += L[c0:c0+128, 0:c0]^T (WT - hatWT)[c0:c0+128, :]
-          launch_gemm_tn_bf16x3_acc(c0, int(C.rows), 128, L + long(c0) * n, n, WT + long(c0) * m + C.r0,
-                                    hatWT + long(c0) * m + C.r0, m, prod32 + C.r0, m, C.s);
         }
         QTIP_HIP(hipEventRecord(pace[k][nbuf_done % (kAhead + 1)], C.s));
       }

@@ -80,7 +80,7 @@ def cpu_baseline(threads=16, group=None):
     """The CPU path timed on this host.  Always: the reference's CPU Viterbi on a sample of tiles.  With `group`
     (n, weights, HRr, L of the benchmark's group, host arrays): the group path as the reference's CPU code would run
     it, from two bounded samples: the CPU LDLQ (oracle port of tests/test_gpu.cpp:180-225: fp64 feedback, fp16
-    rounding, two-pass Viterbi per tile) on 256 weight rows over the last 2048 columns of the group (its own factor),
+    rounding, two-pass Viterbi per tile) on 256 weight rows over the last 4096 columns of the group (its own factor),
     and the reference's compiled block_ldl_to_L on the group's rotated Hessian in full.  `value` extrapolates the
     LDLQ sample's rate to the group's weights and adds the factorization."""
     import numpy as np
@@ -89,7 +89,7 @@ def cpu_baseline(threads=16, group=None):
     if not group:
         return vit
     n, weights, HRr, L = group
-    ncol = min(n, 2048)
+    ncol = min(n, 4096)
     rows = 16 * threads
     Lsub = np.ascontiguousarray(L[n - ncol:, n - ncol:])
     Wr = (ob.rng_normal(78, rows * ncol).reshape(rows, ncol) * (0.9 * ob.Codebook().lut_rms)).astype(np.float32)
@@ -225,6 +225,24 @@ def run_group(args, pkg):
                            host_inputs_same_codes=bool(all(np.array_equal(a.trellis, b.trellis) and a.proxy == b.proxy
                                                            for a, b in zip(hres[-1][0], stats["cmp_outs3"]))))
         del lins_h, H_host, hres
+    fb1 = {}
+    if args.feedback == 0 and not args.no_feedback1_leg:
+        # beside it (outside the timed region): the same groups with the LDLQ feedback in the reference GPU's
+        # arithmetic (fp32 sums, prod cache from bf16 hi/lo split operands on the matrix cores)
+        kf = min(args.steps, 3)
+        fopt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=1,
+                             ldl_device_updates=not args.host_ldl, ldlq_chains=args.chains)
+        q.synchronize()
+        tf = time.time()
+        fres = q.run_groups([(lins, n, H, 3 + k) for k in range(kf)], fopt)
+        q.synchronize()
+        tf = time.time() - tf
+        a, b = fres[-1][0][0], stats["cmp_outs3"][0]
+        same = np.all(a.trellis.reshape(-1, 32) == b.trellis.reshape(-1, 32), axis=1).mean()
+        fb1 = dict(feedback1_Mweights_s=weights_per_step * kf / tf / 1e6, feedback1_groups=kf,
+                   feedback1_ldlq_s=sum(r[1].ldlq for r in fres) / kf, feedback1_proxy=float(a.proxy),
+                   feedback1_word_blocks_equal_to_default=float(same))
+        del fres
     cpu_group = None
     if not args.no_cpu_baseline:
         hp = q.rotate_hessian(H, n, 3)
@@ -246,6 +264,7 @@ def run_group(args, pkg):
                  ldl_device_updates=not args.host_ldl)
     extra.update(host_only)
     extra.update(host_inputs)
+    extra.update(fb1)
     names = {2: "config2: 1024x1024 group", 3: "config3: 12288x12288 q-proj group",
              4: "config4: gate+up 2x(28672x12288) group", 5: "config5: 12288x28672 down-proj group"}
     return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
@@ -300,6 +319,8 @@ def main():
     ap.add_argument("--host-ldl-once", action="store_true", help="with --ldl-only: one host-only factorization instead of three")
     ap.add_argument("--no-host-input-leg", action="store_true",
                     help="skip the extra groups with W and H passed as host pointers reported beside the default run")
+    ap.add_argument("--no-feedback1-leg", action="store_true",
+                    help="skip the extra groups with --feedback 1 reported beside the default run")
     ap.add_argument("--no-host-ldl-leg", action="store_true",
                     help="skip the extra host-only-LDL groups reported beside the default run")
     ap.add_argument("--feedback", type=int, default=0, choices=[0, 1],
