@@ -32,20 +32,29 @@ __global__ __launch_bounds__(256) void transpose_panel_kernel(const double* __re
     if (p0 + r < kb && i0 + tx < nr) Xt[long(p0 + r) * nr + i0 + tx] = tile[tx][r];
 }
 
-// C[i][j] -= sum_p X[i][p] * X[j][p] for the 128 x 128 tile (bi, bj <= bi) of the nr x nr lower triangle, every
-// element one chain over p = 0 .. kb-1 from zero.  Xt: kb x nr (the transposed solved rows, row stride nr, nr a
-// multiple of 4), C: row stride ldc.  256 threads, 2 x 2 waves of 64 x 64, K staged 16 at a time; the next 16 columns
-// travel from HBM while the matrix cores work on the present ones.
+// C[i][j] -= sum_p X[i][p] * X[j][p] for one 128 x 128 tile of the nr x nr lower triangle, every element one chain
+// over p = 0 .. kb-1 from zero.  Xt: kb x nr (the transposed solved rows, row stride ldx; nr and ldx multiples of 4),
+// C: row stride ldc.  strip_tiles = 0: the grid enumerates the tiles (bi, bj <= bi) of the whole triangle;
+// strip_tiles = w > 0: only the first w tile columns, grid = w x row tiles (the columns of the next panel, which the
+// host wants back before the rest of the update has run).  256 threads, 2 x 2 waves of 64 x 64, K staged 16 at a
+// time; the next 16 columns travel from HBM while the matrix cores work on the present ones.
 constexpr int UT = 128, UK = 16;
-__global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double* __restrict__ Xt, int nr, int kb,
-                                                                 double* __restrict__ C, long ldc) {
-  // tile index -> (bi, bj), rows of the triangle enumerated from the top
-  int bi = 0, rem = blockIdx.x;
-  while (rem > bi) {
-    rem -= bi + 1;
-    ++bi;
+__global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double* __restrict__ Xt, long ldx, int nr, int kb,
+                                                                 double* __restrict__ C, long ldc, int strip_tiles) {
+  int bi, bj;
+  if (strip_tiles > 0) {
+    bi = blockIdx.x / strip_tiles;
+    bj = blockIdx.x % strip_tiles;
+    if (bj > bi) return;  // above the diagonal (uniform over the workgroup)
+  } else {
+    // tile index t -> row bi with bi (bi + 1) / 2 <= t: the square root in fp32, then one step either way
+    const int t = blockIdx.x;
+    bi = int((__builtin_sqrtf(8.0f * float(t) + 1.0f) - 1.0f) * 0.5f);
+    while (bi * (bi + 1) / 2 > t) --bi;
+    while ((bi + 1) * (bi + 2) / 2 <= t) ++bi;
+    bj = t - bi * (bi + 1) / 2;
   }
-  const int bj = rem, i0 = bi * UT, j0 = bj * UT;
+  const int i0 = bi * UT, j0 = bj * UT;
   __shared__ __attribute__((aligned(16))) double Xi[UK][UT], Xj[UK][UT];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
   double4_t acc[4][4];
@@ -62,8 +71,8 @@ __global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double*
       const int k = k0 + lk + 8 * r;
       pi[r] = pj[r] = double4_t{0, 0, 0, 0};
       if (k < kb) {
-        if (i_ok) pi[r] = *reinterpret_cast<const double4_t*>(Xt + long(k) * nr + i0 + lc);
-        if (j_ok) pj[r] = *reinterpret_cast<const double4_t*>(Xt + long(k) * nr + j0 + lc);
+        if (i_ok) pi[r] = *reinterpret_cast<const double4_t*>(Xt + long(k) * ldx + i0 + lc);
+        if (j_ok) pj[r] = *reinterpret_cast<const double4_t*>(Xt + long(k) * ldx + j0 + lc);
       }
     }
   };
@@ -102,37 +111,65 @@ __global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double*
       }
 }
 
+// The panels travel one ahead of the updates: as soon as panel k is solved its rows go up, the update of the next
+// panel's columns alone (a strip of the trailing matrix) is queued, those columns start on their way down into the
+// other page-locked buffer, and only then the rest of update k is queued - the host factors and solves panel k + 1
+// while that rest runs.  Every element still receives exactly one update per panel, the same chain as before.
 struct DeviceTrailing final : PanelAssist {
   qtip_ctx* c;
   long n;
   hipStream_t s;
   const float* host_L;
   float* dev_L;  // optional: L is also left on the device, column block by column block as it is assembled
-  DeviceTrailing(qtip_ctx* c_, long n_, const float* hL, float* dL) : c(c_), n(n_), s(c_->ldl_stream), host_L(hL), dev_L(dL) {}
+  hipEvent_t fetched = nullptr;
+  int cur = 0;          // page-locked buffer holding the panel the host works on
+  long ahead_k = -1;    // first column of the panel on its way into buffer cur ^ 1
+  DeviceTrailing(qtip_ctx* c_, long n_, const float* hL, float* dL) : c(c_), n(n_), s(c_->ldl_stream), host_L(hL), dev_L(dL) {
+    QTIP_HIP(hipEventCreateWithFlags(&fetched, hipEventDisableTiming));
+  }
+  ~DeviceTrailing() override {
+    if (fetched) (void)hipEventDestroy(fetched);
+  }
+  void copy_down(long k, long kb, double* dst) {
+    QTIP_HIP(hipMemcpy2DAsync(dst, size_t(kb) * 8, c->ldl_A.p + k * n + k, size_t(n) * 8, size_t(kb) * 8, size_t(n - k),
+                              hipMemcpyDeviceToHost, s));
+  }
   void assembled(int k, int kb) override {
     if (!dev_L) return;
     QTIP_HIP(hipMemcpy2DAsync(dev_L + k, size_t(n) * 4, host_L + k, size_t(n) * 4, size_t(kb) * 4, size_t(n),
                               hipMemcpyHostToDevice, s));
   }
   double* fetch(int k, int kb) override {
-    const long rows = n - k;
-    QTIP_HIP(hipMemcpy2DAsync(c->ldl_panel.p, size_t(kb) * 8, c->ldl_A.p + long(k) * n + k, size_t(n) * 8,
-                              size_t(kb) * 8, size_t(rows), hipMemcpyDeviceToHost, s));
-    QTIP_HIP(hipStreamSynchronize(s));
-    return c->ldl_panel.p;
+    if (ahead_k == k) {
+      cur ^= 1;
+      QTIP_HIP(hipEventSynchronize(fetched));
+    } else {
+      copy_down(k, kb, c->ldl_panel[cur].p);
+      QTIP_HIP(hipStreamSynchronize(s));
+    }
+    ahead_k = -1;
+    return c->ldl_panel[cur].p;
+  }
+  void update(const double* Xt, long ldx, long nr, int kb, double* C, int strip_tiles) {
+    const long nt = (nr + UT - 1) / UT, grid = strip_tiles ? nt * strip_tiles : nt * (nt + 1) / 2;
+    rank_update_lower_kernel<<<dim3(unsigned(grid)), dim3(256), 0, s>>>(Xt, ldx, int(nr), kb, C, n, strip_tiles);
+    QTIP_HIP(hipGetLastError());
   }
   void solved(int k, int kb, const double* panel) override {
     const long r0 = k + kb, nr = n - r0;
     if (nr <= 0) return;
     // the stream orders this copy before the next fetch into the same page-locked buffer
     QTIP_HIP(hipMemcpyAsync(c->ldl_X.p, panel + long(kb) * kb, size_t(nr) * kb * 8, hipMemcpyHostToDevice, s));
-    const long nt = (nr + UT - 1) / UT, tiles = nt * (nt + 1) / 2;
     transpose_panel_kernel<<<dim3(unsigned((nr + 31) / 32), unsigned((kb + 31) / 32)), dim3(256), 0, s>>>(
         c->ldl_X.p, int(nr), kb, c->ldl_Xt.p);
     QTIP_HIP(hipGetLastError());
-    rank_update_lower_kernel<<<dim3(unsigned(tiles)), dim3(256), 0, s>>>(c->ldl_Xt.p, int(nr), kb,
-                                                                        c->ldl_A.p + r0 * n + r0, n);
-    QTIP_HIP(hipGetLastError());
+    double* C = c->ldl_A.p + r0 * n + r0;
+    const long next_kb = std::min<long>(ldl_panel_width(), nr), strip = (next_kb + UT - 1) / UT, done = strip * UT;
+    update(c->ldl_Xt.p, nr, nr, kb, C, int(strip));
+    copy_down(r0, next_kb, c->ldl_panel[cur ^ 1].p);
+    QTIP_HIP(hipEventRecord(fetched, s));
+    ahead_k = r0;
+    if (nr > done) update(c->ldl_Xt.p + done, nr, nr - done, kb, C + done * n + done, 0);
   }
 };
 
@@ -152,7 +189,8 @@ void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int th
   if (!dev_HRr) c->ldl_H.ensure(nn);
   c->ldl_X.ensure(size_t(n) * nb);
   c->ldl_Xt.ensure(size_t(n) * nb);
-  if (c->ldl_panel.n < size_t(n) * nb) c->ldl_panel.alloc(size_t(n) * nb);
+  for (auto& buf : c->ldl_panel)
+    if (buf.n < size_t(n) * nb) buf.alloc(size_t(n) * nb);
   if (!dev_HRr) QTIP_HIP(hipMemcpyAsync(c->ldl_H.p, host_HRr, nn * 4, hipMemcpyHostToDevice, s));
   symmetrize_lower_kernel<<<dim3(unsigned((n + 255) / 256), unsigned(n)), dim3(256), 0, s>>>(dev_HRr ? dev_HRr : c->ldl_H.p, n,
                                                                                               c->ldl_A.p);

@@ -23,11 +23,11 @@ struct qtip_ctx {
   qtipmi::HBuf<float> ring_HRr[3], ring_L[3];  // page-locked staging of run_groups, kept between calls
   qtipmi::DBuf<float> ring_dHRr[3], ring_dL[3];  // run_groups with device-updated LDL: rotated Hessians and factors stay here
   // LDL with the trailing updates on the device (ldl_assist.hip): own stream, fp64 work matrix, fp32 upload of HRr,
-  // solved panel rows, page-locked panel buffer; allocated on first use
+  // solved panel rows, two page-locked panel buffers (the panels travel one ahead); allocated on first use
   hipStream_t ldl_stream = nullptr;
   qtipmi::DBuf<double> ldl_A, ldl_X, ldl_Xt;
   qtipmi::DBuf<float> ldl_H;
-  qtipmi::HBuf<double> ldl_panel;
+  qtipmi::HBuf<double> ldl_panel[2];
 };
 
 namespace qtipmi {
