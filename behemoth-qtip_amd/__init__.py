@@ -114,6 +114,7 @@ def lib():
     L.qtip_rotate_hessian.argtypes = [vp, vp, i, i, u64, d, vp, C.POINTER(d), vp]
     L.qtip_ldl_hessian.argtypes = [vp, i, i, vp]
     L.qtip_ldl_hessian_device_updates.argtypes = [vp, vp, i, i, vp]
+    L.qtip_ldl_hessian_device_updates_dev.argtypes = [vp, vp, i, i, vp, vp]
     L.qtip_ldlq_dev.argtypes = [vp, vp, vp, l, l, vp, vp, i, C.POINTER(d)]
     L.qtip_default_opts.argtypes = [C.POINTER(_OptsC)]
     L.qtip_default_opts.restype = None
@@ -388,6 +389,16 @@ class Quantizer:
             hp.L = None
             _check(rc)
         hp.t_ldl = time.time() - t0
+
+    def ldl_hessian_device_resident(self, dHRr, n, L_host, dL=None, threads=16):
+        """The same with the rotated Hessian on the device (dHRr, never written), as run_groups runs it: L goes to
+        L_host (n x n fp32, page-locked when dL is given) and, column block by column block, to the device buffer
+        dL.  Returns the seconds the call took."""
+        import time
+        t0 = time.time()
+        _check(lib().qtip_ldl_hessian_device_updates_dev(self._h, _ptr(dHRr), n, threads, _ptr(L_host),
+                                                         _ptr(dL) if dL is not None else None))
+        return time.time() - t0
 
     def ldlq_dev(self, dWT, dL, n, m, d_hatWT, dQ, time_viterbi=False, feedback=0):
         vs = C.c_double()

@@ -164,6 +164,40 @@ __attribute__((target("avx512f"))) QTIP_TRI_SOLVE(tri_solve_24, v8d, 8, 24)
 QTIP_TRI_SOLVE(tri_solve_12, v4d, 4, 12)
 #undef QTIP_TRI_SOLVE
 
+// ---- one row of L over nblk 16-column blocks: out[16 b + j] = float(sum_p a[16 b + p] * inv_b[p][j]), p = j .. 15,
+// every sum one fused chain over ascending p from zero (src/qtip_core.cpp:473-483).  The lanes are the 16 values of
+// j: inv_b is lower triangular with +0 above the diagonal, so a lane j > p adds a zero product to its zero and its
+// chain is the scalar one.  false if a sum is not finite.
+typedef float v8f __attribute__((vector_size(32), aligned(4)));
+typedef float v4f __attribute__((vector_size(16), aligned(4)));
+#define QTIP_ASSEMBLE_ROW(NAME, VT, FT, VW)                                                                    \
+  static bool NAME(const double* __restrict__ a, const double* __restrict__ inv, int nblk, float* __restrict__ out) { \
+    constexpr int NV = 16 / VW;                                                                                \
+    VT chk[NV];                                                                                                \
+    for (int v = 0; v < NV; ++v) chk[v] = VT{};                                                                \
+    for (int b = 0; b < nblk; ++b) {                                                                           \
+      const double* ab = a + b * 16;                                                                           \
+      const double* iv = inv + size_t(b) * 256;                                                                \
+      VT s[NV];                                                                                                \
+      for (int v = 0; v < NV; ++v) s[v] = VT{};                                                                \
+      for (int p = 0; p < 16; ++p) {                                                                           \
+        const double ap = ab[p];                                                                               \
+        for (int v = 0; v < NV; ++v) s[v] += ap * *reinterpret_cast<const VT*>(iv + p * 16 + v * VW);          \
+      }                                                                                                        \
+      for (int v = 0; v < NV; ++v) {                                                                           \
+        *reinterpret_cast<FT*>(out + b * 16 + v * VW) = __builtin_convertvector(s[v], FT);                     \
+        chk[v] += s[v] * 0.0; /* NaN as soon as a sum is infinite or NaN */                                    \
+      }                                                                                                        \
+    }                                                                                                          \
+    double c = 0;                                                                                              \
+    for (int v = 0; v < NV; ++v)                                                                               \
+      for (int l = 0; l < VW; ++l) c += chk[v][l];                                                             \
+    return std::isfinite(c);                                                                                   \
+  }
+__attribute__((target("avx512f"))) QTIP_ASSEMBLE_ROW(assemble_row_avx512, v8d, v8f, 8)
+QTIP_ASSEMBLE_ROW(assemble_row_avx2, v4d, v4f, 4)
+#undef QTIP_ASSEMBLE_ROW
+
 }  // namespace
 // lower Cholesky of the kb x kb diagonal block at A (row stride ld) (host_ldl_diag.cpp, built without contraction: it
 // has to say which of its operations are fused); T: scratch of kb * ldt doubles, ldt >= kb rounded up to 32
@@ -176,11 +210,12 @@ struct Kernels {
   void (*micro)(int, const double*, const double*, double*, long, int, int);
   void (*tri_solve)(int, const double*, int, const double*, double*);
   bool (*factor_diag)(double*, long, int, double*, int);
+  bool (*assemble_row)(const double*, const double*, int, float*);
 };
 static Kernels pick_kernels() {
   __builtin_cpu_init();
-  if (__builtin_cpu_supports("avx512f")) return Kernels{8, 24, micro_8x24, tri_solve_24, factor_diag_avx512};
-  return Kernels{4, 12, micro_4x12, tri_solve_12, factor_diag_avx2};
+  if (__builtin_cpu_supports("avx512f")) return Kernels{8, 24, micro_8x24, tri_solve_24, factor_diag_avx512, assemble_row_avx512};
+  return Kernels{4, 12, micro_4x12, tri_solve_12, factor_diag_avx2, assemble_row_avx2};
 }
 
 // Lower Cholesky of the n x n matrix at A (row stride ld) by right-looking panels of width NBT, shared out over the
@@ -207,6 +242,7 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, PanelAssist* ass
     double* Ap = assist ? assist->fetch(k, kb) : A + long(k) * ld + k;
     const long ldp = assist ? kb : ld;
     if (!kn.factor_diag(Ap, ldp, kb, diagT.data(), LDT)) return false;
+    if (assist) assist->factored(k, kb, Ap, ldp);
     const int r0 = k + kb, nr = n - r0;
     if (nr <= 0) {
       if (assist) assist->solved(k, kb, Ap);
@@ -235,6 +271,10 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, PanelAssist* ass
       for (int r = 0; r < rows; ++r) {
         const int i = rb + r;
         double* dst = Ap + long(kb + i) * ldp;
+        if (assist) {  // the update runs elsewhere: no A-side pack
+          for (int p = 0; p < kb; ++p) dst[p] = x[size_t(p) * NR + r];
+          continue;
+        }
         double* pa = packA + size_t(i / MR) * MR * kb + (i % MR);
         for (int p = 0; p < kb; ++p) {
           const double v = x[size_t(p) * NR + r];
@@ -243,9 +283,15 @@ bool cholesky_panels(double* A, long ld, int n, HostTeam* team, PanelAssist* ass
         }
       }
     };
-    if (team) team->parallel_for(nPB, 2, solve_chunk);
+    auto solve_and_hand_over = [&](long gl) {
+      solve_chunk(gl);
+      const int rb = int(gl) * NR;
+      assist->rows_solved(k, kb, r0 + rb, std::min(NR, nr - rb), Ap + long(kb + rb) * ldp, ldp);
+    };
+    if (team && assist) team->parallel_for(nPB, 2, solve_and_hand_over);
+    else if (team) team->parallel_for(nPB, 2, solve_chunk);
     else
-      for (long gl = 0; gl < nPB; ++gl) solve_chunk(gl);
+      for (long gl = 0; gl < nPB; ++gl) assist ? solve_and_hand_over(gl) : solve_chunk(gl);
     if (assist) {
       assist->solved(k, kb, Ap);
       continue;
@@ -287,12 +333,9 @@ bool cholesky_lower_host(double* A, int n, int threads) {
   return cholesky_panels<NB, TILE>(A, n, n, &team);
 }
 
-// L columns c0 .. c0 + nc - 1 from the same columns of C: Cp holds rows c0 .. n-1 of those columns (row stride ldc).
-// L = C * blockdiag(C_bb^-1), 16x16 diagonal blocks and everything above them zero.  false if a value is not finite.
-static bool assemble_L_columns(const double* Cp, long ldc, int c0, int nc, int n, float* L_out, HostTeam& team) {
-  const int nbp = nc / 16;
-  // inverse of every 16x16 lower-triangular diagonal block (column by column, forward substitution)
-  std::vector<double> inv(size_t(nbp) * 256);
+// inverse of every 16 x 16 lower-triangular diagonal block b of C (column by column, forward substitution): Cp holds
+// the rows of the first diagonal block onwards, inv receives nbp blocks of 256 values
+static void invert_diag_blocks(const double* Cp, long ldc, int nbp, double* inv, HostTeam& team) {
   team.parallel_for(nbp, (nbp + team.size() - 1) / team.size(), [&](long bl) {
     const int b = int(bl);
     double D[16][16], V[16][16];
@@ -304,29 +347,27 @@ static bool assemble_L_columns(const double* Cp, long ldc, int c0, int nc, int n
         for (int p = 0; p < i; ++p) s -= D[i][p] * V[p][c];
         V[i][c] = s / D[i][i];
       }
-    std::memcpy(&inv[size_t(b) * 256], V, sizeof V);
+    std::memcpy(inv + size_t(b) * 256, V, sizeof V);
   });
+}
+
+// L columns c0 .. c0 + nc - 1 from the same columns of C, rows 0 .. row_end - 1: Cp holds rows c0 .. of those columns
+// (row stride ldc), inv the inverses of their diagonal blocks.  L = C * blockdiag(C_bb^-1), 16x16 diagonal blocks
+// and everything above them zero.  false if a value is not finite.
+static bool assemble_L_columns(const double* Cp, long ldc, const double* inv, int c0, int nc, int n, int row_end,
+                               float* L_out, HostTeam& team) {
+  const Kernels kn = pick_kernels();
+  const int nbp = nc / 16;
   std::atomic<int> finite{1};
-  team.parallel_for(n, 16, [&](long rl) {
+  team.parallel_for(row_end, 16, [&](long rl) {
     const int r = int(rl);
     float* lr = L_out + long(r) * n + c0;
     if (r < c0) {  // above the diagonal blocks of these columns
       std::memset(lr, 0, sizeof(float) * size_t(nc));
       return;
     }
-    bool ok = true;
-    const double* ar = Cp + long(r - c0) * ldc;
     const int rb = std::min(nbp, (r - c0) / 16);  // column blocks strictly left of this row's diagonal block
-    for (int bj = 0; bj < rb; ++bj) {
-      const double* a = ar + bj * 16;
-      const double* iv = &inv[size_t(bj) * 256];
-      for (int j = 0; j < 16; ++j) {
-        double s = 0;
-        for (int p = j; p < 16; ++p) s += a[p] * iv[p * 16 + j];
-        lr[bj * 16 + j] = float(s);
-        ok = ok && std::isfinite(s);
-      }
-    }
+    const bool ok = kn.assemble_row(Cp + long(r - c0) * ldc, inv, rb, lr);
     if (rb < nbp) std::memset(lr + long(rb) * 16, 0, sizeof(float) * size_t(nc - rb * 16));  // diagonal block and right of it
     if (!ok) finite.store(0, std::memory_order_relaxed);
   });
@@ -337,7 +378,9 @@ bool block_ldl_host(double* A, int n, float* L_out, int threads) {
   if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
   HostTeam& team = team_of_this_thread(threads);
   if (!cholesky_panels<NB, TILE>(A, n, n, &team)) return false;
-  return assemble_L_columns(A, n, 0, n, n, L_out, team);
+  std::vector<double> inv(size_t(n / 16) * 256);
+  invert_diag_blocks(A, n, n / 16, inv.data(), team);
+  return assemble_L_columns(A, n, inv.data(), 0, n, n, n, L_out, team);
 }
 
 int ldl_panel_width() { return NB; }
@@ -345,23 +388,37 @@ int ldl_panel_width() { return NB; }
 bool block_ldl_assisted(int n, float* L_out, int threads, PanelAssist& assist) {
   if (n % 16 != 0) fail(QTIP_E_ARG, "block LDL needs n %% 16 == 0 (n = %d)", n);
   HostTeam& team = team_of_this_thread(threads);
-  // L is assembled panel by panel from the solved columns as they pass through the host
+  // L is assembled panel by panel from the solved columns as they pass through the host: the rows below a panel by
+  // the thread that solved them, while they are in its cache; the rows above (zeros) and those of the diagonal
+  // block after the update has been queued
   struct Wrap : PanelAssist {
     PanelAssist& inner;
     int n;
     float* L;
     HostTeam& team;
-    bool finite = true;
+    const Kernels kn = pick_kernels();
+    std::vector<double> inv;
+    std::atomic<int> finite{1};
     Wrap(PanelAssist& i, int n_, float* L_, HostTeam& t) : inner(i), n(n_), L(L_), team(t) {}
     double* fetch(int k, int kb) override { return inner.fetch(k, kb); }
+    void factored(int k, int kb, const double* diag, long ld) override {
+      inv.resize(size_t(kb / 16) * 256);
+      invert_diag_blocks(diag, ld, kb / 16, inv.data(), team);
+    }
+    void rows_solved(int k, int kb, int row0, int count, const double* rows, long ld) override {
+      bool ok = true;
+      for (int i = 0; i < count; ++i)
+        ok = kn.assemble_row(rows + long(i) * ld, inv.data(), kb / 16, L + long(row0 + i) * n + k) && ok;
+      if (!ok) finite.store(0, std::memory_order_relaxed);
+    }
     void solved(int k, int kb, const double* panel) override {
-      inner.solved(k, kb, panel);  // the update is queued first and runs while L is assembled
-      finite = assemble_L_columns(panel, kb, k, kb, n, L, team) && finite;
+      inner.solved(k, kb, panel);  // the update is queued first and runs while the rest of L's columns is written
+      if (!assemble_L_columns(panel, kb, inv.data(), k, kb, n, k + kb, L, team)) finite.store(0, std::memory_order_relaxed);
       inner.assembled(k, kb);
     }
   } wrap(assist, n, L_out, team);
   if (!cholesky_panels<NB, TILE>(nullptr, 0, n, &team, &wrap)) return false;
-  return wrap.finite;
+  return wrap.finite.load() != 0;
 }
 
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle (tiled so both reads stay in cache)

@@ -32,6 +32,17 @@ __global__ __launch_bounds__(256) void transpose_panel_kernel(const double* __re
     if (p0 + r < kb && i0 + tx < nr) Xt[long(p0 + r) * nr + i0 + tx] = tile[tx][r];
 }
 
+// dst[i][0 .. kb) = A[i][0 .. kb) for `rows` rows (A: row stride lda): the columns of a panel, packed, so that they
+// travel to the host as one contiguous copy (a pitched copy of 2 KB rows runs at a fraction of the link's rate)
+__global__ __launch_bounds__(256) void gather_panel_kernel(const double* __restrict__ A, long lda, long rows, int kb,
+                                                         double* __restrict__ dst) {
+  const long per_row = kb / 2, total = rows * per_row;  // kb is even: two doubles per thread
+  for (long e = long(blockIdx.x) * blockDim.x + threadIdx.x; e < total; e += long(gridDim.x) * blockDim.x) {
+    const long i = e / per_row, c = (e % per_row) * 2;
+    *reinterpret_cast<double2*>(dst + i * kb + c) = *reinterpret_cast<const double2*>(A + i * lda + c);
+  }
+}
+
 // C[i][j] -= sum_p X[i][p] * X[j][p] for one 128 x 128 tile of the nr x nr lower triangle, every element one chain
 // over p = 0 .. kb-1 from zero.  Xt: kb x nr (the transposed solved rows, row stride ldx; nr and ldx multiples of 4),
 // C: row stride ldc.  strip_tiles = 0: the grid enumerates the tiles (bi, bj <= bi) of the whole triangle;
@@ -131,8 +142,11 @@ struct DeviceTrailing final : PanelAssist {
     if (fetched) (void)hipEventDestroy(fetched);
   }
   void copy_down(long k, long kb, double* dst) {
-    QTIP_HIP(hipMemcpy2DAsync(dst, size_t(kb) * 8, c->ldl_A.p + k * n + k, size_t(n) * 8, size_t(kb) * 8, size_t(n - k),
-                              hipMemcpyDeviceToHost, s));
+    const long rows = n - k, pairs = rows * (kb / 2);
+    gather_panel_kernel<<<dim3(unsigned(std::min<long>((pairs + 255) / 256, 4096))), dim3(256), 0, s>>>(
+        c->ldl_A.p + k * n + k, n, rows, int(kb), c->ldl_P.p);
+    QTIP_HIP(hipGetLastError());
+    QTIP_HIP(hipMemcpyAsync(dst, c->ldl_P.p, size_t(rows) * kb * 8, hipMemcpyDeviceToHost, s));
   }
   void assembled(int k, int kb) override {
     if (!dev_L) return;
@@ -189,6 +203,7 @@ void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int th
   if (!dev_HRr) c->ldl_H.ensure(nn);
   c->ldl_X.ensure(size_t(n) * nb);
   c->ldl_Xt.ensure(size_t(n) * nb);
+  c->ldl_P.ensure(size_t(n) * nb);
   for (auto& buf : c->ldl_panel)
     if (buf.n < size_t(n) * nb) buf.alloc(size_t(n) * nb);
   if (!dev_HRr) QTIP_HIP(hipMemcpyAsync(c->ldl_H.p, host_HRr, nn * 4, hipMemcpyHostToDevice, s));

@@ -518,6 +518,15 @@ int qtip_ldl_hessian_device_updates(qtip_ctx* ctx, const float* host_HRr, int n,
   });
 }
 
+int qtip_ldl_hessian_device_updates_dev(qtip_ctx* ctx, const float* dev_HRr, int n, int threads, float* host_L,
+                                        float* dev_L) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && dev_HRr != nullptr, "ldl_hessian (device updates): null context or Hessian");
+    DeviceGuard g(ctx);
+    ldl_hessian_assisted_impl(ctx, nullptr, n, threads, host_L, dev_HRr, dev_L);
+  });
+}
+
 int qtip_ldlq_dev(qtip_ctx* ctx, const float* dev_WT, const float* dev_L, long n, long m, float* dev_hatWT,
                   uint16_t* dev_Q, int feedback, double* vit_seconds) {
   return guarded([&] {

@@ -145,6 +145,12 @@ bool block_ldl_host(double* A, int n, float* L_out, int threads);
 struct PanelAssist {
   virtual double* fetch(int k, int kb) = 0;
   virtual void solved(int k, int kb, const double* panel) = 0;
+  // optional: the kb x kb diagonal block of panel k is factored (lower triangle at diag, row stride ld); called before
+  // the rows below it are solved
+  virtual void factored(int k, int kb, const double* diag, long ld) {}
+  // optional: rows row0 .. row0 + count - 1 of the matrix (below the panel) are solved, `rows` holds their kb values
+  // (row stride ld).  Called from the team's threads, several at a time, while the rows are still in cache.
+  virtual void rows_solved(int k, int kb, int row0, int count, const double* rows, long ld) {}
   // the columns k .. k+kb-1 of L_out are final (all n rows)
   virtual void assembled(int k, int kb) {}
   virtual ~PanelAssist() = default;

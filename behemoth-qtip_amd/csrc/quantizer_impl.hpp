@@ -25,7 +25,7 @@ struct qtip_ctx {
   // LDL with the trailing updates on the device (ldl_assist.hip): own stream, fp64 work matrix, fp32 upload of HRr,
   // solved panel rows, two page-locked panel buffers (the panels travel one ahead); allocated on first use
   hipStream_t ldl_stream = nullptr;
-  qtipmi::DBuf<double> ldl_A, ldl_X, ldl_Xt;
+  qtipmi::DBuf<double> ldl_A, ldl_X, ldl_Xt, ldl_P;
   qtipmi::DBuf<float> ldl_H;
   qtipmi::HBuf<double> ldl_panel[2];
 };

@@ -128,6 +128,14 @@ int qtip_cholesky_inplace(double* host_A, int n, int threads);
  * stream of its own inside ctx; may run on a side thread while another thread quantizes through the same ctx. */
 int qtip_ldl_hessian_device_updates(qtip_ctx* ctx, const float* host_HRr, int n, int threads, float* host_L);
 
+/* The same with the rotated Hessian already on the device (dev_HRr, n x n fp32, read only): the form
+ * qtip_run_groups uses for the groups it schedules (the schedule of run_qtip_groups, src/pipeline.cpp:229-312, where
+ * the reference calls its host-only ldl_hessian).  host_L as above; dev_L (optional, may be NULL): n x n fp32 device
+ * buffer that receives L as well, column block by column block while the factorization runs - host_L is the source
+ * of those copies and should then be page-locked. */
+int qtip_ldl_hessian_device_updates_dev(qtip_ctx* ctx, const float* dev_HRr, int n, int threads, float* host_L,
+                                        float* dev_L);
+
 /* ldlq_gpu, src/quantizer.cpp:30-89.  WT n x m fp32 (scaled), L n x n fp32, both on the device;
  * outputs hatWT n x m fp32 and Q[(m/16)*(n/16)][128] u16 on the device.  feedback as in qtip_opts;
  * vit_seconds may be NULL. */

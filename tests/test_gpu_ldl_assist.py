@@ -1,5 +1,5 @@
 """Block LDL with the trailing updates on the GPU (qtip_ldl_hessian_device_updates): the factor must equal the host
-factorization's bit for bit (same panel code on the host; the rank-512 updates on the fp64 matrix cores in the host
+factorization's bit for bit (same panel code on the host; the rank-256 updates on the fp64 matrix cores in the host
 micro-kernel's order of operations), including ragged last panels, and must fail the same way on a matrix that is not
 positive definite."""
 import numpy as np
@@ -39,6 +39,30 @@ def test_factor_equals_host_factor(qz, pkg, n):
         pkg.Quantizer.ldl_hessian(a2, threads=16)
         qz.ldl_hessian_device_updates(b2, threads=16)
         assert np.array_equal(a2.L.view(np.uint32), b2.L.view(np.uint32))
+
+
+@pytest.mark.parametrize("n", [272, 1040, 2560])
+def test_device_resident_form_equals_host_factor(qz, pkg, n):
+    """qtip_ldl_hessian_device_updates_dev: the rotated Hessian stays on the device and is not written, L arrives in the
+    host buffer and, column block by column block, in the device buffer; both equal the host factorization's words."""
+    import torch
+    say("case: LDL with device updates, Hessian resident on the device, n = %d" % n)
+    H = spd(n, 300 + n)
+    a = pkg.HessPrep(n=n, HRr=H.copy())
+    pkg.Quantizer.ldl_hessian(a, threads=16)
+    dH = torch.from_numpy(H).cuda()
+    L_pin = torch.full((n, n), -1.0, dtype=torch.float32).pin_memory()
+    dL = torch.full((n, n), -1.0, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    for _ in range(2):   # twice through the same context: the panel buffers alternate and are reused
+        qz.ldl_hessian_device_resident(dH, n, L_pin, dL, threads=16)
+        assert np.array_equal(L_pin.numpy().view(np.uint32), a.L.view(np.uint32))
+        assert torch.equal(dL.cpu(), L_pin)
+        assert torch.equal(dH.cpu(), torch.from_numpy(H))
+    # without the device copy of L
+    L2 = np.full((n, n), -1.0, np.float32)
+    qz.ldl_hessian_device_resident(dH, n, L2, None, threads=16)
+    assert np.array_equal(L2.view(np.uint32), a.L.view(np.uint32))
 
 
 def test_rank_deficient_matrix_is_refused(qz, pkg):
