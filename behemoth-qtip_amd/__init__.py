@@ -114,6 +114,7 @@ def lib():
     L.qtip_rotate_hessian.argtypes = [vp, vp, i, i, u64, d, vp, C.POINTER(d), vp]
     L.qtip_ldl_hessian.argtypes = [vp, i, i, vp]
     L.qtip_ldl_hessian_device_updates.argtypes = [vp, vp, i, i, vp]
+    L.qtip_selftest_ldl_panel_handover.argtypes = [vp, i, i, vp]
     L.qtip_ldl_hessian_device_updates_dev.argtypes = [vp, vp, i, i, vp, vp]
     L.qtip_ldlq_dev.argtypes = [vp, vp, vp, l, l, vp, vp, i, C.POINTER(d)]
     L.qtip_default_opts.argtypes = [C.POINTER(_OptsC)]

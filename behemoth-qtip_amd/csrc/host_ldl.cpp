@@ -421,6 +421,38 @@ bool block_ldl_assisted(int n, float* L_out, int threads, PanelAssist& assist) {
   return wrap.finite.load() != 0;
 }
 
+// block_ldl_assisted with the trailing matrix held and updated by plain host code (one fma chain per element over the
+// panel, from zero, then one subtraction): exercises the panel hand-over without a device.  L must come out as
+// block_ldl_host's.
+bool block_ldl_assisted_on_host(const float* HRr, int n, float* L_out, int threads) {
+  struct HostTrailing final : PanelAssist {
+    long n;
+    std::vector<double> A, buf[2];
+    int turn = 0;
+    double* fetch(int k, int kb) override {
+      std::vector<double>& b = buf[turn ^= 1];  // alternate, as the device form's two page-locked buffers do
+      b.resize(size_t(n - k) * kb);
+      for (long i = k; i < n; ++i)
+        for (int p = 0; p < kb; ++p) b[size_t(i - k) * kb + p] = A[size_t(i) * n + k + p];
+      return b.data();
+    }
+    void solved(int k, int kb, const double* panel) override {
+      const long r0 = k + kb;
+      const double* X = panel + size_t(kb) * kb;
+      for (long i = r0; i < n; ++i)
+        for (long j = r0; j <= i; ++j) {
+          double acc = 0;
+          for (int p = 0; p < kb; ++p) acc = __builtin_fma(X[size_t(i - r0) * kb + p], X[size_t(j - r0) * kb + p], acc);
+          A[size_t(i) * n + j] -= acc;
+        }
+    }
+  } host;
+  host.n = n;
+  host.A.assign(size_t(n) * n, 0.0);
+  symmetrize_lower_host(HRr, n, host.A.data(), threads);
+  return block_ldl_assisted(n, L_out, threads, host);
+}
+
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle (tiled so both reads stay in cache)
 void symmetrize_lower_host(const float* HRr, int n, double* A, int threads) {
   HostTeam& team = team_of_this_thread(threads);

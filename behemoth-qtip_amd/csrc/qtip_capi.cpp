@@ -439,6 +439,13 @@ int qtip_selftest_failed_alloc_is_retried(void) {
   });
 }
 
+int qtip_selftest_ldl_panel_handover(const float* host_HRr, int n, int threads, float* host_L) {
+  return guarded([&] {
+    QTIP_REQUIRE(host_HRr && host_L && n > 0 && n % 16 == 0, "ldl self test: bad arguments (n = %d)", n);
+    if (!block_ldl_assisted_on_host(host_HRr, n, host_L, threads)) throw Error(QTIP_E_NOT_PD, "block LDL failed (H not PD)");
+  });
+}
+
 int qtip_st_create(qtip_st_writer** out) {
   return guarded([&] {
     QTIP_REQUIRE(out != nullptr, "st_create: bad arguments");

@@ -157,6 +157,7 @@ struct PanelAssist {
 };
 int ldl_panel_width();
 bool block_ldl_assisted(int n, float* L_out, int threads, PanelAssist& assist);
+bool block_ldl_assisted_on_host(const float* HRr, int n, float* L_out, int threads);
 // lower Cholesky in place (lower triangle of the n x n fp64 matrix A); false if not positive definite
 bool cholesky_lower_host(double* A, int n, int threads);
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle

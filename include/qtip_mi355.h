@@ -286,6 +286,12 @@ int qtip_get_tlut_f16(qtip_ctx* ctx, uint16_t* host_tlut_f16);
  * allocation failed stays empty, so the next call allocates again instead of launching on a null pointer.  0 = ok. */
 int qtip_selftest_failed_alloc_is_retried(void);
 
+/* Host-only self test (no GPU needed, no counterpart in the reference): the block LDL through the panel hand-over
+ * that qtip_ldl_hessian_device_updates uses (a panel's columns fetched, factored and solved by the host, the rows
+ * handed back, L assembled from them as they pass), with the trailing matrix held and updated by plain host code
+ * instead of the device.  host_L must come out as qtip_ldl_hessian's, bit for bit. */
+int qtip_selftest_ldl_panel_handover(const float* host_HRr, int n, int threads, float* host_L);
+
 /* Host packers (pack_trellis / unpack_trellis / swizzle_for_kernel / unswizzle_for_kernel,
  * src/qtip_core.cpp:194-253) */
 void qtip_pack_trellis(const uint16_t* states, long B, uint16_t* packed);

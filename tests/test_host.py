@@ -101,6 +101,24 @@ def test_host_ldl_matches_oracle(pkg, oracle, n, threads):
         assert np.all(hp.L[16 * b:16 * b + 16, 16 * b:] == 0)
 
 
+@pytest.mark.parametrize("n,threads", [(16, 1), (272, 3), (528, 8), (800, 5)])
+def test_ldl_panel_handover_on_host(pkg, n, threads):
+    """The panel hand-over of the device-updated LDL (columns fetched, factored and solved on the host, rows handed
+    back, L assembled from the rows as they pass) with a plain host stand-in for the device's trailing matrix: L equals
+    the host-only factorization's bit for bit, also with a ragged last panel and a single panel."""
+    H = _spd(n, n) + 0.05 * np.eye(n, dtype=np.float32)
+    H[2, 5] += 1e-3
+    H = np.ascontiguousarray(H)
+    hp = pkg.HessPrep(n=n, HRr=H)
+    pkg.Quantizer.ldl_hessian(hp, threads=threads)
+    L2 = np.full((n, n), -1.0, np.float32)
+    assert pkg.lib().qtip_selftest_ldl_panel_handover(H.ctypes.data, n, threads, L2.ctypes.data) == 0
+    assert np.array_equal(L2.view(np.uint32), hp.L.view(np.uint32))
+    bad = H.copy()
+    bad[n // 2, n // 2] = -1.0
+    assert pkg.lib().qtip_selftest_ldl_panel_handover(bad.ctypes.data, n, threads, L2.ctypes.data) != 0
+
+
 def test_cholesky_inplace_fp64_bits(pkg, oracle):
     """qtip_cholesky_inplace: every bit of the fp64 factor equals the compiled reference's committed rows (n = 528) and
     the oracle's factor of a matrix with correlated, badly scaled channels (n = 784)."""
