@@ -43,20 +43,64 @@ __global__ __launch_bounds__(256) void gather_panel_kernel(const double* __restr
   }
 }
 
+// C -= acc for a wave's 64 x 64 outputs (rows i0 .., columns j0 ..; only i < nr, j <= i exist).  A block that lies
+// inside the triangle altogether (nearly all do) fetches the 16 values of a row block together, so it waits for 4
+// round trips to memory, not 64; the others go element by element.
+__device__ __forceinline__ void subtract_tile(const double4_t (&acc)[4][4], double* __restrict__ C, long ldc, int nr,
+                                              int i0, int j0, int lane) {
+  if (i0 + 64 <= nr && j0 + 63 <= i0) {  // the same for the whole wave
+    double* base = C + long(i0 + (lane >> 4)) * ldc + j0 + (lane & 15);
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) {
+      double c[4][4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const double* row = base + long(mi * 16 + 4 * v) * ldc;
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) c[ni][v] = row[ni * 16];
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        double* row = base + long(mi * 16 + 4 * v) * ldc;
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) row[ni * 16] = c[ni][v] - acc[mi][ni][v];
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int gi = i0 + mi * 16 + (lane >> 4) + 4 * v, gj = j0 + ni * 16 + (lane & 15);
+        if (gi < nr && gj <= gi) C[long(gi) * ldc + gj] -= acc[mi][ni][v];
+      }
+}
+
 // C[i][j] -= sum_p X[i][p] * X[j][p] for one 128 x 128 tile of the nr x nr lower triangle, every element one chain
-// over p = 0 .. kb-1 from zero.  Xt: kb x nr (the transposed solved rows, row stride ldx; nr and ldx multiples of 4),
-// C: row stride ldc.  strip_tiles = 0: the grid enumerates the tiles (bi, bj <= bi) of the whole triangle;
-// strip_tiles = w > 0: only the first w tile columns, grid = w x row tiles (the columns of the next panel, which the
-// host wants back before the rest of the update has run).  256 threads, 2 x 2 waves of 64 x 64, K staged 16 at a
-// time; the next 16 columns travel from HBM while the matrix cores work on the present ones.
-constexpr int UT = 128, UK = 16;
-__global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double* __restrict__ Xt, long ldx, int nr, int kb,
-                                                                 double* __restrict__ C, long ldc, int strip_tiles) {
+// over p = 0 .. kb-1 from zero, then one subtraction.  Xt: kb x nr (the transposed solved rows, row stride ldx; nr and
+// ldx multiples of 4, kb a multiple of 8), C: row stride ldc.  strip_tiles = 0: the grid enumerates the tiles
+// (bi, bj <= bi) of the whole triangle; strip_tiles = w > 0: only the first w tile columns, grid = w x row tiles
+// (the columns of the next panel, which the host wants back before the rest of the update has run).
+// 256 threads, 2 x 2 waves of 64 x 64.  The workgroups share the chip with the Viterbi kernel's (168 registers, 50 KB
+// of LDS each, three per CU), so this one stays within 168 registers and 48 KB of LDS and takes the place of one of
+// them, not two: the operand slices go from global memory straight into LDS (global_load_lds_dwordx4: a wave's 64
+// lanes fill one 1 KB row of 128 doubles), eight columns of the panel per stage, three stages in flight, one
+// barrier per stage, no staging registers.
+// Lanes beyond nr in the last tile row read whatever follows in Xt (the caller's buffer extends at least 128 doubles
+// beyond the last row read); those columns only feed outputs that are never stored.
+constexpr int UT = 128;
+constexpr int VK = 8, VSTAGES = 3;
+__global__ __launch_bounds__(256, 3) void rank_update_lower_kernel(const double* __restrict__ Xt, long ldx, int nr,
+                                                                     int kb, double* __restrict__ C, long ldc,
+                                                                     int strip_tiles) {
   int bi, bj;
   if (strip_tiles > 0) {
     bi = blockIdx.x / strip_tiles;
     bj = blockIdx.x % strip_tiles;
-    if (bj > bi) return;  // above the diagonal (uniform over the workgroup)
+    if (bj > bi) return;
   } else {
     // tile index t -> row bi with bi (bi + 1) / 2 <= t: the square root in fp32, then one step either way
     const int t = blockIdx.x;
@@ -66,60 +110,55 @@ __global__ __launch_bounds__(256, 2) void rank_update_lower_kernel(const double*
     bj = t - bi * (bi + 1) / 2;
   }
   const int i0 = bi * UT, j0 = bj * UT;
-  __shared__ __attribute__((aligned(16))) double Xi[UK][UT], Xj[UK][UT];
+  __shared__ __attribute__((aligned(16))) double S[VSTAGES][2][VK][UT];  // [stage][Xi | Xj][k][column]
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
   double4_t acc[4][4];
 #pragma unroll
   for (int a = 0; a < 4; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
-  const int lk = t >> 5, lc = (t & 31) * 4;  // this thread stages rows lk and lk + 8 of a slice, 4 columns at lc
-  const bool i_ok = i0 + lc + 3 < nr, j_ok = j0 + lc + 3 < nr;  // nr is a multiple of 4: a group of 4 is in or out
-  double4_t pi[2], pj[2];
-  auto fetch = [&](int k0) {
+  // wave w brings rows 2w and 2w + 1 of a stage's Xi and Xj slices
+  const double* gi = Xt + long(2 * wave) * ldx + i0 + 2 * lane;
+  const double* gj = Xt + long(2 * wave) * ldx + j0 + 2 * lane;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  auto issue = [&](int slice) {
+    const int st = slice % VSTAGES;
+    const long off = long(slice) * VK * ldx;
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
-      const int k = k0 + lk + 8 * r;
-      pi[r] = pj[r] = double4_t{0, 0, 0, 0};
-      if (k < kb) {
-        if (i_ok) pi[r] = *reinterpret_cast<const double4_t*>(Xt + long(k) * ldx + i0 + lc);
-        if (j_ok) pj[r] = *reinterpret_cast<const double4_t*>(Xt + long(k) * ldx + j0 + lc);
-      }
+      __builtin_amdgcn_global_load_lds(gi + off + r * ldx, (lds_ptr)&S[st][0][2 * wave + r][0], 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(gj + off + r * ldx, (lds_ptr)&S[st][1][2 * wave + r][0], 16, 0, 0);
     }
   };
-  fetch(0);
-  for (int k0 = 0; k0 < kb; k0 += UK) {
+  const int slices = kb / VK;  // kb is a multiple of 16
+  issue(0);
+  if (slices > 1) issue(1);
+  for (int sl = 0; sl < slices; ++sl) {
+    // this wave's loads of slice sl have landed when at most the 4 of slice sl + 1 are outstanding
+    if (sl + 1 < slices) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
+    else __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
+    // everyone's have, and everyone is done reading the stage that slice sl + 2 overwrites (a barrier that orders
+    // LDS only: __syncthreads() would also wait for the loads of slice sl + 1)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (sl + 2 < slices) issue(sl + 2);
+    const int st = sl % VSTAGES;
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      *reinterpret_cast<double4_t*>(&Xi[lk + 8 * r][lc]) = pi[r];
-      *reinterpret_cast<double4_t*>(&Xj[lk + 8 * r][lc]) = pj[r];
-    }
-    __syncthreads();
-    if (k0 + UK < kb) fetch(k0 + UK);
-#pragma unroll
-    for (int kk = 0; kk < UK; kk += 4) {
+    for (int kk = 0; kk < VK; kk += 4) {
       const int kr = kk + (lane >> 4), c = lane & 15;
       double a[4], b[4];
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) a[mi] = Xi[kr][wm * 64 + mi * 16 + c];
+      for (int mi = 0; mi < 4; ++mi) a[mi] = S[st][0][kr][wm * 64 + mi * 16 + c];
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni) b[ni] = Xj[kr][wn * 64 + ni * 16 + c];
+      for (int ni = 0; ni < 4; ++ni) b[ni] = S[st][1][kr][wn * 64 + ni * 16 + c];
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 4; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
     }
-    __syncthreads();
   }
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-    for (int ni = 0; ni < 4; ++ni)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int gi = i0 + wm * 64 + mi * 16 + (lane >> 4) + 4 * v, gj = j0 + wn * 64 + ni * 16 + (lane & 15);
-        if (gi < nr && gj <= gi) C[long(gi) * ldc + gj] -= acc[mi][ni][v];
-      }
+  subtract_tile(acc, C, ldc, nr, i0 + wm * 64, j0 + wn * 64, lane);
 }
 
 // The panels travel one ahead of the updates: as soon as panel k is solved its rows go up, the update of the next
@@ -166,6 +205,10 @@ struct DeviceTrailing final : PanelAssist {
   }
   void update(const double* Xt, long ldx, long nr, int kb, double* C, int strip_tiles) {
     const long nt = (nr + UT - 1) / UT, grid = strip_tiles ? nt * strip_tiles : nt * (nt + 1) / 2;
+    // what the kernel assumes: whole stages of 8 panel columns, and readable memory up to the end of the last tile
+    // row's 128 columns in every row of Xt
+    QTIP_REQUIRE(kb % VK == 0 && Xt >= c->ldl_Xt.p && size_t(Xt - c->ldl_Xt.p) + size_t(kb - 1) * ldx + size_t(nt) * UT <= c->ldl_Xt.n,
+                 "LDL update: operand shape the kernel does not cover (kb = %d, nr = %ld)", kb, nr);
     rank_update_lower_kernel<<<dim3(unsigned(grid)), dim3(256), 0, s>>>(Xt, ldx, int(nr), kb, C, n, strip_tiles);
     QTIP_HIP(hipGetLastError());
   }
