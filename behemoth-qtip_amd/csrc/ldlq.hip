@@ -21,68 +21,74 @@ constexpr int BM = 128, BN = 128, KC = 16;
 // out[y][i][j] = sum over the K slices of split y of A[k][i] * (B1 - B2)[k][j], i < 128: the cross-buffer feedback
 // of one 128-column LDLQ buffer gathered from all rows already quantized ("left-looking": every product term is
 // read once and nothing is read-modified-written).  K is long and the output small, so the K range is shared out
-// over gridDim.y workgroups per column tile and the partial tiles are summed afterwards in a fixed order.  The next
-// K slice is fetched into registers while the matrix cores work on the current one.
-__global__ __launch_bounds__(256, 2) void gemm_tn_f64_splitk_kernel(int N, long K, const float* __restrict__ A, long lda,
+// over gridDim.y workgroups per column tile (boundaries at multiples of 16 rows) and the partial tiles are summed
+// afterwards in a fixed order.
+// The fp32 operand rows go from global memory straight into LDS (global_load_lds_dwordx4: a wave's 64 lanes fill
+// two 128-float rows), 8 rows of K per stage, three stages in flight, one barrier per stage that orders LDS only; a
+// lane widens its fragments to fp64 (and forms B1 - B2) as it reads them.  No staging registers: 168 registers and
+// 36 KB of LDS, so that a workgroup fits beside two workgroups of the Viterbi kernel, which holds the other chain's
+// share of the chip while this one runs.  Columns beyond N (last column tile) read the row's last four floats
+// instead; they only feed outputs that are not stored.
+constexpr int GVK = 8, GST = 3;
+__global__ __launch_bounds__(256, 3) void gemm_tn_f64_splitk_kernel(int N, long K, const float* __restrict__ A, long lda,
                                                                     const float* __restrict__ B1,
                                                                     const float* __restrict__ B2, long ldb,
                                                                     double* __restrict__ out, long ldo) {
-  __shared__ __attribute__((aligned(16))) double As[KC][BM];
-  __shared__ __attribute__((aligned(16))) double Bs[KC][BN];
+  __shared__ __attribute__((aligned(16))) float S[GST][3][GVK][BM];  // [stage][A | B1 | B2][k][column]
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const long j0 = long(blockIdx.x) * BN;
-  const long slices = (K + KC - 1) / KC;
-  const long s0 = slices * blockIdx.y / gridDim.y, s1 = slices * (blockIdx.y + 1) / gridDim.y;
+  const long slices = (K + KC - 1) / KC;  // K is a multiple of 16
+  const long k0 = KC * (slices * blockIdx.y / gridDim.y), k1 = KC * (slices * (blockIdx.y + 1) / gridDim.y);
+  const int stages = int((k1 - k0) / GVK);
   double4_t acc[4][4];
 #pragma unroll
   for (int a = 0; a < 4; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
-  const int lk = t >> 5, lc = (t & 31) * 4;  // this thread stages rows lk and lk + 8 of a slice, 4 columns at lc
-  const bool b_ok = j0 + lc + 3 < N;
-  float4 ga[2], gb[2], gc[2];
-  auto fetch = [&](long slice) {
-#pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      const long k = slice * KC + lk + 8 * r;
-      ga[r] = gb[r] = gc[r] = float4{0.f, 0.f, 0.f, 0.f};
-      if (k < K) {
-        ga[r] = *reinterpret_cast<const float4*>(A + k * lda + lc);
-        if (b_ok) {
-          gb[r] = *reinterpret_cast<const float4*>(B1 + k * ldb + j0 + lc);
-          gc[r] = *reinterpret_cast<const float4*>(B2 + k * ldb + j0 + lc);
-        }
-      }
-    }
+  // wave w brings rows 2w (lanes 0..31) and 2w + 1 (lanes 32..63) of a stage, four floats per lane
+  const long row = k0 + 2 * wave + (lane >> 5), colA = 4 * (lane & 31);
+  long colB = j0 + colA;
+  if (colB + 3 >= N) colB = N - 4;
+  const float* ga = A + row * lda + colA;
+  const float* gb = B1 + row * ldb + colB;
+  const float* gc = B2 + row * ldb + colB;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  auto issue = [&](int stage) {
+    const int st = stage % GST;
+    const long off = long(stage) * GVK;
+    __builtin_amdgcn_global_load_lds(ga + off * lda, (lds_ptr)&S[st][0][2 * wave][0], 16, 0, 0);
+    __builtin_amdgcn_global_load_lds(gb + off * ldb, (lds_ptr)&S[st][1][2 * wave][0], 16, 0, 0);
+    __builtin_amdgcn_global_load_lds(gc + off * ldb, (lds_ptr)&S[st][2][2 * wave][0], 16, 0, 0);
   };
-  if (s0 < s1) fetch(s0);
-  for (long sl = s0; sl < s1; ++sl) {
+  if (stages > 0) issue(0);
+  if (stages > 1) issue(1);
+  for (int sg = 0; sg < stages; ++sg) {
+    // this wave's loads of stage sg have landed when at most the 3 of stage sg + 1 are outstanding
+    if (sg + 1 < stages) __builtin_amdgcn_s_waitcnt(0x0F73);  // vmcnt(3)
+    else __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
+    // everyone's have, and everyone is done reading the stage that stage sg + 2 overwrites (a bare barrier:
+    // __syncthreads() would also wait for the loads of stage sg + 1)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (sg + 2 < stages) issue(sg + 2);
+    const int st = sg % GST;
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      const int k = lk + 8 * r;
-      *reinterpret_cast<double2*>(&As[k][lc]) = double2{double(ga[r].x), double(ga[r].y)};
-      *reinterpret_cast<double2*>(&As[k][lc + 2]) = double2{double(ga[r].z), double(ga[r].w)};
-      *reinterpret_cast<double2*>(&Bs[k][lc]) = double2{double(gb[r].x) - double(gc[r].x), double(gb[r].y) - double(gc[r].y)};
-      *reinterpret_cast<double2*>(&Bs[k][lc + 2]) = double2{double(gb[r].z) - double(gc[r].z), double(gb[r].w) - double(gc[r].w)};
-    }
-    __syncthreads();
-    if (sl + 1 < s1) fetch(sl + 1);
-#pragma unroll
-    for (int kk = 0; kk < KC; kk += 4) {
+    for (int kk = 0; kk < GVK; kk += 4) {
       const int kr = kk + (lane >> 4), c = lane & 15;
       double a[4], b[4];
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) a[mi] = As[kr][wm * 64 + mi * 16 + c];
+      for (int mi = 0; mi < 4; ++mi) a[mi] = double(S[st][0][kr][wm * 64 + mi * 16 + c]);
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni) b[ni] = Bs[kr][wn * 64 + ni * 16 + c];
+      for (int ni = 0; ni < 4; ++ni)
+        b[ni] = double(S[st][1][kr][wn * 64 + ni * 16 + c]) - double(S[st][2][kr][wn * 64 + ni * 16 + c]);
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
         for (int ni = 0; ni < 4; ++ni)
           acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
     }
-    __syncthreads();
   }
   double* o = out + long(blockIdx.y) * BM * ldo;
 #pragma unroll
@@ -245,8 +251,8 @@ int gemm_splitk_splits(long K) {
 
 void launch_gemm_tn_f64_gather(int N, long K, const float* A, long lda, const float* B1, const float* B2, long ldb,
                                double* P, double* partials, hipStream_t s) {
-  QTIP_REQUIRE(N > 0 && K > 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 && B2 != nullptr,
-               "fp64 gather GEMM needs 16-byte aligned fp32 rows");
+  QTIP_REQUIRE(N >= 4 && K > 0 && K % KC == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 && B2 != nullptr,
+               "fp64 gather GEMM needs 16-byte aligned fp32 rows and K %% 16 == 0");
   const int S = gemm_splitk_splits(K);
   dim3 grid(unsigned((N + BN - 1) / BN), unsigned(S));
   gemm_tn_f64_splitk_kernel<<<grid, dim3(256), 0, s>>>(N, K, A, lda, B1, B2, ldb, S == 1 ? P : partials, N);
