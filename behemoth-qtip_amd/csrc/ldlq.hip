@@ -7,6 +7,8 @@
 //    from all rows quantized so far by a K-split kernel.
 //  * gemm_tn_bf16x3_gather: the same gathered product in the arithmetic of the reference's GPU path: every fp32
 //    operand split into bf16 hi + lo, three v_mfma_f32_32x32x16_bf16 terms, fp32 accumulation.
+#include <algorithm>
+
 #include "ldlq.hpp"
 #include "qtip_internal.hpp"
 
@@ -242,18 +244,28 @@ __global__ void sum_splits_f32_kernel(const float* __restrict__ part, int splits
 
 }  // namespace
 
-int gemm_splitk_splits(long K) {
-  // 96 column tiles x 5 splits keep every CU's two workgroup slots busy at m = 12288; short K ranges are not split
-  // below 512 rows
-  const long s = K / 512;
-  return int(s < 1 ? 1 : (s > 5 ? 5 : s));
+int gemm_splitk_splits(long K, int N, int slots) {
+  // The workgroups of a gather take the workgroup slots that the chain's last Viterbi launch has just left (`slots`
+  // of them, half of the chip with two chains), so the number of splits is chosen to fill whole rounds of those
+  // slots: the smallest count that fills at least 95 % of the rounds it needs, else the best there is; a split has
+  // at least 512 rows of K.  m = 12288 in two chains: 48 column tiles x 8 splits = 384 workgroups on 384 slots.
+  const long tiles = (N + BN - 1) / BN, most = std::min<long>(kMaxGatherSplits, std::max<long>(1, K / 512));
+  long best = 1;
+  double best_fill = 0;
+  for (long s = 1; s <= most; ++s) {
+    const long wgs = tiles * s, rounds = (wgs + slots - 1) / slots;
+    const double fill = double(wgs) / double(rounds * slots);
+    if (fill > best_fill + 1e-9) best = s, best_fill = fill;
+    if (fill >= 0.95) return int(s);
+  }
+  return int(best);
 }
 
 void launch_gemm_tn_f64_gather(int N, long K, const float* A, long lda, const float* B1, const float* B2, long ldb,
-                               double* P, double* partials, hipStream_t s) {
+                               double* P, double* partials, int slots, hipStream_t s) {
   QTIP_REQUIRE(N >= 4 && K > 0 && K % KC == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 && B2 != nullptr,
                "fp64 gather GEMM needs 16-byte aligned fp32 rows and K %% 16 == 0");
-  const int S = gemm_splitk_splits(K);
+  const int S = gemm_splitk_splits(K, N, slots);
   dim3 grid(unsigned((N + BN - 1) / BN), unsigned(S));
   gemm_tn_f64_splitk_kernel<<<grid, dim3(256), 0, s>>>(N, K, A, lda, B1, B2, ldb, S == 1 ? P : partials, N);
   QTIP_HIP(hipGetLastError());
@@ -265,10 +277,10 @@ void launch_gemm_tn_f64_gather(int N, long K, const float* A, long lda, const fl
 }
 
 void launch_gemm_tn_bf16x3_gather(int N, long K, const float* A, long lda, const float* B1, const float* B2, long ldb,
-                                  float* P, float* partials, hipStream_t s) {
+                                  float* P, float* partials, int slots, hipStream_t s) {
   QTIP_REQUIRE(N > 0 && K > 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 && B2 != nullptr,
                "split-bf16 gather GEMM needs 16-byte aligned fp32 rows");
-  const int S = gemm_splitk_splits(K);
+  const int S = gemm_splitk_splits(K, N, slots);
   dim3 grid(unsigned((N + SB - 1) / SB), unsigned(S));
   gemm_tn_bf16x3_gather_kernel<<<grid, dim3(256), 0, s>>>(N, K, A, lda, B1, B2, ldb, S == 1 ? P : partials, N);
   QTIP_HIP(hipGetLastError());

@@ -123,7 +123,7 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   }
   // The feedback of the rows quantized in earlier buffers is gathered per buffer into a 128 x rows slab per chain:
   // feedback 0 in fp64 (fp64 MFMA), feedback 1 in fp32 from bf16 hi/lo split operands (the reference GPU's arithmetic)
-  const int max_splits = gemm_splitk_splits(n);
+  const int max_splits = kMaxGatherSplits;
   DBuf<double> prod(feedback == 0 ? size_t(128) * m : 0), parts(feedback == 0 ? size_t(max_splits) * 128 * m : 0);
   DBuf<float> prod32(feedback == 1 ? size_t(128) * m : 0), parts32(feedback == 1 ? size_t(max_splits) * 128 * m : 0);
   for (int k = 0; k < nch; ++k) {
@@ -166,9 +166,9 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
           if (feedback == 0) QTIP_HIP(hipMemsetAsync(C.prod, 0, size_t(128) * C.rows * sizeof(double), C.s));
           else QTIP_HIP(hipMemsetAsync(C.prod32, 0, size_t(128) * C.rows * sizeof(float), C.s));
         } else if (feedback == 0) {
-          launch_gemm_tn_f64_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod, C.parts, C.s);
+          launch_gemm_tn_f64_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod, C.parts, C.slots, C.s);
         } else {
-          launch_gemm_tn_bf16x3_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod32, C.parts32, C.s);
+          launch_gemm_tn_bf16x3_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod32, C.parts32, C.slots, C.s);
         }
         for (int i = 7; i >= 0; --i) {  // the kernel forms the block's targets (in-buffer feedback) itself
           const int col0 = c0 + 16 * i;
