@@ -26,12 +26,12 @@ constexpr int BM = 128, BN = 128, KC = 16;
 // over gridDim.y workgroups per column tile (boundaries at multiples of 16 rows) and the partial tiles are summed
 // afterwards in a fixed order.
 // The fp32 operand rows go from global memory straight into LDS (global_load_lds_dwordx4: a wave's 64 lanes fill
-// two 128-float rows), 8 rows of K per stage, three stages in flight, one barrier per stage that orders LDS only; a
+// two 128-float rows), 8 rows of K per stage, four stages of LDS (three in flight ahead of the one in use), one barrier per stage that orders LDS only; a
 // lane widens its fragments to fp64 (and forms B1 - B2) as it reads them.  No staging registers: 168 registers and
-// 36 KB of LDS, so that a workgroup fits beside two workgroups of the Viterbi kernel, which holds the other chain's
+// 48 KB of LDS, so that a workgroup fits beside two workgroups of the Viterbi kernel, which holds the other chain's
 // share of the chip while this one runs.  Columns beyond N (last column tile) read the row's last four floats
 // instead; they only feed outputs that are not stored.
-constexpr int GVK = 8, GST = 3;
+constexpr int GVK = 8, GST = 4;
 __global__ __launch_bounds__(256, 3) void gemm_tn_f64_splitk_kernel(int N, long K, const float* __restrict__ A, long lda,
                                                                     const float* __restrict__ B1,
                                                                     const float* __restrict__ B2, long ldb,
@@ -63,18 +63,20 @@ __global__ __launch_bounds__(256, 3) void gemm_tn_f64_splitk_kernel(int N, long 
     __builtin_amdgcn_global_load_lds(gb + off * ldb, (lds_ptr)&S[st][1][2 * wave][0], 16, 0, 0);
     __builtin_amdgcn_global_load_lds(gc + off * ldb, (lds_ptr)&S[st][2][2 * wave][0], 16, 0, 0);
   };
-  if (stages > 0) issue(0);
-  if (stages > 1) issue(1);
+  for (int p = 0; p < GST - 1 && p < stages; ++p) issue(p);
   for (int sg = 0; sg < stages; ++sg) {
-    // this wave's loads of stage sg have landed when at most the 3 of stage sg + 1 are outstanding
-    if (sg + 1 < stages) __builtin_amdgcn_s_waitcnt(0x0F73);  // vmcnt(3)
+    // this wave's loads of stage sg have landed when only those of the stages issued after it are outstanding
+    // (3 loads per stage; loads return in order)
+    const int later = stages - 1 - sg < GST - 2 ? stages - 1 - sg : GST - 2;
+    if (later >= 2) __builtin_amdgcn_s_waitcnt(0x0F76);       // vmcnt(6)
+    else if (later == 1) __builtin_amdgcn_s_waitcnt(0x0F73);  // vmcnt(3)
     else __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
-    // everyone's have, and everyone is done reading the stage that stage sg + 2 overwrites (a bare barrier:
-    // __syncthreads() would also wait for the loads of stage sg + 1)
+    // everyone's have, and everyone is done reading the stage that the next issue overwrites (a bare barrier:
+    // __syncthreads() would also wait for the loads still in flight)
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (sg + 2 < stages) issue(sg + 2);
+    if (sg + GST - 1 < stages) issue(sg + GST - 1);
     const int st = sg % GST;
 #pragma unroll
     for (int kk = 0; kk < GVK; kk += 4) {
