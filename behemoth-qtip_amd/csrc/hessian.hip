@@ -235,19 +235,39 @@ __global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __res
 
   // accumulator element v of a lane: row (v % 4) + 8 (v / 4) + 4 (lane / 32), column lane % 32 of the 32 x 32 tile
   double dot = 0.0;
+  if ((ti + 1) * kTile <= n && (tj + 1) * kTile <= n) {
+    // a tile inside the matrix (all of them when n is a multiple of 256): the 16 values of H that go with one
+    // 32 x 32 accumulator are fetched together - one round trip to memory per accumulator, not one per value
+    float* hb = H + (ti * kTile + wm * 128 + 4 * (lane >> 5)) * n + tj * kTile + wn * 128 + rl;
 #pragma unroll
-  for (int mi = 0; mi < 4; ++mi)
+    for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-    for (int ni = 0; ni < 4; ++ni)
+      for (int ni = 0; ni < 4; ++ni) {
+        float h[16];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const long gi = ti * kTile + wm * 128 + mi * 32 + (v & 3) + 8 * (v >> 2) + 4 * (lane >> 5);
-        const long gj = tj * kTile + wn * 128 + ni * 32 + rl;
-        if (gi < n && gj < n) {
-          if (DOT) dot += double(acc[mi][ni][v]) * double(H[gi * n + gj]);
-          else H[gi * n + gj] += acc[mi][ni][v];
+        for (int v = 0; v < 16; ++v) h[v] = hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32];
+        __builtin_amdgcn_sched_barrier(0);  // all 16 loads are issued before the first value is used
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          if (DOT) dot += double(acc[mi][ni][v]) * double(h[v]);
+          else hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32] = h[v] + acc[mi][ni][v];
         }
       }
+  } else {
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const long gi = ti * kTile + wm * 128 + mi * 32 + (v & 3) + 8 * (v >> 2) + 4 * (lane >> 5);
+          const long gj = tj * kTile + wn * 128 + ni * 32 + rl;
+          if (gi < n && gj < n) {
+            if (DOT) dot += double(acc[mi][ni][v]) * double(H[gi * n + gj]);
+            else H[gi * n + gj] += acc[mi][ni][v];
+          }
+        }
+  }
   if (DOT) {
     // lanes, then waves, in a fixed order (the stage loop ended with a barrier: the staging buffers are free)
 #pragma unroll
