@@ -279,6 +279,168 @@ __global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __res
   }
 }
 
+// ---------------------------------------------------------------- the same update from operands stored as LDS images
+// The quadratic forms of the proxy build their operands themselves (split_image_kernel), so they are written as the
+// LDS images of the kernel's stages: [stage of 32 rows of K][column tile of 256][column][32 k], the four 16-byte
+// pieces of a column at position p ^ ((column >> 2) & 3) (free of bank conflicts for the 16-byte fragment reads: the
+// 16 lanes the LDS serves together then touch 16 different 16-byte bank groups).  A stage of an operand is 16 KB of
+// contiguous global memory and goes straight into LDS (global_load_lds_dwordx4, 1 KB per wave and instruction): no
+// staging registers, no transposes, no LDS writes by the waves.  Four stages of LDS; the loads run two stages ahead
+// of the matrix cores, and a wave fetches the fragments of the next 16 k while the 16 MFMAs of the present ones run.
+constexpr int IK = 32, ISTAGES = 4;
+constexpr int kImgSliceU16 = kTile * IK;                                  // one operand slice of a stage, 16 KB
+constexpr size_t kImgLdsBytes = size_t(ISTAGES) * 2 * kImgSliceU16 * 2;   // 128 KB
+
+__host__ __device__ inline size_t img_index(long k, long c, long tiles) {
+  const long st = k / IK, p = (k % IK) >> 3, T = c / kTile, col = c % kTile;
+  return (size_t(st * tiles + T) * kTile + size_t(col)) * IK + size_t((p ^ ((col >> 2) & 3)) * 8 + (k & 7));
+}
+
+template <bool DOT>
+__global__ __launch_bounds__(256, 1) void syrk_img_kernel(const uint16_t* __restrict__ IA, const uint16_t* __restrict__ IB,
+                                                         int stages, long n, float* __restrict__ H,
+                                                         double* __restrict__ partial, int tiles, int patch_cols) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  const long b = blockIdx.x;
+  const long xcd = b & 7, local = b >> 3;
+  const long patch = (local / (kPatchRows * kPatchCols)) * 8 + xcd, within = local % (kPatchRows * kPatchCols);
+  const long ti = (patch / patch_cols) * kPatchRows + within / kPatchCols;
+  const long tj = (patch % patch_cols) * kPatchCols + within % kPatchCols;
+  if (ti >= tiles || tj > ti) return;  // outside the matrix or above the diagonal
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int rl = lane & 31;
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][c][v] = 0.f;
+  {
+    // the accumulators enter the loop as results of a matrix instruction: they live in the accumulation registers
+    bf16x8 z;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) z[e] = __bf16(0.f);
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z, z, acc[a][c], 0, 0, 0);
+  }
+
+  // wave w brings the 1 KB chunks 4 w .. 4 w + 3 of both operand slices of a stage, 16 bytes per lane
+  const size_t stage_stride = size_t(tiles) * kImgSliceU16;
+  const uint16_t* ga = IA + size_t(ti) * kImgSliceU16 + (wave * 4) * 512 + lane * 8;
+  const uint16_t* gb = IB + size_t(tj) * kImgSliceU16 + (wave * 4) * 512 + lane * 8;
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  auto issue = [&](int st) {
+    uint16_t* la = lds + (st % ISTAGES) * 2 * kImgSliceU16 + (wave * 4) * 512;
+    const size_t off = size_t(st) * stage_stride;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      __builtin_amdgcn_global_load_lds(ga + off + q * 512, (lds_ptr)(la + q * 512), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(gb + off + q * 512, (lds_ptr)(la + kImgSliceU16 + q * 512), 16, 0, 0);
+    }
+  };
+  // fragment of 8 k (piece 2 ks + lane / 32) of column wX * 128 + 32 i + rl
+  const int offA = (wm * 128 + rl) * IK, offB = (wn * 128 + rl) * IK, sw = (rl >> 2) & 3, hi = lane >> 5;
+  bf16x8 fa[2][4], fb[2][4];
+  auto fetch = [&](int st, int ks, int set) {
+    const uint16_t* As = lds + (st % ISTAGES) * 2 * kImgSliceU16;
+    const int piece = ((2 * ks + hi) ^ sw) << 3;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      fa[set][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + offA + i * 32 * IK + piece));
+      fb[set][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + kImgSliceU16 + offB + i * 32 * IK + piece));
+    }
+  };
+  auto mfmas = [&](int set, int half) {  // the 8 MFMAs of row tiles 2 half, 2 half + 1
+#pragma unroll
+    for (int mi = 2 * half; mi < 2 * half + 2; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni)
+        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
+  };
+  auto landed = [&](int later_stages) {  // this wave's loads of a stage have landed (8 per stage, in order) ...
+    if (later_stages >= 1) __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
+    else __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();  // ... and so have everyone's (a bare barrier: no wait for the loads in flight)
+    asm volatile("" ::: "memory");
+  };
+  for (int p = 0; p < 2 && p < stages; ++p) issue(p);
+  landed(stages > 1 ? 1 : 0);
+  if (stages > 2) issue(2);
+  fetch(0, 0, 0);
+  // A wave has nothing to hide a wait behind but its own MFMAs, so the fragments of the next 16 k are requested
+  // between the two halves of the 16 MFMAs of the present ones: the wait the compiler puts in front of their first
+  // use then finds them there.
+  for (int st = 0; st < stages; ++st) {
+    mfmas(0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(st, 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(0, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (st + 1 < stages) {
+      // stage st + 1 is needed next; stage st + 2 may still be on its way; the buffer of stage st - 1, which every
+      // wave has read before this barrier, takes stage st + 3
+      landed(st + 2 < stages ? 1 : 0);
+      if (st + 3 < stages) issue(st + 3);
+    }
+    mfmas(1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (st + 1 < stages) fetch(st + 1, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __syncthreads();
+
+  // accumulator element v of a lane: row (v % 4) + 8 (v / 4) + 4 (lane / 32), column lane % 32 of the 32 x 32 tile
+  double dot = 0.0;
+  if ((ti + 1) * kTile <= n && (tj + 1) * kTile <= n) {
+    float* hb = H + (ti * kTile + wm * 128 + 4 * (lane >> 5)) * n + tj * kTile + wn * 128 + rl;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) {
+        float h[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) h[v] = hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32];
+        __builtin_amdgcn_sched_barrier(0);  // all 16 loads are issued before the first value is used
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          if (DOT) dot += double(acc[mi][ni][v]) * double(h[v]);
+          else hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32] = h[v] + acc[mi][ni][v];
+        }
+      }
+  } else {
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const long gi = ti * kTile + wm * 128 + mi * 32 + (v & 3) + 8 * (v >> 2) + 4 * (lane >> 5);
+          const long gj = tj * kTile + wn * 128 + ni * 32 + rl;
+          if (gi < n && gj < n) {
+            if (DOT) dot += double(acc[mi][ni][v]) * double(H[gi * n + gj]);
+            else H[gi * n + gj] += acc[mi][ni][v];
+          }
+        }
+  }
+  if (DOT) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+    double* red = reinterpret_cast<double*>(lds);
+    if (lane == 0) red[wave] = dot;
+    __syncthreads();
+    if (t == 0) partial[ti * tiles + tj] = (ti == tj ? 1.0 : 2.0) * (((red[0] + red[1]) + red[2]) + red[3]);
+  }
+}
+
 __device__ __forceinline__ uint16_t f32_to_bf16_dev(float f) {  // round to nearest even; the inputs here are finite
   uint32_t u = __float_as_uint(f);
   u += 0x7fffu + ((u >> 16) & 1u);
@@ -286,34 +448,38 @@ __device__ __forceinline__ uint16_t f32_to_bf16_dev(float f) {  // round to near
 }
 
 // X[r][c] = A[c][r] - (B ? B[c][r] : 0) for r < m, c < n (A, B: n x m with leading dimension ld), split into bf16 hi + lo
-// and written as the two operand stacks of the three-product form: XA = [hi; hi; lo], XB = [hi; lo; hi] (each 3 m x n),
-// so that XA^T XB = hi^T hi + hi^T lo + lo^T hi.
-__global__ __launch_bounds__(256) void split_transposed_kernel(const float* __restrict__ A, const float* __restrict__ B,
-                                                               long n, long m, long ld, uint16_t* __restrict__ XA,
-                                                               uint16_t* __restrict__ XB) {
-  __shared__ float tile[32][33];
-  const long c0 = long(blockIdx.y) * 32, r0 = long(blockIdx.x) * 32;
-  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+// and written as the stage images (img_index) of the two operand stacks of the three-product form, XA = [hi; hi; lo]
+// and XB = [hi; lo; hi], so that XA^T XB = hi^T hi + hi^T lo + lo^T hi.  Every segment is padded with zero rows to mp
+// (a multiple of 32) and the columns with zeros to tiles x 256.  A thread takes 8 consecutive r of one column: one
+// 16-byte piece of each segment of each image; the rows of A run along r, so no transpose is needed.
+__global__ __launch_bounds__(256) void split_image_kernel(const float* __restrict__ A, const float* __restrict__ B, long n,
+                                                          long m, long ld, long mp, long tiles, uint16_t* __restrict__ IA,
+                                                          uint16_t* __restrict__ IB) {
+  const long pieces = mp / 8, idx = long(blockIdx.x) * 256 + threadIdx.x;
+  const long c = idx / pieces, r0 = (idx % pieces) * 8;
+  if (c >= tiles * kTile) return;
+  uint32_t h[4], l[4];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const long c = c0 + ty + 8 * k, r = r0 + tx;
-    float v = 0.f;
-    if (c < n && r < m) v = A[c * ld + r] - (B ? B[c * ld + r] : 0.f);
-    tile[ty + 8 * k][tx] = v;
-  }
-  __syncthreads();
+  for (int e = 0; e < 8; e += 2) {
+    uint16_t hh[2], ll[2];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const long r = r0 + ty + 8 * k, c = c0 + tx;
-    if (r < m && c < n) {
-      const float v = tile[tx][ty + 8 * k];
-      const uint16_t hi = f32_to_bf16_dev(v);
-      const uint16_t lo = f32_to_bf16_dev(v - __uint_as_float(uint32_t(hi) << 16));
-      const long o = r * n + c, seg = m * n;
-      XA[o] = hi, XA[seg + o] = hi, XA[2 * seg + o] = lo;
-      XB[o] = hi, XB[seg + o] = lo, XB[2 * seg + o] = hi;
+    for (int q = 0; q < 2; ++q) {
+      const long r = r0 + e + q;
+      float v = 0.f;
+      if (c < n && r < m) v = A[c * ld + r] - (B ? B[c * ld + r] : 0.f);
+      hh[q] = f32_to_bf16_dev(v);
+      ll[q] = f32_to_bf16_dev(v - __uint_as_float(uint32_t(hh[q]) << 16));
     }
+    h[e >> 1] = uint32_t(hh[0]) | (uint32_t(hh[1]) << 16);
+    l[e >> 1] = uint32_t(ll[0]) | (uint32_t(ll[1]) << 16);
   }
+  const uint4 hi = {h[0], h[1], h[2], h[3]}, lo = {l[0], l[1], l[2], l[3]};
+  *reinterpret_cast<uint4*>(IA + img_index(r0, c, tiles)) = hi;
+  *reinterpret_cast<uint4*>(IA + img_index(mp + r0, c, tiles)) = hi;
+  *reinterpret_cast<uint4*>(IA + img_index(2 * mp + r0, c, tiles)) = lo;
+  *reinterpret_cast<uint4*>(IB + img_index(r0, c, tiles)) = hi;
+  *reinterpret_cast<uint4*>(IB + img_index(mp + r0, c, tiles)) = lo;
+  *reinterpret_cast<uint4*>(IB + img_index(2 * mp + r0, c, tiles)) = hi;
 }
 
 __global__ __launch_bounds__(256) void sum_doubles_kernel(const double* __restrict__ p, long count, double* __restrict__ out) {
@@ -373,8 +539,8 @@ struct SyrkGrid {
       if (!configured[size_t(dev)]) {
         QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel<false>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
-        QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel<true>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
+        QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_img_kernel<true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(kImgLdsBytes)));
         configured[size_t(dev)] = true;
       }
     }
@@ -406,18 +572,20 @@ double quad_trace_bf16x3(long n, long m, const float* H, const float* A, const f
                          DBuf<double>& scratch, hipStream_t s) {
   if (n <= 0 || m <= 0) return 0.0;
   QTIP_REQUIRE(n % 8 == 0, "proxy: n must be a multiple of 8 (n = %ld)", n);
-  const size_t seg = size_t(m) * size_t(n);
-  stack.ensure(6 * seg);
-  uint16_t* XA = stack.p;
-  uint16_t* XB = stack.p + 3 * seg;
-  split_transposed_kernel<<<dim3(unsigned((m + 31) / 32), unsigned((n + 31) / 32)), dim3(256), 0, s>>>(A, B, n, m, ld, XA, XB);
-  QTIP_HIP(hipGetLastError());
   SyrkGrid g(n);
+  const long mp = (m + IK - 1) / IK * IK, tiles = g.tiles;
+  const size_t img = size_t(3 * mp) * size_t(tiles) * kTile;  // one operand stack as stage images
+  stack.ensure(2 * img);
+  uint16_t* IA = stack.p;
+  uint16_t* IB = stack.p + img;
+  const long threads = tiles * kTile * (mp / 8);
+  split_image_kernel<<<dim3(unsigned((threads + 255) / 256)), dim3(256), 0, s>>>(A, B, n, m, ld, mp, tiles, IA, IB);
+  QTIP_HIP(hipGetLastError());
   const size_t np = size_t(g.tiles) * g.tiles;
   scratch.ensure(np + 1);
   QTIP_HIP(hipMemsetAsync(scratch.p, 0, np * sizeof(double), s));
-  syrk_bf16_kernel<true><<<dim3(g.grid), dim3(256), kLdsBytes, s>>>(XA, XB, 3 * m, n, const_cast<float*>(H), scratch.p,
-                                                                    g.tiles, g.patch_cols);
+  syrk_img_kernel<true><<<dim3(g.grid), dim3(256), kImgLdsBytes, s>>>(IA, IB, int(3 * mp / IK), n, const_cast<float*>(H),
+                                                                     scratch.p, g.tiles, g.patch_cols);
   QTIP_HIP(hipGetLastError());
   sum_doubles_kernel<<<dim3(1), dim3(256), 0, s>>>(scratch.p, long(np), scratch.p + np);
   QTIP_HIP(hipGetLastError());
