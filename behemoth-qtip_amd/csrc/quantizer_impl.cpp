@@ -145,7 +145,7 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
       launch_delay(launch_us * k / nch, ch[k].s);
     }
   }
-  // The queue is kept kAhead buffers (8 launches of ~2 ms each) ahead of the GPU and no further: without a bound the
+  // The queue is kept kAhead buffers (a gather and a Viterbi launch of ~10 ms each) ahead of the GPU and no further: without a bound the
   // submitting thread would spin on a full queue and take a core from the host LDL of the next group; with less
   // slack a submitting thread that the scheduler holds back for a few milliseconds leaves the GPU idle.
   constexpr long kAhead = 4;
@@ -170,8 +170,9 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
         } else {
           launch_gemm_tn_bf16x3_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod32, C.parts32, C.slots, C.s);
         }
-        for (int i = 7; i >= 0; --i) {  // the kernel forms the block's targets (in-buffer feedback) itself
-          const int col0 = c0 + 16 * i;
+        {
+          // one launch per buffer: a workgroup takes its tile row through the 8 column blocks, last to first, and
+          // forms each block's targets (in-buffer feedback) itself; no workgroup waits for another between blocks
           TileJob job;
           job.tiles = C.tiles;
           job.WT = WT + C.r0;
@@ -183,10 +184,11 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
           job.prod_row0 = c0, job.ldp = C.rows;
           job.states = Q + size_t(C.tile0) * nblk * 128;
           job.q_tile_stride = nblk;
-          job.q_offset = col0 / 16;
+          job.q_offset = c0 / 16;
           job.hatWT = hatWT + C.r0;
           job.ldw = m;
-          job.col0 = col0;
+          job.col0 = c0;
+          job.blocks = 8;
           hipEvent_t t0 = nullptr, t1 = nullptr;
           if (vit_seconds) t0 = timed.add(hipEventDefault), t1 = timed.add(hipEventDefault);
           launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws.p + viterbi_workspace_bytes(C.slot0), C.slots,

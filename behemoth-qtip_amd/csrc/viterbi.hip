@@ -319,9 +319,10 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
 // form tests/test_gpu.cpp:196-207).  The (<= 112) x 16 blocks of L, WT and hatWT the tile needs are staged in the
 // metric array, which is idle between tiles; thread u then owns the sequence position u.
 template <typename Acc>
-__device__ __forceinline__ void tile_targets(Smem& sm, const TileJob& job, long tile, const Acc* __restrict__ prod) {
+__device__ __forceinline__ void tile_targets(Smem& sm, const TileJob& job, long col0, long tile,
+                                             const Acc* __restrict__ prod) {
   const int u = threadIdx.x;
-  const int k0 = int(job.col0) + 16, nk = job.bufend - k0;
+  const int k0 = int(col0) + 16, nk = job.bufend - k0;
   float* Ls = reinterpret_cast<float*>(sm.M);
   float* Ws = Ls + 112 * 16;
   float* Hs = Ws + 112 * 16;
@@ -329,13 +330,13 @@ __device__ __forceinline__ void tile_targets(Smem& sm, const TileJob& job, long 
   for (int idx = u; idx < nk * 16; idx += kThreads) {
     const long k = k0 + (idx >> 4);
     const int e = idx & 15;
-    Ls[idx] = job.L[k * job.ldl + job.col0 + e];
+    Ls[idx] = job.L[k * job.ldl + col0 + e];
     Ws[idx] = job.WT[k * job.ldw + row0 + e];
     Hs[idx] = job.hatWT[k * job.ldw + row0 + e];
   }
   __syncthreads();
   const int q = perm_fwd(u), r = q >> 4, c = q & 15;
-  const long col = job.col0 + c;
+  const long col = col0 + c;
   Acc acc = Acc(job.WT[col * job.ldw + row0 + r]) + prod[(col - job.prod_row0) * (job.ldp ? job.ldp : job.ldw) + row0 + r];
   for (int kk = 0; kk < nk; ++kk) acc += Acc(Ls[kk * 16 + c]) * (Acc(Ws[kk * 16 + r]) - Acc(Hs[kk * 16 + r]));
   sm.x[u] = float(_Float16(float(acc)));
@@ -443,10 +444,14 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
   __shared__ Smem sm;
   const int u = threadIdx.x;
   double* hist = hist_all + size_t(blockIdx.x) * kHistWordsPerTile;
-  for (long tile = blockIdx.x; tile < job.tiles; tile += gridDim.x) {
+  for (long tile = blockIdx.x; tile < job.tiles; tile += gridDim.x)
+  for (int blk = job.blocks - 1; blk >= 0; --blk) {
+    // the column block of this turn; the hatWT values the previous turn wrote for this tile row are visible after
+    // the barrier that ended it
+    const long col0 = job.col0 + 16 * blk;
     if (job.X) sm.x[u] = job.X[tile * kSeq + u];
-    else if (job.prod64) tile_targets<double>(sm, job, tile, job.prod64);
-    else tile_targets<float>(sm, job, tile, job.prod32);
+    else if (job.prod64) tile_targets<double>(sm, job, col0, tile, job.prod64);
+    else tile_targets<float>(sm, job, col0, tile, job.prod32);
     __syncthreads();
     // pass 1 on the sequence rotated by half its length, free ends, traced back to step 64 for the overlap group;
     // pass 2 on the sequence itself, tail-biting through that group, traced back in full.  One loop, so that the
@@ -474,7 +479,7 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
       ov = sm.overlap;
     }
     // ---- outputs
-    if (job.states && u < kSteps) job.states[(tile * job.q_tile_stride + job.q_offset) * kSteps + u] = sm.st[u];
+    if (job.states && u < kSteps) job.states[(tile * job.q_tile_stride + job.q_offset + blk) * kSteps + u] = sm.st[u];
     if (job.packed && u < kWords) {
       uint32_t v;
       if (u == 0) v = sm.st[0];
@@ -489,7 +494,7 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
       const uint32_t s = sm.st[u >> 1];
       const uint32_t e = ((s * (s + 1u)) >> 6) & 1023u;
       const int q = perm_fwd(u), r = q >> 4, c = q & 15;
-      job.hatWT[(job.col0 + c) * job.ldw + tile * 16 + r] = entry_f[2 * e + (u & 1)];
+      job.hatWT[(col0 + c) * job.ldw + tile * 16 + r] = entry_f[2 * e + (u & 1)];
     }
     __syncthreads();
   }
@@ -532,10 +537,12 @@ void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const flo
     QTIP_REQUIRE(job.WT && job.L && job.hatWT && ((job.prod64 != nullptr) != (job.prod32 != nullptr)),
                  "viterbi: neither inputs nor complete LDLQ feedback operands");
     const long nk = job.bufend - job.col0 - 16;
-    QTIP_REQUIRE(job.col0 >= 0 && nk >= 0 && nk <= 112, "viterbi: column block outside its 128-column buffer");
+    QTIP_REQUIRE(job.col0 >= 0 && nk >= 0 && nk <= 112 && job.blocks >= 1 && job.col0 + 16 * job.blocks <= job.bufend,
+                 "viterbi: column blocks outside their 128-column buffer");
     QTIP_REQUIRE(job.col0 >= job.prod_row0 && job.ldw >= 16 * job.tiles && job.ldl >= job.bufend,
                  "viterbi: LDLQ operand geometry");
   }
+  QTIP_REQUIRE(job.blocks == 1 || (!job.X && !job.packed), "viterbi: several blocks per tile row only for LDLQ launches");
   const unsigned grid = unsigned(job.tiles < slots ? job.tiles : slots);
   if (start || stop) {
     // the runtime stamps the two events at the kernel's own start and end: the time between them is the kernel's,

@@ -251,7 +251,7 @@ def run_group(args, pkg):
     stats.pop("cmp_outs", None)
     stats.pop("cmp_outs3", None)
     ntr = sum(ms) // 16
-    launches = n // 16
+    launches = n // 128   # one Viterbi launch per 128-column buffer and chain: a workgroup takes its tile row through 8 column blocks
     nch = args.chains or 2        # the library's rule: a chain must fill its share of the 768 resident workgroups
     while nch > 1 and ntr < 768:
         nch -= 1
@@ -268,7 +268,7 @@ def run_group(args, pkg):
     names = {2: "config2: 1024x1024 group", 3: "config3: 12288x12288 q-proj group",
              4: "config4: gate+up 2x(28672x12288) group", 5: "config5: 12288x28672 down-proj group"}
     return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
-                vit_launch_weights=ntr * 256, workload=names[cfg] + (" (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)" if args.host_ldl else
+                vit_launch_weights=ntr * 256 * 8, blocks_per_launch=8, workload=names[cfg] + (" (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)" if args.host_ldl else
                                        " (RHT + fp64 LDL: host panels, GPU trailing updates + LDLQ + 2-pass Viterbi + pack)"),
                 extra=extra, cpu_group=cpu_group, concurrent=nch)
 
@@ -376,6 +376,8 @@ def main():
             "config%d_bytes_per_launch" % args.config)
     except Exception:
         traffic = None
+    if traffic is not None:
+        traffic *= res.get("blocks_per_launch", 1)   # the file gives bytes per column block of the group (768 tiles)
     try:
         counters = json.load(open(os.path.join(ROOT, "profiles", "viterbi_counters.json"))).get("config%d" % args.config, {})
     except Exception:
@@ -387,14 +389,15 @@ def main():
         "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": dict({"workload": res["workload"]}, **res["extra"]),
         # launch_ms: the average duration of one Viterbi launch (a start and a stop event stamped by every launch of
-        # the timed region itself); concurrent_launches of them run side by side, each on tiles_per_launch tiles, so
-        # weights_per_launch weights pass in that time
+        # the timed region itself); concurrent_launches of them run side by side, each taking tiles_per_launch tile
+        # rows through column_blocks_per_launch column blocks, so weights_per_launch weights pass in that time
         "roofline": {"bound": "valu", "kernel": "viterbi_tiles_kernel", "achieved": achieved, "peak": PEAK_FP64_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP64_TFLOPS, "traffic": traffic,
                      "traffic_source": "profiles/viterbi_traffic.json (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; offline)",
                      "launch_ms": res["vit_launch_s"] * 1e3, "weights_per_launch": res["vit_launch_weights"],
                      "concurrent_launches": res.get("concurrent", 1),
-                     "tiles_per_launch": res["vit_launch_weights"] // 256 // res.get("concurrent", 1),
+                     "tiles_per_launch": res["vit_launch_weights"] // 256 // res.get("concurrent", 1) // res.get("blocks_per_launch", 1),
+                     "column_blocks_per_launch": res.get("blocks_per_launch", 1),
                      "flop_per_weight": FLOP_PER_WEIGHT,
                      "lds_frac": counters.get("lds_active_frac"), "valu_frac": counters.get("valu_busy_frac"),
                      "counters_source": "profiles/viterbi_counters.json (rocprofv3 --pmc SQ_*; offline)"},
