@@ -202,7 +202,7 @@ class QuantOpts:  # src/quantizer.hpp:11-19
     feedback: int = 0          # 0: fp64 feedback (default), 1: fp32 feedback + bf16 hi/lo split MFMA
     skip_proxy: bool = False
     ldl_device_updates: bool = True    # the LDL's trailing updates run on the GPU (same L bit for bit); False: host alone
-    ldlq_chains: int = 0       # independent chains of launches the tile rows are dealt to (0: the library's default, 2)
+    ldlq_chains: int = 0       # independent chains of launches the tile rows are dealt to (0: the library's default: 3 with GPU_MAX_HW_QUEUES >= 6, else 2)
 
 
 @dataclass

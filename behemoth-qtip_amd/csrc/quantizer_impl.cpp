@@ -94,14 +94,20 @@ void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L) 
 void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, float* hatWT, uint16_t* Q, int feedback,
                double* vit_seconds, int chains) {
   QTIP_REQUIRE(n % 128 == 0, "LDLQ needs n %% 128 == 0 (n = %ld)", n);
-  QTIP_REQUIRE(chains >= 0 && chains <= 3, "LDLQ runs as 1 to 3 chains (0: default), not %d", chains);
+  QTIP_REQUIRE(chains >= 0 && chains <= qtip_ctx::kMaxChains, "LDLQ runs as 1 to %d chains (0: default), not %d", qtip_ctx::kMaxChains, chains);
   QTIP_REQUIRE(m % 16 == 0 && m > 0, "LDLQ needs m %% 16 == 0 (m = %ld)", m);
   QTIP_REQUIRE(feedback == 0 || feedback == 1, "unknown feedback mode %d", feedback);
   hipStream_t s = c->stream;
   ensure_viterbi_workspace(c);
   const long ntr = m / 16, nblk = n / 16;
-  // chains: only where every chain still fills its share of the chip
-  int nch = chains == 0 ? 2 : chains;
+  // chains: only where every chain still fills its share of the chip.  Default: three where the process was given
+  // enough hardware queues for them (context stream, two chain streams, the LDL's stream and the caller's own: with
+  // HIP's default of four queues two of these would share one and run one after the other), else two.
+  static const int default_chains = [] {
+    const char* q = getenv("GPU_MAX_HW_QUEUES");
+    return q && atoi(q) >= 6 ? 3 : 2;
+  }();
+  int nch = chains == 0 ? default_chains : chains;
   while (nch > 1 && ntr < long(nch) * (c->vit_slots / nch)) --nch;
   struct Chain {
     hipStream_t s;
@@ -110,7 +116,7 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
     int slot0, slots;    // share of the kept-metrics workspace
     double *prod, *parts;     // feedback 0: 128 x rows slab and the split-K partial slabs
     float *prod32, *parts32;  // feedback 1: the same in fp32
-  } ch[3];
+  } ch[qtip_ctx::kMaxChains];
   for (int k = 0; k < nch; ++k) {
     if (k > 0 && !c->chain_stream[k - 1]) QTIP_HIP(hipStreamCreateWithFlags(&c->chain_stream[k - 1], hipStreamNonBlocking));
     ch[k].s = k == 0 ? s : c->chain_stream[k - 1];
@@ -149,7 +155,7 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   // submitting thread would spin on a full queue and take a core from the host LDL of the next group; with less
   // slack a submitting thread that the scheduler holds back for a few milliseconds leaves the GPU idle.
   constexpr long kAhead = 4;
-  hipEvent_t pace[3][kAhead + 1];
+  hipEvent_t pace[qtip_ctx::kMaxChains][kAhead + 1];
   for (int k = 0; k < nch; ++k)
     for (auto& e : pace[k]) e = pacing.add(hipEventBlockingSync | hipEventDisableTiming);
   try {

@@ -15,9 +15,10 @@ struct qtip_ctx {
   bool lut_h2_valid = false;
   qtipmi::DBuf<unsigned char> vit_ws;  // kept-metrics slots of the resident Viterbi workgroups
   int vit_slots = 0;
-  // LDLQ runs its tile rows as up to three independent chains of launches, on the context's stream and these two,
-  // a third of a tile's time apart, so that one chain's trace-backs run under the others' forward passes
-  hipStream_t chain_stream[2] = {nullptr, nullptr};
+  // LDLQ runs its tile rows as up to kMaxChains independent chains of launches, on the context's stream and these,
+  // so that one chain's trace-backs and gathers run under the others' forward passes
+  static constexpr int kMaxChains = 3;
+  hipStream_t chain_stream[kMaxChains - 1] = {};
   qtipmi::Rht rht;
   qtipmi::DBuf<double> scratch;
   qtipmi::HBuf<float> ring_HRr[3], ring_L[3];  // page-locked staging of run_groups, kept between calls

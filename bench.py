@@ -252,7 +252,9 @@ def run_group(args, pkg):
     stats.pop("cmp_outs3", None)
     ntr = sum(ms) // 16
     launches = n // 128   # one Viterbi launch per 128-column buffer and chain: a workgroup takes its tile row through 8 column blocks
-    nch = args.chains or 2        # the library's rule: a chain must fill its share of the 768 resident workgroups
+    # the library's rule: three chains with at least 6 hardware queues, else two; a chain must fill its share of the
+    # 768 resident workgroups
+    nch = args.chains or (3 if int(os.environ.get("GPU_MAX_HW_QUEUES", "4")) >= 6 else 2)
     while nch > 1 and ntr < 768:
         nch -= 1
     gpu_s = stats["rht_s"] + stats["load_s"] + stats["ldlq_s"] + stats["proxy_s"] + stats["pack_s"]
@@ -261,6 +263,7 @@ def run_group(args, pkg):
                  serial_Mweights_s=weights_per_step / (gpu_s + stats["ldl_s"]) / 1e6,
                  viterbi_only_Mweights_s=weights_per_step / stats["viterbi_s"] / 1e6,
                  proxy_in_timed_region=True, ldl_threads=args.ldl_threads, feedback=args.feedback,
+                 hw_queues=int(os.environ.get("GPU_MAX_HW_QUEUES", "4")), ldlq_chains=nch,
                  ldl_device_updates=not args.host_ldl)
     extra.update(host_only)
     extra.update(host_inputs)
@@ -343,6 +346,10 @@ def main():
                     help="0: fp64 LDLQ feedback (default); 1: fp32 feedback + bf16 hi/lo split MFMA prod cache")
     ap.add_argument("--chains", type=int, default=0, choices=[0, 1, 2, 3],
                     help="independent chains of launches LDLQ deals the tile rows to (0: the library's default, 2)")
+    ap.add_argument("--hw-queues", type=int, default=8,
+                    help="GPU_MAX_HW_QUEUES for this process (set before the HIP runtime starts; 0: leave the environment "
+                         "alone).  With HIP's default of 4 the library runs two chains of launches per group, with 6 or "
+                         "more three")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="first run one plain 1 GiB device copy kernel (known traffic, scales the rocprof byte counters)")
     args = ap.parse_args()
@@ -351,6 +358,8 @@ def main():
               "tile row of a group is independent, so the path would shard by tile rows without any exchange)" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
+    if args.hw_queues > 0:
+        os.environ["GPU_MAX_HW_QUEUES"] = str(min(args.hw_queues, 32))   # read by the HIP runtime when it starts, below
     import torch
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)

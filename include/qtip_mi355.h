@@ -176,8 +176,10 @@ typedef struct { /* QuantOpts, src/quantizer.hpp:11-19 */
                             bit for bit); 0: block LDL on the host alone, as in the reference */
   int ldlq_chains;       /* LDLQ deals the tile rows of a group to this many independent chains of launches (each on
                             a stream of its own inside ctx), so that the trace-backs of one run under the forward
-                            passes of the others; same codes whatever the number.  0 (default): 2; at most 3, which
-                            pays only with more than HIP's default of four hardware queues per process */
+                            passes of the others; same codes whatever the number.  At most 3.  0 (default): 3 if the
+                            environment gave the process at least 6 hardware queues (GPU_MAX_HW_QUEUES, read by
+                            the HIP runtime when it starts), else 2 - with HIP's default of four queues a third
+                            chain would share a queue with another stream and run after it, not beside it */
 } qtip_opts;
 void qtip_default_opts(qtip_opts* o);
 
