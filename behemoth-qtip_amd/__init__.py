@@ -60,7 +60,7 @@ class _LinearOutC(C.Structure):
 class _OptsC(C.Structure):
     _fields_ = [("sigma_reg", C.c_double), ("scale_override", C.c_double), ("ldl_threads", C.c_int),
                 ("feedback", C.c_int), ("skip_proxy", C.c_int), ("ldl_device_updates", C.c_int),
-                ("ldlq_chains", C.c_int)]
+                ("ldlq_chains", C.c_int), ("group_lanes", C.c_int)]
 
 
 class _TimingC(C.Structure):
@@ -135,6 +135,8 @@ def lib():
     L.qtip_nvfp4_quantize_group.argtypes = [vp, i, vp, i, vp, C.POINTER(_Nvfp4OptsC), C.POINTER(i)]
     L.qtip_run_groups.argtypes = [vp, i, vp, C.POINTER(_OptsC), vp, vp]
     L.qtip_reserve_groups.argtypes = [vp, i]
+    L.qtip_group_lanes.argtypes = [vp, i, vp, C.POINTER(_OptsC), C.POINTER(C.c_int)]
+    L.qtip_selftest_group_lanes.argtypes = [i, i, i, i, i, C.POINTER(C.c_int)]
     L.qtip_st_create.argtypes = [C.POINTER(vp)]
     L.qtip_st_destroy.argtypes = [vp]
     L.qtip_st_destroy.restype = None
@@ -203,6 +205,7 @@ class QuantOpts:  # src/quantizer.hpp:11-19
     skip_proxy: bool = False
     ldl_device_updates: bool = True    # the LDL's trailing updates run on the GPU (same L bit for bit); False: host alone
     ldlq_chains: int = 0       # independent chains of launches the tile rows are dealt to (0: the library's default: 3 with GPU_MAX_HW_QUEUES >= 6, else 2)
+    group_lanes: int = 0       # run_groups: groups run side by side on this many lanes (0: as many as fit the chip, 1 for large groups; 1: one after the other)
 
 
 @dataclass
@@ -435,7 +438,7 @@ class Quantizer:
             cout[k].hatW = _ptr(o.hatW)
             outs.append(o)
         co = _OptsC(opt.sigma_reg, opt.scale_override, opt.ldl_threads, opt.feedback, 1 if opt.skip_proxy else 0,
-                    1 if opt.ldl_device_updates else 0, opt.ldlq_chains)
+                    1 if opt.ldl_device_updates else 0, opt.ldlq_chains, opt.group_lanes)
         return cin, cout, outs, co, keep
 
     @staticmethod
@@ -541,6 +544,24 @@ class Quantizer:
             o, tm = self._finish(cout, outs, tms[g])
             res.append((o, tm, waits[g]))
         return res
+
+    def group_lanes(self, shapes, opt: QuantOpts = None):
+        """How many groups run_groups would run side by side for groups of these shapes: a list of (ms, n) with ms
+        the out-features of the group's linears."""
+        opt = opt or QuantOpts()
+        G = (_GroupC * len(shapes))()
+        keep = []
+        for g, (ms, n) in enumerate(shapes):
+            cin = (_LinearInC * len(ms))()
+            for k, m in enumerate(ms):
+                cin[k].m = m
+            keep.append(cin)
+            G[g].nlin, G[g].lins, G[g].n = len(ms), C.addressof(cin), n
+        co = _OptsC(opt.sigma_reg, opt.scale_override, opt.ldl_threads, opt.feedback, 1 if opt.skip_proxy else 0,
+                    1 if opt.ldl_device_updates else 0, opt.ldlq_chains, opt.group_lanes)
+        lanes = C.c_int()
+        _check(lib().qtip_group_lanes(self._h, len(shapes), C.addressof(G), C.byref(co), C.byref(lanes)))
+        return lanes.value
 
     def tlut_f16(self):
         out = np.zeros((512, 2), np.uint16)

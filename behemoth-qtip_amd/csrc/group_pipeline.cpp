@@ -6,10 +6,12 @@
 // host memory stays at 6 n^2 floats however many groups are queued.
 #include <chrono>
 #include <condition_variable>
+#include <cstdlib>
 #include <cstring>
 #include <exception>
 #include <mutex>
 #include <thread>
+#include <vector>
 
 #include "quantizer_impl.hpp"
 
@@ -33,16 +35,12 @@ void reserve_group_ring(qtip_ctx* c, int n, int depth) {
   }
 }
 
-void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opts& opt, qtip_timing* tms,
-                     double* ldl_wait) {
-  QTIP_REQUIRE(ng >= 0 && (ng == 0 || groups), "run_groups: bad arguments");
-  if (ng == 0) return;
+namespace {
+// the groups one after the other through context c, the factorization of the next under the GPU work of the present
+void run_groups_on(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opts& opt, qtip_timing* tms,
+                   double* ldl_wait) {
   int nmax = 0;
-  for (int g = 0; g < ng; ++g) {
-    QTIP_REQUIRE(groups[g].n > 0 && groups[g].H && groups[g].nlin > 0 && groups[g].lins && groups[g].outs,
-                 "run_groups: group %d is incomplete", g);
-    nmax = std::max(nmax, groups[g].n);
-  }
+  for (int g = 0; g < ng; ++g) nmax = std::max(nmax, groups[g].n);
   const int R = std::min(3, ng);
   reserve_group_ring(c, nmax, R);
   // with the LDL's updates on the device the rotated Hessian never leaves it: the factorization reads it there and so
@@ -142,6 +140,145 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
   feed();
   ldl_thread.join();
   if (feed_err) std::rethrow_exception(feed_err);
+}
+
+// A lane's schedule: its groups one after the other on the lane's one stream - rotate, factor, quantize.  Nothing of a
+// lane overlaps with itself; the other lanes fill the chip meanwhile.
+void run_groups_in_line(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opts& opt, qtip_timing* tms,
+                        double* ldl_wait) {
+  int nmax = 0;
+  for (int g = 0; g < ng; ++g) nmax = std::max(nmax, groups[g].n);
+  reserve_group_ring(c, nmax, 1);
+  const bool keep_dev = opt.ldl_device_updates != 0;
+  if (keep_dev) {
+    c->ring_dHRr[0].ensure(size_t(nmax) * nmax);
+    c->ring_dL[0].ensure(size_t(nmax) * nmax);
+  }
+  std::vector<float> su(static_cast<size_t>(nmax), 0.0f);
+  for (int g = 0; g < ng; ++g) {
+    qtip_timing T{};
+    double creg = 0.0;
+    double t0 = now_s();
+    rotate_hessian_impl(c, groups[g].H, groups[g].h_on_device != 0, groups[g].n, groups[g].seed, opt.sigma_reg, su.data(),
+                        &creg, keep_dev ? nullptr : c->ring_HRr[0].p, keep_dev ? c->ring_dHRr[0].p : nullptr);
+    T.rht = now_s() - t0;
+    t0 = now_s();
+    if (keep_dev)
+      ldl_hessian_assisted_impl(c, nullptr, groups[g].n, opt.ldl_threads, c->ring_L[0].p, c->ring_dHRr[0].p,
+                                c->ring_dL[0].p);
+    else
+      ldl_hessian_impl(c->ring_HRr[0].p, groups[g].n, opt.ldl_threads, c->ring_L[0].p);
+    T.ldl_cpu = now_s() - t0;
+    if (ldl_wait) ldl_wait[g] = T.ldl_cpu;  // all of it: the lane's GPU work waits for its own factorization
+    quantize_group_impl(c, groups[g].nlin, groups[g].lins, groups[g].n, groups[g].seed, su.data(), creg,
+                        keep_dev ? nullptr : c->ring_HRr[0].p, c->ring_L[0].p, opt, groups[g].outs, &T,
+                        keep_dev ? c->ring_dHRr[0].p : nullptr, keep_dev ? c->ring_dL[0].p : nullptr);
+    if (tms) tms[g] = T;
+  }
+}
+
+long tile_rows_of(const qtip_group& g) {
+  long m = 0;
+  for (int i = 0; i < g.nlin; ++i) m += g.lins[i].m;
+  return (m + 15) / 16;
+}
+}  // namespace
+
+// Lanes.  A group keeps as many Viterbi workgroups busy as it has 16-row tile rows, and the chip holds
+// `device_slots` of them (three per compute unit); the reference's schedule (one group at a time,
+// src/pipeline.cpp:229-312) leaves most of the chip idle when the groups are small.  Groups do not depend on each
+// other, so such groups run side by side, each lane with streams, workspaces and a ring of its own and the
+// groups one after the other on its one stream.  Every group is computed by the same code on the same inputs: same
+// results whatever the number of lanes.  Automatic: as many lanes as the largest group's tile rows fit into the
+// chip's slots, while the lanes' staging (2 n^2 floats each, on the host and on the device) and fp64 work matrices
+// (2 n^2 floats more) stay under 8 GiB.  Lanes whose streams share a hardware queue (a process has
+// GPU_MAX_HW_QUEUES of them, 4 unless the environment says more) run one after the other; measured on 1024 x 1024
+// groups, 12 lanes were still the fastest choice with 4 queues (54 Mweights/s against 26 for one lane), with 8 (92)
+// and with 16 (134), so the rule does not look at the queues.
+int group_lanes_for(int ng, const qtip_group* groups, const qtip_opts& opt, int device_slots) {
+  QTIP_REQUIRE(opt.group_lanes >= 0 && opt.group_lanes <= qtip_ctx::kMaxLanes,
+               "run_groups: 1 to %d lanes (0: automatic), not %d", qtip_ctx::kMaxLanes, opt.group_lanes);
+  if (ng < 2 || opt.group_lanes == 1) return 1;
+  if (opt.group_lanes > 1) return std::min(opt.group_lanes, ng);
+  long rows = 1, nmax = 1;
+  for (int g = 0; g < ng; ++g) {
+    rows = std::max(rows, tile_rows_of(groups[g]));
+    nmax = std::max<long>(nmax, groups[g].n);
+  }
+  const long by_slots = device_slots / rows;
+  const long by_memory = (8L << 30) / (16 * nmax * nmax);
+  const long lanes = std::min<long>({by_slots, by_memory, long(qtip_ctx::kMaxLanes), long(ng)});
+  return lanes < 2 ? 1 : int(lanes);
+}
+
+void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opts& opt, qtip_timing* tms,
+                     double* ldl_wait) {
+  QTIP_REQUIRE(ng >= 0 && (ng == 0 || groups), "run_groups: bad arguments");
+  if (ng == 0) return;
+  for (int g = 0; g < ng; ++g)
+    QTIP_REQUIRE(groups[g].n > 0 && groups[g].H && groups[g].nlin > 0 && groups[g].lins && groups[g].outs,
+                 "run_groups: group %d is incomplete", g);
+  const int lanes = group_lanes_for(ng, groups, opt, viterbi_max_slots(c->device));
+  if (lanes == 1) {
+    // the per-group device buffers of the quantizing thread come from the context's arena and stay there between
+    // groups and calls: a hipFree waits for the whole device, the factorization's queued updates included (a dozen
+    // of them per group cost 10 ms of a 2.5 s config-5 group)
+    ArenaScope memory(&c->arena);
+    run_groups_on(c, ng, groups, opt, tms, ldl_wait);
+    return;
+  }
+  // group g goes to lane g % lanes; a lane's context keeps kept-metrics slots for its largest group only, and the
+  // host threads of the factorizations are shared out
+  struct Lane {
+    qtip_ctx* c = nullptr;
+    std::vector<qtip_group> groups;
+    std::vector<int> index;
+    std::vector<qtip_timing> tms;
+    std::vector<double> wait;
+    std::exception_ptr err;
+  };
+  std::vector<Lane> L(static_cast<size_t>(lanes));
+  qtip_opts lopt = opt;
+  lopt.group_lanes = 1;
+  lopt.ldlq_chains = 1;  // the other lanes are what runs under a lane's trace-backs; a chain more is a stream more
+  lopt.ldl_threads = std::max(1, opt.ldl_threads / lanes);
+  for (int k = 0; k < lanes; ++k) {
+    Lane& l = L[size_t(k)];
+    l.c = lane_context(c, k);
+    long rows = 1;
+    for (int g = k; g < ng; g += lanes) {
+      l.groups.push_back(groups[g]);
+      l.index.push_back(g);
+      rows = std::max(rows, tile_rows_of(groups[g]));
+    }
+    l.c->vit_slots_limit = std::max<int>(l.c->vit_slots_limit, int(std::min<long>(rows, 1L << 20)));
+    l.tms.resize(l.groups.size());
+    l.wait.resize(l.groups.size());
+    order_streams(c->stream, l.c->stream);  // inputs the caller ordered before the context's stream
+  }
+  std::vector<std::thread> th;
+  for (int k = 0; k < lanes; ++k)
+    th.emplace_back([&, k] {
+      Lane& l = L[size_t(k)];
+      try {
+        QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
+        // the lane's per-group buffers come from its own arena: a hipFree would wait for every other lane's work
+        ArenaScope lane_memory(&l.c->arena);
+        run_groups_in_line(l.c, int(l.groups.size()), l.groups.data(), lopt, l.tms.data(), l.wait.data());
+      } catch (...) {
+        l.err = std::current_exception();
+      }
+    });
+  for (std::thread& t : th) t.join();
+  for (Lane& l : L) {
+    order_streams(l.c->stream, c->stream);
+    for (size_t i = 0; i < l.index.size(); ++i) {
+      if (tms) tms[l.index[i]] = l.tms[i];
+      if (ldl_wait) ldl_wait[l.index[i]] = l.wait[i];
+    }
+  }
+  for (Lane& l : L)
+    if (l.err) std::rethrow_exception(l.err);
 }
 
 }  // namespace qtipmi

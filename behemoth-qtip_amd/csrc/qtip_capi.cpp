@@ -51,8 +51,19 @@ void upload_codebook(qtip_ctx* c) {
   QTIP_HIP(hipStreamSynchronize(c->stream));
 }
 
+
+void ensure_viterbi_workspace(qtip_ctx* c) {
+  int slots = viterbi_max_slots(c->device);
+  if (c->vit_slots_limit > 0) slots = std::min(slots, c->vit_slots_limit);
+  if (c->vit_slots >= slots) return;
+  QTIP_HIP(hipStreamSynchronize(c->stream));  // nothing may still use the smaller workspace
+  c->vit_slots = 0;
+  c->vit_ws.alloc(viterbi_workspace_bytes(slots));
+  c->vit_slots = slots;  // only once the workspace exists
+}
+
 // the context's stream waits for `other` (or the reverse): an event recorded on one, waited for on the other
-static void order_streams(hipStream_t first, hipStream_t then) {
+void order_streams(hipStream_t first, hipStream_t then) {
   hipEvent_t e;
   QTIP_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
   hipError_t rc = hipEventRecord(e, first);
@@ -61,11 +72,75 @@ static void order_streams(hipStream_t first, hipStream_t then) {
   QTIP_HIP(rc);
 }
 
-void ensure_viterbi_workspace(qtip_ctx* c) {
-  if (c->vit_slots > 0) return;
-  const int slots = viterbi_max_slots(c->device);
-  c->vit_ws.alloc(viterbi_workspace_bytes(slots));
-  c->vit_slots = slots;  // only once the workspace exists
+namespace {
+// a context on the current device: stream, codebook (cb_from's, or the default one), Hadamard tables
+qtip_ctx* make_context(int device, const HostCodebook* cb_from) {
+  struct Cleanup {
+    qtip_ctx* c;
+    ~Cleanup() {
+      if (c) {
+        if (c->stream) (void)hipStreamDestroy(c->stream);
+        delete c;
+      }
+    }
+  } guard{new qtip_ctx()};
+  qtip_ctx* c = guard.c;
+  c->device = device;
+  QTIP_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+  c->arena.streams.push_back(&c->stream);
+  for (hipStream_t& cs : c->chain_stream) c->arena.streams.push_back(&cs);
+  if (cb_from) c->cb = *cb_from;
+  else c->cb.build(nullptr);
+  upload_codebook(c);
+  c->rht.init(device, c->stream);
+  guard.c = nullptr;
+  return c;
+}
+
+void destroy_context(qtip_ctx* ctx) {
+  for (qtip_ctx*& l : ctx->lane)
+    if (l) {
+      destroy_context(l);
+      l = nullptr;
+    }
+  if (ctx->ldl_stream && ctx->ldl_stream != ctx->stream) {  // (a lane factors on its one stream)
+    (void)hipStreamSynchronize(ctx->ldl_stream);
+    (void)hipStreamDestroy(ctx->ldl_stream);
+  }
+  ctx->ldl_stream = nullptr;
+  for (hipStream_t& cs : ctx->chain_stream)
+    if (cs) {
+      (void)hipStreamSynchronize(cs);
+      (void)hipStreamDestroy(cs);
+      cs = nullptr;  // the context's buffers go back to its arena below, which must not wait for a stream that is gone
+    }
+  if (ctx->stream) {
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipStreamDestroy(ctx->stream);
+    ctx->stream = nullptr;
+  }
+  delete ctx;
+}
+}  // namespace
+
+qtip_ctx* lane_context(qtip_ctx* parent, int k) {
+  QTIP_REQUIRE(k >= 0 && k < qtip_ctx::kMaxLanes, "lane %d of %d", k, qtip_ctx::kMaxLanes);
+  if (!parent->lane[k]) {
+    parent->lane[k] = make_context(parent->device, &parent->cb);
+    // one stream per lane, the factorization's work included: a stream only runs beside the others if it has a
+    // hardware queue to itself, and a process has few of them (GPU_MAX_HW_QUEUES, 4 unless the environment says
+    // more); with a stream more per lane for the factorization 1024 x 1024 groups ran at 59 instead of 134 Mweights/s
+    parent->lane[k]->ldl_stream = parent->lane[k]->stream;
+  }
+  return parent->lane[k];
+}
+
+void release_lanes(qtip_ctx* parent) {
+  for (qtip_ctx*& l : parent->lane)
+    if (l) {
+      destroy_context(l);
+      l = nullptr;
+    }
 }
 }  // namespace qtipmi
 
@@ -89,27 +164,19 @@ int qtip_create(int device, qtip_ctx** out) {
     int prev = 0;
     QTIP_HIP(hipGetDevice(&prev));
     QTIP_HIP(hipSetDevice(device));
-    // a failure below must not leak the stream or leave another device current
-    struct Cleanup {
-      qtip_ctx* c;
+    // a failure below must not leave another device current
+    struct Restore {
       int prev;
-      ~Cleanup() {
-        if (c) {
-          if (c->stream) (void)hipStreamDestroy(c->stream);
-          delete c;
-        }
-        (void)hipSetDevice(prev);
-      }
-    } guard{new qtip_ctx(), prev};
-    qtip_ctx* c = guard.c;
-    c->device = device;
-    QTIP_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-    c->cb.build(nullptr);
-    upload_codebook(c);
-    c->rht.init(device, c->stream);
-    viterbi_static_scratch_init(device);
+      ~Restore() { (void)hipSetDevice(prev); }
+    } restore{prev};
+    qtip_ctx* c = make_context(device, nullptr);
+    try {
+      viterbi_static_scratch_init(device);
+    } catch (...) {
+      destroy_context(c);
+      throw;
+    }
     *out = c;
-    guard.c = nullptr;
   });
 }
 
@@ -118,20 +185,7 @@ void qtip_destroy(qtip_ctx* ctx) {
   int prev = 0;
   (void)hipGetDevice(&prev);
   (void)hipSetDevice(ctx->device);
-  if (ctx->ldl_stream) {
-    (void)hipStreamSynchronize(ctx->ldl_stream);
-    (void)hipStreamDestroy(ctx->ldl_stream);
-  }
-  for (hipStream_t cs : ctx->chain_stream)
-    if (cs) {
-      (void)hipStreamSynchronize(cs);
-      (void)hipStreamDestroy(cs);
-    }
-  if (ctx->stream) {
-    (void)hipStreamSynchronize(ctx->stream);
-    (void)hipStreamDestroy(ctx->stream);
-  }
-  delete ctx;
+  destroy_context(ctx);
   (void)hipSetDevice(prev);
 }
 
@@ -152,6 +206,7 @@ int qtip_set_tlut(qtip_ctx* ctx, const float* host_tlut) {
     ctx->cb.build(host_tlut);
     upload_codebook(ctx);
     ctx->lut_h2_valid = false;
+    release_lanes(ctx);  // they carry the old codebook; the next call that wants lanes makes new ones
   });
 }
 
@@ -320,6 +375,7 @@ void qtip_default_opts(qtip_opts* o) {
   o->skip_proxy = 0;
   o->ldl_device_updates = 1;
   o->ldlq_chains = 0;
+  o->group_lanes = 0;
 }
 
 void qtip_pack_trellis(const uint16_t* states, long B, uint16_t* packed) { pack_trellis_host(states, B, packed); }
@@ -408,6 +464,35 @@ int qtip_run_groups(qtip_ctx* ctx, int ngroups, const qtip_group* groups, const 
   });
 }
 
+int qtip_group_lanes(qtip_ctx* ctx, int ngroups, const qtip_group* groups, const qtip_opts* opts, int* lanes) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && lanes != nullptr && ngroups >= 0 && (ngroups == 0 || groups),
+                 "group_lanes: bad arguments");
+    qtip_opts o;
+    qtip_default_opts(&o);
+    if (opts) o = *opts;
+    *lanes = group_lanes_for(ngroups, groups, o, viterbi_max_slots(ctx->device));
+  });
+}
+
+int qtip_selftest_group_lanes(int device_slots, int ngroups, int m, int n, int requested, int* lanes) {
+  // host only: the lane rule for `ngroups` equal groups of one m x n linear each
+  return guarded([&] {
+    QTIP_REQUIRE(lanes != nullptr && ngroups >= 0 && ngroups <= 4096 && m > 0 && n > 0, "selftest: bad arguments");
+    qtip_linear_in lin{};
+    lin.m = m;
+    std::vector<qtip_group> groups(static_cast<size_t>(ngroups));
+    for (qtip_group& g : groups) {
+      g = qtip_group{};
+      g.nlin = 1, g.lins = &lin, g.n = n;
+    }
+    qtip_opts o;
+    qtip_default_opts(&o);
+    o.group_lanes = requested;
+    *lanes = group_lanes_for(ngroups, groups.data(), o, device_slots);
+  });
+}
+
 int qtip_reserve_groups(qtip_ctx* ctx, int n) {
   return guarded([&] {
     QTIP_REQUIRE(ctx != nullptr && n > 0, "reserve_groups: bad arguments");
@@ -436,6 +521,23 @@ int qtip_selftest_failed_alloc_is_retried(void) {
       QTIP_REQUIRE(b.p == nullptr && b.n == 0, "attempt %d: a failed allocation left n = %zu", attempt, b.n);
     }
     test_fail_next_device_allocs(0);
+    // the same through an arena: a failed allocation is tried once more after the arena has let go of its idle
+    // blocks, and a second failure leaves the buffer empty
+    DeviceArena arena;
+    ArenaScope scope(&arena);
+    DBuf<float> a;
+    test_fail_next_device_allocs(2);
+    const long calls = test_device_alloc_calls();
+    bool threw = false;
+    try {
+      a.ensure(4096);
+    } catch (const Error& e) {
+      threw = e.code == QTIP_E_HIP;
+    }
+    test_fail_next_device_allocs(0);
+    QTIP_REQUIRE(threw, "arena: a failed allocation did not raise");
+    QTIP_REQUIRE(test_device_alloc_calls() == calls + 2, "arena: a failed allocation was not tried again once");
+    QTIP_REQUIRE(a.p == nullptr && a.n == 0 && a.from == nullptr, "arena: a failed allocation left n = %zu", a.n);
   });
 }
 

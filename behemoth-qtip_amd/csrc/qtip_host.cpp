@@ -7,6 +7,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <vector>
 
 #include "data/qtip_tables.h"
 #include "qtip_internal.hpp"
@@ -37,6 +38,82 @@ hipError_t device_malloc(void** p, size_t bytes) {
 }
 void test_fail_next_device_allocs(int count) { g_fail_allocs.store(count); }
 long test_device_alloc_calls() { return g_alloc_calls.load(); }
+
+struct DeviceArena::Impl {
+  struct Block {
+    void* p;
+    size_t cap;
+    bool busy;
+  };
+  std::mutex mu;
+  std::vector<Block> blocks;
+};
+DeviceArena::~DeviceArena() {
+  if (!impl) return;
+  for (auto& b : impl->blocks) (void)hipFree(b.p);
+  delete impl;
+}
+hipError_t DeviceArena::acquire(void** p, size_t bytes) {
+  if (!impl) impl = new Impl();
+  {
+    std::lock_guard<std::mutex> lk(impl->mu);
+    Impl::Block* fit = nullptr;
+    for (auto& b : impl->blocks)
+      if (!b.busy && b.cap >= bytes && b.cap / 2 <= bytes && (!fit || b.cap < fit->cap)) fit = &b;
+    if (fit) {
+      fit->busy = true;
+      *p = fit->p;
+      return hipSuccess;
+    }
+  }
+  // nothing idle fits: a new block.  Idle blocks go back to the runtime first when they hold more than 32 GiB (groups
+  // of many different shapes would otherwise pile them up), and all of them when the device is out of memory
+  const size_t cap = (bytes + 255) / 256 * 256;
+  auto drop_idle = [&] {
+    std::vector<void*> gone;
+    {
+      std::lock_guard<std::mutex> lk(impl->mu);
+      for (size_t i = impl->blocks.size(); i-- > 0;)
+        if (!impl->blocks[i].busy) {
+          gone.push_back(impl->blocks[i].p);
+          impl->blocks.erase(impl->blocks.begin() + long(i));
+        }
+    }
+    for (void* q : gone) (void)hipFree(q);
+  };
+  {
+    size_t idle = 0;
+    {
+      std::lock_guard<std::mutex> lk(impl->mu);
+      for (auto& b : impl->blocks)
+        if (!b.busy) idle += b.cap;
+    }
+    if (idle > (size_t(32) << 30)) drop_idle();
+  }
+  hipError_t rc = device_malloc(p, cap);
+  if (rc == hipErrorOutOfMemory) {
+    (void)hipGetLastError();
+    drop_idle();
+    rc = device_malloc(p, cap);
+  }
+  if (rc != hipSuccess) return rc;
+  std::lock_guard<std::mutex> lk(impl->mu);
+  impl->blocks.push_back(Impl::Block{*p, cap, true});
+  return hipSuccess;
+}
+void DeviceArena::give_back(void* p) {
+  // the next user of the block may run on another of the arena's streams: everything queued on them so far is over
+  // before the block counts as idle (hipFree would have waited for the whole device)
+  for (hipStream_t* s : streams)
+    if (s && *s) (void)hipStreamSynchronize(*s);
+  std::lock_guard<std::mutex> lk(impl->mu);
+  for (auto& b : impl->blocks)
+    if (b.p == p) b.busy = false;
+}
+static thread_local DeviceArena* g_arena = nullptr;
+DeviceArena* current_arena() { return g_arena; }
+ArenaScope::ArenaScope(DeviceArena* a) : prev(g_arena) { g_arena = a; }
+ArenaScope::~ArenaScope() { g_arena = prev; }
 
 // IEEE binary16 <-> binary32, round to nearest even (src/common.hpp:49-78 of the reference)
 uint16_t f32_to_fp16(float f) {

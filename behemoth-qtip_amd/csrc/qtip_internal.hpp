@@ -43,11 +43,39 @@ hipError_t device_malloc(void** p, size_t bytes);
 void test_fail_next_device_allocs(int count);
 long test_device_alloc_calls();
 
+// Device memory kept by a context instead of going back to the runtime.  hipFree waits for the whole device, every
+// stream of every thread, and the per-group buffers of the quantizer are a dozen such waits per group: harmless
+// while one group at a time uses the chip, but groups that run side by side on lanes would wait for each other at
+// every one of them.  A thread that has made an arena current (ArenaScope) gets its DBuf allocations from the
+// arena's idle blocks (smallest one that is large enough and at most twice the size; else a new hipMalloc) and hands
+// them back on release, after waiting for the arena's own streams only - the streams the lane's kernels run on.
+// The blocks are freed with the arena.
+struct DeviceArena {
+  DeviceArena() = default;
+  DeviceArena(const DeviceArena&) = delete;
+  DeviceArena& operator=(const DeviceArena&) = delete;
+  ~DeviceArena();
+  hipError_t acquire(void** p, size_t bytes);
+  void give_back(void* p);
+  std::vector<hipStream_t*> streams;  // slots holding the streams whose work may use the blocks (null slots are skipped)
+  struct Impl;
+  Impl* impl = nullptr;
+};
+DeviceArena* current_arena();
+struct ArenaScope {  // makes `a` the calling thread's arena until the scope ends
+  DeviceArena* prev;
+  explicit ArenaScope(DeviceArena* a);
+  ~ArenaScope();
+  ArenaScope(const ArenaScope&) = delete;
+  ArenaScope& operator=(const ArenaScope&) = delete;
+};
+
 // Device buffer released on scope exit.
 template <class T>
 struct DBuf {
   T* p = nullptr;
   size_t n = 0;
+  DeviceArena* from = nullptr;  // the arena the block came from (null: hipMalloc)
   DBuf() = default;
   explicit DBuf(size_t count) { alloc(count); }
   DBuf(const DBuf&) = delete;
@@ -55,16 +83,25 @@ struct DBuf {
   ~DBuf() { release(); }
   void alloc(size_t count) {
     release();
-    if (count) QTIP_HIP(device_malloc(reinterpret_cast<void**>(&p), count * sizeof(T)));
+    if (count) {
+      DeviceArena* a = current_arena();
+      QTIP_HIP(a ? a->acquire(reinterpret_cast<void**>(&p), count * sizeof(T))
+                 : device_malloc(reinterpret_cast<void**>(&p), count * sizeof(T)));
+      from = a;
+    }
     n = count;  // only after the allocation succeeded: a failed one leaves an empty buffer that ensure() retries
   }
   void ensure(size_t count) {
     if (count > n) alloc(count);
   }
   void release() {
-    if (p) (void)hipFree(p);
+    if (p) {
+      if (from) from->give_back(p);
+      else (void)hipFree(p);
+    }
     p = nullptr;
     n = 0;
+    from = nullptr;
   }
   size_t bytes() const { return n * sizeof(T); }
   operator T*() const { return p; }

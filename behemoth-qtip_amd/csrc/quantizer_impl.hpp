@@ -6,6 +6,8 @@
 #include "rht.hpp"
 
 struct qtip_ctx {
+  // first member, so that it outlives every buffer below: a lane's per-group device buffers come from here
+  qtipmi::DeviceArena arena;
   int device = 0;
   hipStream_t stream = nullptr;
   qtipmi::HostCodebook cb;
@@ -15,6 +17,11 @@ struct qtip_ctx {
   bool lut_h2_valid = false;
   qtipmi::DBuf<unsigned char> vit_ws;  // kept-metrics slots of the resident Viterbi workgroups
   int vit_slots = 0;
+  int vit_slots_limit = 0;  // a lane (below) keeps slots for this many workgroups only; 0: all the device can hold
+  // qtip_run_groups runs groups too small to fill the chip side by side, each on a lane: a context of its own
+  // (streams, workspaces, rings) made on first use, kept here and released with this context
+  static constexpr int kMaxLanes = 12;
+  qtip_ctx* lane[kMaxLanes] = {};
   // LDLQ runs its tile rows as up to kMaxChains independent chains of launches, on the context's stream and these,
   // so that one chain's trace-backs and gathers run under the others' forward passes
   static constexpr int kMaxChains = 3;
@@ -45,6 +52,13 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
                          qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr = nullptr,
                          const float* dev_L = nullptr);
 void reserve_group_ring(qtip_ctx* c, int n, int depth);
+// lane k of a context (made on first use with the parent's codebook), and the release of all of them
+qtip_ctx* lane_context(qtip_ctx* parent, int k);
+void release_lanes(qtip_ctx* parent);
+// stream `then` waits for everything queued on `first` so far
+void order_streams(hipStream_t first, hipStream_t then);
+// how many groups qtip_run_groups runs side by side (1: one after the other on the context itself)
+int group_lanes_for(int ngroups, const qtip_group* groups, const qtip_opts& opt, int device_slots);
 void run_groups_impl(qtip_ctx* c, int ngroups, const qtip_group* groups, const qtip_opts& opt, qtip_timing* timings,
                      double* ldl_wait);
 uint8_t f32_to_fp8e4m3(float x);

@@ -162,7 +162,7 @@ def run_group(args, pkg):
     ms = [int(w.shape[0]) for w in Ws]
     lins = [pkg.LinearIn("w%d" % i, m, w_f32=w) for i, (m, w) in enumerate(zip(ms, Ws))]
     opt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback,
-                        ldl_device_updates=not args.host_ldl, ldlq_chains=args.chains)
+                        ldl_device_updates=not args.host_ldl, ldlq_chains=args.chains, group_lanes=args.lanes)
     weights_per_step = sum(ms) * n
 
     stats = {}
@@ -198,7 +198,7 @@ def run_group(args, pkg):
         # reference factors; fewer groups, so the one exposed factorization at the start weighs more
         kh = min(args.steps, 6)
         hopt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback,
-                             ldl_device_updates=False, ldlq_chains=args.chains)
+                             ldl_device_updates=False, ldlq_chains=args.chains, group_lanes=args.lanes)
         q.synchronize()
         th = time.time()
         hres = q.run_groups([(lins, n, H, 3 + k) for k in range(kh)], hopt)
@@ -231,7 +231,7 @@ def run_group(args, pkg):
         # arithmetic (fp32 sums, prod cache from bf16 hi/lo split operands on the matrix cores)
         kf = min(args.steps, 3)
         fopt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=1,
-                             ldl_device_updates=not args.host_ldl, ldlq_chains=args.chains)
+                             ldl_device_updates=not args.host_ldl, ldlq_chains=args.chains, group_lanes=args.lanes)
         q.synchronize()
         tf = time.time()
         fres = q.run_groups([(lins, n, H, 3 + k) for k in range(kf)], fopt)
@@ -257,13 +257,16 @@ def run_group(args, pkg):
     nch = args.chains or (3 if int(os.environ.get("GPU_MAX_HW_QUEUES", "4")) >= 6 else 2)
     while nch > 1 and ntr < 768:
         nch -= 1
+    # groups too small to fill the chip run side by side (qtip_opts.group_lanes): that many times as many launches
+    # share the chip
+    lanes = q.group_lanes([(ms, n)] * args.steps, opt)
     gpu_s = stats["rht_s"] + stats["load_s"] + stats["ldlq_s"] + stats["proxy_s"] + stats["pack_s"]
     extra = dict(stats)
     extra.update(gpu_only_Mweights_s=weights_per_step / gpu_s / 1e6,
                  serial_Mweights_s=weights_per_step / (gpu_s + stats["ldl_s"]) / 1e6,
                  viterbi_only_Mweights_s=weights_per_step / stats["viterbi_s"] / 1e6,
                  proxy_in_timed_region=True, ldl_threads=args.ldl_threads, feedback=args.feedback,
-                 hw_queues=int(os.environ.get("GPU_MAX_HW_QUEUES", "4")), ldlq_chains=nch,
+                 hw_queues=int(os.environ.get("GPU_MAX_HW_QUEUES", "4")), ldlq_chains=nch, group_lanes=lanes,
                  ldl_device_updates=not args.host_ldl)
     extra.update(host_only)
     extra.update(host_inputs)
@@ -271,9 +274,9 @@ def run_group(args, pkg):
     names = {2: "config2: 1024x1024 group", 3: "config3: 12288x12288 q-proj group",
              4: "config4: gate+up 2x(28672x12288) group", 5: "config5: 12288x28672 down-proj group"}
     return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
-                vit_launch_weights=ntr * 256 * 8, blocks_per_launch=8, workload=names[cfg] + (" (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)" if args.host_ldl else
+                vit_launch_weights=ntr * 256 * 8 * lanes, blocks_per_launch=8, workload=names[cfg] + (" (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)" if args.host_ldl else
                                        " (RHT + fp64 LDL: host panels, GPU trailing updates + LDLQ + 2-pass Viterbi + pack)"),
-                extra=extra, cpu_group=cpu_group, concurrent=nch)
+                extra=extra, cpu_group=cpu_group, concurrent=nch * lanes)
 
 
 def run_ldl_only(args, pkg):
@@ -324,8 +327,9 @@ def run_ldl_only(args, pkg):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=16)
-    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed groups (default 16; 48 for --config 2, whose groups run twelve at a time)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed groups before them (default 1; 12 for --config 2)")
     ap.add_argument("--config", type=int, default=5, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--ldl-threads", type=int, default=16, help="OpenMP team of the host LDL")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -345,11 +349,15 @@ def main():
     ap.add_argument("--feedback", type=int, default=0, choices=[0, 1],
                     help="0: fp64 LDLQ feedback (default); 1: fp32 feedback + bf16 hi/lo split MFMA prod cache")
     ap.add_argument("--chains", type=int, default=0, choices=[0, 1, 2, 3],
-                    help="independent chains of launches LDLQ deals the tile rows to (0: the library's default, 2)")
-    ap.add_argument("--hw-queues", type=int, default=8,
+                    help="independent chains of launches LDLQ deals the tile rows to (0: the library's default)")
+    ap.add_argument("--lanes", type=int, default=0,
+                    help="groups qtip_run_groups runs side by side (0: the library's rule: as many as fit the chip, 1 "
+                         "for the large configurations; 1: one after the other)")
+    ap.add_argument("--hw-queues", type=int, default=None,
                     help="GPU_MAX_HW_QUEUES for this process (set before the HIP runtime starts; 0: leave the environment "
-                         "alone).  With HIP's default of 4 the library runs two chains of launches per group, with 6 or "
-                         "more three")
+                         "alone; default: 8, and 16 for --config 2).  With HIP's default of 4 the library runs two chains "
+                         "of launches per group, with 6 or more three; small groups run side by side on as many lanes "
+                         "as there are queues")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="first run one plain 1 GiB device copy kernel (known traffic, scales the rocprof byte counters)")
     args = ap.parse_args()
@@ -358,6 +366,12 @@ def main():
               "tile row of a group is independent, so the path would shard by tile rows without any exchange)" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
+    if args.hw_queues is None:
+        args.hw_queues = 16 if args.config == 2 else 8
+    if args.steps is None:
+        args.steps = 48 if args.config == 2 else 16
+    if args.warmup is None:
+        args.warmup = 12 if args.config == 2 else 1
     if args.hw_queues > 0:
         os.environ["GPU_MAX_HW_QUEUES"] = str(min(args.hw_queues, 32))   # read by the HIP runtime when it starts, below
     import torch

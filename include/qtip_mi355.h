@@ -180,6 +180,14 @@ typedef struct { /* QuantOpts, src/quantizer.hpp:11-19 */
                             environment gave the process at least 6 hardware queues (GPU_MAX_HW_QUEUES, read by
                             the HIP runtime when it starts), else 2 - with HIP's default of four queues a third
                             chain would share a queue with another stream and run after it, not beside it */
+  int group_lanes;       /* qtip_run_groups runs this many groups side by side, each on a lane of its own inside ctx
+                            (one stream, workspaces, staging), group g on lane g mod lanes; same results whatever
+                            the number.  At most 12.  1: one group after the other, as the reference schedules them.
+                            0 (default): as many as the largest group's 16-row tile rows fit into the chip's 768
+                            Viterbi workgroup slots (a 1024-row group fills a twelfth of them), 1 for large groups.
+                            Lanes whose streams share a hardware queue run one after the other: small groups gain
+                            most where the process has a queue per lane (GPU_MAX_HW_QUEUES=16 in the environment
+                            when the HIP runtime starts; HIP's default is 4) */
 } qtip_opts;
 void qtip_default_opts(qtip_opts* o);
 
@@ -248,7 +256,11 @@ int qtip_nvfp4_quantize_prepared(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mat
  * quantized as soon as its factor is ready (the LDL of group g+1 overlaps the GPU work of group g).  HRr and L live
  * in page-locked staging buffers owned by the context (a ring of three pairs, 6 n^2 floats, kept between calls).
  * timings / ldl_wait_s (seconds the GPU side waited for each group's factor) may be NULL.  On an error the
- * groups before the failing one are complete. */
+ * groups before the failing one are complete.
+ * Groups too small to fill the chip run side by side (qtip_opts.group_lanes: group g on lane g mod lanes, each lane
+ * takes its groups one after the other on a stream of its own; same results); then an error leaves the groups before the
+ * failing one on its lane complete, the other lanes finish their groups, and the first failing lane's error is
+ * reported. */
 typedef struct {
   int nlin;
   const qtip_linear_in* lins;
@@ -260,6 +272,12 @@ typedef struct {
 } qtip_group;
 int qtip_run_groups(qtip_ctx* ctx, int ngroups, const qtip_group* groups, const qtip_opts* opts, qtip_timing* timings,
                     double* ldl_wait_s);
+/* The number of lanes qtip_run_groups would use for these groups and options (1: one group after the other).  Reads
+ * only nlin, lins[].m and n of each group.  No counterpart in the reference, which runs one group at a time. */
+int qtip_group_lanes(qtip_ctx* ctx, int ngroups, const qtip_group* groups, const qtip_opts* opts, int* lanes);
+/* Host-only check of the lane rule: `ngroups` equal groups of one m x n linear on a device with `device_slots`
+ * Viterbi workgroup slots, qtip_opts.group_lanes = requested. */
+int qtip_selftest_group_lanes(int device_slots, int ngroups, int m, int n, int requested, int* lanes);
 /* Allocates the staging ring of qtip_run_groups for Hessians up to n x n ahead of the first call (optional). */
 int qtip_reserve_groups(qtip_ctx* ctx, int n);
 

@@ -327,6 +327,60 @@ def test_group_config2(qz, oracle, pkg, hyb, synth):
     assert rel1 < 0.01
 
 
+def test_run_groups_lanes_give_the_same_results(qz, pkg, synth):
+    """Small groups run side by side on lanes (qtip_opts.group_lanes): seven groups of four shapes through one lane
+    (the reference's schedule, src/pipeline.cpp:229-312), two, three and the automatic number give the same words,
+    scales and proxy errors; a lane that gets several groups pipelines them; a new tlut reaches the lanes."""
+    say("case: run_groups lanes")
+    qz.set_tlut(None)
+    cases, shapes = [], []
+    for g, (n, ms) in enumerate([(256, (64, 32)), (512, (32,)), (256, (32,)), (1024, (64, 64)), (512, (32, 64)),
+                                 (256, (32,)), (1024, (128,))]):
+        Ws, H = synth.small_group(seed=70 + g, n=n, ms=ms)
+        lins = [pkg.LinearIn("g%d_%d" % (g, k), w.shape[0], w_f32=w) for k, w in enumerate(Ws)]
+        cases.append((lins, n, H, 200 + g))
+        shapes.append((ms, n))
+    assert qz.group_lanes(shapes) == 7            # 8 tile rows at most: all of them side by side
+    assert qz.group_lanes(shapes, pkg.QuantOpts(group_lanes=1)) == 1
+    assert qz.group_lanes(shapes, pkg.QuantOpts(group_lanes=3)) == 3
+    assert qz.group_lanes([((12288,), 28672)] * 4) == 1
+
+    def same(ra, rb):
+        for (oa, ta, _), (ob, _, _) in zip(ra, rb):
+            for a, b in zip(oa, ob):
+                assert a.name == b.name
+                assert np.array_equal(a.trellis, b.trellis) and np.array_equal(a.sv, b.sv)
+                assert np.array_equal(a.su_bf16, b.su_bf16)
+                assert a.wscale == b.wscale and a.proxy == b.proxy and a.proxy_rot_reg == b.proxy_rot_reg
+            assert ta.total > 0 and ta.ldl_cpu > 0
+
+    one = qz.run_groups(cases, pkg.QuantOpts(ldl_threads=8, group_lanes=1))
+    for lanes in (2, 3, 0):
+        say("  lanes %d" % lanes)
+        same(qz.run_groups(cases, pkg.QuantOpts(ldl_threads=8, group_lanes=lanes)), one)
+    same(qz.run_groups(cases, pkg.QuantOpts(ldl_threads=8, group_lanes=3, ldl_device_updates=False)), one)
+    # the lanes keep their device buffers between calls: a second call of the same shape allocates nothing
+    import torch
+    torch.cuda.synchronize()
+    free1 = torch.cuda.mem_get_info()[0]
+    same(qz.run_groups(cases, pkg.QuantOpts(ldl_threads=8, group_lanes=3, ldl_device_updates=False)), one)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] >= free1 - (1 << 20)
+    # a codebook set after the lanes exist
+    rng = np.random.default_rng(9)
+    tl = (rng.standard_normal((512, 2)) * 0.9).astype(np.float32)
+    qz.set_tlut(tl)
+    try:
+        a = qz.run_groups(cases[:4], pkg.QuantOpts(ldl_threads=8, group_lanes=4))
+        b = qz.run_groups(cases[:4], pkg.QuantOpts(ldl_threads=8, group_lanes=1))
+        same(a, b)
+        assert not np.array_equal(a[0][0][0].trellis, one[0][0][0].trellis)
+    finally:
+        qz.set_tlut(None)
+    with pytest.raises(pkg.QtipError):
+        qz.run_groups(cases, pkg.QuantOpts(group_lanes=13))
+
+
 def test_run_groups_equals_group_by_group(qz, oracle, pkg, synth):
     """The overlapped scheduler (run_qtip_groups, src/pipeline.cpp:229-312) returns, for five groups of three
     different widths through its ring of three staging buffers, exactly what quantize_group returns one at a time;

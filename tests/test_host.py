@@ -119,6 +119,40 @@ def test_ldl_panel_handover_on_host(pkg, n, threads):
     assert pkg.lib().qtip_selftest_ldl_panel_handover(bad.ctypes.data, n, threads, L2.ctypes.data) != 0
 
 
+def test_group_lane_rule(pkg):
+    """qtip_run_groups' lane rule on a chip with 768 Viterbi workgroup slots: groups that fill the chip run one at a
+    time, small groups share it, bounded by the slots, the lanes' staging memory, the number of groups and the
+    library's maximum; an explicit request is honoured up to the number of groups and refused beyond the maximum."""
+    import ctypes as C
+    L = pkg.lib()
+
+    def lanes(ng, m, n, req=0, slots=768):
+        out = C.c_int(-1)
+        rc = L.qtip_selftest_group_lanes(slots, ng, m, n, req, C.byref(out))
+        return rc, out.value
+
+    assert lanes(16, 12288, 28672) == (0, 1)        # 768 tile rows: the chip is full
+    assert lanes(16, 12288, 12288) == (0, 1)
+    assert lanes(16, 6144, 4096) == (0, 2)          # 384 tile rows: two side by side
+    assert lanes(16, 4096, 4096) == (0, 3)
+    assert lanes(16, 1024, 1024) == (0, 12)         # 64 tile rows: 12 fit, which is also the maximum
+    assert lanes(16, 256, 1024) == (0, 12)
+    assert lanes(5, 1024, 1024) == (0, 5)           # no more lanes than groups
+    assert lanes(1, 1024, 1024) == (0, 1)
+    assert lanes(0, 1024, 1024) == (0, 1)
+    assert lanes(16, 1024, 8192) == (0, 8)          # 4 n^2 floats of staging and work matrices per lane, 8 GiB in all
+    assert lanes(16, 1024, 12288) == (0, 3)
+    assert lanes(16, 1024, 28672) == (0, 1)
+    assert lanes(16, 1024, 1024, req=1) == (0, 1)   # the reference's schedule on request
+    assert lanes(16, 12288, 28672, req=3) == (0, 3)
+    assert lanes(2, 1024, 1024, req=8) == (0, 2)
+    assert lanes(16, 1024, 1024, slots=304) == (0, 4)
+    rc, _ = lanes(16, 1024, 1024, req=13)
+    assert rc != 0 and b"lanes" in L.qtip_last_error()
+    rc, _ = lanes(16, 1024, 1024, req=-1)
+    assert rc != 0
+
+
 def test_cholesky_inplace_fp64_bits(pkg, oracle):
     """qtip_cholesky_inplace: every bit of the fp64 factor equals the compiled reference's committed rows (n = 528) and
     the oracle's factor of a matrix with correlated, badly scaled channels (n = 784)."""
