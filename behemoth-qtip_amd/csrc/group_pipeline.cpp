@@ -189,9 +189,9 @@ long tile_rows_of(const qtip_group& g) {
 // src/pipeline.cpp:229-312) leaves most of the chip idle when the groups are small.  Groups do not depend on each
 // other, so such groups run side by side, each lane with streams, workspaces and a ring of its own and the
 // groups one after the other on its one stream.  Every group is computed by the same code on the same inputs: same
-// results whatever the number of lanes.  Automatic: as many lanes as the largest group's tile rows fit into the
-// chip's slots, while the lanes' staging (2 n^2 floats each, on the host and on the device) and fp64 work matrices
-// (2 n^2 floats more) stay under 8 GiB.  Lanes whose streams share a hardware queue (a process has
+// results whatever the number of lanes.  Automatic: as many lanes as it takes for the largest group's tile rows to
+// fill the chip's slots, while the lanes' staging (2 n^2 floats each, on the host and on the device) and fp64 work
+// matrices (2 n^2 floats more) stay under 32 GiB.  Lanes whose streams share a hardware queue (a process has
 // GPU_MAX_HW_QUEUES of them, 4 unless the environment says more) run one after the other; measured on 1024 x 1024
 // groups, 12 lanes were still the fastest choice with 4 queues (54 Mweights/s against 26 for one lane), with 8 (92)
 // and with 16 (134), so the rule does not look at the queues.
@@ -205,8 +205,10 @@ int group_lanes_for(int ng, const qtip_group* groups, const qtip_opts& opt, int 
     rows = std::max(rows, tile_rows_of(groups[g]));
     nmax = std::max<long>(nmax, groups[g].n);
   }
-  const long by_slots = device_slots / rows;
-  const long by_memory = (8L << 30) / (16 * nmax * nmax);
+  // rounded up: the workgroups beyond the chip's slots wait at the dispatcher and fill the slots the first lane's
+  // finished workgroups leave (8192 x 4096 groups, 512 tile rows: 132 Mweights/s on one lane, 150 on two)
+  const long by_slots = rows >= device_slots ? 1 : (device_slots + rows - 1) / rows;
+  const long by_memory = (32L << 30) / (16 * nmax * nmax);
   const long lanes = std::min<long>({by_slots, by_memory, long(qtip_ctx::kMaxLanes), long(ng)});
   return lanes < 2 ? 1 : int(lanes);
 }

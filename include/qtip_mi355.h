@@ -183,8 +183,9 @@ typedef struct { /* QuantOpts, src/quantizer.hpp:11-19 */
   int group_lanes;       /* qtip_run_groups runs this many groups side by side, each on a lane of its own inside ctx
                             (one stream, workspaces, staging), group g on lane g mod lanes; same results whatever
                             the number.  At most 12.  1: one group after the other, as the reference schedules them.
-                            0 (default): as many as the largest group's 16-row tile rows fit into the chip's 768
-                            Viterbi workgroup slots (a 1024-row group fills a twelfth of them), 1 for large groups.
+                            0 (default): as many as it takes for the largest group's 16-row tile rows to fill the
+                            chip's 768 Viterbi workgroup slots (a 1024-row group fills a twelfth of them), 1 for
+                            groups of 12288 rows and more.
                             Lanes whose streams share a hardware queue run one after the other: small groups gain
                             most where the process has a queue per lane (GPU_MAX_HW_QUEUES=16 in the environment
                             when the HIP runtime starts; HIP's default is 4) */

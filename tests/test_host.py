@@ -133,20 +133,23 @@ def test_group_lane_rule(pkg):
 
     assert lanes(16, 12288, 28672) == (0, 1)        # 768 tile rows: the chip is full
     assert lanes(16, 12288, 12288) == (0, 1)
-    assert lanes(16, 6144, 4096) == (0, 2)          # 384 tile rows: two side by side
+    assert lanes(16, 57344, 12288) == (0, 1)
+    assert lanes(16, 8192, 4096) == (0, 2)          # 512 tile rows: a second lane fills the slots the first leaves
+    assert lanes(16, 6144, 4096) == (0, 2)
     assert lanes(16, 4096, 4096) == (0, 3)
-    assert lanes(16, 1024, 1024) == (0, 12)         # 64 tile rows: 12 fit, which is also the maximum
+    assert lanes(16, 1024, 1024) == (0, 12)         # 64 tile rows: 12 fill the chip, which is also the maximum
     assert lanes(16, 256, 1024) == (0, 12)
     assert lanes(5, 1024, 1024) == (0, 5)           # no more lanes than groups
     assert lanes(1, 1024, 1024) == (0, 1)
     assert lanes(0, 1024, 1024) == (0, 1)
-    assert lanes(16, 1024, 8192) == (0, 8)          # 4 n^2 floats of staging and work matrices per lane, 8 GiB in all
-    assert lanes(16, 1024, 12288) == (0, 3)
-    assert lanes(16, 1024, 28672) == (0, 1)
+    assert lanes(16, 1024, 16384) == (0, 8)         # 4 n^2 floats of staging and work matrices per lane, 32 GiB in all
+    assert lanes(16, 8192, 28672) == (0, 2)
+    assert lanes(16, 1024, 28672) == (0, 2)
+    assert lanes(16, 1024, 40960) == (0, 1)
     assert lanes(16, 1024, 1024, req=1) == (0, 1)   # the reference's schedule on request
     assert lanes(16, 12288, 28672, req=3) == (0, 3)
     assert lanes(2, 1024, 1024, req=8) == (0, 2)
-    assert lanes(16, 1024, 1024, slots=304) == (0, 4)
+    assert lanes(16, 1024, 1024, slots=304) == (0, 5)
     rc, _ = lanes(16, 1024, 1024, req=13)
     assert rc != 0 and b"lanes" in L.qtip_last_error()
     rc, _ = lanes(16, 1024, 1024, req=-1)
