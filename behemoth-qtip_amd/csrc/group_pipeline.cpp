@@ -258,19 +258,31 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
     l.wait.resize(l.groups.size());
     order_streams(c->stream, l.c->stream);  // inputs the caller ordered before the context's stream
   }
+  auto run_lane = [&](int k) {
+    Lane& l = L[size_t(k)];
+    try {
+      QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
+      // the lane's per-group buffers come from its own arena: a hipFree would wait for every other lane's work
+      ArenaScope lane_memory(&l.c->arena);
+      run_groups_in_line(l.c, int(l.groups.size()), l.groups.data(), lopt, l.tms.data(), l.wait.data());
+    } catch (...) {
+      l.err = std::current_exception();
+    }
+  };
   std::vector<std::thread> th;
-  for (int k = 0; k < lanes; ++k)
-    th.emplace_back([&, k] {
-      Lane& l = L[size_t(k)];
-      try {
-        QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
-        // the lane's per-group buffers come from its own arena: a hipFree would wait for every other lane's work
-        ArenaScope lane_memory(&l.c->arena);
-        run_groups_in_line(l.c, int(l.groups.size()), l.groups.data(), lopt, l.tms.data(), l.wait.data());
-      } catch (...) {
-        l.err = std::current_exception();
-      }
-    });
+  for (int k = 1; k < lanes; ++k) {
+    try {
+      th.emplace_back(run_lane, k);
+    } catch (...) {  // no thread to be had: the lane's groups run on this one, after lane 0's
+      L[size_t(k)].index.push_back(-1);
+    }
+  }
+  run_lane(0);  // the calling thread takes the first lane
+  for (int k = 1; k < lanes; ++k)
+    if (!L[size_t(k)].index.empty() && L[size_t(k)].index.back() == -1) {
+      L[size_t(k)].index.pop_back();
+      run_lane(k);
+    }
   for (std::thread& t : th) t.join();
   for (Lane& l : L) {
     order_streams(l.c->stream, c->stream);

@@ -379,6 +379,14 @@ def test_run_groups_lanes_give_the_same_results(qz, pkg, synth):
         qz.set_tlut(None)
     with pytest.raises(pkg.QtipError):
         qz.run_groups(cases, pkg.QuantOpts(group_lanes=13))
+    # groups of 384 tile rows: two lanes of one LDLQ chain each against one lane that deals the rows to two chains
+    say("  lanes, 6144 x 512 groups")
+    big = []
+    for g in range(3):
+        Ws, H = synth.small_group(seed=90 + g, n=512, ms=(4096, 2048))
+        big.append(([pkg.LinearIn("b%d_%d" % (g, k), w.shape[0], w_f32=w) for k, w in enumerate(Ws)], 512, H, 300 + g))
+    assert qz.group_lanes([((4096, 2048), 512)] * 3) == 2
+    same(qz.run_groups(big, pkg.QuantOpts(ldl_threads=8)), qz.run_groups(big, pkg.QuantOpts(ldl_threads=8, group_lanes=1)))
 
 
 def test_run_groups_equals_group_by_group(qz, oracle, pkg, synth):
