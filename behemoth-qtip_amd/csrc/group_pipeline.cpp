@@ -187,8 +187,8 @@ long tile_rows_of(const qtip_group& g) {
 // Lanes.  A group keeps as many Viterbi workgroups busy as it has 16-row tile rows, and the chip holds
 // `device_slots` of them (three per compute unit); the reference's schedule (one group at a time,
 // src/pipeline.cpp:229-312) leaves most of the chip idle when the groups are small.  Groups do not depend on each
-// other, so such groups run side by side, each lane with streams, workspaces and a ring of its own and the
-// groups one after the other on its one stream.  Every group is computed by the same code on the same inputs: same
+// other, so such groups run side by side on lanes: a lane has a context of its own (one stream, workspaces, staging)
+// and takes its groups one after the other.  Every group is computed by the same code on the same inputs: same
 // results whatever the number of lanes.  Automatic: as many lanes as it takes for the largest group's tile rows to
 // fill the chip's slots, while the lanes' staging (2 n^2 floats each, on the host and on the device) and fp64 work
 // matrices (2 n^2 floats more) stay under 32 GiB.  Lanes whose streams share a hardware queue (a process has
@@ -238,6 +238,7 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
     std::vector<qtip_timing> tms;
     std::vector<double> wait;
     std::exception_ptr err;
+    bool deferred = false;  // no thread could be started for it: its groups run on the calling thread after lane 0's
   };
   std::vector<Lane> L(static_cast<size_t>(lanes));
   qtip_opts lopt = opt;
@@ -273,16 +274,13 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
   for (int k = 1; k < lanes; ++k) {
     try {
       th.emplace_back(run_lane, k);
-    } catch (...) {  // no thread to be had: the lane's groups run on this one, after lane 0's
-      L[size_t(k)].index.push_back(-1);
+    } catch (...) {
+      L[size_t(k)].deferred = true;
     }
   }
   run_lane(0);  // the calling thread takes the first lane
   for (int k = 1; k < lanes; ++k)
-    if (!L[size_t(k)].index.empty() && L[size_t(k)].index.back() == -1) {
-      L[size_t(k)].index.pop_back();
-      run_lane(k);
-    }
+    if (L[size_t(k)].deferred) run_lane(k);
   for (std::thread& t : th) t.join();
   for (Lane& l : L) {
     order_streams(l.c->stream, c->stream);
