@@ -220,6 +220,33 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
   for (int g = 0; g < ng; ++g)
     QTIP_REQUIRE(groups[g].n > 0 && groups[g].H && groups[g].nlin > 0 && groups[g].lins && groups[g].outs,
                  "run_groups: group %d is incomplete", g);
+  // Mixed sizes (a layer's gate/up group beside its o-proj group): the groups that fill the chip on their own go
+  // through the overlapped schedule first, in their order, the others then share the chip on lanes.
+  if (opt.group_lanes == 0 && ng >= 3) {
+    const long slots = viterbi_max_slots(c->device);
+    std::vector<int> large, small;
+    for (int g = 0; g < ng; ++g) (tile_rows_of(groups[g]) >= slots ? large : small).push_back(g);
+    if (!large.empty() && small.size() >= 2) {
+      for (const std::vector<int>* part : {&large, &small}) {
+        std::vector<qtip_group> sub;
+        for (int g : *part) sub.push_back(groups[g]);
+        std::vector<qtip_timing> st(sub.size());
+        std::vector<double> sw(sub.size(), 0.0);
+        std::exception_ptr err;
+        try {
+          run_groups_impl(c, int(sub.size()), sub.data(), opt, st.data(), sw.data());
+        } catch (...) {
+          err = std::current_exception();
+        }
+        for (size_t i = 0; i < part->size(); ++i) {
+          if (tms) tms[(*part)[i]] = st[i];
+          if (ldl_wait) ldl_wait[(*part)[i]] = sw[i];
+        }
+        if (err) std::rethrow_exception(err);
+      }
+      return;
+    }
+  }
   const int lanes = group_lanes_for(ng, groups, opt, viterbi_max_slots(c->device));
   if (lanes == 1) {
     // the per-group device buffers of the quantizing thread come from the context's arena and stay there between

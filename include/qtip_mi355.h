@@ -261,7 +261,8 @@ int qtip_nvfp4_quantize_prepared(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mat
  * Groups too small to fill the chip run side by side (qtip_opts.group_lanes: group g on lane g mod lanes, each lane
  * takes its groups one after the other on a stream of its own; same results); then an error leaves the groups before the
  * failing one on its lane complete, the other lanes finish their groups, and the first failing lane's error is
- * reported. */
+ * reported.  With group_lanes = 0 and groups of mixed sizes, the groups of 12288 rows and more run first, in their
+ * order, one after the other, and the smaller ones then share the chip on lanes. */
 typedef struct {
   int nlin;
   const qtip_linear_in* lins;

@@ -379,6 +379,12 @@ def test_run_groups_lanes_give_the_same_results(qz, pkg, synth):
         qz.set_tlut(None)
     with pytest.raises(pkg.QtipError):
         qz.run_groups(cases, pkg.QuantOpts(group_lanes=13))
+    # mixed sizes: a group that fills the chip runs through the overlapped schedule, the small ones on lanes
+    say("  lanes, mixed sizes")
+    Ws, H = synth.small_group(seed=99, n=256, ms=(8192, 4096))
+    wide = ([pkg.LinearIn("wide%d" % k, w.shape[0], w_f32=w) for k, w in enumerate(Ws)], 256, H, 400)
+    mixed = [cases[0], wide, cases[2], cases[5]]
+    same(qz.run_groups(mixed, pkg.QuantOpts(ldl_threads=8)), qz.run_groups(mixed, pkg.QuantOpts(ldl_threads=8, group_lanes=1)))
     # groups of 384 tile rows: two lanes of one LDLQ chain each against one lane that deals the rows to two chains
     say("  lanes, 6144 x 512 groups")
     big = []
