@@ -48,13 +48,12 @@ struct DeviceArena::Impl {
   std::mutex mu;
   std::vector<Block> blocks;
 };
+DeviceArena::DeviceArena() : impl(new Impl()) {}
 DeviceArena::~DeviceArena() {
-  if (!impl) return;
   for (auto& b : impl->blocks) (void)hipFree(b.p);
   delete impl;
 }
 hipError_t DeviceArena::acquire(void** p, size_t bytes) {
-  if (!impl) impl = new Impl();
   {
     std::lock_guard<std::mutex> lk(impl->mu);
     Impl::Block* fit = nullptr;

@@ -51,7 +51,7 @@ long test_device_alloc_calls();
 // them back on release, after waiting for the arena's own streams only - the streams the lane's kernels run on.
 // The blocks are freed with the arena.
 struct DeviceArena {
-  DeviceArena() = default;
+  DeviceArena();
   DeviceArena(const DeviceArena&) = delete;
   DeviceArena& operator=(const DeviceArena&) = delete;
   ~DeviceArena();
@@ -59,7 +59,7 @@ struct DeviceArena {
   void give_back(void* p);
   std::vector<hipStream_t*> streams;  // slots holding the streams whose work may use the blocks (null slots are skipped)
   struct Impl;
-  Impl* impl = nullptr;
+  Impl* impl;
 };
 DeviceArena* current_arena();
 struct ArenaScope {  // makes `a` the calling thread's arena until the scope ends
