@@ -14,7 +14,7 @@
 // in opposite order.  A lane therefore owns 8 groups of one metric column c (one for each value m of the low
 // three bits, so that the stride 2m+1 is a compile-time constant) and their mirrors in column 255-c: per step it
 // keeps the two metric columns (2 x 16 fp64) in registers and streams 8 rows of E (16 fp64 each) from LDS, i.e.
-// 160 LDS reads for 256 add-compare-selects.
+// 128 + 16 LDS reads for 256 add-compare-selects.
 //
 // LDS layout: free of bank conflicts.  An 8-byte LDS access is served 16 lanes at a time, and a 16-lane quarter
 // takes as many cycles as the largest number of distinct addresses that fall on one of the 16 bank pairs.
@@ -25,10 +25,15 @@
 //     so the bank pair of a read is row mod 16 = those bits, whatever the rotation b4; the 16 positions are stored
 //     twice (q = 0..31) so that the rotation is a per-lane base address and the stride d*(2m+1) mod 16 a
 //     compile-time offset.
-//   * The metric of (column c, digit d) sits at c*16 + (pi(d) ^ ((c >> 2) & 15) ^ (c >> 6)) with
-//     pi(d) = 4 (d & 3) + (d >> 2): the 16 lanes of a quarter read 16 different bank pairs for every d, write 16
-//     different ones for every slot, a read address is one XOR of a per-lane base with a constant, and the mirror
-//     group's slot is the group's XOR 0xff3.
+//   * The metric of (column c, digit d) sits at pos(c)*16 + (d ^ swz(c)): pos(c) is c with bits 0 and 2 exchanged and
+//     swz(c) = 2 ((c >> 3 & 7) ^ 2 (c >> 6)) is even, so the digits 2k and 2k+1 of a column are one 16-byte piece, in
+//     that order for every lane: a column comes in as eight 16-byte reads whose addresses are one XOR of a per-lane
+//     base with 16k.  A 16-byte LDS access is served 16 lanes at a time as well, but in the turns {0-3, 12-15, 20-27}
+//     and {4-11, 16-19, 28-31} of each half-wave, at full rate when the 16 lanes of a turn touch 16 different 16-byte
+//     bank groups: bits 4..6 of the address are (k ^ u >> 1) and bit 7 is u & 1 here, a different value for each of
+//     the 16 values u of a turn.  The 16 lanes of a quarter write 16 different bank pairs for every slot (their
+//     digits differ in the low two bits, their target columns in bits 6 and 7, which swz moves to slot bits 2 and 3),
+//     and the mirror group's slot is the group's XOR 0xffd.
 // LDS per workgroup ~50 KB, three workgroups per CU; metrics single-buffered (the columns are read into registers
 // before the step's results are written).
 // No back-pointers.  A step's 16-way search keeps the minimum only (add + min per candidate); which digit won
@@ -62,9 +67,11 @@ constexpr int kMaxDevices = 64;
 double* g_scratch_ptr[kMaxDevices] = {};
 std::mutex g_scratch_mutex;
 
-__device__ __forceinline__ constexpr int pi16(int d) { return 4 * (d & 3) + (d >> 2); }
-__device__ __forceinline__ int m_swz(int col) { return ((col >> 2) & 15) ^ (col >> 6); }
-__device__ __forceinline__ int m_slot(int col, int d) { return col * 16 + (pi16(d) ^ m_swz(col)); }
+// metric array: column `col` lives at position m_pos(col) (bits 0 and 2 of the column exchanged), digit d in slot
+// d ^ m_swz(col) of its 16; m_swz is even, so the digits 2k and 2k + 1 are the halves of one 16-byte piece
+__device__ __forceinline__ int m_pos(int col) { return (col & ~5) | ((col & 1) << 2) | ((col >> 2) & 1); }
+__device__ __forceinline__ int m_swz(int col) { return (((col >> 3) & 7) ^ (((col >> 6) & 3) << 1)) << 1; }
+__device__ __forceinline__ int m_slot(int col, int d) { return m_pos(col) * 16 + (d ^ m_swz(col)); }
 
 struct Smem {
   double E[kESlots];  // first: its reads use 8-bit immediate offsets from a per-lane base
@@ -115,15 +122,15 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
 
   // per slot: E base (b4 * 64 + row) and the metric slot written for the group; the mirror group's is that ^ kMirror
   int ebase[8], wslot[8];
-  constexpr int kMirror = 0xff3;
+  constexpr int kMirror = 0xffd;
 #pragma unroll
   for (int m = 0; m < 8; ++m) {
     const uint32_t j = 16u * colA + 8u * uint32_t(half) + m, p = j * (j + 1u);
     ebase[m] = int((p >> 12) & 15u) * 64 + int((p >> 6) & 63u);
     wslot[m] = m_slot(int(j & 255u), int(j >> 8));
   }
-  // byte offsets of digit pi^-1(0) of the two metric columns; the other digits are XORs with 8 pi(d)
-  int xA = colA * 128 + m_swz(colA) * 8, xB = colB * 128 + m_swz(colB) * 8;
+  // byte offsets of digit 0 of the two metric columns; the pair of digits (2k, 2k + 1) is at that ^ 16 k
+  int xA = m_pos(colA) * 128 + m_swz(colA) * 8, xB = m_pos(colB) * 128 + m_swz(colB) * 8;
   const char* const Mb = reinterpret_cast<const char*>(sm.M);
 
   // initial metrics: M_0[g] = 0, or +inf outside group ov
@@ -142,13 +149,15 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
     if constexpr (kind == kStore) hs = hist + size_t(it >> 1) * kGroups + tid;
     // ---- phase R: metric columns -> registers, error table of this step -> LDS
     double MA[16], MB[16];
-    // the 32 read addresses are recomputed in every step (one XOR each): kept across the loop they would take 32
-    // registers the accumulators need
+    // 16-byte reads, two digits each; the 16 read addresses are recomputed in every step (one XOR each): kept
+    // across the loop they would take 16 registers the accumulators need
     asm volatile("" : "+v"(xA), "+v"(xB));
 #pragma unroll
-    for (int d = 0; d < 16; ++d) {
-      MA[d] = *reinterpret_cast<const double*>(Mb + (xA ^ (8 * pi16(d))));
-      MB[d] = *reinterpret_cast<const double*>(Mb + (xB ^ (8 * pi16(d))));
+    for (int k = 0; k < 8; ++k) {
+      const double2 a = *reinterpret_cast<const double2*>(Mb + (xA ^ (16 * k)));
+      const double2 b = *reinterpret_cast<const double2*>(Mb + (xB ^ (16 * k)));
+      MA[2 * k] = a.x, MA[2 * k + 1] = a.y;
+      MB[2 * k] = b.x, MB[2 * k + 1] = b.y;
     }
     {
       const int t = (2 * it + roll) & 255;
