@@ -39,6 +39,9 @@ struct QuantOpts {  // src/quantizer.hpp:11-19
   // not in the reference: the group calls hand the trailing updates of the host LDL to the GPU (the factor is the
   // host's bit for bit); false keeps the factorization on the host alone
   bool ldl_device_updates = true;
+  // not in the reference: run_groups runs groups that cannot fill the chip side by side (0: as many as fit, 1: one at
+  // a time, as the reference schedules them); the outputs do not depend on it
+  int group_lanes = 0;
 };
 
 struct LinearIn {  // src/quantizer.hpp:21-28
@@ -286,6 +289,7 @@ inline std::vector<std::vector<LinearOut>> run_groups(const std::vector<GroupSpe
   qtip_default_opts(&co);
   co.sigma_reg = opt.sigma_reg, co.scale_override = opt.scale_override, co.ldl_threads = opt.ldl_threads;
   co.ldl_device_updates = opt.ldl_device_updates ? 1 : 0;
+  co.group_lanes = opt.group_lanes;
   std::vector<qtip_timing> ct(ng);
   std::vector<double> waits(ng, 0.0);
   detail::check(qtip_run_groups(detail::context(), int(ng), cg.data(), &co, ct.data(), waits.data()), "run_groups");
