@@ -338,6 +338,9 @@ def test_run_groups_lanes_give_the_same_results(qz, pkg, synth):
                                  (256, (32,)), (1024, (128,))]):
         Ws, H = synth.small_group(seed=70 + g, n=n, ms=ms)
         lins = [pkg.LinearIn("g%d_%d" % (g, k), w.shape[0], w_f32=w) for k, w in enumerate(Ws)]
+        if g == 2:   # one group with bf16 weights, one with feedback through the other arithmetic below
+            wb = (Ws[0].view(np.uint32) >> 16).astype(np.uint16)
+            lins = [pkg.LinearIn("g2_0", Ws[0].shape[0], w_bf16=wb)]
         cases.append((lins, n, H, 200 + g))
         shapes.append((ms, n))
     assert qz.group_lanes(shapes) == 7            # 8 tile rows at most: all of them side by side
@@ -359,6 +362,8 @@ def test_run_groups_lanes_give_the_same_results(qz, pkg, synth):
         say("  lanes %d" % lanes)
         same(qz.run_groups(cases, pkg.QuantOpts(ldl_threads=8, group_lanes=lanes)), one)
     same(qz.run_groups(cases, pkg.QuantOpts(ldl_threads=8, group_lanes=3, ldl_device_updates=False)), one)
+    same(qz.run_groups(cases, pkg.QuantOpts(ldl_threads=8, group_lanes=4, feedback=1)),
+         qz.run_groups(cases, pkg.QuantOpts(ldl_threads=8, group_lanes=1, feedback=1)))
     # the lanes keep their device buffers between calls: a second call of the same shape allocates nothing
     import torch
     torch.cuda.synchronize()
