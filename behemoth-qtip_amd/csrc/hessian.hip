@@ -10,12 +10,11 @@
 //
 // One 256-thread workgroup per tile, one workgroup per CU: a wave owns 128 x 128 outputs (4 x 4 MFMA tiles, 256
 // accumulator registers).  Both operands are column slices of X and the contraction runs over the rows of X, so the
-// matrix cores want, per lane, 8 consecutive rows of one column, while memory has the columns contiguous: every
-// thread loads an 8 row x 8 column block (eight 16-byte loads, whole 128-byte lines per wave), transposes it in
-// registers (v_perm_b32) and writes eight 16-byte column pieces to LDS ([column][row], 128-byte pitch with the pieces
-// XOR-swizzled: conflict-free for the writes and for the lanes' 16-byte fragment reads).  Two LDS stages of 64 rows: the next stage is fetched
-// and written while the matrix cores work on the current one.  Workgroups are numbered so that the 32 that share an
-// XCD (and its L2) at a time form an 8 x 4 patch of tiles, which needs 12 operand slices instead of 33.
+// matrix cores want, per lane, 8 consecutive rows of one column, while memory has the columns contiguous.  The batch
+// is therefore first rewritten (batch_image_kernel, one pass over it) as the LDS images of the update kernel's stages,
+// and the update kernel (syrk_img_kernel, which the proxy's quadratic forms use as well) moves them from global memory
+// straight into LDS.  Workgroups are numbered so that the 32 that share an XCD (and its L2) at a time form an 8 x 4
+// patch of tiles, which needs 12 operand slices instead of 33.
 #include <mutex>
 #include <vector>
 
@@ -29,259 +28,10 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kTile = 256;    // output tile edge
-constexpr int kStage = 64;    // rows of X per LDS stage
-constexpr int kPitch = 64;    // u16 per LDS row: the 64 rows of X of one stage (128 bytes), 16-byte pieces XOR-swizzled
-constexpr int kSliceU16 = kTile * kPitch;                 // one operand slice in LDS
-constexpr size_t kLdsBytes = size_t(4) * kSliceU16 * 2;   // 2 stages x (A, B)
 constexpr int kPatchRows = 8, kPatchCols = 4;             // tiles per XCD patch
 
-struct Block8x8 {
-  uint4 r[8];  // r[q]: 8 consecutive columns of row q
-};
-
-// Rows beyond `rows` read as zero (they would add to every output); columns beyond n only feed outputs that are
-// never stored, so their address is clamped instead.  FULL: the caller knows that all 8 rows exist.
-template <bool FULL>
-__device__ __forceinline__ void fetch_block(Block8x8& b, const uint16_t* __restrict__ X, long rows, long n, long row0,
-                                            long col0) {
-  const long c = col0 + 7 < n ? col0 : 0;
-#pragma unroll
-  for (int q = 0; q < 8; ++q) {
-    if (FULL) {
-      b.r[q] = *reinterpret_cast<const uint4*>(X + (row0 + q) * n + c);
-    } else {
-      const bool ok = row0 + q < rows;
-      const uint4 v = *reinterpret_cast<const uint4*>(X + (ok ? row0 + q : 0) * n + c);
-      b.r[q] = ok ? v : uint4{0u, 0u, 0u, 0u};
-    }
-  }
-}
-
-// LDS layout of an operand slice: column `col` of X occupies 128 bytes; its 16-byte piece holding rows 8 p .. 8 p + 7 of
-// the stage sits at piece position p ^ (col & 7) ^ ((col >> 3) & 7).  The writers of one instruction are 8 lanes with
-// the same column offset in 8 neighbouring column groups, the readers 8 lanes on 8 neighbouring columns: both then
-// touch 8 different 16-byte bank groups.
-//
-// column c of the block as 8 consecutive rows (4 dwords), written to piece (sw ^ c) of row c of dst; sw = p ^ (group & 7)
-template <int D>
-__device__ __forceinline__ void store_chunk_transposed(const Block8x8& b, uint16_t* dst, int sw) {
-  const uint32_t w[8] = {D == 0 ? b.r[0].x : D == 1 ? b.r[0].y : D == 2 ? b.r[0].z : b.r[0].w,
-                         D == 0 ? b.r[1].x : D == 1 ? b.r[1].y : D == 2 ? b.r[1].z : b.r[1].w,
-                         D == 0 ? b.r[2].x : D == 1 ? b.r[2].y : D == 2 ? b.r[2].z : b.r[2].w,
-                         D == 0 ? b.r[3].x : D == 1 ? b.r[3].y : D == 2 ? b.r[3].z : b.r[3].w,
-                         D == 0 ? b.r[4].x : D == 1 ? b.r[4].y : D == 2 ? b.r[4].z : b.r[4].w,
-                         D == 0 ? b.r[5].x : D == 1 ? b.r[5].y : D == 2 ? b.r[5].z : b.r[5].w,
-                         D == 0 ? b.r[6].x : D == 1 ? b.r[6].y : D == 2 ? b.r[6].z : b.r[6].w,
-                         D == 0 ? b.r[7].x : D == 1 ? b.r[7].y : D == 2 ? b.r[7].z : b.r[7].w};
-  uint4 even, odd;  // columns 2 D and 2 D + 1: (row 0, row 1), (2, 3), (4, 5), (6, 7)
-  even.x = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u);
-  even.y = __builtin_amdgcn_perm(w[3], w[2], 0x05040100u);
-  even.z = __builtin_amdgcn_perm(w[5], w[4], 0x05040100u);
-  even.w = __builtin_amdgcn_perm(w[7], w[6], 0x05040100u);
-  odd.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
-  odd.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
-  odd.z = __builtin_amdgcn_perm(w[5], w[4], 0x07060302u);
-  odd.w = __builtin_amdgcn_perm(w[7], w[6], 0x07060302u);
-  *reinterpret_cast<uint4*>(dst + (2 * D) * kPitch + ((sw ^ (2 * D)) << 3)) = even;
-  *reinterpret_cast<uint4*>(dst + (2 * D + 1) * kPitch + ((sw ^ (2 * D + 1)) << 3)) = odd;
-}
-__device__ __forceinline__ void store_block_transposed(const Block8x8& b, uint16_t* dst, int sw) {
-  store_chunk_transposed<0>(b, dst, sw);
-  store_chunk_transposed<1>(b, dst, sw);
-  store_chunk_transposed<2>(b, dst, sw);
-  store_chunk_transposed<3>(b, dst, sw);
-}
-
-// One 64-row stage of a workgroup: 64 MFMAs per wave on the LDS buffers As / Bs while (FETCH != 0) the next stage
-// travels global memory -> registers -> transpose -> the other LDS buffer.  FETCH: 0 nothing follows, 1 the next
-// stage is complete, 2 it is the ragged last one.  The function is one basic block; the group barriers at its end
-// give the order the instruction scheduler is asked for: loads first, then fragment reads of k-slice ks + 1 between
-// the MFMAs of slice ks, and the transposes and LDS writes of the next stage between the MFMAs of the last slice.
-template <bool DIAG, int FETCH>
-__device__ __forceinline__ void syrk_stage(floatx16 (&acc)[4][4], const uint16_t* As, const uint16_t* Bs, uint16_t* nxt,
-                                           Block8x8& ga, Block8x8& gb, const uint16_t* __restrict__ X,
-                                           const uint16_t* __restrict__ XB, long rows, long n, long r0, long ci, long cj,
-                                           int offA, int offB, int swr, int sww) {
-  if (FETCH) {
-    fetch_block<FETCH == 1>(ga, X, rows, n, r0, ci);
-    if (!DIAG) fetch_block<FETCH == 1>(gb, XB, rows, n, r0, cj);
-  }
-  bf16x8 fa[2][4], fb[2][4];
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi) {
-    const int piece = (swr ^ (4 * (mi & 1))) << 3;
-    fa[0][mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + offA + mi * 32 * kPitch + piece));
-    fb[0][mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Bs + offB + mi * 32 * kPitch + piece));
-  }
-  __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-  for (int ks = 0; ks < kStage / 16; ++ks) {
-    if (ks + 1 < kStage / 16) {
-      // the fragments of the next k-slice are requested before the 16 MFMAs of this one are queued
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        const int piece = (swr ^ (2 * (ks + 1)) ^ (4 * (mi & 1))) << 3;
-        fa[(ks + 1) & 1][mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + offA + mi * 32 * kPitch + piece));
-        fb[(ks + 1) & 1][mi] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(Bs + offB + mi * 32 * kPitch + piece));
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni) {
-        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][mi], fb[ks & 1][ni], acc[mi][ni], 0, 0, 0);
-        if (FETCH && ks == kStage / 16 - 1) {
-          // last k-slice: the next stage's blocks are transposed and written to the other LDS buffer in the shadow of
-          // the matrix instructions, one quarter block (8 permutes, 2 writes) after every second (fourth) MFMA
-          const int i = mi * 4 + ni;
-          if (!DIAG) {
-            if (i == 0) store_chunk_transposed<0>(ga, nxt, sww);
-            if (i == 2) store_chunk_transposed<1>(ga, nxt, sww);
-            if (i == 4) store_chunk_transposed<2>(ga, nxt, sww);
-            if (i == 6) store_chunk_transposed<3>(ga, nxt, sww);
-            if (i == 8) store_chunk_transposed<0>(gb, nxt + kSliceU16, sww);
-            if (i == 10) store_chunk_transposed<1>(gb, nxt + kSliceU16, sww);
-            if (i == 12) store_chunk_transposed<2>(gb, nxt + kSliceU16, sww);
-            if (i == 14) store_chunk_transposed<3>(gb, nxt + kSliceU16, sww);
-          } else {
-            if (i == 0) store_chunk_transposed<0>(ga, nxt, sww);
-            if (i == 4) store_chunk_transposed<1>(ga, nxt, sww);
-            if (i == 8) store_chunk_transposed<2>(ga, nxt, sww);
-            if (i == 12) store_chunk_transposed<3>(ga, nxt, sww);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  __syncthreads();
-}
-
-template <bool DIAG>
-__device__ __forceinline__ void syrk_tile(floatx16 (&acc)[4][4], uint16_t* lds, const uint16_t* __restrict__ X,
-                                          const uint16_t* __restrict__ XB, long rows, long n, long ci, long cj, int ro,
-                                          int cg, int offA, int offB, int swr) {
-  const long stages = (rows + kStage - 1) / kStage;
-  Block8x8 ga, gb;
-  uint16_t* const wr = lds + (8 * cg) * kPitch;  // row of this thread's first column within a slice
-  const int sww = ro ^ (cg & 7);
-  fetch_block<false>(ga, X, rows, n, 8 * ro, ci);
-  if (!DIAG) fetch_block<false>(gb, XB, rows, n, 8 * ro, cj);
-  store_block_transposed(ga, wr, sww);
-  if (!DIAG) store_block_transposed(gb, wr + kSliceU16, sww);
-  __syncthreads();
-  // stages whose successor is complete run in one loop body; the ragged successor and the last stage follow
-  long st = 0;
-#define QTIP_SYRK_STAGE(F)                                                                                   \
-  syrk_stage<DIAG, F>(acc, lds + (st & 1) * 2 * kSliceU16, lds + (st & 1) * 2 * kSliceU16 + (DIAG ? 0 : kSliceU16), \
-                      wr + ((st + 1) & 1) * 2 * kSliceU16, ga, gb, X, XB, rows, n, (st + 1) * kStage + 8 * ro, ci, cj, offA, offB, swr, sww)
-  for (; (st + 2) * kStage <= rows; ++st) QTIP_SYRK_STAGE(1);
-  if (st + 1 < stages) {
-    QTIP_SYRK_STAGE(2);
-    ++st;
-  }
-  QTIP_SYRK_STAGE(0);
-#undef QTIP_SYRK_STAGE
-}
-
-// DOT = false: H += X^T X on the tiles on or below the diagonal (XB == X).
-// DOT = true:  nothing is stored; partial[ti * tiles + tj] = w * sum_ij (X^T XB)_ij H_ij over the tile, w = 2 below the
-//              diagonal and 1 on it: with X^T XB symmetric the partials add up to sum_ij (X^T XB)_ij H_ij of a symmetric
-//              H.  The tiles above the diagonal keep the zero the caller wrote.
-template <bool DOT>
-__global__ __launch_bounds__(256, 1) void syrk_bf16_kernel(const uint16_t* __restrict__ X, const uint16_t* __restrict__ XB,
-                                                          long rows, long n, float* __restrict__ H,
-                                                          double* __restrict__ partial, int tiles, int patch_cols) {
-  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  // workgroup -> tile: ids that differ by 8 run on different XCDs; the 32 ids an XCD holds at a time are one patch
-  const long b = blockIdx.x;
-  const long xcd = b & 7, local = b >> 3;
-  const long patch = (local / (kPatchRows * kPatchCols)) * 8 + xcd, within = local % (kPatchRows * kPatchCols);
-  const long ti = (patch / patch_cols) * kPatchRows + within / kPatchCols;
-  const long tj = (patch % patch_cols) * kPatchCols + within % kPatchCols;
-  if (ti >= tiles || tj > ti) return;  // outside the matrix or above the diagonal
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  // this thread stages rows 8 ro .. 8 ro + 7, columns 8 cg .. 8 cg + 7 of a slice; 8 neighbouring lanes read one
-  // 128-byte line of a row of X
-  const int ro = (t >> 3) & 7, cg = (t & 7) + 8 * (t >> 6);
-  const long ci = ti * kTile + 8 * cg, cj = tj * kTile + 8 * cg;
-  const int rl = lane & 31;
-  const int offA = (wm * 128 + rl) * kPitch, offB = (wn * 128 + rl) * kPitch;
-  const int swr = (lane >> 5) ^ (rl & 7) ^ (rl >> 3);  // piece of k-slice 0, row tile 0; the others differ by constants
-
-  floatx16 acc[4][4];
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[a][c][v] = 0.f;
-  {
-    // The accumulators enter the stage loop as results of a matrix instruction (of zero operands): they then live in
-    // the accumulation registers from the start.  Entering as plain zeros, the compiler keeps them in ordinary
-    // registers at the loop head and copies all 256 of them to the accumulation registers and back in every stage.
-    bf16x8 z;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) z[e] = __bf16(0.f);
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int c = 0; c < 4; ++c) acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z, z, acc[a][c], 0, 0, 0);
-  }
-  if (!DOT && ti == tj) syrk_tile<true>(acc, lds, X, XB, rows, n, ci, cj, ro, cg, offA, offB, swr);
-  else syrk_tile<false>(acc, lds, X, XB, rows, n, ci, cj, ro, cg, offA, offB, swr);
-
-  // accumulator element v of a lane: row (v % 4) + 8 (v / 4) + 4 (lane / 32), column lane % 32 of the 32 x 32 tile
-  double dot = 0.0;
-  if ((ti + 1) * kTile <= n && (tj + 1) * kTile <= n) {
-    // a tile inside the matrix (all of them when n is a multiple of 256): the 16 values of H that go with one
-    // 32 x 32 accumulator are fetched together - one round trip to memory per accumulator, not one per value
-    float* hb = H + (ti * kTile + wm * 128 + 4 * (lane >> 5)) * n + tj * kTile + wn * 128 + rl;
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni) {
-        float h[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) h[v] = hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32];
-        __builtin_amdgcn_sched_barrier(0);  // all 16 loads are issued before the first value is used
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          if (DOT) dot += double(acc[mi][ni][v]) * double(h[v]);
-          else hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32] = h[v] + acc[mi][ni][v];
-        }
-      }
-  } else {
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const long gi = ti * kTile + wm * 128 + mi * 32 + (v & 3) + 8 * (v >> 2) + 4 * (lane >> 5);
-          const long gj = tj * kTile + wn * 128 + ni * 32 + rl;
-          if (gi < n && gj < n) {
-            if (DOT) dot += double(acc[mi][ni][v]) * double(H[gi * n + gj]);
-            else H[gi * n + gj] += acc[mi][ni][v];
-          }
-        }
-  }
-  if (DOT) {
-    // lanes, then waves, in a fixed order (the stage loop ended with a barrier: the staging buffers are free)
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
-    double* red = reinterpret_cast<double*>(lds);
-    if (lane == 0) red[wave] = dot;
-    __syncthreads();
-    if (t == 0) partial[ti * tiles + tj] = (ti == tj ? 1.0 : 2.0) * (((red[0] + red[1]) + red[2]) + red[3]);
-  }
-}
-
-// ---------------------------------------------------------------- the same update from operands stored as LDS images
-// The quadratic forms of the proxy build their operands themselves (split_image_kernel), so they are written as the
-// LDS images of the kernel's stages: [stage of 32 rows of K][column tile of 256][column][32 k], the four 16-byte
+// The operands of the update kernel are written (batch_image_kernel for a Hessian batch, split_image_kernel for the
+// proxy's quadratic forms) as the LDS images of its stages: [stage of 32 rows of K][column tile of 256][column][32 k], the four 16-byte
 // pieces of a column at position p ^ ((column >> 2) & 3) (free of bank conflicts for the 16-byte fragment reads: the
 // 16 lanes the LDS serves together then touch 16 different 16-byte bank groups).  A stage of an operand is 16 KB of
 // contiguous global memory and goes straight into LDS (global_load_lds_dwordx4, 1 KB per wave and instruction): no
@@ -441,6 +191,34 @@ __global__ __launch_bounds__(256, 1) void syrk_img_kernel(const uint16_t* __rest
   }
 }
 
+// The batch of a Hessian accumulation (rows x n bf16, row-major) as the stage images of syrk_img_kernel: one workgroup
+// per stage of 32 rows and tile of 256 columns brings the 32 x 256 block in with 16-byte loads (zeros beyond the
+// matrix), turns it in LDS and writes each column's 32 values as the four swizzled 16-byte pieces of its image: 16 KB
+// of contiguous global memory per workgroup.
+__global__ __launch_bounds__(256) void batch_image_kernel(const uint16_t* __restrict__ X, long rows, long n, int tiles,
+                                                          uint16_t* __restrict__ I) {
+  __shared__ __attribute__((aligned(16))) uint16_t blk[IK][kTile + 8];
+  const long st = blockIdx.y, T = blockIdx.x;
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = t + 256 * i, r = idx >> 5, c8 = idx & 31;
+    const long gr = st * IK + r, gc = T * kTile + 8 * c8;
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (gr < rows && gc + 8 <= n) v = *reinterpret_cast<const uint4*>(X + gr * n + gc);
+    *reinterpret_cast<uint4*>(&blk[r][8 * c8]) = v;
+  }
+  __syncthreads();
+  uint16_t* out = I + (size_t(st) * tiles + size_t(T)) * kImgSliceU16 + size_t(t) * IK;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = uint32_t(blk[8 * p + 2 * e][t]) | (uint32_t(blk[8 * p + 2 * e + 1][t]) << 16);
+    *reinterpret_cast<uint4*>(out + ((p ^ ((t >> 2) & 3)) << 3)) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
 __device__ __forceinline__ uint16_t f32_to_bf16_dev(float f) {  // round to nearest even; the inputs here are finite
   uint32_t u = __float_as_uint(f);
   u += 0x7fffu + ((u >> 16) & 1u);
@@ -537,9 +315,9 @@ struct SyrkGrid {
       std::lock_guard<std::mutex> lk(mu);
       if (configured.size() <= size_t(dev)) configured.resize(size_t(dev) + 1, false);
       if (!configured[size_t(dev)]) {
-        QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_bf16_kernel<false>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
         QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_img_kernel<true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(kImgLdsBytes)));
+        QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(syrk_img_kernel<false>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(kImgLdsBytes)));
         configured[size_t(dev)] = true;
       }
@@ -556,12 +334,20 @@ struct SyrkGrid {
 };
 }  // namespace
 
-void launch_hessian_accumulate(const uint16_t* X, long rows, long n, float* H, hipStream_t s) {
+void launch_hessian_accumulate(const uint16_t* X, long rows, long n, float* H, DBuf<uint16_t>& image, hipStream_t s) {
   QTIP_REQUIRE(X != nullptr && H != nullptr && rows >= 0 && n > 0, "hessian_accumulate: bad arguments");
   QTIP_REQUIRE(n % 8 == 0 && (reinterpret_cast<uintptr_t>(X) & 15) == 0, "hessian_accumulate: rows of X must be 16-byte aligned (n = %ld)", n);
   if (rows == 0) return;
   SyrkGrid g(n);
-  syrk_bf16_kernel<false><<<dim3(g.grid), dim3(256), kLdsBytes, s>>>(X, X, rows, n, H, nullptr, g.tiles, g.patch_cols);
+  // the batch is first written as the LDS images of the update kernel's stages (a pass over the batch, 4 % of the
+  // update's time), which then feeds its matrix cores with direct global-to-LDS loads; both operands are the batch
+  const long stages = (rows + IK - 1) / IK;
+  QTIP_REQUIRE(stages <= 65535, "hessian_accumulate: at most %d rows per call (rows = %ld)", 65535 * IK, rows);
+  image.ensure(size_t(stages) * size_t(g.tiles) * kImgSliceU16);
+  batch_image_kernel<<<dim3(unsigned(g.tiles), unsigned(stages)), dim3(256), 0, s>>>(X, rows, n, g.tiles, image.p);
+  QTIP_HIP(hipGetLastError());
+  syrk_img_kernel<false><<<dim3(g.grid), dim3(256), kImgLdsBytes, s>>>(image.p, image.p, int(stages), n, H, nullptr,
+                                                                      g.tiles, g.patch_cols);
   QTIP_HIP(hipGetLastError());
 }
 

@@ -10,7 +10,7 @@ void launch_pack_swizzle(const uint16_t* Q, long m, long n, uint16_t* out, hipSt
 void launch_decode_trellis(const uint16_t* trellis, long m, long n, const float* entry_f, float* out, long ld,
                            hipStream_t s);
 // H (n x n fp32) += X^T X for X = rows x n bf16, tiles on or below the diagonal only; then mirror + scale (hessian.hip)
-void launch_hessian_accumulate(const uint16_t* X, long rows, long n, float* H, hipStream_t s);
+void launch_hessian_accumulate(const uint16_t* X, long rows, long n, float* H, DBuf<uint16_t>& image, hipStream_t s);
 void launch_hessian_finish(float* H, long n, float scale, hipStream_t s);
 // tr(D H D^T) for D = A^T - B^T (m x n; A, B n x m fp32 with leading dimension ld, B may be null), H symmetric n x n
 // fp32, from bf16 hi/lo products on the matrix cores; synchronises the stream

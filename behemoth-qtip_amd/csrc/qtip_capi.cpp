@@ -395,7 +395,7 @@ int qtip_hessian_accumulate_dev(qtip_ctx* ctx, const uint16_t* dev_X_bf16, long 
   return guarded([&] {
     QTIP_REQUIRE(ctx != nullptr, "hessian_accumulate: bad arguments");
     DeviceGuard g(ctx);
-    launch_hessian_accumulate(dev_X_bf16, rows, n, dev_H, ctx->stream);
+    launch_hessian_accumulate(dev_X_bf16, rows, n, dev_H, ctx->hess_img, ctx->stream);
   });
 }
 int qtip_hessian_finish_dev(qtip_ctx* ctx, float* dev_H, int n, double scale) {

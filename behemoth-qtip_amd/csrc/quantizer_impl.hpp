@@ -28,6 +28,7 @@ struct qtip_ctx {
   hipStream_t chain_stream[kMaxChains - 1] = {};
   qtipmi::Rht rht;
   qtipmi::DBuf<double> scratch;
+  qtipmi::DBuf<uint16_t> hess_img;  // a batch of qtip_hessian_accumulate_dev as the stage images of its update kernel
   qtipmi::HBuf<float> ring_HRr[3], ring_L[3];  // page-locked staging of run_groups, kept between calls
   qtipmi::DBuf<float> ring_dHRr[3], ring_dL[3];  // run_groups with device-updated LDL: rotated Hessians and factors stay here
   // LDL with the trailing updates on the device (ldl_assist.hip): own stream, fp64 work matrix, fp32 upload of HRr,

@@ -211,8 +211,10 @@ int qtip_quantize_group_h(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, i
  * dev_H (n x n fp32, row-major) += X^T X for a batch of `rows` activation vectors dev_X (rows x n raw bf16 bits,
  * row-major), bf16 products with fp32 accumulation on the matrix cores.  Only the 256 x 256 tiles on or below the
  * diagonal are updated; qtip_hessian_finish_dev mirrors them into the other triangle and multiplies by `scale`
- * (symmetrize_hess, src/model.cpp:260-264, and the 1 / token count of src/pipeline.cpp:160-166).  n % 8 == 0.
- * Asynchronous on the context's stream. */
+ * (symmetrize_hess, src/model.cpp:260-264, and the 1 / token count of src/pipeline.cpp:160-166).  n % 8 == 0, at
+ * most 2097120 rows per call.  The batch is first rewritten in the layout the matrix cores are fed from, into a
+ * buffer of the context (rows rounded up to 32 x n rounded up to 256 values of 2 bytes) that stays with it.
+ * Asynchronous on the context's stream; calls on one context use that buffer one after the other. */
 int qtip_hessian_accumulate_dev(qtip_ctx* ctx, const uint16_t* dev_X_bf16, long rows, int n, float* dev_H);
 int qtip_hessian_finish_dev(qtip_ctx* ctx, float* dev_H, int n, double scale);
 
