@@ -131,6 +131,7 @@ def lib():
     L.qtip_nvfp4_dequantize.argtypes = [vp, vp, C.c_float, i, i, vp]
     L.qtip_nvfp4_proxy_error.argtypes = [vp, vp, i, i, vp, C.POINTER(d)]
     L.qtip_nvfp4_prepare.argtypes = [vp, i, d, i, i, vp, vp]
+    L.qtip_nvfp4_prepare_device_updates.argtypes = [vp, vp, i, d, i, vp, vp]
     L.qtip_nvfp4_quantize_prepared.argtypes = [vp, i, vp, i, vp, vp, i]
     L.qtip_nvfp4_quantize_group.argtypes = [vp, i, vp, i, vp, C.POINTER(_Nvfp4OptsC), C.POINTER(i)]
     L.qtip_run_groups.argtypes = [vp, i, vp, C.POINTER(_OptsC), vp, vp]
@@ -164,7 +165,8 @@ class _Nvfp4MatrixC(C.Structure):
 
 
 class _Nvfp4OptsC(C.Structure):
-    _fields_ = [("scale_search", C.c_int), ("calibrate", C.c_int), ("sigma_reg", C.c_double)]
+    _fields_ = [("scale_search", C.c_int), ("calibrate", C.c_int), ("sigma_reg", C.c_double),
+                ("factor_on_host", C.c_int)]
 
 
 def _check(rc):
@@ -494,10 +496,12 @@ class Quantizer:
             keep.append(w)
         return mats, outs, keep
 
-    def nvfp4_quantize_group(self, ws, n, H=None, scale_search=True, calibrate=True, sigma_reg=1e-2):
-        """nvfp4_quantize_group, src/nvfp4_gpu.hip:174-241 -> (tensors, calibrated)."""
+    def nvfp4_quantize_group(self, ws, n, H=None, scale_search=True, calibrate=True, sigma_reg=1e-2,
+                             factor_on_host=False):
+        """nvfp4_quantize_group, src/nvfp4_gpu.hip:174-241 -> (tensors, calibrated).  factor_on_host: the calibration's
+        Cholesky factorization on the host alone (default: its trailing updates on the GPU, same bits)."""
         mats, outs, keep = self._nvfp4_marshal(ws, n)
-        o = _Nvfp4OptsC(1 if scale_search else 0, 1 if calibrate else 0, sigma_reg)
+        o = _Nvfp4OptsC(1 if scale_search else 0, 1 if calibrate else 0, sigma_reg, 1 if factor_on_host else 0)
         used = C.c_int()
         Hc = None if H is None else np.ascontiguousarray(H, np.float32)
         _check(lib().qtip_nvfp4_quantize_group(self._h, len(ws), C.addressof(mats), n, _ptr(Hc), C.byref(o), C.byref(used)))
@@ -562,6 +566,15 @@ class Quantizer:
         lanes = C.c_int()
         _check(lib().qtip_group_lanes(self._h, len(shapes), C.addressof(G), C.byref(co), C.byref(lanes)))
         return lanes.value
+
+    def nvfp4_prepare_device_updates(self, H, sigma_reg=1e-2, threads=16):
+        """nvfp4_prepare (calibrated) with the factorization's trailing updates on the GPU -> (L, dw), same bits."""
+        H = np.ascontiguousarray(H, np.float32)
+        n = H.shape[0]
+        L = np.zeros((n, n), np.float32)
+        dw = np.zeros(n, np.float32)
+        _check(lib().qtip_nvfp4_prepare_device_updates(self._h, _ptr(H), n, sigma_reg, threads, _ptr(L), _ptr(dw)))
+        return L, dw
 
     def tlut_f16(self):
         out = np.zeros((512, 2), np.uint16)

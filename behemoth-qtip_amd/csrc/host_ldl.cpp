@@ -421,6 +421,48 @@ bool block_ldl_assisted(int n, float* L_out, int threads, PanelAssist& assist) {
   return wrap.finite.load() != 0;
 }
 
+// The scalar LDL of the NVFP4 calibration (nvfp4_quantize_group, src/nvfp4_gpu.hip:181-207: H = L D L^T from the
+// Cholesky factor C, L_ij = C_ij / C_jj unit lower, dw_j = C_jj^2) from the same panel factorization, written as the
+// panels pass through the host: the rows below a panel by the thread that solved them, the rows of the diagonal
+// block, with the zeros on and right of the diagonal, once the update is queued.
+bool scalar_ldl_assisted(int n, float* L_out, float* dw, int threads, PanelAssist& assist) {
+  if (n % 16 != 0) fail(QTIP_E_ARG, "NVFP4 calibration needs n %% 16 == 0 (n = %d)", n);
+  HostTeam& team = team_of_this_thread(threads);
+  struct Wrap : PanelAssist {
+    PanelAssist& inner;
+    int n;
+    float* L;
+    float* dw;
+    std::vector<double> diag;
+    Wrap(PanelAssist& i, int n_, float* L_, float* dw_) : inner(i), n(n_), L(L_), dw(dw_) {}
+    double* fetch(int k, int kb) override { return inner.fetch(k, kb); }
+    void factored(int k, int kb, const double* d, long ld) override {
+      diag.resize(size_t(kb));
+      for (int j = 0; j < kb; ++j) {
+        diag[size_t(j)] = d[long(j) * ld + j];
+        dw[k + j] = float(diag[size_t(j)] * diag[size_t(j)]);
+      }
+    }
+    void rows_solved(int k, int kb, int row0, int count, const double* rows, long ld) override {
+      for (int i = 0; i < count; ++i) {
+        float* li = L + long(row0 + i) * n + k;
+        const double* r = rows + long(i) * ld;
+        for (int j = 0; j < kb; ++j) li[j] = float(r[j] / diag[size_t(j)]);
+      }
+    }
+    void solved(int k, int kb, const double* panel) override {
+      inner.solved(k, kb, panel);  // the update is queued first
+      for (int i = 0; i < kb; ++i) {
+        float* li = L + long(k + i) * n;
+        for (int j = 0; j < i; ++j) li[k + j] = float(panel[long(i) * kb + j] / diag[size_t(j)]);
+        std::memset(li + k + i, 0, sizeof(float) * size_t(n - k - i));
+      }
+      inner.assembled(k, kb);
+    }
+  } wrap(assist, n, L_out, dw);
+  return cholesky_panels<NB, TILE>(nullptr, 0, n, &team, &wrap);
+}
+
 // block_ldl_assisted with the trailing matrix held and updated by plain host code (one fma chain per element over the
 // panel, from zero, then one subtraction): exercises the panel hand-over without a device.  L must come out as
 // block_ldl_host's.

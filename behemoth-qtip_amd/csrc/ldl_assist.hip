@@ -230,7 +230,48 @@ struct DeviceTrailing final : PanelAssist {
   }
 };
 
+__global__ void add_to_diagonal_kernel(double* __restrict__ A, long n, double v) {
+  const long i = blockIdx.x * long(blockDim.x) + threadIdx.x;
+  if (i < n) A[i * n + i] += v;
+}
+
 }  // namespace
+
+// The Hessian preparation of the calibrated NVFP4 quantizer (nvfp4_prepare_host) with the trailing updates of its
+// Cholesky factorization on the device: same panels, same chains, hence the same L and dw bit for bit.
+void nvfp4_prepare_assisted_impl(qtip_ctx* c, const float* host_H, int n, double sigma_reg, int threads, float* host_L,
+                                 float* host_dw) {
+  QTIP_REQUIRE(c && host_H && host_L && host_dw && n > 0 && n % 16 == 0, "nvfp4_prepare (device updates): bad arguments (n = %d)", n);
+  QTIP_REQUIRE(n <= 65535, "nvfp4_prepare (device updates): n = %d is beyond one grid dimension", n);
+  double dsum = 0;
+  for (int i = 0; i < n; ++i) dsum += host_H[size_t(i) * n + i];
+  const double creg = sigma_reg * dsum / n;
+  if (!c->ldl_stream) QTIP_HIP(hipStreamCreateWithFlags(&c->ldl_stream, hipStreamNonBlocking));
+  hipStream_t s = c->ldl_stream;
+  const size_t nn = size_t(n) * n, nb = size_t(ldl_panel_width());
+  c->ldl_A.ensure(nn);
+  c->ldl_H.ensure(nn);
+  c->ldl_X.ensure(size_t(n) * nb);
+  c->ldl_Xt.ensure(size_t(n) * nb);
+  c->ldl_P.ensure(size_t(n) * nb);
+  for (auto& buf : c->ldl_panel)
+    if (buf.n < size_t(n) * nb) buf.alloc(size_t(n) * nb);
+  QTIP_HIP(hipMemcpyAsync(c->ldl_H.p, host_H, nn * 4, hipMemcpyHostToDevice, s));
+  symmetrize_lower_kernel<<<dim3(unsigned((n + 255) / 256), unsigned(n)), dim3(256), 0, s>>>(c->ldl_H.p, n, c->ldl_A.p);
+  QTIP_HIP(hipGetLastError());
+  add_to_diagonal_kernel<<<dim3(unsigned((n + 255) / 256)), dim3(256), 0, s>>>(c->ldl_A.p, n, creg);
+  QTIP_HIP(hipGetLastError());
+  DeviceTrailing dev(c, n, nullptr, nullptr);
+  bool ok = false;
+  try {
+    ok = scalar_ldl_assisted(n, host_L, host_dw, threads, dev);
+  } catch (...) {
+    (void)hipStreamSynchronize(s);
+    throw;
+  }
+  QTIP_HIP(hipStreamSynchronize(s));
+  if (!ok) throw Error(QTIP_E_NOT_PD, "NVFP4 calibration: Hessian not positive definite");
+}
 
 // dev_HRr (optional): the rotated Hessian already on the device (then host_HRr is not read)
 // dev_L (optional): n x n device buffer that receives L as well

@@ -424,6 +424,14 @@ int qtip_nvfp4_prepare(const float* host_H, int n, double sigma_reg, int calibra
                        float* host_dw) {
   return guarded([&] { nvfp4_prepare_host(host_H, n, sigma_reg, calibrate != 0, threads, host_L, host_dw); });
 }
+int qtip_nvfp4_prepare_device_updates(qtip_ctx* ctx, const float* host_H, int n, double sigma_reg, int threads,
+                                      float* host_L, float* host_dw) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "nvfp4_prepare_device_updates: bad arguments");
+    DeviceGuard g(ctx);
+    nvfp4_prepare_assisted_impl(ctx, host_H, n, sigma_reg, threads, host_L, host_dw);
+  });
+}
 int qtip_nvfp4_quantize_prepared(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mats, int n, const float* host_L,
                                  const float* host_dw, int scale_search) {
   return guarded([&] {
@@ -437,7 +445,7 @@ int qtip_nvfp4_quantize_group(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mats, 
   return guarded([&] {
     QTIP_REQUIRE(ctx != nullptr && n > 0 && n % 16 == 0, "nvfp4_quantize_group: bad arguments");
     DeviceGuard g(ctx);
-    qtip_nvfp4_opts o{1, 1, 1e-2};
+    qtip_nvfp4_opts o{1, 1, 1e-2, 0};
     if (opts) o = *opts;
     const bool cal = o.calibrate != 0 && host_H != nullptr;
     if (calibrated) *calibrated = cal ? 1 : 0;
@@ -445,7 +453,8 @@ int qtip_nvfp4_quantize_group(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mats, 
     if (host_H) {
       dw.resize(static_cast<size_t>(n));
       if (cal) L.resize(size_t(n) * n);
-      nvfp4_prepare_host(host_H, n, o.sigma_reg, cal, 16, cal ? L.data() : nullptr, dw.data());
+      if (cal && !o.factor_on_host) nvfp4_prepare_assisted_impl(ctx, host_H, n, o.sigma_reg, 16, L.data(), dw.data());
+      else nvfp4_prepare_host(host_H, n, o.sigma_reg, cal, 16, cal ? L.data() : nullptr, dw.data());
     }
     nvfp4_quantize_prepared_impl(ctx, nmat, mats, n, cal ? L.data() : nullptr, host_H ? dw.data() : nullptr,
                                  o.scale_search != 0);

@@ -195,6 +195,8 @@ struct PanelAssist {
 int ldl_panel_width();
 bool block_ldl_assisted(int n, float* L_out, int threads, PanelAssist& assist);
 bool block_ldl_assisted_on_host(const float* HRr, int n, float* L_out, int threads);
+// the scalar LDL of the NVFP4 calibration through the same panels: L_ij = C_ij / C_jj, dw_j = C_jj^2
+bool scalar_ldl_assisted(int n, float* L_out, float* dw, int threads, PanelAssist& assist);
 // lower Cholesky in place (lower triangle of the n x n fp64 matrix A); false if not positive definite
 bool cholesky_lower_host(double* A, int n, int threads);
 // A[i][j] = (HRr[i][j] + HRr[j][i]) / 2 in fp64, lower triangle

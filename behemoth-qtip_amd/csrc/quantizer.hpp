@@ -375,7 +375,7 @@ inline std::vector<Nvfp4Tensor> nvfp4_quantize_group(hipStream_t, const std::vec
     out[i].scales.resize(size_t(ms[i] > 0 ? ms[i] : 0) * size_t(n > 0 ? n / 16 : 0));
     mats[i] = qtip_nvfp4_matrix{ms[i], ws[i], out[i].packed.data(), out[i].scales.data(), 1.f};
   }
-  qtip_nvfp4_opts o{opt.scale_search ? 1 : 0, opt.calibrate ? 1 : 0, opt.sigma_reg};
+  qtip_nvfp4_opts o{opt.scale_search ? 1 : 0, opt.calibrate ? 1 : 0, opt.sigma_reg, 0};
   int used = 0;
   detail::check(qtip_nvfp4_quantize_group(detail::context(), int(mats.size()), mats.data(), n, H, &o, &used),
                 "nvfp4_quantize_group");

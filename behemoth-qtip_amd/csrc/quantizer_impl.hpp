@@ -46,6 +46,8 @@ void rotate_hessian_impl(qtip_ctx* c, const float* H, bool on_device, int n, uin
 void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L);
 void ldl_hessian_assisted_impl(qtip_ctx* c, const float* host_HRr, int n, int threads, float* host_L,
                                const float* dev_HRr = nullptr, float* dev_L = nullptr);
+void nvfp4_prepare_assisted_impl(qtip_ctx* c, const float* host_H, int n, double sigma_reg, int threads, float* host_L,
+                                 float* host_dw);
 void ldlq_impl(qtip_ctx* c, const float* dWT, const float* dL, long n, long m, float* d_hatWT, uint16_t* dQ,
                int feedback, double* vit_seconds, int chains);
 void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,

@@ -101,6 +101,33 @@ def test_group_bytes_equal_the_reference_device_path(qz, oracle, name):
             assert np.array_equal(t.scales, sc) and np.array_equal(t.packed, pk)
 
 
+@pytest.mark.parametrize("n", [272, 1040, 2560])
+def test_prepare_with_device_updates_equals_host_prepare(qz, pkg, n):
+    """The calibration's factor with the trailing updates of its Cholesky factorization on the GPU (one panel, a ragged
+    last panel, ten panels): L and dw equal the host preparation's bit for bit; a Hessian that is not positive definite
+    is refused with the same code; the group call gives the same bytes either way."""
+    say("case: nvfp4 prepare, device updates, n = %d" % n)
+    rng = np.random.default_rng(n)
+    X = rng.standard_normal((2 * n, n)).astype(np.float32) * np.exp(0.8 * rng.standard_normal(n)).astype(np.float32)
+    H = np.ascontiguousarray(X.T @ X / (2 * n), np.float32)
+    H[3, 7] += 1e-3      # not exactly symmetric: the preparation takes the mean of the two triangles
+    L0, dw0 = pkg.nvfp4_prepare(H, 1e-2, True, 5)
+    L1, dw1 = qz.nvfp4_prepare_device_updates(H, 1e-2, 7)
+    assert np.array_equal(L0.view(np.uint32), L1.view(np.uint32))
+    assert np.array_equal(dw0.view(np.uint32), dw1.view(np.uint32))
+    assert np.all(np.triu(L1) == 0)
+    bad = H.copy()
+    bad[n // 2, n // 2] = -10.0
+    with pytest.raises(pkg.QtipError) as e:
+        qz.nvfp4_prepare_device_updates(bad, 1e-2, 7)
+    assert e.value.code == pkg.QTIP_E_NOT_PD
+    if n == 272:
+        w = (rng.standard_normal((64, n)) * 0.02).astype(np.float32)
+        (a,), ua = qz.nvfp4_quantize_group([w], n, H)
+        (b,), ub = qz.nvfp4_quantize_group([w], n, H, factor_on_host=True)
+        assert ua and ub and np.array_equal(a.packed, b.packed) and np.array_equal(a.scales, b.scales)
+
+
 def test_nvfp4_layer_shape(qz, pkg, oracle):
     """A 4096 x 4096 matrix with a dense Hessian: calibrated result beats the plain quantizer in the proxy (fp64 on the
     device), format valid; prints the time."""
@@ -159,8 +186,12 @@ def test_nvfp4_config5_shape(qz, pkg):
     t1 = time.time()
     cal = qz.nvfp4_quantize_prepared([w], n, L, dw, True)[0]
     t2 = time.time()
-    say("  preparation %.2f s, block loop %.2f s (%.0f Mweights/s)" % (t1 - t0, t2 - t1, m * n / (t2 - t1) / 1e6))
-    del L
+    Ld, dwd = qz.nvfp4_prepare_device_updates(H, 1e-2, 16)
+    t3 = time.time()
+    say("  preparation %.2f s on the host, %.2f s with the updates on the GPU; block loop %.2f s (%.0f Mweights/s)" %
+        (t1 - t0, t3 - t2, t2 - t1, m * n / (t2 - t1) / 1e6))
+    assert np.array_equal(Ld.view(np.uint32), L.view(np.uint32)) and np.array_equal(dwd.view(np.uint32), dw.view(np.uint32))
+    del L, Ld
     plain = pkg.nvfp4_quantize(w)
     assert cal.global_scale == plain.global_scale and np.all((cal.scales & 0x7f) <= 126)
 
