@@ -449,15 +449,21 @@ int qtip_nvfp4_quantize_group(qtip_ctx* ctx, int nmat, qtip_nvfp4_matrix* mats, 
     if (opts) o = *opts;
     const bool cal = o.calibrate != 0 && host_H != nullptr;
     if (calibrated) *calibrated = cal ? 1 : 0;
-    std::vector<float> L, dw;
+    std::vector<float> dw;
+    float* L = nullptr;
     if (host_H) {
       dw.resize(static_cast<size_t>(n));
-      if (cal) L.resize(size_t(n) * n);
-      if (cal && !o.factor_on_host) nvfp4_prepare_assisted_impl(ctx, host_H, n, o.sigma_reg, 16, L.data(), dw.data());
-      else nvfp4_prepare_host(host_H, n, o.sigma_reg, cal, 16, cal ? L.data() : nullptr, dw.data());
+      if (cal) {
+        // the factor goes through a page-locked buffer the context keeps (the staging of qtip_run_groups): no 3.3 GB
+        // of fresh pages per call at n = 28672, and an upload at the bus's rate
+        const size_t nn = size_t(n) * n;
+        if (ctx->ring_L[0].n < nn) ctx->ring_L[0].alloc(nn);
+        L = ctx->ring_L[0].p;
+      }
+      if (cal && !o.factor_on_host) nvfp4_prepare_assisted_impl(ctx, host_H, n, o.sigma_reg, 16, L, dw.data());
+      else nvfp4_prepare_host(host_H, n, o.sigma_reg, cal, 16, L, dw.data());
     }
-    nvfp4_quantize_prepared_impl(ctx, nmat, mats, n, cal ? L.data() : nullptr, host_H ? dw.data() : nullptr,
-                                 o.scale_search != 0);
+    nvfp4_quantize_prepared_impl(ctx, nmat, mats, n, L, host_H ? dw.data() : nullptr, o.scale_search != 0);
   });
 }
 
