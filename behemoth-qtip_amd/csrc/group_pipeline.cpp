@@ -59,16 +59,120 @@ void run_groups_on(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opt
 
   std::mutex mu;
   std::condition_variable cv;
-  int rotated = 0, factored = 0;
+  int rotated = 0, factored = 0, loaded = 0, finished = 0;
   bool stop = false;
-  std::exception_ptr ldl_err;
+  std::exception_ptr ldl_err, load_err;
+
+  // Inputs that arrive as host pointers (the reference's interface, src/quantizer.hpp:21-28, 75-77) are brought to the
+  // device by a side thread on a stream of its own, up to three groups ahead, into a ring of four staging slots the
+  // context keeps: the quantizing stream then only sees device-to-device copies.  On that stream a Hessian's 3.3 GB
+  // and a group's 1.4 GB of weights from pageable memory held one of the LDLQ chains up for their whole length.
+  constexpr int U = qtip_ctx::kUploadSlots;
+  bool any_host = false;
+  for (int g = 0; g < ng; ++g) {
+    any_host = any_host || !groups[g].h_on_device;
+    for (int i = 0; i < groups[g].nlin; ++i) any_host = any_host || !groups[g].lins[i].on_device;
+  }
+  std::vector<const float*> dH(ngz);
+  std::vector<std::vector<qtip_linear_in>> dl(ngz);
+  for (int g = 0; g < ng; ++g) {
+    dH[size_t(g)] = groups[g].H;
+    dl[size_t(g)].assign(groups[g].lins, groups[g].lins + groups[g].nlin);
+  }
+  auto upload = [&](int g) {
+    const int b = g % U;
+    hipStream_t us = c->upload_stream;
+    const size_t nn = size_t(groups[g].n) * groups[g].n;
+    if (!groups[g].h_on_device) {
+      c->up_H[b].ensure(nn);
+      QTIP_HIP(hipMemcpyAsync(c->up_H[b].p, groups[g].H, nn * 4, hipMemcpyHostToDevice, us));
+      dH[size_t(g)] = c->up_H[b].p;
+    }
+    auto padded = [](size_t bytes) { return (bytes + 255) / 256 * 256; };
+    size_t total = 0;
+    for (const qtip_linear_in& l : dl[size_t(g)]) {
+      if (l.on_device) continue;
+      const size_t mn = size_t(l.m) * size_t(groups[g].n);
+      total += padded(l.w_f32 ? mn * 4 : l.w_bf16 ? mn * 2 : mn) + (l.w_fp8 && l.scale_bf16 ? padded(size_t(l.m) * 2) : 0);
+    }
+    c->up_W[b].ensure(total);
+    size_t at = 0;
+    for (qtip_linear_in& l : dl[size_t(g)]) {
+      if (l.on_device) continue;
+      const size_t mn = size_t(l.m) * size_t(groups[g].n);
+      const void* src = l.w_f32 ? static_cast<const void*>(l.w_f32) : l.w_bf16 ? static_cast<const void*>(l.w_bf16)
+                                                                            : static_cast<const void*>(l.w_fp8);
+      if (!src) continue;  // refused with its message when the group is quantized
+      const size_t bytes = l.w_f32 ? mn * 4 : l.w_bf16 ? mn * 2 : mn;
+      uint8_t* dst = c->up_W[b].p + at;
+      QTIP_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, us));
+      at += padded(bytes);
+      if (l.w_f32) l.w_f32 = reinterpret_cast<const float*>(dst);
+      else if (l.w_bf16) l.w_bf16 = reinterpret_cast<const uint16_t*>(dst);
+      else l.w_fp8 = dst;
+      if (l.w_fp8 && l.scale_bf16) {
+        uint8_t* sd = c->up_W[b].p + at;
+        QTIP_HIP(hipMemcpyAsync(sd, l.scale_bf16, size_t(l.m) * 2, hipMemcpyHostToDevice, us));
+        at += padded(size_t(l.m) * 2);
+        l.scale_bf16 = reinterpret_cast<const uint16_t*>(sd);
+      }
+      l.on_device = 1;
+    }
+    QTIP_HIP(hipStreamSynchronize(us));
+  };
+  std::thread loader;
+  if (any_host) {
+    if (!c->upload_stream) QTIP_HIP(hipStreamCreateWithFlags(&c->upload_stream, hipStreamNonBlocking));
+    loader = std::thread([&] {
+      try {
+        QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
+        for (int g = 0; g < ng; ++g) {
+          {
+            std::unique_lock<std::mutex> lk(mu);
+            cv.wait(lk, [&] { return finished >= g - (U - 1) || stop; });  // the slot's last user is through
+            if (stop) return;
+          }
+          upload(g);
+          std::lock_guard<std::mutex> lk(mu);
+          loaded = g + 1;
+          cv.notify_all();
+        }
+      } catch (...) {
+        std::lock_guard<std::mutex> lk(mu);
+        load_err = std::current_exception();
+        cv.notify_all();
+      }
+    });
+  } else {
+    loaded = ng;
+  }
+  struct JoinLoader {  // whatever ends this call, the loader is told and waited for
+    std::thread& t;
+    std::mutex& mu;
+    std::condition_variable& cv;
+    bool& stop;
+    ~JoinLoader() {
+      if (!t.joinable()) return;
+      {
+        std::lock_guard<std::mutex> lk(mu);
+        stop = true;
+        cv.notify_all();
+      }
+      t.join();
+    }
+  } join_loader{loader, mu, cv, stop};
 
   auto rotate = [&](int g) {
+    {
+      std::unique_lock<std::mutex> lk(mu);
+      cv.wait(lk, [&] { return loaded > g || load_err; });
+      if (loaded <= g) std::rethrow_exception(load_err);
+    }
     const double t0 = now_s();
     const int b = g % R;
-    rotate_hessian_impl(c, groups[g].H, groups[g].h_on_device != 0, groups[g].n, groups[g].seed, opt.sigma_reg,
-                        su[size_t(b)].data(), &creg[size_t(g)], keep_dev ? nullptr : c->ring_HRr[b].p,
-                        keep_dev ? c->ring_dHRr[b].p : nullptr);
+    rotate_hessian_impl(c, dH[size_t(g)], groups[g].h_on_device != 0 || dH[size_t(g)] != groups[g].H, groups[g].n,
+                        groups[g].seed, opt.sigma_reg, su[size_t(b)].data(), &creg[size_t(g)],
+                        keep_dev ? nullptr : c->ring_HRr[b].p, keep_dev ? c->ring_dHRr[b].p : nullptr);
     t_rot[size_t(g)] = now_s() - t0;
     std::lock_guard<std::mutex> lk(mu);
     rotated = g + 1;
@@ -125,10 +229,15 @@ void run_groups_on(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opt
         qtip_timing T{};
         T.rht = t_rot[size_t(g)];
         T.ldl_cpu = t_ldl[size_t(g)];
-        quantize_group_impl(c, groups[g].nlin, groups[g].lins, groups[g].n, groups[g].seed, su[size_t(b)].data(),
+        quantize_group_impl(c, groups[g].nlin, dl[size_t(g)].data(), groups[g].n, groups[g].seed, su[size_t(b)].data(),
                             creg[size_t(g)], keep_dev ? nullptr : c->ring_HRr[b].p, c->ring_L[b].p, opt, groups[g].outs, &T,
                             keep_dev ? c->ring_dHRr[b].p : nullptr, keep_dev ? c->ring_dL[b].p : nullptr);
         if (tms) tms[g] = T;
+        {
+          std::lock_guard<std::mutex> lk(mu);
+          finished = g + 1;
+          cv.notify_all();
+        }
       }
     } catch (...) {
       feed_err = std::current_exception();

@@ -108,6 +108,11 @@ void destroy_context(qtip_ctx* ctx) {
     (void)hipStreamDestroy(ctx->ldl_stream);
   }
   ctx->ldl_stream = nullptr;
+  if (ctx->upload_stream) {
+    (void)hipStreamSynchronize(ctx->upload_stream);
+    (void)hipStreamDestroy(ctx->upload_stream);
+    ctx->upload_stream = nullptr;
+  }
   for (hipStream_t& cs : ctx->chain_stream)
     if (cs) {
       (void)hipStreamSynchronize(cs);

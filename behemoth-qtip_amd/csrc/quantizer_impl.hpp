@@ -30,6 +30,11 @@ struct qtip_ctx {
   qtipmi::DBuf<double> scratch;
   qtipmi::DBuf<uint16_t> hess_img;  // a batch of qtip_hessian_accumulate_dev as the stage images of its update kernel
   qtipmi::HBuf<float> ring_HRr[3], ring_L[3];  // page-locked staging of run_groups, kept between calls
+  // host inputs of qtip_run_groups on their way to the device: a stream and four staging slots (Hessian, weights)
+  static constexpr int kUploadSlots = 4;
+  hipStream_t upload_stream = nullptr;
+  qtipmi::DBuf<float> up_H[kUploadSlots];
+  qtipmi::DBuf<uint8_t> up_W[kUploadSlots];
   qtipmi::DBuf<float> ring_dHRr[3], ring_dL[3];  // run_groups with device-updated LDL: rotated Hessians and factors stay here
   // LDL with the trailing updates on the device (ldl_assist.hip): own stream, fp64 work matrix, fp32 upload of HRr,
   // solved panel rows, two page-locked panel buffers (the panels travel one ahead); allocated on first use

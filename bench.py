@@ -212,7 +212,7 @@ def run_group(args, pkg):
     if not args.no_host_input_leg:
         # beside it (outside the timed region): the same groups with W and H handed over as host pointers, as the
         # reference's entry point takes them (src/quantizer.hpp:21-28,75-77): pageable host memory, PCIe inside
-        kq = min(args.steps, 3)
+        kq = min(args.steps, 6)
         lins_h = [pkg.LinearIn("w%d" % i, m, w_f32=w.cpu().numpy()) for i, (m, w) in enumerate(zip(ms, Ws))]
         H_host = H.cpu().numpy()
         q.synchronize()
@@ -223,7 +223,7 @@ def run_group(args, pkg):
         host_inputs = dict(host_inputs_Mweights_s=weights_per_step * kq / th / 1e6, host_inputs_groups=kq,
                            host_inputs_load_s=sum(r[1].load for r in hres) / kq,
                            host_inputs_same_codes=bool(all(np.array_equal(a.trellis, b.trellis) and a.proxy == b.proxy
-                                                           for a, b in zip(hres[-1][0], stats["cmp_outs3"]))))
+                                                           for a, b in zip(hres[-1][0], stats["cmp_outs"]))))
         del lins_h, H_host, hres
     fb1 = {}
     if args.feedback == 0 and not args.no_feedback1_leg:
