@@ -343,7 +343,15 @@ def test_run_groups_lanes_give_the_same_results(qz, pkg, synth):
             lins = [pkg.LinearIn("g2_0", Ws[0].shape[0], w_bf16=wb)]
         cases.append((lins, n, H, 200 + g))
         shapes.append((ms, n))
-    assert qz.group_lanes(shapes) == 7            # 8 tile rows at most: all of them side by side
+    # an eighth group with fp8 weights and a per-row scale: with one lane the side thread that uploads host inputs
+    # takes every format through its four staging slots twice over
+    rng8 = np.random.default_rng(8)
+    codes = rng8.integers(0, 256, (64, 512)).astype(np.uint8)
+    codes[(codes & 0x7f) == 0x7f] = 0x30        # no NaN codes
+    _, H8 = synth.small_group(seed=78, n=512, ms=(64,))
+    cases.append(([pkg.LinearIn("g7_0", 64, w_fp8=codes, scale_bf16=np.full(64, 0x3c00, np.uint16))], 512, H8, 207))
+    shapes.append(((64,), 512))
+    assert qz.group_lanes(shapes) == 8            # 8 tile rows at most: all of them side by side
     assert qz.group_lanes(shapes, pkg.QuantOpts(group_lanes=1)) == 1
     assert qz.group_lanes(shapes, pkg.QuantOpts(group_lanes=3)) == 3
     assert qz.group_lanes([((12288,), 28672)] * 4) == 1
