@@ -101,6 +101,8 @@ def lib():
     L.qtip_viterbi_tiles.argtypes = [vp, vp, l, vp, vp]
     L.qtip_viterbi_tiles_dev.argtypes = [vp, vp, l, vp, vp]
     L.qtip_viterbi_tiles_dev_noalloc.argtypes = [vp, vp, l, vp, vp]
+    L.qtip_set_viterbi_mode.argtypes = [vp, i, C.c_uint]
+    L.qtip_viterbi_stats.argtypes = [vp, C.POINTER(C.c_ulonglong), C.POINTER(C.c_ulonglong), i]
     L.qtip_stream_wait.argtypes = [vp, vp]
     L.qtip_stream_signal.argtypes = [vp, vp]
     L.qtip_device_lut.argtypes = [vp, C.POINTER(vp)]
@@ -327,6 +329,17 @@ class Quantizer:
         pk = np.zeros((B, 32), np.uint16) if want_packed else None
         _check(lib().qtip_viterbi_tiles(self._h, _ptr(X), B, _ptr(st), _ptr(pk)))
         return st, pk
+
+    def set_viterbi_mode(self, mode=0, margin_units=0):
+        """0: 32-bit metrics first, fp64 again where a traced decision is closer than margin_units (default 160)
+        units of 2^-26; 1: fp64 metrics only.  Same states either way."""
+        _check(lib().qtip_set_viterbi_mode(self._h, int(mode), C.c_uint(int(margin_units))))
+
+    def viterbi_stats(self, reset=False):
+        """(first passes, second passes) that mode 0 ran again on fp64 metrics."""
+        a, b = C.c_ulonglong(0), C.c_ulonglong(0)
+        _check(lib().qtip_viterbi_stats(self._h, C.byref(a), C.byref(b), 1 if reset else 0))
+        return int(a.value), int(b.value)
 
     def viterbi_tiles_dev(self, dX, B, d_states=None, d_packed=None):
         _check(lib().qtip_viterbi_tiles_dev(self._h, _ptr(dX), B, _ptr(d_states), _ptr(d_packed)))

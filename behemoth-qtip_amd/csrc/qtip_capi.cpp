@@ -93,6 +93,8 @@ qtip_ctx* make_context(int device, const HostCodebook* cb_from) {
   else c->cb.build(nullptr);
   upload_codebook(c);
   c->rht.init(device, c->stream);
+  c->vit_stats.alloc(4);
+  QTIP_HIP(hipMemset(c->vit_stats.p, 0, 4 * sizeof(unsigned)));
   guard.c = nullptr;
   return c;
 }
@@ -136,6 +138,8 @@ qtip_ctx* lane_context(qtip_ctx* parent, int k) {
     // hardware queue to itself, and a process has few of them (GPU_MAX_HW_QUEUES, 4 unless the environment says
     // more); with a stream more per lane for the factorization 1024 x 1024 groups ran at 59 instead of 134 Mweights/s
     parent->lane[k]->ldl_stream = parent->lane[k]->stream;
+    parent->lane[k]->vit_mode = parent->vit_mode;
+    parent->lane[k]->vit_margin = parent->vit_margin;
   }
   return parent->lane[k];
 }
@@ -264,6 +268,36 @@ int qtip_get_lut(qtip_ctx* ctx, float* lut0, float* lut1) {
   });
 }
 
+int qtip_set_viterbi_mode(qtip_ctx* ctx, int mode, unsigned margin_units) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && (mode == 0 || mode == 1), "set_viterbi_mode: mode must be 0 or 1");
+    ctx->vit_mode = mode;
+    ctx->vit_margin = margin_units ? margin_units : kViterbiMargin;
+    for (qtip_ctx* l : ctx->lane)
+      if (l) l->vit_mode = ctx->vit_mode, l->vit_margin = ctx->vit_margin;
+  });
+}
+
+int qtip_viterbi_stats(qtip_ctx* ctx, unsigned long long* redone_first, unsigned long long* redone_second, int reset) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "null context");
+    DeviceGuard g(ctx);
+    unsigned long long sum[2] = {0, 0};
+    auto take = [&](qtip_ctx* c) {
+      QTIP_HIP(hipDeviceSynchronize());
+      unsigned v[4];
+      QTIP_HIP(hipMemcpy(v, c->vit_stats.p, sizeof v, hipMemcpyDeviceToHost));
+      sum[0] += v[0], sum[1] += v[1];
+      if (reset) QTIP_HIP(hipMemset(c->vit_stats.p, 0, sizeof v));
+    };
+    take(ctx);
+    for (qtip_ctx* l : ctx->lane)
+      if (l) take(l);
+    if (redone_first) *redone_first = sum[0];
+    if (redone_second) *redone_second = sum[1];
+  });
+}
+
 int qtip_viterbi_tiles_dev(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* dev_states, uint16_t* dev_packed) {
   return guarded([&] {
     QTIP_REQUIRE(ctx != nullptr && B >= 0, "viterbi_tiles: bad arguments");
@@ -276,6 +310,7 @@ int qtip_viterbi_tiles_dev(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* 
     job.tiles = B;
     job.states = dev_states;
     job.packed = dev_packed;
+    ctx->viterbi_settings(job);
     launch_viterbi_tiles(job, ctx->d_entry_d, ctx->d_entry_f, ctx->vit_ws, ctx->vit_slots, ctx->stream);
   });
 }
@@ -296,6 +331,7 @@ int qtip_viterbi_tiles_dev_noalloc(qtip_ctx* ctx, const float* dev_X, long B, ui
     job.tiles = B;
     job.states = dev_states;
     job.packed = dev_packed;
+    ctx->viterbi_settings(job);
     launch_viterbi_tiles(job, ctx->d_entry_d, ctx->d_entry_f, ws, viterbi_static_slots(), ctx->stream);
   });
 }

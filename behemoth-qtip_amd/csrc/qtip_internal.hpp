@@ -19,6 +19,9 @@ constexpr int kStates = 65536; // L = 16
 constexpr int kGroups = 4096;  // states sharing a successor group
 constexpr int kWords = 32;     // packed u16 words per trellis
 constexpr int kLutEntries = 1024;  // distinct codebook entries: bits 6..15 of s*(s+1)
+// A decision of a 32-bit Viterbi pass stands when it is won by this many units of 2^-26: a metric of at most 128
+// rounded terms is within 64 units of the fp64 one, so two candidates 129 units apart are ordered alike in fp64.
+constexpr uint32_t kViterbiMargin = 160;
 
 struct Error : std::runtime_error {
   int code;
@@ -239,6 +242,11 @@ struct TileJob {
   // col0 + 16 (blocks - 1) ..) down to the first (col0 ..), state words at q_offset + block: the blocks of a tile row
   // depend on each other only through that row's own hatWT values, so nothing has to wait for another workgroup
   int blocks = 1;
+  // 0: both passes run on 32-bit metrics first and a pass whose traced decisions are not all won by `margin` units of
+  // 2^-26 is run again on fp64 metrics (same results as mode 1, bit for bit); 1: fp64 metrics only
+  int mode = 0;
+  uint32_t margin = kViterbiMargin;
+  unsigned* stats = nullptr;  // device counters (optional): [0], [1] += passes of the first / second kind run again
 };
 size_t viterbi_workspace_bytes(int slots);
 int viterbi_max_slots(int device);

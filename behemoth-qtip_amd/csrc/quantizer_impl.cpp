@@ -195,6 +195,7 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
           job.ldw = m;
           job.col0 = c0;
           job.blocks = 8;
+          c->viterbi_settings(job);
           hipEvent_t t0 = nullptr, t1 = nullptr;
           if (vit_seconds) t0 = timed.add(hipEventDefault), t1 = timed.add(hipEventDefault);
           launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws.p + viterbi_workspace_bytes(C.slot0), C.slots,

@@ -17,6 +17,16 @@ struct qtip_ctx {
   bool lut_h2_valid = false;
   qtipmi::DBuf<unsigned char> vit_ws;  // kept-metrics slots of the resident Viterbi workgroups
   int vit_slots = 0;
+  // Viterbi passes: 0 = 32-bit metrics first, fp64 again where a traced decision is too close (same results);
+  // 1 = fp64 only.  vit_stats: two device counters, passes of the first / second kind that were run again.
+  int vit_mode = 0;
+  uint32_t vit_margin = qtipmi::kViterbiMargin;
+  qtipmi::DBuf<unsigned> vit_stats;
+  void viterbi_settings(qtipmi::TileJob& job) const {
+    job.mode = vit_mode;
+    job.margin = vit_margin;
+    job.stats = vit_stats.p;
+  }
   int vit_slots_limit = 0;  // a lane (below) keeps slots for this many workgroups only; 0: all the device can hold
   // qtip_run_groups runs groups too small to fill the chip side by side, each on a lane: a context of its own
   // (streams, workspaces, rings) made on first use, kept here and released with this context

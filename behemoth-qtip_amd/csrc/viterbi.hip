@@ -73,6 +73,16 @@ __device__ __forceinline__ int m_pos(int col) { return (col & ~5) | ((col & 1) <
 __device__ __forceinline__ int m_swz(int col) { return (((col >> 3) & 7) ^ (((col >> 6) & 3) << 1)) << 1; }
 __device__ __forceinline__ int m_slot(int col, int d) { return m_pos(col) * 16 + (d ^ m_swz(col)); }
 
+// threadIdx.x through a barrier for the optimizer: what a pass derives from it (table rows, metric slots, read
+// addresses: some twenty registers per kind of pass) is then formed where the pass starts instead of once at the top
+// of the kernel, where the three kinds together would sit in registers for the whole launch and push the passes' own
+// values out to scratch memory
+__device__ __forceinline__ int opaque_tid() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+
 struct Smem {
   double E[kESlots];  // first: its reads use 8-bit immediate offsets from a per-lane base
   double M[kMSlots];
@@ -82,6 +92,8 @@ struct Smem {
   uint32_t red_s[4];
   double tr_c[2][4];    // trace-back: the four waves' best candidates of a round (cost; d | d1 << 8), two sets
   uint32_t tr_d[2][4];
+  uint32_t tr32[2][4][4];  // the same for the 32-bit passes: best, second best, d | d1 << 8, gap inside the best's row
+  uint32_t red32[4][3];    // end of the free 32-bit pass: per wave the best group's metric, the second best, the group
   int overlap;
   uint32_t final_state;
 };
@@ -109,7 +121,7 @@ __device__ __forceinline__ uint32_t hist_index(uint32_t g) {
 // Returns nothing; the final state is left in sm.final_state.
 __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict__ entry_d, int roll, int ov,
                                              double* __restrict__ hist, int first_kept) {
-  const int tid = threadIdx.x;
+  const int tid = opaque_tid();
   const int colA = 4 * (tid & 15) + ((tid >> 4) & 3) + 64 * ((tid >> 6) & 1), colB = 255 - colA;
   const int half = tid >> 7;  // owns 16c + 8 half + m, m = 0..7
   const double INF = __builtin_inf();
@@ -330,7 +342,7 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
 template <typename Acc>
 __device__ __forceinline__ void tile_targets(Smem& sm, const TileJob& job, long col0, long tile,
                                              const Acc* __restrict__ prod) {
-  const int u = threadIdx.x;
+  const int u = opaque_tid();
   const int k0 = int(col0) + 16, nk = job.bufend - k0;
   float* Ls = reinterpret_cast<float*>(sm.M);
   float* Ws = Ls + 112 * 16;
@@ -384,7 +396,8 @@ __device__ __forceinline__ double read_lane_f64(double v, int lane) {
 __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restrict__ entry_d,
                                                const double* __restrict__ hist, int roll, uint32_t s, int it_min,
                                                bool record) {
-  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, dp = lane & 15u, d = 4u * wave + (lane >> 4);
+  const uint32_t tid = uint32_t(opaque_tid());
+  const uint32_t lane = tid & 63u, wave = tid >> 6, dp = lane & 15u, d = 4u * wave + (lane >> 4);
   int set = 0;
 #pragma nounroll
   for (int it = kSteps - 2; it >= it_min; it -= 2, set ^= 1) {
@@ -447,6 +460,337 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
   return s;
 }
 
+// ================================================================= the same two passes on 32-bit metrics
+// The fp64 passes above are bound by the issue rate of fp64 vector instructions and, behind it, by 8-byte LDS reads.
+// Both passes are therefore first run on unsigned 32-bit metrics in units of 2^-26: the squared error of a codebook
+// entry is formed in fp64 exactly as above and rounded to the nearest unit once (|error| <= 1/2 unit), the adds are
+// integer adds that saturate at 2^32 - 1 (= 64.0, which also stands for +inf), so a path metric of n terms differs from
+// the fp64 one by at most n/2 units, whatever the path.  Only the decisions on the surviving path matter: the
+// trace-back redoes them from the kept metrics as above and also looks at the runner-up.  If every decision it takes
+// (the final state, and the 16-way choice of each step it walks) is won by at least `thr` > 128 units and the winner is
+// below 2^31, the fp64 recursion takes the same decisions and the pass's result is the fp64 result.  Otherwise the
+// workgroup runs that pass again through the fp64 code above (a fraction of a percent of the passes: near-ties of
+// 2e-6 relative, and the exact ties between states that share predecessor and codebook entry).
+// Integer adds issue at twice the rate of fp64 adds on this chip and a three-way minimum covers two candidates, so an
+// add-compare-select costs 1.5 instructions of 4.5 ns per pair instead of 2 of 8.2 ns; the table and the metrics are
+// 4 bytes, half the LDS traffic, and the kept metrics half the HBM traffic.
+//
+// Free ends (first pass): state s and its complement 65535 - s decode to the same values and the complement of a
+// predecessor is a predecessor of the complement, so with equal initial metrics the metric of group 4095 - j equals
+// that of group j at every step, exactly.  The pass computes the groups below 2048 only (half of the candidates) and
+// copies them to their mirrors; of the two best final states, complements of each other, the smaller one is taken,
+// which is what the first-minimum rule of the CPU algorithm does.
+//
+// LDS layout for 4-byte values (32 banks of 4 bytes, a 4-byte access served 32 lanes at a time): lane t runs metric
+// column c = 4 (t & 31) + (t >> 5 & 3) and owns the groups j = 16 c + 8 (t >> 7) + m, m = 0..7, and their mirrors.
+// Bits 6..10 of j(j+1) then run through all 32 values over the 32 lanes of a half wave, so the table E32[q][row]
+// (64 rows of 4 bytes per entry position q, positions stored twice for the rotation as above) is read without
+// conflicts.  The metric of (column, digit d) sits at pos(column) * 16 + (d ^ swz(column)) with swz a multiple of 4,
+// so a column comes in as four 16-byte reads; pos and swz are chosen so that those reads, the 4-byte writes of a
+// group's result (32 lanes: 4 columns x 8 digits) and of its mirror (slot ^ 0xfeb) are free of bank conflicts.
+constexpr uint32_t kSat = 0xffffffffu;
+constexpr int kMirror32 = 0xfeb;
+static_assert(64 * kGroups <= 2 * kHistWordsPerTile, "the 32-bit kept metrics (64 steps) must fit the fp64 slot");
+
+__device__ __forceinline__ int m32_pos(int col) {  // bits 7..0: b7 b6 b5 b4 b1 b0 b3 (b2 ^ b6)
+  return (col & 0xf0) | ((col & 3) << 2) | (((col >> 3) & 1) << 1) | (((col >> 2) ^ (col >> 6)) & 1);
+}
+__device__ __forceinline__ int m32_swz(int col) { return (((col >> 4) & 1) << 2) | ((((col >> 5) ^ (col >> 7)) & 1) << 3); }
+__device__ __forceinline__ int m32_slot(int col, int d) { return m32_pos(col) * 16 + (d ^ m32_swz(col)); }
+// thread that owns group jj < 2048 in the 32-bit passes
+__device__ __forceinline__ uint32_t owner32(uint32_t jj) {
+  const uint32_t c = jj >> 4;
+  return (c >> 2) | ((c & 3u) << 5) | (((jj >> 3) & 1u) << 7);
+}
+// place of group g in one kept step (value-major: a wave's store is 256 contiguous bytes); kSym: the mirror groups
+// are not kept, their metrics are those of the groups they mirror
+template <bool kSym>
+__device__ __forceinline__ uint32_t hist32_index(uint32_t g) {
+  const uint32_t jj = g < 2048u ? g : 4095u - g;
+  return ((jj & 7u) + ((kSym || g < 2048u) ? 0u : 8u)) * kThreads + owner32(jj);
+}
+__device__ __forceinline__ uint32_t sat_add(uint32_t a, uint32_t b) { return __builtin_elementwise_add_sat(a, b); }
+__device__ __forceinline__ uint32_t min3u(uint32_t a, uint32_t b, uint32_t c) {
+  uint32_t r;  // written out: the compiler forms the three-way minimum for only half of the chains
+  asm("v_min3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+// squared error of a codebook entry against the two inputs of a step, the fp64 value of the passes above in units of
+// 2^-26, rounded to nearest; 64.0 and more (and NaN) become 2^32 - 1
+__device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, double x1) {
+  const double a = l0 - x0, b = l1 - x1;
+  const double v = __builtin_rint(__builtin_fma(a, a, b * b) * 67108864.0);
+  return uint32_t(__builtin_fmin(v, 4294967295.0));
+}
+
+// One forward pass on 32-bit metrics.  kSym: free ends, the groups below 2048 only (their mirrors get copies), all
+// 128 steps, and the best final group, its metric and the gap to the runner-up are left in sm.red32[0]; otherwise:
+// start in group ov, steps 0 .. 126 (the last step's decision is taken by the trace-back from the metrics entering
+// it).  The results of the even steps first_kept .. 126 (the metrics entering the next, odd step) go to hist.
+// Metrics and error table are double-buffered in LDS (2 x 16 KB, 2 x 8 KB: the footprint of the fp64 arrays): a step
+// reads the present buffers and writes the next metrics and the next step's table, so one barrier per step suffices;
+// a thread keeps its four codebook entries in registers.
+template <bool kSym>
+__device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restrict__ entry_d, int roll, int ov,
+                                               uint32_t* __restrict__ hist, int first_kept) {
+  const int tid = opaque_tid();
+  const int colA = 4 * (tid & 31) + ((tid >> 5) & 3), colB = 255 - colA;
+  const int half = tid >> 7;
+  uint32_t* const E32 = reinterpret_cast<uint32_t*>(sm.E);  // [2][32 positions][64 rows]
+  uint32_t* const M32 = reinterpret_cast<uint32_t*>(sm.M);  // [2][4096]
+  static_assert(sizeof(sm.E) >= 2 * kESlots * sizeof(uint32_t) && sizeof(sm.M) >= 2 * kMSlots * sizeof(uint32_t));
+#ifndef QTIP_V_ENTREG
+#define QTIP_V_ENTREG 1
+#endif
+#ifndef QTIP_V_TABLE_LATE
+#define QTIP_V_TABLE_LATE 0
+#endif
+  double2 ent[4];
+  const double2* __restrict__ entries = reinterpret_cast<const double2*>(entry_d) + tid;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) ent[q] = entries[256 * q];
+  const int e_wr = (tid >> 6) * 64 + (tid & 63);
+  int ebase[8], wslot[8];
+#pragma unroll
+  for (int m = 0; m < 8; ++m) {
+    const uint32_t j = 16u * colA + 8u * uint32_t(half) + m, p = j * (j + 1u);
+    ebase[m] = int((p >> 12) & 15u) * 64 + int((p >> 6) & 63u);
+    wslot[m] = m32_slot(int(j & 255u), int(j >> 8));
+  }
+  int xA = m32_pos(colA) * 64 + m32_swz(colA) * 4, xB = m32_pos(colB) * 64 + m32_swz(colB) * 4;  // bytes
+  // the error table of step `it` into table buffer it & 1
+  auto table = [&](int it) __attribute__((always_inline)) {
+    const int t = (2 * it + roll) & 255;
+    const double x0 = double(sm.x[t]), x1 = double(sm.x[t + 1]);
+    uint32_t* const Ew = E32 + (it & 1) * kESlots + e_wr;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+#if QTIP_V_ENTREG
+      const double2 l = ent[q];
+#else
+      const double2 l = entries[256 * q];
+#endif
+      const uint32_t v = err_units(l.x, l.y, x0, x1);
+      Ew[256 * q] = v;
+      Ew[256 * q + 1024] = v;
+    }
+  };
+  for (int g = tid; g < kGroups; g += kThreads) M32[m32_slot(g & 255, g >> 8)] = (ov < 0 || g == ov) ? 0u : kSat;
+  table(0);
+  __syncthreads();
+
+  uint32_t fin[8];
+  // step `it`: metrics of buffer it & 1 and table buffer it & 1 -> metrics of buffer (it + 1) & 1
+  auto step = [&](int it, auto kind_tag) __attribute__((always_inline)) {
+    constexpr int kind = decltype(kind_tag)::value;  // kDigits: the free pass's last step, results to fin only
+    uint32_t* hs = nullptr;
+    if constexpr (kind == kStore) hs = hist + size_t(it >> 1) * kGroups + tid;
+    const char* const Mb = reinterpret_cast<const char*>(M32 + (it & 1) * kMSlots);
+    uint32_t* const Mw = M32 + ((it + 1) & 1) * kMSlots;
+    const uint32_t* const Er = E32 + (it & 1) * kESlots;
+    uint32_t MA[16], MB[16];
+    asm volatile("" : "+v"(xA), "+v"(xB));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint4 a = *reinterpret_cast<const uint4*>(Mb + (xA ^ (16 * k)));
+      MA[4 * k] = a.x, MA[4 * k + 1] = a.y, MA[4 * k + 2] = a.z, MA[4 * k + 3] = a.w;
+      if constexpr (!kSym) {
+        const uint4 b = *reinterpret_cast<const uint4*>(Mb + (xB ^ (16 * k)));
+        MB[4 * k] = b.x, MB[4 * k + 1] = b.y, MB[4 * k + 2] = b.z, MB[4 * k + 3] = b.w;
+      }
+    }
+#if !QTIP_V_TABLE_LATE
+    if constexpr (kind != kDigits) table(it + 1);
+#endif
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+      const int g = 2 * m + 1;
+      const uint32_t* er = Er + ebase[m];
+      uint32_t ev[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) ev[k] = er[((k * g) & 15) * 64];
+      // the table value at position k is the candidate of digit k of the group and of digit 15 - k of its mirror
+      uint32_t ba = min(sat_add(ev[0], MA[0]), sat_add(ev[1], MA[1]));
+#pragma unroll
+      for (int k = 1; k < 8; ++k) ba = min3u(ba, sat_add(ev[2 * k], MA[2 * k]), sat_add(ev[2 * k + 1], MA[2 * k + 1]));
+      uint32_t bb = ba;
+      if constexpr (!kSym) {
+        bb = min(sat_add(ev[0], MB[15]), sat_add(ev[1], MB[14]));
+#pragma unroll
+        for (int k = 1; k < 8; ++k)
+          bb = min3u(bb, sat_add(ev[2 * k], MB[15 - 2 * k]), sat_add(ev[2 * k + 1], MB[14 - 2 * k]));
+      }
+      if constexpr (kind == kDigits) {
+        fin[m] = ba;
+      } else {
+        Mw[wslot[m]] = ba;
+        Mw[wslot[m] ^ kMirror32] = bb;
+      }
+      if constexpr (kind == kStore) {
+        hs[m * kThreads] = ba;
+        if constexpr (!kSym) hs[(8 + m) * kThreads] = bb;
+      }
+    }
+#if QTIP_V_TABLE_LATE
+    if constexpr (kind != kDigits) table(it + 1);
+#endif
+    __syncthreads();
+  };
+  using Plain = std::integral_constant<int, kPlain>;
+  using Store = std::integral_constant<int, kStore>;
+  using Last = std::integral_constant<int, kDigits>;
+#pragma nounroll
+  for (int it = 0; it < kSteps - 1; ++it) {
+    if (!(it & 1) && it >= first_kept) step(it, Store{});
+    else step(it, Plain{});
+  }
+  if constexpr (kSym) {
+    step(kSteps - 1, Last{});
+    // best final group among the groups below 2048 (each stands for a pair of complementary states), and the runner-up
+    uint32_t b1 = kSat, b2 = kSat, bj = 0;
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+      const uint32_t v = fin[m], j = 16u * colA + 8u * uint32_t(half) + m;
+      const bool take = v < b1;
+      b2 = take ? b1 : min(b2, v);
+      bj = take ? j : bj;
+      b1 = take ? v : b1;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const uint32_t o1 = __shfl_xor(b1, off, 64), o2 = __shfl_xor(b2, off, 64), oj = __shfl_xor(bj, off, 64);
+      const bool take = o1 < b1 || (o1 == b1 && oj < bj);  // equal metrics: same choice in both lanes, gap 0 either way
+      b2 = take ? min(b1, o2) : min(b2, o1);
+      bj = take ? oj : bj;
+      b1 = take ? o1 : b1;
+    }
+    if ((tid & 63) == 0) sm.red32[tid >> 6][0] = b1, sm.red32[tid >> 6][1] = b2, sm.red32[tid >> 6][2] = bj;
+    __syncthreads();
+    b1 = sm.red32[0][0], b2 = sm.red32[0][1], bj = sm.red32[0][2];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const uint32_t o1 = sm.red32[w][0], o2 = sm.red32[w][1], oj = sm.red32[w][2];
+      const bool take = o1 < b1 || (o1 == b1 && oj < bj);
+      b2 = take ? min(b1, o2) : min(b2, o1);
+      bj = take ? oj : bj;
+      b1 = take ? o1 : b1;
+    }
+    __syncthreads();
+    if (tid == 0) sm.red32[0][0] = b1, sm.red32[0][1] = b2 - b1, sm.red32[0][2] = bj;
+    __syncthreads();
+  }
+}
+
+__device__ __forceinline__ uint32_t row_min16_u32(uint32_t c) {
+#define QTIP_ROW_STEP32(CTRL) c = min(c, uint32_t(__builtin_amdgcn_update_dpp(0, int(c), CTRL, 0xf, 0xf, false)));
+  QTIP_ROW_STEP32(0xB1)   // quad_perm [1, 0, 3, 2]
+  QTIP_ROW_STEP32(0x4E)   // quad_perm [2, 3, 0, 1]
+  QTIP_ROW_STEP32(0x141)  // row_half_mirror
+  QTIP_ROW_STEP32(0x140)  // row_mirror
+#undef QTIP_ROW_STEP32
+  return c;
+}
+
+// Trace-back of a 32-bit pass, the scheme of trace_back above with the runner-up of every decision looked at as well.
+// j_last: low 12 bits of the final state (the group the pass ends in).  The decision of step 127 is taken from the
+// metrics entering it (kept slot 63), then two steps per round trip.  flag is raised (in every thread alike) when a
+// decision is won by less than thr units or the winner is not below 2^31.
+// Returns the state of step it_min - 1; record: the states of the steps walked are written to sm.st.
+template <bool kSym>
+__device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restrict__ entry_d,
+                                                 const uint32_t* __restrict__ hist, int roll, uint32_t j_last,
+                                                 int it_min, bool record, uint32_t thr, uint32_t& flag) {
+  const uint32_t tid = uint32_t(opaque_tid());
+  const uint32_t lane = tid & 63u, wave = tid >> 6, dp = lane & 15u, d = 4u * wave + (lane >> 4);
+  // written by this workgroup's own waves before the barrier that ended the forward pass: workgroup scope suffices
+  auto kept = [&](int slot, uint32_t g) -> uint32_t {
+    return __hip_atomic_load(hist + size_t(slot) * kGroups + hist32_index<kSym>(g), __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_WORKGROUP);
+  };
+  auto err_of = [&](uint32_t st, double x0, double x1) -> uint32_t {
+    const uint32_t e = ((st * (st + 1u)) >> 6) & 1023u;
+    return err_units(entry_d[2 * e], entry_d[2 * e + 1], x0, x1);
+  };
+  // over the 16 lanes of a row: the smallest value (returned), the first lane that holds it, the gap to the runner-up
+  auto row_pick = [&](uint32_t c, uint32_t& first, uint32_t& gap) -> uint32_t {
+    const uint32_t m = row_min16_u32(c);
+    const unsigned long long at_min = __builtin_amdgcn_ballot_w64(c == m);
+    const uint32_t bits = uint32_t(at_min >> (lane & 48u)) & 0xffffu;
+    first = bits ? uint32_t(__builtin_ctz(bits)) : 0u;
+    gap = row_min16_u32(dp == first ? kSat : c) - m;
+    return m;
+  };
+  uint32_t s;
+  {  // step 127: the 16 states (digit << 12) | j_last, one per lane of a row; every row does the same
+    const int t = (2 * (kSteps - 1) + roll) & 255;
+    const double x0 = double(sm.x[t]), x1 = double(sm.x[t + 1]);
+    const uint32_t st = (dp << 12) | j_last;
+    const uint32_t c = sat_add(err_of(st, x0, x1), kept(63, st >> 4));
+    uint32_t k, gap;
+    const uint32_t m = row_pick(c, k, gap);
+    flag |= uint32_t(gap < thr) | uint32_t(m >= 0x80000000u);
+    s = (k << 12) | j_last;
+    if (kSym && k >= 8u) s = 65535u - s;  // the smaller state of the pair
+    if (record && threadIdx.x == 0) sm.st[kSteps - 1] = uint16_t(s);
+  }
+  int set = 0;
+#pragma nounroll
+  for (int it = kSteps - 2; it >= it_min; it -= 2, set ^= 1) {
+    const uint32_t j = s >> 4;
+    const int ta = (2 * (it - 1) + roll) & 255, tb = (2 * it + roll) & 255;
+    const double xa0 = double(sm.x[ta]), xa1 = double(sm.x[ta + 1]);
+    const double xb0 = double(sm.x[tb]), xb1 = double(sm.x[tb + 1]);
+    const uint32_t g = (d << 8) | (j >> 4);
+    const uint32_t s1 = (dp << 12) | g;
+    const uint32_t c1 = sat_add(err_of(s1, xa0, xa1), kept(it / 2 - 1, s1 >> 4));
+    uint32_t k1, gap1;
+    const uint32_t m1 = row_pick(c1, k1, gap1);  // the metric of group g entering step it, as the forward pass had it
+    const uint32_t c0 = sat_add(err_of((d << 12) | j, xb0, xb1), m1);
+    // every lane of row r holds that row's (c0, k1, gap1) for d = 4 wave + r: best and runner-up of the wave's four
+    uint32_t bc = uint32_t(__builtin_amdgcn_readlane(int(c0), 0)), sc = kSat, bd = 4u * wave;
+    uint32_t bd1 = uint32_t(__builtin_amdgcn_readlane(int(k1), 0)), bg = uint32_t(__builtin_amdgcn_readlane(int(gap1), 0));
+#pragma unroll
+    for (int r = 1; r < 4; ++r) {
+      const uint32_t oc = uint32_t(__builtin_amdgcn_readlane(int(c0), 16 * r));
+      const uint32_t od1 = uint32_t(__builtin_amdgcn_readlane(int(k1), 16 * r));
+      const uint32_t og = uint32_t(__builtin_amdgcn_readlane(int(gap1), 16 * r));
+      const bool take = oc < bc;
+      sc = take ? bc : min(sc, oc);
+      bd = take ? 4u * wave + uint32_t(r) : bd;
+      bd1 = take ? od1 : bd1;
+      bg = take ? og : bg;
+      bc = take ? oc : bc;
+    }
+    if (lane == 0) {
+      sm.tr32[set][wave][0] = bc;
+      sm.tr32[set][wave][1] = sc;
+      sm.tr32[set][wave][2] = bd | (bd1 << 8);
+      sm.tr32[set][wave][3] = bg;
+    }
+    __syncthreads();
+    bc = sm.tr32[set][0][0], sc = sm.tr32[set][0][1];
+    uint32_t bdd = sm.tr32[set][0][2];
+    bg = sm.tr32[set][0][3];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const uint32_t oc = sm.tr32[set][w][0], os = sm.tr32[set][w][1];
+      const bool take = oc < bc;
+      sc = take ? min(bc, os) : min(sc, oc);
+      bdd = take ? sm.tr32[set][w][2] : bdd;
+      bg = take ? sm.tr32[set][w][3] : bg;
+      bc = take ? oc : bc;
+    }
+    flag |= uint32_t(sc - bc < thr) | uint32_t(bg < thr) | uint32_t(bc >= 0x80000000u);
+    const uint32_t s_it = ((bdd & 15u) << 12) | j;
+    s = (((bdd >> 8) & 15u) << 12) | (s_it >> 4);
+    if (record && threadIdx.x == 0) {
+      sm.st[it] = uint16_t(s_it);
+      sm.st[it - 1] = uint16_t(s);
+    }
+  }
+  return s;
+}
+
 __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job, const double* __restrict__ entry_d,
                                                                  const float* __restrict__ entry_f,
                                                                  double* __restrict__ hist_all) {
@@ -469,6 +813,25 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
 #pragma nounroll
     for (int pass = 0; pass < 2; ++pass) {
       const int roll = pass == 0 ? kSeq / 2 : 0;
+      bool done = false;
+      if (job.mode == 0) {
+        uint32_t* const hist32 = reinterpret_cast<uint32_t*>(hist);
+        uint32_t flag = 0;
+        if (pass == 0) {
+          forward_pass32<true>(sm, entry_d, roll, -1, hist32, 62);
+          flag |= uint32_t(sm.red32[0][1] < job.margin) | uint32_t(sm.red32[0][0] >= 0x80000000u);
+          const uint32_t s = trace_back32<true>(sm, entry_d, hist32, roll, sm.red32[0][2], 64, false, job.margin, flag);
+          if (!flag && u == 0) sm.overlap = int(s & 0xfffu);  // s is the state of step 63
+        } else {
+          forward_pass32<false>(sm, entry_d, roll, ov, hist32, 0);
+          const uint32_t s = trace_back32<false>(sm, entry_d, hist32, roll, uint32_t(ov), 2, true, job.margin, flag);
+          // s is the state of step 1; at step 0 the one predecessor group with a finite initial metric is ov
+          if (!flag && u == 0) sm.st[0] = uint16_t((s >> 4) | ((uint32_t(ov) >> 8) << 12));
+        }
+        done = !flag;
+        if (flag && u == 0 && job.stats) atomicAdd(job.stats + pass, 1u);
+      }
+      if (!done) {
       forward_pass(sm, entry_d, roll, ov, hist, pass == 0 ? 62 : 0);
       {
         const uint32_t s_last = sm.final_state;  // state of step 127
@@ -483,6 +846,7 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
             sm.st[0] = uint16_t((s >> 4) | ((uint32_t(ov) >> 8) << 12));
           }
         }
+      }
       }
       __syncthreads();
       ov = sm.overlap;

@@ -83,6 +83,23 @@ int qtip_viterbi_tiles_dev(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* 
 int qtip_viterbi_tiles_dev_noalloc(qtip_ctx* ctx, const float* dev_X, long B, uint16_t* dev_states,
                                    uint16_t* dev_packed);
 
+/* How the Viterbi passes of this context (tile calls, LDLQ, groups) keep their path metrics.  No counterpart in the
+ * reference, whose device kernel scores in fp32 with the predecessor tag in the low mantissa bits and is exact most of
+ * the time only (src/viterbi.hip:106-140).
+ * mode 0 (default): each pass runs on unsigned 32-bit metrics first (squared errors formed in fp64 as the CPU
+ * algorithm forms them, src/qtip_core.cpp:123-127, rounded once to units of 2^-26; saturating integer adds), and its
+ * trace-back checks that every decision on the surviving path was won by at least margin_units units, which is more
+ * than the rounding of 128 terms can move two candidates against each other; a pass that fails the check runs again on
+ * fp64 metrics.  The states are those of mode 1 bit for bit.
+ * mode 1: fp64 metrics only (viterbi_ref's own arithmetic, src/qtip_core.cpp:129-164).
+ * margin_units: 0 = the default of 160; values below 129 give up the guarantee (tests only), UINT32_MAX sends every
+ * pass to fp64. */
+int qtip_set_viterbi_mode(qtip_ctx* ctx, int mode, unsigned margin_units);
+/* Passes that mode 0 ran again on fp64 metrics since the context was made (or since the last call with reset != 0):
+ * first passes (free ends, on the rotated sequence) and second passes (tail-biting).  Waits for the device.
+ * Either pointer may be NULL. */
+int qtip_viterbi_stats(qtip_ctx* ctx, unsigned long long* redone_first, unsigned long long* redone_second, int reset);
+
 /* hat[i] = lut[state[i]] (k_decode_states, src/viterbi.hip:231-238): B x 128 states -> B x 256 fp32 */
 int qtip_decode_states_dev(qtip_ctx* ctx, const uint16_t* dev_states, long B, float* dev_hat);
 

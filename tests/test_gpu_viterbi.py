@@ -161,3 +161,47 @@ def test_non_finite_inputs_leave_other_tiles_alone(qz, oracle, hyb):
     st, pk = qz.viterbi_tiles(X)
     assert np.array_equal(st[good], want)
     assert np.array_equal(pk[good], oracle.pack_trellis(want))
+
+
+def test_metric_modes_give_the_same_states(qz, oracle, hyb):
+    """The default runs each pass on 32-bit metrics and repeats it on fp64 metrics when a decision on the surviving
+    path is too close to call; fp64-only, and the default with a margin no decision can reach (every pass repeated),
+    must give the same states, the CPU algorithm's, on raw inputs, fp16-rounded inputs (the LDLQ case) and inputs full
+    of exact ties.  The counters say how many passes were repeated."""
+    say("case: 32-bit-first, fp64-only and all-repeated passes agree")
+    qz.set_tlut(None)
+    rng = np.random.default_rng(11)
+    B = 320
+    X = oracle.rng_normal(4242, B * 256).astype(np.float32).reshape(B, 256)
+    X[64:128] = X[64:128].astype(np.float16).astype(np.float32)           # fp16-representable, as LDLQ feeds them
+    X[128:160] = (X[128:160] * np.float32(0.87)).astype(np.float16).astype(np.float32)
+    X[160:176] = np.round(X[160:176] * 2) / 2                              # coarse grid: many equal errors
+    X[176] = 0.0
+    X[177] = 1.0
+    X[178] = 40.0                                                          # squared errors beyond the 32-bit range
+    X[179, ::2] = -3.0
+    X[180] = X[180] * np.float32(1e-3)
+    X[181:192] = rng.standard_t(3, size=(11, 256)).astype(np.float32) * 2
+    want = oracle.quantize_tiles(hyb, X, fast=True)
+    try:
+        qz.viterbi_stats(reset=True)
+        qz.set_viterbi_mode(0)
+        st0, pk0 = qz.viterbi_tiles(X)
+        r0 = qz.viterbi_stats(reset=True)
+        say("  default: %d first and %d second passes of %d tiles repeated on fp64 metrics" % (r0[0], r0[1], B))
+        qz.set_viterbi_mode(1)
+        st1, pk1 = qz.viterbi_tiles(X)
+        assert qz.viterbi_stats(reset=True) == (0, 0)
+        qz.set_viterbi_mode(0, 0xffffffff)
+        st2, pk2 = qz.viterbi_tiles(X)
+        r2 = qz.viterbi_stats(reset=True)
+    finally:
+        qz.set_viterbi_mode(0)
+    for name, st in (("default", st0), ("fp64 only", st1), ("all repeated", st2)):
+        same = np.all(st == want, axis=1)
+        assert same.all(), "%s: tiles differing from the CPU algorithm: %s" % (name, np.nonzero(~same)[0][:10])
+    assert np.array_equal(pk0, pk1) and np.array_equal(pk0, pk2)
+    assert r2 == (B, B)
+    # near-ties of 2e-6 relative are rare: the bulk of the passes stands on 32-bit metrics (the tie-laden tiles
+    # 160..179 may all be repeated)
+    assert r0[0] <= 40 and r0[1] <= 40
