@@ -10,57 +10,18 @@
 // 256-byte line for every column it touches.  Columns are processed in 16-wide blocks from the last to the first;
 // the residual of a finished block goes to all remaining columns before the next block starts.
 #include "misc.hpp"
+#include "nvfp4_codec.hpp"
 #include "qtip_internal.hpp"
 
 namespace qtipmi {
 namespace {
 
-__device__ __forceinline__ float nv_fp8_dec(unsigned b) {  // non-negative E4M3 code -> value
-  const unsigned e = (b >> 3) & 0xf, m = b & 7;
-  return e == 0 ? ldexpf(float(m), -9) : ldexpf(float(m | 8), int(e) - 10);
-}
-__device__ __forceinline__ unsigned nv_round_even(float v) {
-  const float f = floorf(v), r = v - f;
-  const unsigned n = unsigned(f);
-  return n + unsigned(r > .5f || (r == .5f && (n & 1u)));
-}
-__device__ __forceinline__ unsigned nv_fp8_enc(float x) {  // non-negative finite x, saturating at 448 = code 126
-  x = fminf(fabsf(x), 448.f);
-  if (x < ldexpf(1.f, -6)) return nv_round_even(x * 512.f);
-  int exp;
-  const float frac = frexpf(x, &exp) * 2;
-  unsigned mant = nv_round_even((frac - 1) * 8);
-  int ee = exp + 6;
-  if (mant == 8) {
-    mant = 0;
-    ++ee;
-  }
-  const unsigned c = (unsigned(ee) << 3) | mant;
-  return c < 126u ? c : 126u;
-}
-__device__ __forceinline__ float nv_bf16_round(float f) {
-  uint32_t u = __float_as_uint(f);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return __uint_as_float(u & 0xffff0000u);
-}
-__device__ __forceinline__ float nv_level(int c) {
-  // 0, .5, 1, 1.5, 2, 3, 4, 6
-  return c < 4 ? 0.5f * float(c) : (c < 6 ? float(c - 2) : (c == 6 ? 4.f : 6.f));
-}
-// nearest E2M1 magnitude code of a >= 0, ties to the even code
-__device__ __forceinline__ int nv_fp4_code(float a) {
-  float best = __builtin_inff();
-  int code = 0;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float e = fabsf(a - nv_level(i));
-    if (e < best || (e == best && (i % 2 == 0))) {
-      best = e;
-      code = i;
-    }
-  }
-  return code;
-}
+// the scalar codec (nvfp4_codec.hpp) under the names the kernels use
+__device__ __forceinline__ float nv_fp8_dec(unsigned c) { return nvcodec::e4m3_value(c); }           // code <= 126 -> value
+__device__ __forceinline__ unsigned nv_fp8_enc(float x) { return nvcodec::e4m3_of_magnitude(x); }    // finite x -> code of |x|
+__device__ __forceinline__ float nv_bf16_round(float f) { return nvcodec::through_bf16(f); }
+__device__ __forceinline__ float nv_level(int c) { return nvcodec::e2m1_value(unsigned(c)); }
+__device__ __forceinline__ int nv_fp4_code(float a) { return int(nvcodec::e2m1_of_magnitude(a)); }  // a >= 0
 
 constexpr int kCand = 11;       // scale candidates of the search: the plain one, 8 shrink factors, one code down, one up
 constexpr int kBlockRows = 64;  // matrix rows per workgroup: one per lane

@@ -4,118 +4,119 @@
 #include <cmath>
 #include <cstring>
 
+#include "host_team.hpp"
+#include "nvfp4_codec.hpp"
 #include "quantizer_impl.hpp"
 
 namespace qtipmi {
 namespace {
 
-unsigned round_even(float v) {
-  const float f = std::floor(v), r = v - f;
-  const unsigned n = unsigned(f);
-  return n + unsigned(r > .5f || (r == .5f && (n & 1u)));
-}
-float fp8e4m3_to_f32(uint8_t b) {  // src/common.hpp:81-88
-  const uint32_t s = b >> 7, e = (b >> 3) & 0xf, m = b & 7;
-  float v;
-  if (e == 0) v = std::ldexp(float(m), -9);
-  else if (e == 15 && m == 7) v = NAN;
-  else v = std::ldexp(float(m | 8), int(e) - 10);
-  return s ? -v : v;
-}
-const float kLevels[8] = {0, .5f, 1, 1.5f, 2, 3, 4, 6};
-uint8_t fp4_code(float x) {  // nearest E2M1 value, ties to the even code (src/nvfp4.cpp:27-38)
-  const float a = std::fabs(x);
-  float best = INFINITY;
-  int code = 0;
-  for (int i = 0; i < 8; ++i) {
-    const float e = std::fabs(a - kLevels[i]);
-    if (e < best || (e == best && (i % 2 == 0))) {
-      best = e;
-      code = i;
-    }
-  }
-  return uint8_t(code | (std::signbit(x) ? 8 : 0));
-}
+// one fp32 global scale per matrix: the largest magnitude lands on the largest representable product 448 * 6
 float global_scale(const float* w, size_t numel) {
-  float maximum = 0;
+  float top = 0;
+  bool finite = true;
   for (size_t i = 0; i < numel; ++i) {
-    QTIP_REQUIRE(std::isfinite(w[i]), "nonfinite NVFP4 input");
-    maximum = std::max(maximum, std::fabs(w[i]));
+    const float a = std::fabs(w[i]);
+    finite = finite && a <= 3.4028234663852886e38f;  // false for infinity and NaN
+    top = a > top ? a : top;
   }
-  const float g = maximum ? maximum / (448.f * 6) : 1.f;
-  QTIP_REQUIRE(g > 0 && std::isfinite(g), "NVFP4 global scale underflow/overflow");
+  QTIP_REQUIRE(finite, "NVFP4: the matrix holds a value that is not finite");
+  const float g = top > 0 ? top / (448.f * 6) : 1.f;
+  QTIP_REQUIRE(g > 0 && g <= 3.4028234663852886e38f, "NVFP4: global scale %g is not a positive finite float", double(g));
   return g;
+}
+
+// value of a scale byte as stored: NaN for the two NaN codes, negative for a set sign bit
+inline float scale_byte_value(uint8_t b) {
+  if ((b & 0x7f) == 0x7f) return NAN;
+  const float v = nvcodec::e4m3_value(b & 0x7fu);
+  return b & 0x80 ? -v : v;
 }
 
 }  // namespace
 
 uint8_t f32_to_fp8e4m3(float x) {  // src/nvfp4.hpp:15-33
-  const uint8_t sign = std::signbit(x) ? 128 : 0;
-  if (std::isnan(x)) return uint8_t(sign | 127);
-  x = std::min(std::fabs(x), 448.f);
-  if (x < std::ldexp(1.f, -6)) return uint8_t(sign | round_even(x * 512.f));
-  int exp;
-  const float frac = std::frexp(x, &exp) * 2;
-  unsigned mant = round_even((frac - 1) * 8);
-  int ee = exp + 6;
-  if (mant == 8) {
-    mant = 0;
-    ++ee;
-  }
-  return uint8_t(sign | std::min(126u, (unsigned(ee) << 3) | mant));
+  const uint8_t sign = uint8_t(nvcodec::bits_of(x) >> 31 << 7);
+  if (x != x) return uint8_t(sign | 127);
+  return uint8_t(sign | nvcodec::e4m3_of_magnitude(x));
 }
 
 void nvfp4_quantize_host(const float* w, int m, int n, uint8_t* packed, uint8_t* scales, float* global) {
   QTIP_REQUIRE(w && packed && scales && global && m > 0 && n > 0 && n % 16 == 0, "NVFP4 needs n %% 16 == 0 (m=%d n=%d)", m, n);
-  const size_t numel = size_t(m) * n;
-  const float g = global_scale(w, numel);
+  const long blocks = long(m) * n / 16;
+  const float g = global_scale(w, size_t(blocks) * 16);
   *global = g;
-#pragma omp parallel for schedule(static) if (numel >= (1u << 20))
-  for (size_t b = 0; b < numel / 16; ++b) {
-    float mx = 0;
-    for (int j = 0; j < 16; ++j) mx = std::max(mx, std::fabs(w[b * 16 + j]));
-    const uint8_t sc = f32_to_fp8e4m3(mx / (6 * g));
-    scales[b] = sc;
-    const float scale = fp8e4m3_to_f32(sc) * g;
-    for (int j = 0; j < 16; j += 2)
-      packed[b * 8 + j / 2] = uint8_t(fp4_code(scale ? w[b * 16 + j] / scale : 0) | (fp4_code(scale ? w[b * 16 + j + 1] / scale : 0) << 4));
-  }
+  HostTeam team(blocks >= (1 << 16) ? 16 : 1);
+  team.parallel_for(blocks, 4096, [&](long b) {
+    const float* x = w + b * 16;
+    float top = 0;
+    for (int j = 0; j < 16; ++j) top = std::fmax(top, std::fabs(x[j]));
+    const uint32_t code = nvcodec::e4m3_of_magnitude(top / (6 * g));
+    scales[b] = uint8_t(code);
+    const float unit = nvcodec::e4m3_value(code) * g;
+    uint8_t* out = packed + b * 8;
+    for (int j = 0; j < 8; ++j) {
+      // a zero unit (an all-zero block, or one below the smallest scale) stores plain zeros
+      const float lo = unit ? x[2 * j] / unit : 0.f, hi = unit ? x[2 * j + 1] / unit : 0.f;
+      const uint32_t nl = (nvcodec::bits_of(lo) >> 31 << 3) | nvcodec::e2m1_of_magnitude(std::fabs(lo));
+      const uint32_t nh = (nvcodec::bits_of(hi) >> 31 << 3) | nvcodec::e2m1_of_magnitude(std::fabs(hi));
+      out[j] = uint8_t(nl | (nh << 4));
+    }
+  });
 }
 
 void nvfp4_dequantize_host(const uint8_t* packed, const uint8_t* scales, float global, int m, int n, float* out) {
-  QTIP_REQUIRE(packed && scales && out && m > 0 && n > 0 && n % 16 == 0 && global > 0 && std::isfinite(global),
-               "invalid NVFP4 payload");
-  const size_t numel = size_t(m) * n;
-  bool bad = false;
-#pragma omp parallel for schedule(static) reduction(|| : bad) if (numel >= (1u << 20))
-  for (size_t i = 0; i < numel; ++i) {
-    const uint8_t code = (packed[i / 2] >> (i % 2 * 4)) & 15;
-    const float s = fp8e4m3_to_f32(scales[i / 16]);
-    bad = bad || !(s >= 0 && std::isfinite(s));
-    out[i] = bf16_to_f32(f32_to_bf16((code & 8 ? -1.f : 1.f) * kLevels[code & 7] * s * global));
+  QTIP_REQUIRE(packed && scales && out && m > 0 && n > 0 && n % 16 == 0, "NVFP4 dequantize: bad arguments (m=%d n=%d)", m, n);
+  QTIP_REQUIRE(global > 0 && global <= 3.4028234663852886e38f, "NVFP4 dequantize: global scale %g is not a positive finite float",
+               double(global));
+  const long blocks = long(m) * n / 16;
+  for (long b = 0; b < blocks; ++b) {
+    const float s = scale_byte_value(scales[b]);
+    QTIP_REQUIRE(s >= 0 && s <= 448.f, "NVFP4 dequantize: block %ld has the scale byte 0x%02x (NaN or negative)", b, scales[b]);
   }
-  QTIP_REQUIRE(!bad, "invalid NVFP4 block scale");
+  HostTeam team(blocks >= (1 << 16) ? 16 : 1);
+  team.parallel_for(blocks, 4096, [&](long b) {
+    const float s = scale_byte_value(scales[b]);
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t nib = (packed[b * 8 + j / 2] >> (4 * (j & 1))) & 15u;
+      const float mag = nvcodec::e2m1_value(nib & 7u);
+      out[b * 16 + j] = nvcodec::through_bf16((nib & 8u ? -mag : mag) * s * global);
+    }
+  });
 }
 
+// tr((W - What) H (W - What)^T) / m in fp64.  Four rows of the difference share a pass over H; every row's sums run
+// over ascending columns, and the rows' results are added in row order.
 double nvfp4_proxy_error_host(const float* w, const float* what, int m, int n, const float* H) {
   QTIP_REQUIRE(w && what && m > 0 && n > 0, "nvfp4_proxy_error: bad arguments");
-  double total = 0;
-#pragma omp parallel for reduction(+ : total) schedule(static)
-  for (int r = 0; r < m; ++r) {
-    std::vector<double> e(static_cast<size_t>(n), 0.0);
-    for (int j = 0; j < n; ++j) e[size_t(j)] = double(w[size_t(r) * n + j]) - what[size_t(r) * n + j];
-    double row = 0;
+  constexpr int kRows = 4;
+  const long groups = (long(m) + kRows - 1) / kRows;
+  std::vector<double> per_row(size_t(m), 0.0);
+  HostTeam team(16);
+  team.parallel_for(groups, 1, [&](long gi) {
+    const int r0 = int(gi) * kRows, rows = std::min(kRows, m - r0);
+    std::vector<double> e(size_t(kRows) * n, 0.0);
+    for (int r = 0; r < rows; ++r)
+      for (int j = 0; j < n; ++j) e[size_t(r) * n + j] = double(w[size_t(r0 + r) * n + j]) - double(what[size_t(r0 + r) * n + j]);
+    double quad[kRows] = {0, 0, 0, 0};
     if (!H) {
-      for (int j = 0; j < n; ++j) row += e[size_t(j)] * e[size_t(j)];
+      for (int r = 0; r < rows; ++r)
+        for (int j = 0; j < n; ++j) quad[r] += e[size_t(r) * n + j] * e[size_t(r) * n + j];
     } else {
       for (int i = 0; i < n; ++i) {
-        double acc = 0;
-        for (int j = 0; j < n; ++j) acc += double(H[size_t(i) * n + j]) * e[size_t(j)];
-        row += e[size_t(i)] * acc;
+        const float* hi = H + size_t(i) * n;
+        double dot[kRows] = {0, 0, 0, 0};
+        for (int j = 0; j < n; ++j) {
+          const double h = double(hi[j]);
+          for (int r = 0; r < kRows; ++r) dot[r] += h * e[size_t(r) * n + j];
+        }
+        for (int r = 0; r < kRows; ++r) quad[r] += e[size_t(r) * n + i] * dot[r];
       }
     }
-    total += row;
-  }
+    for (int r = 0; r < rows; ++r) per_row[size_t(r0 + r)] = quad[r];
+  });
+  double total = 0;
+  for (double v : per_row) total += v;
   return total / m;
 }
 

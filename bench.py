@@ -24,6 +24,8 @@ sys.path.insert(0, ROOT)
 
 FLOP_PER_WEIGHT = 393216.0      # 2^16 add-compare-selects per weight, counted as 6 flop each
 PEAK_FP64_TFLOPS = 78.6         # MI355X vector fp64
+PEAK_32BIT_TFLOPS = 157.3       # MI355X vector fp32: the rate of 32-bit lanes, which the u32 path metrics run on
+HBM_BYTES_PER_WEIGHT = 2040.0   # algorithmic HBM traffic of the Viterbi per weight (4-bit back-pointers of two passes + X)
 
 
 def load_pkg():
@@ -127,6 +129,7 @@ def run_viterbi_only(args, pkg):
     import torch
     synth = load_synth()
     q = pkg.Quantizer(0, tlut=synth.synthetic_tlut(1))
+    q.set_viterbi_mode(1 if args.viterbi_fp64 else 0)
     X = torch.from_numpy(synth.splitmix_normal(1234, 4096 * 256).astype(np.float32).reshape(4096, 256)).cuda()
     S = torch.zeros((4096, 128), dtype=torch.int16, device="cuda")
     P = torch.zeros((4096, 32), dtype=torch.int16, device="cuda")
@@ -183,15 +186,56 @@ def run_group(args, pkg):
                          cmp_outs3=res[min(K, 3) - 1][0])
 
     q.reserve_groups(n)   # page-locked staging ring (3 x (HRr, L)); a worker keeps it for its lifetime
+    q.set_viterbi_mode(1 if args.viterbi_fp64 else 0)
     if args.warmup > 0:
         run_steps(args.warmup, False)
     q.synchronize()
     torch.cuda.synchronize()
+    q.viterbi_stats(reset=True)
     t0 = time.time()
     run_steps(args.steps, True)
     q.synchronize()
     torch.cuda.synchronize()
     wall = time.time() - t0
+    redone = q.viterbi_stats(reset=True)   # passes of the timed region that were run again on fp64 metrics
+    tiles_timed = (sum(ms) // 16) * (n // 16) * args.steps
+    vit = dict(viterbi_metrics="fp64" if args.viterbi_fp64 else
+               "u32 in units of 2^-26 (errors formed in fp64), a pass repeated on fp64 metrics when a traced decision "
+               "is won by less than 160 units",
+               viterbi_first_passes_repeated=redone[0], viterbi_second_passes_repeated=redone[1],
+               viterbi_repeated_share=(redone[0] + redone[1]) / (2.0 * tiles_timed))
+    legs = {}
+    if not args.viterbi_fp64 and not args.no_fp64_leg:
+        # beside it (outside the timed region): three groups with fp64 path metrics only, the arithmetic of the CPU
+        # algorithm; every word of the output must be the same
+        kf = min(args.steps, 3)
+        q.set_viterbi_mode(1)
+        q.synchronize()
+        tf = time.time()
+        fres = q.run_groups([(lins, n, H, 3 + k) for k in range(kf)], opt)
+        q.synchronize()
+        tf = time.time() - tf
+        q.set_viterbi_mode(0)
+        legs.update(fp64_metrics_Mweights_s=weights_per_step * kf / tf / 1e6, fp64_metrics_groups=kf,
+                    fp64_metrics_viterbi_s=sum(r[1].viterbi for r in fres) / kf,
+                    fp64_metrics_same_codes=bool(all(np.array_equal(a.trellis, b.trellis) and a.proxy == b.proxy
+                                                     for a, b in zip(fres[-1][0], stats["cmp_outs3"]))))
+        del fres
+    if args.chains == 0 and not args.no_chains2_leg:
+        # beside it: three groups with two LDLQ chains, what a caller gets whose process runs on HIP's default of four
+        # hardware queues (the third chain needs GPU_MAX_HW_QUEUES >= 6 in the environment when the runtime starts)
+        kc = min(args.steps, 3)
+        copt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback,
+                             ldl_device_updates=not args.host_ldl, ldlq_chains=2, group_lanes=args.lanes)
+        q.synchronize()
+        tc = time.time()
+        cres = q.run_groups([(lins, n, H, 3 + k) for k in range(kc)], copt)
+        q.synchronize()
+        tc = time.time() - tc
+        legs.update(chains2_Mweights_s=weights_per_step * kc / tc / 1e6, chains2_groups=kc,
+                    chains2_same_codes=bool(all(np.array_equal(a.trellis, b.trellis) and a.proxy == b.proxy
+                                                for a, b in zip(cres[-1][0], stats["cmp_outs3"]))))
+        del cres
     host_only = {}
     if not args.host_ldl and not args.no_host_ldl_leg:
         # beside it (outside the timed region): the same groups with the block LDL on the host alone, as the
@@ -268,6 +312,8 @@ def run_group(args, pkg):
                  proxy_in_timed_region=True, ldl_threads=args.ldl_threads, feedback=args.feedback,
                  hw_queues=int(os.environ.get("GPU_MAX_HW_QUEUES", "4")), ldlq_chains=nch, group_lanes=lanes,
                  ldl_device_updates=not args.host_ldl)
+    extra.update(vit)
+    extra.update(legs)
     extra.update(host_only)
     extra.update(host_inputs)
     extra.update(fb1)
@@ -276,7 +322,8 @@ def run_group(args, pkg):
     return dict(weights=weights_per_step * args.steps, wall=wall, vit_launch_s=stats["viterbi_s"] / launches,
                 vit_launch_weights=ntr * 256 * 8 * lanes, blocks_per_launch=8, workload=names[cfg] + (" (RHT + host fp64 LDL + LDLQ + 2-pass Viterbi + pack)" if args.host_ldl else
                                        " (RHT + fp64 LDL: host panels, GPU trailing updates + LDLQ + 2-pass Viterbi + pack)"),
-                extra=extra, cpu_group=cpu_group, concurrent=nch * lanes)
+                extra=extra, cpu_group=cpu_group, concurrent=nch * lanes,
+                ldlq_s=stats["ldlq_s"], weights_per_step=weights_per_step)
 
 
 def run_ldl_only(args, pkg):
@@ -358,6 +405,13 @@ def main():
                          "alone; default: 8, and 16 for --config 2).  With HIP's default of 4 the library runs two chains "
                          "of launches per group, with 6 or more three; small groups run side by side on as many lanes "
                          "as there are queues")
+    ap.add_argument("--viterbi-fp64", action="store_true",
+                    help="fp64 path metrics only (default: 32-bit metrics first, a pass repeated on fp64 metrics when a "
+                         "traced decision is too close; same codes)")
+    ap.add_argument("--no-fp64-leg", action="store_true",
+                    help="skip the extra groups with fp64 path metrics only reported beside the default run")
+    ap.add_argument("--no-chains2-leg", action="store_true",
+                    help="skip the extra groups with two LDLQ chains reported beside the default run")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="first run one plain 1 GiB device copy kernel (known traffic, scales the rocprof byte counters)")
     args = ap.parse_args()
@@ -396,34 +450,49 @@ def main():
     traffic, counters = None, {}
     try:
         traffic = json.load(open(os.path.join(ROOT, "profiles", "viterbi_traffic.json"))).get(
-            "config%d_bytes_per_launch" % args.config)
+            "config%d_bytes_per_launch%s" % (args.config, "_fp64" if args.viterbi_fp64 else ""))
     except Exception:
         traffic = None
     if traffic is not None:
         traffic *= res.get("blocks_per_launch", 1)   # the file gives bytes per column block of the group (768 tiles)
     try:
-        counters = json.load(open(os.path.join(ROOT, "profiles", "viterbi_counters.json"))).get("config%d" % args.config, {})
+        counters = json.load(open(os.path.join(ROOT, "profiles", "viterbi_counters.json"))).get(
+            "config%d%s" % (args.config, "_fp64" if args.viterbi_fp64 else ""), {})
     except Exception:
         counters = {}
+    fp64_only = args.viterbi_fp64
+    peak = PEAK_FP64_TFLOPS if fp64_only else PEAK_32BIT_TFLOPS
+    alg_traffic = HBM_BYTES_PER_WEIGHT * res["vit_launch_weights"] / res.get("concurrent", 1)
+    roof = {"bound": "valu", "kernel": "viterbi_tiles_kernel", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+            "frac": achieved / peak,
+            "peak_is": "MI355X vector fp64" if fp64_only else
+                       "MI355X vector rate of 32-bit lanes (the published fp32 figure): the path metrics are u32",
+            "frac_of_fp64_vector_peak": achieved / PEAK_FP64_TFLOPS,
+            # HBM bytes of one launch: measured (rocprofv3 --pmc, offline) against the algorithmic figure
+            "traffic": traffic, "traffic_algorithmic": alg_traffic,
+            "traffic_ratio": (traffic / alg_traffic) if traffic else None,
+            "traffic_source": "profiles/viterbi_traffic.json (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; offline)",
+            "launch_ms": res["vit_launch_s"] * 1e3, "weights_per_launch": res["vit_launch_weights"],
+            "concurrent_launches": res.get("concurrent", 1),
+            "tiles_per_launch": res["vit_launch_weights"] // 256 // res.get("concurrent", 1) // res.get("blocks_per_launch", 1),
+            "column_blocks_per_launch": res.get("blocks_per_launch", 1),
+            "flop_per_weight": FLOP_PER_WEIGHT,
+            "lds_frac": counters.get("lds_active_frac"), "valu_frac": counters.get("valu_busy_frac"),
+            "counters_source": "profiles/viterbi_counters.json (rocprofv3 --pmc SQ_*; offline)"}
+    if res.get("ldlq_s"):
+        # the same algorithmic work over the whole LDLQ stage (gathers included) and over a whole step (everything)
+        roof["frac_ldlq"] = res["weights_per_step"] * FLOP_PER_WEIGHT / res["ldlq_s"] / 1e12 / peak
+        roof["frac_step"] = res["weights_per_step"] * FLOP_PER_WEIGHT / (res["wall"] / args.steps) / 1e12 / peak
     out = {
         "metric": "Mweights/s quantized (RHT+LDLQ+2-pass Viterbi) 12288x28672; % VALU/LDS peak",
         "value": value, "unit": "Mweights/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": res["wall"] / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f64" if fp64_only else "u32", "data": "synthetic",
         "config": dict({"workload": res["workload"]}, **res["extra"]),
         # launch_ms: the average duration of one Viterbi launch (a start and a stop event stamped by every launch of
         # the timed region itself); concurrent_launches of them run side by side, each taking tiles_per_launch tile
         # rows through column_blocks_per_launch column blocks, so weights_per_launch weights pass in that time
-        "roofline": {"bound": "valu", "kernel": "viterbi_tiles_kernel", "achieved": achieved, "peak": PEAK_FP64_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_FP64_TFLOPS, "traffic": traffic,
-                     "traffic_source": "profiles/viterbi_traffic.json (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; offline)",
-                     "launch_ms": res["vit_launch_s"] * 1e3, "weights_per_launch": res["vit_launch_weights"],
-                     "concurrent_launches": res.get("concurrent", 1),
-                     "tiles_per_launch": res["vit_launch_weights"] // 256 // res.get("concurrent", 1) // res.get("blocks_per_launch", 1),
-                     "column_blocks_per_launch": res.get("blocks_per_launch", 1),
-                     "flop_per_weight": FLOP_PER_WEIGHT,
-                     "lds_frac": counters.get("lds_active_frac"), "valu_frac": counters.get("valu_busy_frac"),
-                     "counters_source": "profiles/viterbi_counters.json (rocprofv3 --pmc SQ_*; offline)"},
+        "roofline": roof,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(threads=min(16, os.cpu_count() or 1), group=res.get("cpu_group"))

@@ -59,11 +59,11 @@ def agreement_by_depth(same, nblk, label):
 def test_config3_group_rows_against_reference_chain(qz, pkg, oracle, hyb, synth):
     """Configuration 3 on its own inputs (12288 x 12288, 1 % of the weights x 10, 32 outlier channels) through the group
     call, whose factor comes from the library's default LDL (host panels, trailing updates on the GPU).  The reference
-    chain beside it: block_ldl_to_L of the compiled reference on the same rotated Hessian, then the CPU LDLQ on two
+    chain beside it: block_ldl_to_L of the compiled reference on the same rotated Hessian, then the CPU LDLQ on three
     tile rows.  The two factors must be the same 32-bit words and the codes of those rows identical (>= 99 % is the
-    bar) over all 768 column blocks."""
+    bar) over all 768 column blocks.  Three LDLQ chains are asked for and one tile row of each chain's share is compared."""
     import torch
-    say("case: config 3 through the group call, 32 rows against reference LDL + CPU LDLQ")
+    say("case: config 3 through the group call (three chains), 48 rows against reference LDL + CPU LDLQ")
     qz.set_tlut(None)
     Ws, H = synth.large_config(3)
     n, m = H.shape[0], Ws[0].shape[0]
@@ -75,7 +75,7 @@ def test_config3_group_rows_against_reference_chain(qz, pkg, oracle, hyb, synth)
     diff = int(np.count_nonzero(hp.L.view(np.uint32) != L_ref.view(np.uint32)))
     say("  words of L differing from the reference's factor: %d of %d" % (diff, L_ref.size))
     assert diff == 0
-    outs, tm = qz.quantize_group([pkg.LinearIn("q", m, w_f32=Ws[0])], hp, pkg.QuantOpts(ldl_threads=16))
+    outs, tm = qz.quantize_group([pkg.LinearIn("q", m, w_f32=Ws[0])], hp, pkg.QuantOpts(ldl_threads=16, ldlq_chains=3))
     lo = outs[0]
     say("  ldlq %.1fs viterbi %.1fs (%.1f Mweights/s) proxy %.5f wscale %.6f"
         % (tm.ldlq, tm.viterbi, m * n / tm.viterbi / 1e6, lo.proxy, lo.wscale))
@@ -95,12 +95,12 @@ def test_config3_group_rows_against_reference_chain(qz, pkg, oracle, hyb, synth)
     torch.cuda.synchronize()
     qz.hadamard_rows_dev(AT, n, m, m, True)
     qz.synchronize()
-    rows = np.r_[0:16, 6400:6416]
+    rows = np.r_[0:16, 6400:6416, 11200:11216]                   # tile rows 0, 400, 700: one from each of the three chains
     sub = (AT[:, torch.from_numpy(rows).cuda()] * float(np.float32(1.0) / np.float32(lo.wscale))).T.contiguous().cpu().numpy()
     del AT
     hat_o, Q_o = oracle.ldlq(hyb, sub, L_ref, threads=16)
-    Q_g = st.reshape(m // 16, n // 16, 128)[[0, 400]].reshape(-1, 128)
-    same = np.all(Q_g == Q_o, axis=1).reshape(2, n // 16)
+    Q_g = st.reshape(m // 16, n // 16, 128)[[0, 400, 700]].reshape(-1, 128)
+    same = np.all(Q_g == Q_o, axis=1).reshape(3, n // 16)
     agreement_by_depth(same, n // 16, "config 3")
     say("  identical trellises: %d of %d" % (int(same.sum()), same.size))
     assert same.mean() >= 0.99
@@ -131,43 +131,97 @@ def test_config5_group_properties(qz, pkg, oracle, synth):
     assert hist.min() > 0.04 and hist.max() < 0.09
 
 
-def test_config5_depth_rows_against_reference_chain(qz, pkg, oracle, hyb, synth):
-    """n = 28672, the headline depth: a tile row is a chain of 1792 tiles, each depending on every later column.
-    Product chain: the library's default LDL (host panels, trailing updates on the GPU) of the headline
-    configuration's rotated Hessian, then the GPU LDLQ on two tile rows (LDLQ is row-independent).  Reference chain:
-    block_ldl_to_L of the compiled reference on the same rotated Hessian, then the CPU LDLQ on the same rows.  The
-    factors must be the same 32-bit words and the codes identical (>= 99 % is the bar) down the whole chain."""
+def rotated_scaled_rows(qz, W, sv, su, wscale, rows):
+    """Rows `rows` of Wr / Wscale: Wr^T = U^T_m (U^T_n (diag(SV) W diag(SU)))^T with the library's transform (pinned bit for
+    bit elsewhere), then the fp32 multiplication by 1 / Wscale.  W: m x n device tensor.  Returns a host array."""
     import torch
-    say("case: config-5 depth, own LDL + GPU LDLQ against reference LDL + CPU LDLQ on 32 rows")
+    m, n = W.shape
+    A = W * torch.from_numpy(sv).cuda()[:, None] * torch.from_numpy(su).cuda()[None, :]
+    torch.cuda.synchronize()                                     # the library works on a stream of its own
+    qz.hadamard_rows_dev(A, m, n, n, True)
+    qz.synchronize()
+    AT = A.T.contiguous()
+    del A
+    torch.cuda.synchronize()
+    qz.hadamard_rows_dev(AT, n, m, m, True)
+    qz.synchronize()
+    sub = (AT[:, torch.from_numpy(rows).cuda()] * float(np.float32(1.0) / np.float32(wscale))).T.contiguous()
+    return sub.cpu().numpy(), AT
+
+
+def test_config5_timed_path_rows_against_reference_chain(qz, pkg, oracle, hyb, synth):
+    """The path the benchmark times, at its own size: two 12288 x 28672 groups through qtip_run_groups with W and H
+    handed over as host pointers (loader thread, staging slots), the LDL's trailing updates on the GPU and the factor
+    resident on the device (ring), three LDLQ chains (each with its own split-K gather sums and share of the
+    kept-metrics slots).  n = 28672 is the headline depth: a tile row is a chain of 1792 tiles, each depending on every
+    later column.  Of the second group, one tile row from each chain's share is compared with the reference chain -
+    block_ldl_to_L of the compiled reference on the same rotated Hessian, then the CPU LDLQ on those rows - per depth
+    octile (>= 99 % is the bar); the library's own factor must equal the reference's in every 32-bit word, and the
+    reported proxy errors must agree with an fp64 recomputation over the whole group."""
+    import torch
+    say("case: config 5 through run_groups (host inputs, device-updated LDL, three chains), rows against the reference chain")
     qz.set_tlut(None)
     Ws, H = synth.large_config(5)
-    n, m = H.shape[0], 32
-    W = Ws[0][4000:4000 + m]
-    WT = (W / W.pow(2).mean().sqrt() * 0.9).T.contiguous()        # unit-scale rows at the codebook's working point
-    hp = qz.rotate_hessian(H, n, 3)
-    del Ws, H
+    n, m = H.shape[0], Ws[0].shape[0]
+    Wh, Hh = Ws[0].cpu().numpy(), H.cpu().numpy()
+    opt = pkg.QuantOpts(ldl_threads=16, ldl_device_updates=True, ldlq_chains=3, group_lanes=1)
+    seeds = (21, 22)
+    res = qz.run_groups([([pkg.LinearIn("down", m, w_f32=Wh)], n, Hh, sd) for sd in seeds], opt)
+    (outs, tm, wait) = res[1]
+    lo, seed = outs[0], seeds[1]
+    say("  second group: ldlq %.2fs viterbi %.2fs (%.1f Mweights/s) ldl wait %.3fs proxy %.6f rot_reg %.6f wscale %.6f; "
+        "passes repeated on fp64 metrics: %s" % (tm.ldlq, tm.viterbi, m * n / tm.viterbi / 1e6, wait, lo.proxy,
+                                                  lo.proxy_rot_reg, lo.wscale, qz.viterbi_stats()))
+    st = pkg.unpack_trellis(pkg.unswizzle_for_kernel(lo.trellis, m, n))
+    check_trellis_paths(st)
+    su, sv = pkg.sign_vector(seed, n), pkg.sign_vector(seed * 1000003 + 1, m)
+    assert np.array_equal((lo.su_bf16.astype(np.uint32) << 16).view(np.float32), su) and np.array_equal(lo.sv, sv)
+    # the reference chain's factor, and the library's own (as run_groups forms it) word for word
+    hp = qz.rotate_hessian(H, n, seed)
+    del H, Hh
     qz.ldl_hessian_device_updates(hp, threads=16)
     say("  own factor done; reference block_ldl_to_L on 16 threads ...")
     L_ref = reference_factor(oracle, hp.HRr)
     diff = int(np.count_nonzero(hp.L.view(np.uint32) != L_ref.view(np.uint32)))
     say("  words of L differing from the reference's factor: %d of %d" % (diff, L_ref.size))
-    dL = torch.from_numpy(hp.L).cuda()
-    dH = torch.zeros((n, m), device="cuda")
-    dQ = torch.zeros(((m // 16) * (n // 16), 128), dtype=torch.int16, device="cuda")
-    torch.cuda.synchronize()
-    qz.ldlq_dev(WT, dL, n, m, dH, dQ)
-    qz.synchronize()
-    Q = dQ.cpu().numpy().view(np.uint16)
-    check_trellis_paths(Q)
-    say("  GPU LDLQ done; CPU form on 16 threads ...")
-    hat_o, Q_o = oracle.ldlq(hyb, np.ascontiguousarray(WT.cpu().numpy().T), L_ref, threads=16)
-    same = np.all(Q == Q_o, axis=1).reshape(m // 16, n // 16)
-    agreement_by_depth(same, n // 16, "config 5")
-    say("  identical trellises: %d of %d" % (int(same.sum()), same.size))
     assert diff == 0
+    hp.L = None
+    # one tile row from each chain's share (768 tile rows dealt to three chains: 0..255, 256..511, 512..767)
+    tile_rows = [5, 300, 700]
+    rows = np.concatenate([np.arange(16 * t, 16 * t + 16) for t in tile_rows])
+    sub, AT = rotated_scaled_rows(qz, Ws[0], sv, su, lo.wscale, rows)
+    say("  CPU LDLQ on %d rows x %d columns, 16 threads ..." % (len(rows), n))
+    hat_o, Q_o = oracle.ldlq(hyb, sub, L_ref, threads=16)
+    Q_g = st.reshape(m // 16, n // 16, 128)[tile_rows].reshape(-1, 128)
+    same = np.all(Q_g == Q_o, axis=1).reshape(len(tile_rows), n // 16)
+    for k, t in enumerate(tile_rows):
+        agreement_by_depth(same[k:k + 1], n // 16, "config 5, chain %d (tile row %d)" % (k, t))
+    say("  identical trellises: %d of %d" % (int(same.sum()), same.size))
     assert same.mean() >= 0.99
-    if same.all():
-        assert np.array_equal(dH.cpu().numpy().T, hat_o)
+    # proxy errors over the whole group in fp64: D = Wr / Wscale - decode(trellis), num = tr(D HRr D^T), den likewise
+    del L_ref
+    dT = torch.from_numpy(lo.trellis.view(np.int16)).cuda()
+    hatWr = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    qz.decode_trellis_dev(dT, m, n, hatWr)
+    qz.synchronize()
+    assert np.array_equal(hatWr[torch.from_numpy(rows).cuda()].cpu().numpy()[same.all(axis=1).repeat(16)],
+                          hat_o[same.all(axis=1).repeat(16)])
+    Wr = (AT * float(np.float32(1.0) / np.float32(lo.wscale))).T      # m x n view of the scaled rotated weights
+    HR = torch.from_numpy(hp.HRr).cuda().double()
+    num = den = nd = nw = 0.0
+    for r0 in range(0, m, 2048):
+        w = Wr[r0:r0 + 2048].double()
+        dlt = w - hatWr[r0:r0 + 2048].double()
+        num += float(((dlt @ HR) * dlt).sum())
+        den += float(((w @ HR) * w).sum())
+        nd += float((dlt * dlt).sum())
+        nw += float((w * w).sum())
+    rot_reg = num / den
+    plain = (num - hp.creg * nd) / (den - hp.creg * nw)
+    say("  proxy_rot_reg %.8f (fp64 %.8f), proxy %.8f (fp64 %.8f)" % (lo.proxy_rot_reg, rot_reg, lo.proxy, plain))
+    assert abs(lo.proxy_rot_reg - rot_reg) <= 1e-3 * rot_reg
+    assert abs(lo.proxy - plain) <= 1e-3 * plain
 
 
 def test_config4_two_linears_shared_hessian_rows_against_cpu(qz, pkg, oracle, hyb, synth):
