@@ -101,6 +101,8 @@ def lib():
     L.qtip_viterbi_tiles.argtypes = [vp, vp, l, vp, vp]
     L.qtip_viterbi_tiles_dev.argtypes = [vp, vp, l, vp, vp]
     L.qtip_viterbi_tiles_dev_noalloc.argtypes = [vp, vp, l, vp, vp]
+    L.qtip_trim.argtypes = [vp, C.POINTER(C.c_ulonglong)]
+    L.qtip_selftest_device_alloc_calls.restype = l
     L.qtip_set_viterbi_mode.argtypes = [vp, i, C.c_uint]
     L.qtip_viterbi_stats.argtypes = [vp, C.POINTER(C.c_ulonglong), C.POINTER(C.c_ulonglong), i]
     L.qtip_stream_wait.argtypes = [vp, vp]
@@ -330,9 +332,15 @@ class Quantizer:
         _check(lib().qtip_viterbi_tiles(self._h, _ptr(X), B, _ptr(st), _ptr(pk)))
         return st, pk
 
+    def trim(self):
+        """Idle device memory the context keeps for reuse goes back to the runtime; returns the bytes released."""
+        b = C.c_ulonglong(0)
+        _check(lib().qtip_trim(self._h, C.byref(b)))
+        return int(b.value)
+
     def set_viterbi_mode(self, mode=0, margin_units=0):
         """0: 32-bit metrics first, fp64 again where a traced decision is closer than margin_units (default 160)
-        units of 2^-26; 1: fp64 metrics only.  Same states either way."""
+        units of 2^-25; 1: fp64 metrics only.  Same states either way."""
         _check(lib().qtip_set_viterbi_mode(self._h, int(mode), C.c_uint(int(margin_units))))
 
     def viterbi_stats(self, reset=False):
@@ -701,6 +709,11 @@ class LayerFileWriter:
 
 
 # ---------------------------------------------------------------- host packers
+def device_alloc_calls():
+    """Device allocations (hipMalloc) the library has made in this process so far."""
+    return int(lib().qtip_selftest_device_alloc_calls())
+
+
 def pack_trellis(states):
     states = np.ascontiguousarray(states, np.uint16).reshape(-1, 128)
     out = np.zeros((states.shape[0], 32), np.uint16)

@@ -79,23 +79,27 @@ void run_groups_on(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opt
     dH[size_t(g)] = groups[g].H;
     dl[size_t(g)].assign(groups[g].lins, groups[g].lins + groups[g].nlin);
   }
-  auto upload = [&](int g) {
-    const int b = g % U;
-    hipStream_t us = c->upload_stream;
-    const size_t nn = size_t(groups[g].n) * groups[g].n;
-    if (!groups[g].h_on_device) {
-      c->up_H[b].ensure(nn);
-      QTIP_HIP(hipMemcpyAsync(c->up_H[b].p, groups[g].H, nn * 4, hipMemcpyHostToDevice, us));
-      dH[size_t(g)] = c->up_H[b].p;
-    }
-    auto padded = [](size_t bytes) { return (bytes + 255) / 256 * 256; };
+  auto padded = [](size_t bytes) { return (bytes + 255) / 256 * 256; };
+  // bytes of staging group g's host weights take
+  auto weight_bytes = [&](int g) {
     size_t total = 0;
     for (const qtip_linear_in& l : dl[size_t(g)]) {
       if (l.on_device) continue;
       const size_t mn = size_t(l.m) * size_t(groups[g].n);
       total += padded(l.w_f32 ? mn * 4 : l.w_bf16 ? mn * 2 : mn) + (l.w_fp8 && l.scale_bf16 ? padded(size_t(l.m) * 2) : 0);
     }
-    c->up_W[b].ensure(total);
+    return total;
+  };
+  auto upload = [&](int g) {
+    const int b = g % U;
+    hipStream_t us = c->upload_stream;
+    const size_t nn = size_t(groups[g].n) * groups[g].n;
+    if (!groups[g].h_on_device) {
+      QTIP_REQUIRE(c->up_H[b].n >= nn, "run_groups: staging slot %d too small for the Hessian of group %d", b, g);
+      QTIP_HIP(hipMemcpyAsync(c->up_H[b].p, groups[g].H, nn * 4, hipMemcpyHostToDevice, us));
+      dH[size_t(g)] = c->up_H[b].p;
+    }
+    QTIP_REQUIRE(c->up_W[b].n >= weight_bytes(g), "run_groups: staging slot %d too small for the weights of group %d", b, g);
     size_t at = 0;
     for (qtip_linear_in& l : dl[size_t(g)]) {
       if (l.on_device) continue;
@@ -123,6 +127,17 @@ void run_groups_on(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opt
   std::thread loader;
   if (any_host) {
     if (!c->upload_stream) QTIP_HIP(hipStreamCreateWithFlags(&c->upload_stream, hipStreamNonBlocking));
+    // every slot a group will use is sized here, for the largest group that goes through it, before anything runs:
+    // growing one later would be a hipFree (a wait for the whole device) and a hipMalloc in the middle of the pipeline
+    for (int b = 0; b < std::min(U, ng); ++b) {
+      size_t h_need = 0, w_need = 0;
+      for (int g = b; g < ng; g += U) {
+        if (!groups[g].h_on_device) h_need = std::max(h_need, size_t(groups[g].n) * groups[g].n);
+        w_need = std::max(w_need, weight_bytes(g));
+      }
+      c->up_H[b].ensure(h_need);
+      c->up_W[b].ensure(w_need);
+    }
     loader = std::thread([&] {
       try {
         QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
@@ -138,6 +153,8 @@ void run_groups_on(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opt
           cv.notify_all();
         }
       } catch (...) {
+        // copies queued before the failure still read the caller's memory: they are through before the error is seen
+        (void)hipStreamSynchronize(c->upload_stream);
         std::lock_guard<std::mutex> lk(mu);
         load_err = std::current_exception();
         cv.notify_all();
@@ -146,11 +163,12 @@ void run_groups_on(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opt
   } else {
     loaded = ng;
   }
-  struct JoinLoader {  // whatever ends this call, the loader is told and waited for
+  struct JoinLoader {  // whatever ends this call, the loader is told and waited for, and so are its copies
     std::thread& t;
     std::mutex& mu;
     std::condition_variable& cv;
     bool& stop;
+    hipStream_t& us;
     ~JoinLoader() {
       if (!t.joinable()) return;
       {
@@ -159,8 +177,9 @@ void run_groups_on(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_opt
         cv.notify_all();
       }
       t.join();
+      if (us) (void)hipStreamSynchronize(us);
     }
-  } join_loader{loader, mu, cv, stop};
+  } join_loader{loader, mu, cv, stop, c->upload_stream};
 
   auto rotate = [&](int g) {
     {
@@ -380,7 +399,9 @@ void run_groups_impl(qtip_ctx* c, int ng, const qtip_group* groups, const qtip_o
   qtip_opts lopt = opt;
   lopt.group_lanes = 1;
   lopt.ldlq_chains = 1;  // the other lanes are what runs under a lane's trace-backs; a chain more is a stream more
-  lopt.ldl_threads = std::max(1, opt.ldl_threads / lanes);
+  // ldl_threads <= 0 stands for the machine's hardware concurrency (host_ldl.cpp): resolve it before the lanes share it
+  const int team = opt.ldl_threads > 0 ? opt.ldl_threads : std::max(1, int(std::thread::hardware_concurrency()));
+  lopt.ldl_threads = std::max(1, team / lanes);
   for (int k = 0; k < lanes; ++k) {
     Lane& l = L[size_t(k)];
     l.c = lane_context(c, k);

@@ -100,6 +100,7 @@ qtip_ctx* make_context(int device, const HostCodebook* cb_from) {
 }
 
 void destroy_context(qtip_ctx* ctx) {
+  ctx->arena.children.clear();
   for (qtip_ctx*& l : ctx->lane)
     if (l) {
       destroy_context(l);
@@ -138,6 +139,8 @@ qtip_ctx* lane_context(qtip_ctx* parent, int k) {
     // hardware queue to itself, and a process has few of them (GPU_MAX_HW_QUEUES, 4 unless the environment says
     // more); with a stream more per lane for the factorization 1024 x 1024 groups ran at 59 instead of 134 Mweights/s
     parent->lane[k]->ldl_stream = parent->lane[k]->stream;
+    parent->lane[k]->arena.parent = &parent->arena;
+    parent->arena.children.push_back(&parent->lane[k]->arena);
     parent->lane[k]->vit_mode = parent->vit_mode;
     parent->lane[k]->vit_margin = parent->vit_margin;
   }
@@ -145,6 +148,7 @@ qtip_ctx* lane_context(qtip_ctx* parent, int k) {
 }
 
 void release_lanes(qtip_ctx* parent) {
+  parent->arena.children.clear();
   for (qtip_ctx*& l : parent->lane)
     if (l) {
       destroy_context(l);
@@ -267,6 +271,19 @@ int qtip_get_lut(qtip_ctx* ctx, float* lut0, float* lut1) {
     }
   });
 }
+
+int qtip_trim(qtip_ctx* ctx, unsigned long long* bytes_released) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr, "null context");
+    DeviceGuard g(ctx);
+    unsigned long long total = ctx->arena.trim();
+    for (qtip_ctx* l : ctx->lane)
+      if (l) total += l->arena.trim();
+    if (bytes_released) *bytes_released = total;
+  });
+}
+
+long qtip_selftest_device_alloc_calls(void) { return test_device_alloc_calls(); }
 
 int qtip_set_viterbi_mode(qtip_ctx* ctx, int mode, unsigned margin_units) {
   return guarded([&] {

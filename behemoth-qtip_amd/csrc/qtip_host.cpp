@@ -68,37 +68,46 @@ hipError_t DeviceArena::acquire(void** p, size_t bytes) {
   // nothing idle fits: a new block.  Idle blocks go back to the runtime first when they hold more than 32 GiB (groups
   // of many different shapes would otherwise pile them up), and all of them when the device is out of memory
   const size_t cap = (bytes + 255) / 256 * 256;
-  auto drop_idle = [&] {
-    std::vector<void*> gone;
-    {
-      std::lock_guard<std::mutex> lk(impl->mu);
-      for (size_t i = impl->blocks.size(); i-- > 0;)
-        if (!impl->blocks[i].busy) {
-          gone.push_back(impl->blocks[i].p);
-          impl->blocks.erase(impl->blocks.begin() + long(i));
-        }
-    }
-    for (void* q : gone) (void)hipFree(q);
-  };
-  {
-    size_t idle = 0;
-    {
-      std::lock_guard<std::mutex> lk(impl->mu);
-      for (auto& b : impl->blocks)
-        if (!b.busy) idle += b.cap;
-    }
-    if (idle > (size_t(32) << 30)) drop_idle();
-  }
+  if (idle_bytes() > (size_t(32) << 30)) trim();
   hipError_t rc = device_malloc(p, cap);
   if (rc == hipErrorOutOfMemory) {
+    // the idle blocks of the whole family go back first: a lane's arena may be empty while its parent's or a
+    // sibling's holds the memory of an earlier, larger call
     (void)hipGetLastError();
-    drop_idle();
+    DeviceArena* root = this;
+    while (root->parent) root = root->parent;
+    root->trim();
+    for (DeviceArena* a : root->children) a->trim();
     rc = device_malloc(p, cap);
   }
   if (rc != hipSuccess) return rc;
   std::lock_guard<std::mutex> lk(impl->mu);
   impl->blocks.push_back(Impl::Block{*p, cap, true});
   return hipSuccess;
+}
+size_t DeviceArena::idle_bytes() const {
+  std::lock_guard<std::mutex> lk(impl->mu);
+  size_t idle = 0;
+  for (auto& b : impl->blocks)
+    if (!b.busy) idle += b.cap;
+  return idle;
+}
+size_t DeviceArena::trim() {
+  std::vector<Impl::Block> gone;
+  {
+    std::lock_guard<std::mutex> lk(impl->mu);
+    for (size_t i = impl->blocks.size(); i-- > 0;)
+      if (!impl->blocks[i].busy) {
+        gone.push_back(impl->blocks[i]);
+        impl->blocks.erase(impl->blocks.begin() + long(i));
+      }
+  }
+  size_t bytes = 0;
+  for (auto& b : gone) {
+    (void)hipFree(b.p);
+    bytes += b.cap;
+  }
+  return bytes;
 }
 void DeviceArena::give_back(void* p) {
   // the next user of the block may run on another of the arena's streams: everything queued on them so far is over

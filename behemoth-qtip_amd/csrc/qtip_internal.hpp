@@ -19,7 +19,7 @@ constexpr int kStates = 65536; // L = 16
 constexpr int kGroups = 4096;  // states sharing a successor group
 constexpr int kWords = 32;     // packed u16 words per trellis
 constexpr int kLutEntries = 1024;  // distinct codebook entries: bits 6..15 of s*(s+1)
-// A decision of a 32-bit Viterbi pass stands when it is won by this many units of 2^-26: a metric of at most 128
+// A decision of a 32-bit Viterbi pass stands when it is won by this many units of 2^-25: a metric of at most 128
 // rounded terms is within 64 units of the fp64 one, so two candidates 129 units apart are ordered alike in fp64.
 constexpr uint32_t kViterbiMargin = 160;
 
@@ -60,6 +60,12 @@ struct DeviceArena {
   ~DeviceArena();
   hipError_t acquire(void** p, size_t bytes);
   void give_back(void* p);
+  size_t idle_bytes() const;
+  size_t trim();  // idle blocks back to the runtime; returns their bytes.  An idle block is one whose last user has waited for the arena's streams, so any thread may do this
+  // a lane's arena names its context's arena as parent (set while no lane thread runs): an allocation that finds the
+  // device out of memory trims the whole family before it gives up
+  DeviceArena* parent = nullptr;
+  std::vector<DeviceArena*> children;
   std::vector<hipStream_t*> streams;  // slots holding the streams whose work may use the blocks (null slots are skipped)
   struct Impl;
   Impl* impl;
@@ -243,7 +249,7 @@ struct TileJob {
   // depend on each other only through that row's own hatWT values, so nothing has to wait for another workgroup
   int blocks = 1;
   // 0: both passes run on 32-bit metrics first and a pass whose traced decisions are not all won by `margin` units of
-  // 2^-26 is run again on fp64 metrics (same results as mode 1, bit for bit); 1: fp64 metrics only
+  // 2^-25 is run again on fp64 metrics (same results as mode 1, bit for bit); 1: fp64 metrics only
   int mode = 0;
   uint32_t margin = kViterbiMargin;
   unsigned* stats = nullptr;  // device counters (optional): [0], [1] += passes of the first / second kind run again

@@ -103,11 +103,15 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   // chains: only where every chain still fills its share of the chip.  Default: three where the process was given
   // enough hardware queues for them (context stream, two chain streams, the LDL's stream and the caller's own: with
   // HIP's default of four queues two of these would share one and run one after the other), else two.
-  static const int default_chains = [] {
+  // The library cannot see how many queues the runtime was started with, only what the environment says now, so a
+  // default of three is on probation: the first call that runs three chains looks at its launches' own time stamps
+  // and the context goes back to two for good when the first launches of the chains ran one after the other.
+  static const int env_chains = [] {
     const char* q = getenv("GPU_MAX_HW_QUEUES");
     return q && atoi(q) >= 6 ? 3 : 2;
   }();
-  int nch = chains == 0 ? default_chains : chains;
+  if (c->default_chains == 0) c->default_chains = env_chains;
+  int nch = chains == 0 ? c->default_chains : chains;
   while (nch > 1 && ntr < long(nch) * (c->vit_slots / nch)) --nch;
   struct Chain {
     hipStream_t s;
@@ -141,13 +145,14 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
   Events timed, pacing, joins;  // timed: a (start, stop) pair per Viterbi launch, stamped by the launch itself
   // the other chains start once the caller's inputs and the cleared outputs are there, a third (two thirds) of a
-  // tile's time later; a resident workgroup takes about 1.25 ms for a tile, and a launch walks tiles / slots of them
+  // tile's time later; a launch walks tiles / slots of them
   if (nch > 1) {
     hipEvent_t ready = joins.add(hipEventDisableTiming);
     QTIP_HIP(hipEventRecord(ready, s));
     for (int k = 1; k < nch; ++k) {
       QTIP_HIP(hipStreamWaitEvent(ch[k].s, ready, 0));
-      const double launch_us = 1250.0 * double((ch[k].tiles + ch[k].slots - 1) / ch[k].slots);
+      // (tile_us: what a resident workgroup took per tile in this context's last timed call)
+      const double launch_us = c->vit_tile_us * double((ch[k].tiles + ch[k].slots - 1) / ch[k].slots);
       launch_delay(launch_us * k / nch, ch[k].s);
     }
   }
@@ -225,6 +230,23 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
       t += ms * 1e-3;
     }
     *vit_seconds = t / nch;
+    // per tile and resident workgroup: a launch takes its tile rows through 8 column blocks, tiles / slots rounds of them
+    const size_t launches = timed.ev.size() / 2;
+    if (launches > 0) {
+      const double rounds = double((ch[0].tiles + ch[0].slots - 1) / ch[0].slots);
+      const double tile_us = t / double(launches) / (8.0 * rounds) * 1e6;
+      if (tile_us > 50.0 && tile_us < 20000.0) c->vit_tile_us = tile_us;
+    }
+    // three chains by default, on probation: did the first launches of the chains run side by side?  (One pair of
+    // events per launch, in the order chain 0, 1, 2 of the first buffer.)
+    if (chains == 0 && nch == 3 && !c->chains_checked && timed.ev.size() >= 6) {
+      c->chains_checked = true;
+      float first_ms = 0, start1 = 0, start2 = 0;
+      QTIP_HIP(hipEventElapsedTime(&first_ms, timed.ev[0], timed.ev[1]));
+      QTIP_HIP(hipEventElapsedTime(&start1, timed.ev[0], timed.ev[2]));
+      QTIP_HIP(hipEventElapsedTime(&start2, timed.ev[0], timed.ev[4]));
+      if (start1 >= first_ms || start2 >= first_ms) c->default_chains = 2;  // a chain waited for another's launch to end
+    }
   }
 }
 

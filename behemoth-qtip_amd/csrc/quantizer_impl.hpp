@@ -36,6 +36,9 @@ struct qtip_ctx {
   // so that one chain's trace-backs and gathers run under the others' forward passes
   static constexpr int kMaxChains = 3;
   hipStream_t chain_stream[kMaxChains - 1] = {};
+  int default_chains = 0;       // 0: not decided yet (the environment's queue count decides, then the first call checks)
+  bool chains_checked = false;
+  double vit_tile_us = 800.0;   // a resident Viterbi workgroup's time per tile, from the last timed LDLQ call
   qtipmi::Rht rht;
   qtipmi::DBuf<double> scratch;
   qtipmi::DBuf<uint16_t> hess_img;  // a batch of qtip_hessian_accumulate_dev as the stage images of its update kernel

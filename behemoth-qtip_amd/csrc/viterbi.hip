@@ -462,15 +462,17 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
 
 // ================================================================= the same two passes on 32-bit metrics
 // The fp64 passes above are bound by the issue rate of fp64 vector instructions and, behind it, by 8-byte LDS reads.
-// Both passes are therefore first run on unsigned 32-bit metrics in units of 2^-26: the squared error of a codebook
-// entry is formed in fp64 exactly as above and rounded to the nearest unit once (|error| <= 1/2 unit), the adds are
-// integer adds that saturate at 2^32 - 1 (= 64.0, which also stands for +inf), so a path metric of n terms differs from
-// the fp64 one by at most n/2 units, whatever the path.  Only the decisions on the surviving path matter: the
+// Both passes are therefore first run on unsigned 32-bit metrics in units of 2^-25: the squared error of a codebook
+// entry is formed in fp64 exactly as above and rounded to the nearest unit once (|error| <= 1/2 unit); errors and
+// metrics are held to 2^31 - 1 (= 64.0, which also stands for +inf: every chain of minima starts from it), so the adds
+// are plain integer adds that cannot wrap, and a path metric of n terms differs from the fp64 one by at most n/2
+// units, whatever the path.  Only the decisions on the surviving path matter: the
 // trace-back redoes them from the kept metrics as above and also looks at the runner-up.  If every decision it takes
 // (the final state, and the 16-way choice of each step it walks) is won by at least `thr` > 128 units and the winner is
-// below 2^31, the fp64 recursion takes the same decisions and the pass's result is the fp64 result.  Otherwise the
+// below 2^30 (32.0: nothing on its path was cut off at 64.0), the fp64 recursion takes the same decisions and the
+// pass's result is the fp64 result.  Otherwise the
 // workgroup runs that pass again through the fp64 code above (a fraction of a percent of the passes: near-ties of
-// 2e-6 relative, and the exact ties between states that share predecessor and codebook entry).
+// 5e-6, and the exact ties between states that share predecessor and codebook entry).
 // Integer adds issue at twice the rate of fp64 adds on this chip and a three-way minimum covers two candidates, so an
 // add-compare-select costs 1.5 instructions of 4.5 ns per pair instead of 2 of 8.2 ns; the table and the metrics are
 // 4 bytes, half the LDS traffic, and the kept metrics half the HBM traffic.
@@ -488,7 +490,8 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
 // conflicts.  The metric of (column, digit d) sits at pos(column) * 16 + (d ^ swz(column)) with swz a multiple of 4,
 // so a column comes in as four 16-byte reads; pos and swz are chosen so that those reads, the 4-byte writes of a
 // group's result (32 lanes: 4 columns x 8 digits) and of its mirror (slot ^ 0xfeb) are free of bank conflicts.
-constexpr uint32_t kSat = 0xffffffffu;
+constexpr uint32_t kSat = 0x7fffffffu;      // 64.0: the largest metric, and +inf
+constexpr uint32_t kWinnerMax = 0x40000000u;  // 32.0: a decision's winner must be below this
 constexpr int kMirror32 = 0xfeb;
 static_assert(64 * kGroups <= 2 * kHistWordsPerTile, "the 32-bit kept metrics (64 steps) must fit the fp64 slot");
 
@@ -509,18 +512,19 @@ __device__ __forceinline__ uint32_t hist32_index(uint32_t g) {
   const uint32_t jj = g < 2048u ? g : 4095u - g;
   return ((jj & 7u) + ((kSym || g < 2048u) ? 0u : 8u)) * kThreads + owner32(jj);
 }
-__device__ __forceinline__ uint32_t sat_add(uint32_t a, uint32_t b) { return __builtin_elementwise_add_sat(a, b); }
+// metrics and errors are at most kSat = 2^31 - 1, so a plain add cannot wrap; every chain of minima starts from kSat
+__device__ __forceinline__ uint32_t sat_add(uint32_t a, uint32_t b) { return a + b; }
 __device__ __forceinline__ uint32_t min3u(uint32_t a, uint32_t b, uint32_t c) {
   uint32_t r;  // written out: the compiler forms the three-way minimum for only half of the chains
   asm("v_min3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
 }
 // squared error of a codebook entry against the two inputs of a step, the fp64 value of the passes above in units of
-// 2^-26, rounded to nearest; 64.0 and more (and NaN) become 2^32 - 1
+// 2^-25, rounded to nearest; 64.0 and more (and NaN) become 2^31 - 1
 __device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, double x1) {
   const double a = l0 - x0, b = l1 - x1;
-  const double v = __builtin_rint(__builtin_fma(a, a, b * b) * 67108864.0);
-  return uint32_t(__builtin_fmin(v, 4294967295.0));
+  const double v = __builtin_rint(__builtin_fma(a, a, b * b) * 33554432.0);
+  return uint32_t(__builtin_fmin(v, 2147483647.0));
 }
 
 // One forward pass on 32-bit metrics.  kSym: free ends, the groups below 2048 only (their mirrors get copies), all
@@ -602,22 +606,28 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
 #if !QTIP_V_TABLE_LATE
     if constexpr (kind != kDigits) table(it + 1);
 #endif
+    // the 16 table values of a slot are fetched while the slot before it is worked on
+    uint32_t evb[2][16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) evb[0][k] = Er[ebase[0] + k * 64];  // slot 0: stride 1
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
-      const int g = 2 * m + 1;
-      const uint32_t* er = Er + ebase[m];
-      uint32_t ev[16];
+      if (m < 7) {
+        const int gn = 2 * (m + 1) + 1;
+        const uint32_t* er = Er + ebase[m < 7 ? m + 1 : 7];
 #pragma unroll
-      for (int k = 0; k < 16; ++k) ev[k] = er[((k * g) & 15) * 64];
+        for (int k = 0; k < 16; ++k) evb[(m + 1) & 1][k] = er[((k * gn) & 15) * 64];
+      }
+      const uint32_t* ev = evb[m & 1];
       // the table value at position k is the candidate of digit k of the group and of digit 15 - k of its mirror
-      uint32_t ba = min(sat_add(ev[0], MA[0]), sat_add(ev[1], MA[1]));
+      uint32_t ba = kSat;
 #pragma unroll
-      for (int k = 1; k < 8; ++k) ba = min3u(ba, sat_add(ev[2 * k], MA[2 * k]), sat_add(ev[2 * k + 1], MA[2 * k + 1]));
+      for (int k = 0; k < 8; ++k) ba = min3u(ba, sat_add(ev[2 * k], MA[2 * k]), sat_add(ev[2 * k + 1], MA[2 * k + 1]));
       uint32_t bb = ba;
       if constexpr (!kSym) {
-        bb = min(sat_add(ev[0], MB[15]), sat_add(ev[1], MB[14]));
+        bb = kSat;
 #pragma unroll
-        for (int k = 1; k < 8; ++k)
+        for (int k = 0; k < 8; ++k)
           bb = min3u(bb, sat_add(ev[2 * k], MB[15 - 2 * k]), sat_add(ev[2 * k + 1], MB[14 - 2 * k]));
       }
       if constexpr (kind == kDigits) {
@@ -694,7 +704,7 @@ __device__ __forceinline__ uint32_t row_min16_u32(uint32_t c) {
 // Trace-back of a 32-bit pass, the scheme of trace_back above with the runner-up of every decision looked at as well.
 // j_last: low 12 bits of the final state (the group the pass ends in).  The decision of step 127 is taken from the
 // metrics entering it (kept slot 63), then two steps per round trip.  flag is raised (in every thread alike) when a
-// decision is won by less than thr units or the winner is not below 2^31.
+// decision is won by less than thr units or the winner is not below 2^30.
 // Returns the state of step it_min - 1; record: the states of the steps walked are written to sm.st.
 template <bool kSym>
 __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restrict__ entry_d,
@@ -728,7 +738,7 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
     const uint32_t c = sat_add(err_of(st, x0, x1), kept(63, st >> 4));
     uint32_t k, gap;
     const uint32_t m = row_pick(c, k, gap);
-    flag |= uint32_t(gap < thr) | uint32_t(m >= 0x80000000u);
+    flag |= uint32_t(gap < thr) | uint32_t(m >= kWinnerMax);
     s = (k << 12) | j_last;
     if (kSym && k >= 8u) s = 65535u - s;  // the smaller state of the pair
     if (record && threadIdx.x == 0) sm.st[kSteps - 1] = uint16_t(s);
@@ -744,7 +754,8 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
     const uint32_t s1 = (dp << 12) | g;
     const uint32_t c1 = sat_add(err_of(s1, xa0, xa1), kept(it / 2 - 1, s1 >> 4));
     uint32_t k1, gap1;
-    const uint32_t m1 = row_pick(c1, k1, gap1);  // the metric of group g entering step it, as the forward pass had it
+    // the metric of group g entering step it, as the forward pass had it
+    const uint32_t m1 = min(row_pick(c1, k1, gap1), kSat);
     const uint32_t c0 = sat_add(err_of((d << 12) | j, xb0, xb1), m1);
     // every lane of row r holds that row's (c0, k1, gap1) for d = 4 wave + r: best and runner-up of the wave's four
     uint32_t bc = uint32_t(__builtin_amdgcn_readlane(int(c0), 0)), sc = kSat, bd = 4u * wave;
@@ -780,7 +791,7 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
       bg = take ? sm.tr32[set][w][3] : bg;
       bc = take ? oc : bc;
     }
-    flag |= uint32_t(sc - bc < thr) | uint32_t(bg < thr) | uint32_t(bc >= 0x80000000u);
+    flag |= uint32_t(sc - bc < thr) | uint32_t(bg < thr) | uint32_t(bc >= kWinnerMax);
     const uint32_t s_it = ((bdd & 15u) << 12) | j;
     s = (((bdd >> 8) & 15u) << 12) | (s_it >> 4);
     if (record && threadIdx.x == 0) {
@@ -819,7 +830,7 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
         uint32_t flag = 0;
         if (pass == 0) {
           forward_pass32<true>(sm, entry_d, roll, -1, hist32, 62);
-          flag |= uint32_t(sm.red32[0][1] < job.margin) | uint32_t(sm.red32[0][0] >= 0x80000000u);
+          flag |= uint32_t(sm.red32[0][1] < job.margin) | uint32_t(sm.red32[0][0] >= kWinnerMax);
           const uint32_t s = trace_back32<true>(sm, entry_d, hist32, roll, sm.red32[0][2], 64, false, job.margin, flag);
           if (!flag && u == 0) sm.overlap = int(s & 0xfffu);  // s is the state of step 63
         } else {

@@ -87,7 +87,7 @@ int qtip_viterbi_tiles_dev_noalloc(qtip_ctx* ctx, const float* dev_X, long B, ui
  * reference, whose device kernel scores in fp32 with the predecessor tag in the low mantissa bits and is exact most of
  * the time only (src/viterbi.hip:106-140).
  * mode 0 (default): each pass runs on unsigned 32-bit metrics first (squared errors formed in fp64 as the CPU
- * algorithm forms them, src/qtip_core.cpp:123-127, rounded once to units of 2^-26; saturating integer adds), and its
+ * algorithm forms them, src/qtip_core.cpp:123-127, rounded once to units of 2^-25; integer adds, values held to 2^31 - 1), and its
  * trace-back checks that every decision on the surviving path was won by at least margin_units units, which is more
  * than the rounding of 128 terms can move two candidates against each other; a pass that fails the check runs again on
  * fp64 metrics.  The states are those of mode 1 bit for bit.
@@ -329,6 +329,17 @@ int qtip_st_write(qtip_st_writer* w, const char* path, const char* const* metada
                   uint64_t* bytes_written);
 /* fp16 bits of the context's codebook table [512][2] (Codebook::tlut_h, src/qtip_core.hpp:24-31) */
 int qtip_get_tlut_f16(qtip_ctx* ctx, uint16_t* host_tlut_f16);
+
+/* Device memory the context keeps between calls for reuse (per-group buffers of qtip_run_groups and
+ * qtip_quantize_group*, about 13 GB after 12288 x 28672 groups, and the same per lane) goes back to the runtime;
+ * buffers in use are not touched.  No counterpart in the reference, whose buffers are freed on return
+ * (RAII DBuf, src/gpu.hpp:139-160).  The library does the same by itself when an allocation finds the device out of
+ * memory.  *bytes_released may be NULL.  Must not overlap another call on the same context. */
+int qtip_trim(qtip_ctx* ctx, unsigned long long* bytes_released);
+
+/* Host-only: the number of device allocations (hipMalloc) the library has made in this process so far; a test of
+ * qtip_viterbi_tiles_dev_noalloc reads it before and after the call.  No counterpart in the reference. */
+long qtip_selftest_device_alloc_calls(void);
 
 /* Host-only self test (no GPU needed, no counterpart in the reference): a device buffer of the context whose
  * allocation failed stays empty, so the next call allocates again instead of launching on a null pointer.  0 = ok. */

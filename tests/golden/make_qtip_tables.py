@@ -6,7 +6,10 @@ reference carries as data (src/qtip_constants.hpp) and re-encodes them in this
 library's own compact form: each Hadamard row is bit-packed (bit k of the row
 word array set <=> entry +1), the tlut is kept as fp32 bit patterns.
 
-usage: gen_tables.py /root/reference/src/qtip_constants.hpp > qtip_tables.h
+It sits beside the other provenance scripts of committed data (the make_ref_* scripts of this folder); the header it
+writes lives with the library, behemoth-qtip_amd/csrc/data/qtip_tables.h.
+
+usage: make_qtip_tables.py /root/reference/src/qtip_constants.hpp > behemoth-qtip_amd/csrc/data/qtip_tables.h
 """
 import re
 import sys
@@ -17,7 +20,7 @@ def main():
     order = [int(v) for v in re.search(r"kHadOrder\[\d+\]\s*=\s*\{([^}]*)\}", src).group(1).split(",")]
     out = []
     out.append("/* Hadamard factor matrices (bit-packed rows, bit set = +1) and the default HYB tlut")
-    out.append(" * (fp32 bit patterns, [512][2]).  Data only; generated by gen_tables.py. */")
+    out.append(" * (fp32 bit patterns, [512][2]).  Data only; written by tests/golden/make_qtip_tables.py. */")
     out.append("#ifndef QTIP_TABLES_H_")
     out.append("#define QTIP_TABLES_H_")
     out.append("#include <stdint.h>")

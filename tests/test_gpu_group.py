@@ -207,7 +207,7 @@ def test_group_small_end_to_end(qz, oracle, pkg, hyb, synth):
         m = lo.m
         words = (m // 16) * (n // 16) * 32
         want = ref["trellis"][off // 16 * (n // 16) * 32: off // 16 * (n // 16) * 32 + words]
-        tiles_same = np.all(lo.trellis.reshape(-1, 32) == _deswz(pkg, want, lo.trellis, m, n), axis=1).mean()
+        tiles_same = np.all(lo.trellis.reshape(-1, 32) == want.reshape(-1, 32), axis=1).mean()
         say("  %s: proxy %.5f (cpu %.5f) rot_reg %.5f Wscale %.6f (cpu %.6f) tiles identical %.4f" %
             (lo.name, lo.proxy, ref["proxy"][k], lo.proxy_rot_reg, lo.wscale, ref["wscale"][k], tiles_same))
         assert lo.trellis.size == words
@@ -224,11 +224,6 @@ def test_group_small_end_to_end(qz, oracle, pkg, hyb, synth):
         assert np.max(np.abs(hat - lo.hatW)) < 1e-5 * max(1.0, np.max(np.abs(hat)) / 1e-2)
         off += m
     assert tm.total > 0 and tm.ldlq > 0 and tm.viterbi > 0
-
-
-def _deswz(pkg, want, got, m, n):
-    # both in kernel layout: compare tile-wise after undoing the swizzle
-    return pkg.unswizzle_for_kernel(want, m, n).reshape(-1, 32) if False else want.reshape(-1, 32)
 
 
 def test_ldlq_chains_give_the_same_codes(qz, oracle, pkg, hyb):

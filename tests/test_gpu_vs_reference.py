@@ -146,13 +146,16 @@ def test_config2_vs_reference_device_group(qz, pkg, ref, hyb, synth):
             assert agree >= 0.99
 
 
-def test_config5_vs_reference_device_group(qz, pkg, ref, synth):
-    """The headline shape (12288 x 28672 down-proj group, rank-deficient damped Hessian) through the reference's device
-    path and through this library on the same host arrays: sign vectors and Wscale equal, proxy within 1 %.  Each of
-    the 768 tile rows is a chain of 1792 tiles in which every tile depends on all later columns, so the first rounding
-    that falls differently (the two host LDL codes differ in the last bit of a few entries of L, the two cross-buffer
-    GEMMs in their summation order) changes the rest of that chain: the share of identical tiles is reported per
-    depth, and only the chains' starts (the last 128-column buffer, which no GEMM has touched) are held to 99 %."""
+def test_config5_prefix_and_proxy_vs_reference_device_group(qz, pkg, ref, synth):
+    """A prefix-and-proxy check, not a code-agreement check: the headline shape (12288 x 28672 down-proj group,
+    rank-deficient damped Hessian) through the reference's DEVICE path and through this library on the same host arrays.
+    The device path is not the accuracy target (the CPU chain is, and tests/test_gpu_fullsize.py holds the library to
+    it over the full depth): it feeds back in fp32, so along a chain of 1792 tiles, each depending on all later columns,
+    its own roundings fall differently from the CPU algorithm's (and from this library's) sooner or later, and the rest
+    of that tile row's chain then differs.  Asserted: sign vectors and Wscale equal, both proxy errors within 1 % of the
+    device path's (the bound the comparison prints), and the chains' starts - the last 128-column buffer, which no
+    cross-buffer GEMM has touched - identical in at least 99 % of the tiles.  The share of identical tiles by depth is
+    printed for the record."""
     say("case: config 5 vs reference device group (12288 x 28672)")
     qz.set_tlut(None)
     Ws, H = synth.large_config(5)

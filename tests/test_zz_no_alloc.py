@@ -41,6 +41,27 @@ def test_noalloc_equals_allocating_entry_point(qz, pkg, oracle, hyb):
         assert np.array_equal(st[idx], oracle.quantize_tiles(hyb, X[idx], fast=True))
 
 
+def test_noalloc_call_allocates_nothing(qz, pkg, oracle):
+    """The property the entry point exists for: across the call the library makes no device allocation (its own
+    counter of hipMalloc calls) and the device's free memory does not move."""
+    import torch
+    say("case: no-alloc Viterbi makes no device allocation")
+    qz.set_tlut(None)
+    B = 96
+    X = oracle.rng_normal(77, B * 256).astype(np.float32).reshape(B, 256)
+    dX = torch.from_numpy(X).cuda()
+    dS = torch.zeros((B, 128), dtype=torch.int16, device="cuda")
+    dP = torch.zeros((B, 32), dtype=torch.int16, device="cuda")
+    torch.cuda.synchronize()
+    calls0, free0 = pkg.device_alloc_calls(), torch.cuda.mem_get_info()[0]
+    qz.viterbi_tiles_dev_noalloc(dX, B, dS, dP)
+    qz.synchronize()
+    calls1, free1 = pkg.device_alloc_calls(), torch.cuda.mem_get_info()[0]
+    assert calls1 == calls0, "the call made %d device allocations" % (calls1 - calls0)
+    assert free1 == free0, "free device memory moved by %d bytes across the call" % (free0 - free1)
+    # (the allocating entry point, by contrast, is allowed to: its workspace comes from hipMalloc on first use)
+
+
 def test_noalloc_limits(qz, pkg):
     import torch
     say("case: no-alloc Viterbi, B = 0 and B above the limit")
