@@ -453,8 +453,6 @@ def main():
             "config%d_bytes_per_launch%s" % (args.config, "_fp64" if args.viterbi_fp64 else ""))
     except Exception:
         traffic = None
-    if traffic is not None:
-        traffic *= res.get("blocks_per_launch", 1)   # the file gives bytes per column block of the group (768 tiles)
     try:
         counters = json.load(open(os.path.join(ROOT, "profiles", "viterbi_counters.json"))).get(
             "config%d%s" % (args.config, "_fp64" if args.viterbi_fp64 else ""), {})
