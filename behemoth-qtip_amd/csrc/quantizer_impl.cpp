@@ -251,20 +251,27 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
 }
 
 // ---------------------------------------------------------------- quantize_group, src/quantizer.cpp:176-346
-void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
-                         double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
-                         qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr, const float* dev_L) {
-  QTIP_REQUIRE(nlin > 0 && lins && outs && host_su && host_L, "quantize_group: bad arguments");
+// In three phases: prepare (weights -> rotated, scaled Wr^T, Wscale), LDLQ + Viterbi, finish (proxy errors, packing,
+// optional reconstruction); each is synchronous on return.  (A scheduler that ran the first and the last phase of
+// neighbouring groups on a second context beside a group's LDLQ was built on this split and measured: the proxy's
+// matrix-core kernel, 256 accumulators and 64 KB of LDS per workgroup, takes the place of two Viterbi workgroups
+// wherever it gets in and takes 1.39 s instead of 0.067 s; with only the rotation and the weight transform run ahead
+// those take 0.99 s instead of 0.02 s.  210.8 and 212.0 Mweights/s against 215-217 with the phases one after the
+// other on one stream: the chip has no idle capacity beside the Viterbi launches.)
+void group_prepare(qtip_ctx* c, GroupWork& w, int nlin, const qtip_linear_in* lins, int n, uint64_t seed,
+                   const float* host_su, const qtip_opts& opt, qtip_linear_out* outs, const qtip_timing* tm) {
+  QTIP_REQUIRE(nlin > 0 && lins && outs && host_su, "quantize_group: bad arguments");
   QTIP_REQUIRE(n % 128 == 0, "LDLQ needs n %% 128 == 0 (n = %d)", n);
   QTIP_REQUIRE(had_K(n) > 0 && n / had_K(n) <= 8192, "unsupported hadamard dim %d", n);
-  QTIP_REQUIRE(opt.skip_proxy || host_HRr || dev_HRr, "quantize_group: HRr is needed for the proxy");
   hipStream_t s = c->stream;
-  qtip_timing T{};
+  qtip_timing& T = w.T;
+  T = qtip_timing{};
   if (tm) T.rht = tm->rht, T.ldl_cpu = tm->ldl_cpu;
-  const double t_start = now_s();
-  double t0 = t_start;
+  w.t_start = now_s();
+  w.carried = (tm ? tm->rht : 0.0);
+  double t0 = w.t_start;
   long mt = 0, maxm = 0;
-  std::vector<long> off;
+  w.off.clear();
   for (int li = 0; li < nlin; ++li) {
     const qtip_linear_in& l = lins[li];
     QTIP_REQUIRE(l.m > 0 && l.m % 32 == 0 && n % 32 == 0, "kernel layout needs m, n multiples of 32 (m=%d n=%d)", l.m, n);
@@ -272,15 +279,20 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
     QTIP_REQUIRE((l.w_f32 != nullptr) + (l.w_bf16 != nullptr) + (l.w_fp8 != nullptr) == 1,
                  "linear %d: exactly one of w_f32 / w_bf16 / w_fp8 must be set", li);
     QTIP_REQUIRE(outs[li].trellis && outs[li].su_bf16 && outs[li].sv, "linear %d: output buffers missing", li);
-    off.push_back(mt);
+    w.off.push_back(mt);
     mt += l.m;
     maxm = std::max<long>(maxm, l.m);
   }
-  DBuf<float> d_su{size_t(n)}, d_sv{size_t(mt)};
+  w.mt = mt;
+  const std::vector<long>& off = w.off;
+  w.d_su.alloc(size_t(n));
+  w.d_sv.alloc(size_t(mt));
+  DBuf<float>&d_su = w.d_su, &d_sv = w.d_sv;
   QTIP_HIP(hipMemcpyAsync(d_su, host_su, size_t(n) * 4, hipMemcpyHostToDevice, s));
 
   // ---- weights -> Wr^T (n x mt), each linear's column block scaled by 1/Wscale (src/quantizer.cpp:195-249)
-  DBuf<float> WT(size_t(n) * mt);
+  w.WT.alloc(size_t(n) * mt);
+  DBuf<float>& WT = w.WT;
   {
     DBuf<float> Wt(size_t(maxm) * n);
     DBuf<uint8_t> raw;
@@ -325,24 +337,39 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
       t0 = now_s();
     }
   }
+}
 
+void group_ldlq(qtip_ctx* c, GroupWork& w, int n, const float* host_L, const float* dev_L, const qtip_opts& opt) {
+  QTIP_REQUIRE(host_L || dev_L, "quantize_group: no factor");
+  hipStream_t s = c->stream;
+  qtip_timing& T = w.T;
+  const long mt = w.mt;
+  double t0 = now_s();
   // the factor: the caller's device copy if it kept one, else uploaded
   DBuf<float> Ld(dev_L ? 0 : size_t(n) * n);
   if (!dev_L) QTIP_HIP(hipMemcpyAsync(Ld, host_L, size_t(n) * n * 4, hipMemcpyHostToDevice, s));
   QTIP_HIP(hipStreamSynchronize(s));
   T.load += now_s() - t0;
   t0 = now_s();
-
-  // ---- LDLQ + Viterbi
-  DBuf<float> hatWT(size_t(n) * mt);
-  DBuf<uint16_t> Q(size_t(mt / 16) * (n / 16) * 128);
+  w.hatWT.alloc(size_t(n) * mt);
+  w.Q.alloc(size_t(mt / 16) * (n / 16) * 128);
   double vit = 0;
-  ldlq_impl(c, WT, dev_L ? dev_L : Ld.p, n, mt, hatWT, Q, opt.feedback, &vit, opt.ldlq_chains);
+  ldlq_impl(c, w.WT, dev_L ? dev_L : Ld.p, n, mt, w.hatWT, w.Q, opt.feedback, &vit, opt.ldlq_chains);
   T.ldlq += now_s() - t0;
   T.viterbi += vit;
-  t0 = now_s();
-  Ld.release();
+}
 
+void group_finish(qtip_ctx* c, GroupWork& w, int nlin, const qtip_linear_in* lins, int n, double creg,
+                  const float* host_HRr, const float* dev_HRr, const qtip_opts& opt, qtip_linear_out* outs,
+                  qtip_timing* tm) {
+  QTIP_REQUIRE(opt.skip_proxy || host_HRr || dev_HRr, "quantize_group: HRr is needed for the proxy");
+  hipStream_t s = c->stream;
+  qtip_timing& T = w.T;
+  const long mt = w.mt;
+  const std::vector<long>& off = w.off;
+  DBuf<float>&WT = w.WT, &hatWT = w.hatWT, &d_su = w.d_su, &d_sv = w.d_sv;
+  DBuf<uint16_t>& Q = w.Q;
+  double t0 = now_s();
   // ---- proxy (rotated, scaled domain; Wscale cancels), src/quantizer.cpp:268-303
   if (!opt.skip_proxy) {
     // the rotated Hessian: the caller's device copy if it kept one, else uploaded
@@ -395,11 +422,23 @@ void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int 
     QTIP_HIP(hipStreamSynchronize(s));
   }
   T.pack += now_s() - t0;
-  T.total = (now_s() - t_start) + (tm ? tm->rht : 0.0) + T.ldl_cpu;
+  T.total = (now_s() - w.t_start) + w.carried + T.ldl_cpu;
   double wsum = 0;
   for (int li = 0; li < nlin; ++li) wsum += double(lins[li].m) * n;
   for (int li = 0; li < nlin; ++li) outs[li].seconds = T.total * double(lins[li].m) * n / wsum;
   if (tm) *tm = T;
+  w.release();
+}
+
+void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
+                         double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
+                         qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr, const float* dev_L) {
+  QTIP_REQUIRE(host_L != nullptr, "quantize_group: bad arguments");
+  QTIP_REQUIRE(opt.skip_proxy || host_HRr || dev_HRr, "quantize_group: HRr is needed for the proxy");
+  GroupWork w;
+  group_prepare(c, w, nlin, lins, n, seed, host_su, opt, outs, tm);
+  group_ldlq(c, w, n, host_L, dev_L, opt);
+  group_finish(c, w, nlin, lins, n, creg, host_HRr, dev_HRr, opt, outs, tm);
 }
 
 }  // namespace qtipmi

@@ -32,6 +32,7 @@ struct qtip_ctx {
   // (streams, workspaces, rings) made on first use, kept here and released with this context
   static constexpr int kMaxLanes = 12;
   qtip_ctx* lane[kMaxLanes] = {};
+
   // LDLQ runs its tile rows as up to kMaxChains independent chains of launches, on the context's stream and these,
   // so that one chain's trace-backs and gathers run under the others' forward passes
   static constexpr int kMaxChains = 3;
@@ -68,6 +69,24 @@ void nvfp4_prepare_assisted_impl(qtip_ctx* c, const float* host_H, int n, double
                                  float* host_dw);
 void ldlq_impl(qtip_ctx* c, const float* dWT, const float* dL, long n, long m, float* d_hatWT, uint16_t* dQ,
                int feedback, double* vit_seconds, int chains);
+// what a group carries from one phase of its quantization to the next (device buffers, offsets of its linears, times)
+struct GroupWork {
+  long mt = 0;
+  std::vector<long> off;
+  DBuf<float> d_su, d_sv, WT, hatWT;
+  DBuf<uint16_t> Q;
+  qtip_timing T{};
+  double t_start = 0, carried = 0;
+  void release() {
+    d_su.release(), d_sv.release(), WT.release(), hatWT.release(), Q.release();
+  }
+};
+void group_prepare(qtip_ctx* c, GroupWork& w, int nlin, const qtip_linear_in* lins, int n, uint64_t seed,
+                   const float* host_su, const qtip_opts& opt, qtip_linear_out* outs, const qtip_timing* tm);
+void group_ldlq(qtip_ctx* c, GroupWork& w, int n, const float* host_L, const float* dev_L, const qtip_opts& opt);
+void group_finish(qtip_ctx* c, GroupWork& w, int nlin, const qtip_linear_in* lins, int n, double creg,
+                  const float* host_HRr, const float* dev_HRr, const qtip_opts& opt, qtip_linear_out* outs,
+                  qtip_timing* tm);
 void quantize_group_impl(qtip_ctx* c, int nlin, const qtip_linear_in* lins, int n, uint64_t seed, const float* host_su,
                          double creg, const float* host_HRr, const float* host_L, const qtip_opts& opt,
                          qtip_linear_out* outs, qtip_timing* tm, const float* dev_HRr = nullptr,
