@@ -121,6 +121,7 @@ def lib():
     L.qtip_selftest_ldl_panel_handover.argtypes = [vp, i, i, vp]
     L.qtip_ldl_hessian_device_updates_dev.argtypes = [vp, vp, i, i, vp, vp]
     L.qtip_ldlq_dev.argtypes = [vp, vp, vp, l, l, vp, vp, i, C.POINTER(d)]
+    L.qtip_prod_cache_bf16x3_dev.argtypes = [vp, i, l, vp, l, vp, vp, l, vp]
     L.qtip_default_opts.argtypes = [C.POINTER(_OptsC)]
     L.qtip_default_opts.restype = None
     L.qtip_quantize_group.argtypes = [vp, i, C.POINTER(_LinearInC), i, u64, vp, d, vp, vp, C.POINTER(_OptsC),
@@ -432,6 +433,10 @@ class Quantizer:
         _check(lib().qtip_ldlq_dev(self._h, _ptr(dWT), _ptr(dL), n, m, _ptr(d_hatWT), _ptr(dQ), feedback,
                                    C.byref(vs) if time_viterbi else None))
         return vs.value
+
+    def prod_cache_bf16x3_dev(self, N, K, dLrows, ldl, dWT, d_hatWT, ldw, dP):
+        """P[128][N] = sum_k Lrows[k][r] (WT - hatWT)[k][j] in split-bf16 arithmetic (device fp32 tensors)."""
+        _check(lib().qtip_prod_cache_bf16x3_dev(self._h, N, K, _ptr(dLrows), ldl, _ptr(dWT), _ptr(d_hatWT), ldw, _ptr(dP)))
 
     def _marshal(self, lins, n, opt):
         if not opt.share_su:

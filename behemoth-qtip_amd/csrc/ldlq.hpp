@@ -8,8 +8,14 @@ constexpr int kMaxGatherSplits = 16;
 int gemm_splitk_splits(long K, int N, int slots);
 void launch_gemm_tn_f64_gather(int N, long K, const float* A, long lda, const float* B1, const float* B2, long ldb,
                                double* P, double* partials, int slots, hipStream_t s);
-// the gathered product with every operand split into bf16 hi + lo (three MFMA terms, fp32 accumulate), P and the
-// partials (up to kMaxGatherSplits x 128 x N) in fp32
-void launch_gemm_tn_bf16x3_gather(int N, long K, const float* A, long lda, const float* B1, const float* B2, long ldb,
-                                  float* P, float* partials, int slots, hipStream_t s);
+// The gathered product in the reference GPU path's arithmetic: operands as bf16 hi + lo images with k contiguous,
+// three MFMA terms, fp32 accumulate; P and the partials (up to kMaxGatherSplits x 128 x N) in fp32.
+//   a: Ah / Al[i * lda + k], i < 128   (launch_split_transpose_bf16 of L, offset to the buffer's columns and rows)
+//   b: Bh / Bl[j * ldb + k], j < N     (written by the Viterbi kernel, TileJob::dimg_h / dimg_l)
+void launch_gemm_img_gather(int N, long K, const uint16_t* Ah, const uint16_t* Al, long lda, const uint16_t* Bh,
+                            const uint16_t* Bl, long ldb, float* P, float* partials, int slots, hipStream_t s);
+// Th / Tl[i * ldt + k] = bf16 hi / lo of X[k * ldx + i] (minus X2[k * ldx + i] when X2 is given), k < rows_k,
+// i < cols_i, both multiples of 64; lower_only: the 64 x 64 tiles wholly above the diagonal are skipped
+void launch_split_transpose_bf16(const float* X, const float* X2, long ldx, long rows_k, long cols_i, uint16_t* Th,
+                                 uint16_t* Tl, long ldt, bool lower_only, hipStream_t s);
 }  // namespace qtipmi

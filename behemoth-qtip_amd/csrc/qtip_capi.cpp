@@ -718,6 +718,25 @@ int qtip_ldlq_dev(qtip_ctx* ctx, const float* dev_WT, const float* dev_L, long n
   });
 }
 
+int qtip_prod_cache_bf16x3_dev(qtip_ctx* ctx, int N, long K, const float* dev_Lrows, long ldl, const float* dev_WT,
+                               const float* dev_hatWT, long ldw, float* dev_P) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && dev_Lrows && dev_WT && dev_hatWT && dev_P, "prod_cache: bad arguments");
+    QTIP_REQUIRE(N > 0 && N % 64 == 0 && K > 0 && K % 64 == 0 && ldl >= 128 && ldw >= N && ldl % 4 == 0 && ldw % 4 == 0,
+                 "prod_cache: N and K must be multiples of 64 and the rows 16-byte aligned (N = %d, K = %ld)", N, K);
+    DeviceGuard g(ctx);
+    hipStream_t s = ctx->stream;
+    // images [row][k], k contiguous: L's 128 columns, then the N columns of the residual
+    DBuf<uint16_t> img(size_t(2) * (128 + N) * K);
+    uint16_t *ah = img.p, *al = ah + size_t(128) * K, *bh = al + size_t(128) * K, *bl = bh + size_t(N) * K;
+    launch_split_transpose_bf16(dev_Lrows, nullptr, ldl, K, 128, ah, al, K, false, s);
+    launch_split_transpose_bf16(dev_WT, dev_hatWT, ldw, K, N, bh, bl, K, false, s);
+    DBuf<float> parts(size_t(kMaxGatherSplits) * 128 * N);
+    launch_gemm_img_gather(N, K, ah, al, K, bh, bl, K, dev_P, parts.p, ctx->vit_slots > 0 ? ctx->vit_slots : 768, s);
+    QTIP_HIP(hipStreamSynchronize(s));
+  });
+}
+
 int qtip_quantize_group(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, int n, uint64_t seed,
                         const float* host_su, double creg, const float* host_HRr, const float* host_L,
                         const qtip_opts* opts, qtip_linear_out* outs, qtip_timing* timing) {

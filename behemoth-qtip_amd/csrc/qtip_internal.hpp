@@ -244,6 +244,10 @@ struct TileJob {
   uint16_t* packed = nullptr;  // tiles x 32, pack_trellis layout
   float* hatWT = nullptr;      // scatter of decoded values: hatWT[(col0 + c) * ldw + 16 * t + r]
   long ldw = 0, col0 = 0;
+  // with hatWT and WT: the residual WT - hatWT of the decoded values as bf16 hi / lo bit patterns, weight row major:
+  // dimg[(16 t + r) * ldd + col0 + c] (the operand images of the split-bf16 gathered product)
+  uint16_t *dimg_h = nullptr, *dimg_l = nullptr;
+  long ldd = 0;
   // LDLQ: a workgroup takes its tile row through `blocks` consecutive 16-column blocks, from the last (columns
   // col0 + 16 (blocks - 1) ..) down to the first (col0 ..), state words at q_offset + block: the blocks of a tile row
   // depend on each other only through that row's own hatWT values, so nothing has to wait for another workgroup

@@ -142,6 +142,10 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
     ch[k].prod32 = feedback == 1 ? prod32.p + size_t(128) * ch[k].r0 : nullptr;
     ch[k].parts32 = feedback == 1 ? parts32.p + size_t(max_splits) * 128 * ch[k].r0 : nullptr;
   }
+  // feedback 1: the operands of the gathered product as bf16 hi / lo images with k contiguous: L transposed, made
+  // here once; the residual WT - hatWT, weight row major, written by the Viterbi launches as they decode
+  DBuf<uint16_t> limg(feedback == 1 ? size_t(2) * n * n : 0), dimg(feedback == 1 ? size_t(2) * m * n : 0);
+  if (feedback == 1) launch_split_transpose_bf16(L, nullptr, n, n, n, limg.p, limg.p + size_t(n) * n, n, true, s);
   QTIP_HIP(hipMemsetAsync(hatWT, 0, size_t(n) * m * 4, s));
   Events timed, pacing, joins;  // timed: a (start, stop) pair per Viterbi launch, stamped by the launch itself
   // the other chains start once the caller's inputs and the cleared outputs are there, a third (two thirds) of a
@@ -179,7 +183,10 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
         } else if (feedback == 0) {
           launch_gemm_tn_f64_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod, C.parts, C.slots, C.s);
         } else {
-          launch_gemm_tn_bf16x3_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod32, C.parts32, C.slots, C.s);
+          const uint16_t* la = limg.p + size_t(c0) * n + bufend;
+          const uint16_t* da = dimg.p + size_t(C.r0) * n + bufend;
+          launch_gemm_img_gather(int(C.rows), n - bufend, la, la + size_t(n) * n, n, da, da + size_t(m) * n, n, C.prod32,
+                                 C.parts32, C.slots, C.s);
         }
         {
           // one launch per buffer: a workgroup takes its tile row through the 8 column blocks, last to first, and
@@ -198,6 +205,7 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
           job.q_offset = c0 / 16;
           job.hatWT = hatWT + C.r0;
           job.ldw = m;
+          if (feedback == 1) job.dimg_h = dimg.p + size_t(C.r0) * n, job.dimg_l = job.dimg_h + size_t(m) * n, job.ldd = n;
           job.col0 = c0;
           job.blocks = 8;
           c->viterbi_settings(job);

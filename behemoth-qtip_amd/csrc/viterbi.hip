@@ -46,6 +46,7 @@
 #include <mutex>
 #include <type_traits>
 
+#include "bf16_split.hpp"
 #include "qtip_internal.hpp"
 
 namespace qtipmi {
@@ -878,7 +879,15 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
       const uint32_t s = sm.st[u >> 1];
       const uint32_t e = ((s * (s + 1u)) >> 6) & 1023u;
       const int q = perm_fwd(u), r = q >> 4, c = q & 15;
-      job.hatWT[(col0 + c) * job.ldw + tile * 16 + r] = entry_f[2 * e + (u & 1)];
+      const long wi = (col0 + c) * job.ldw + tile * 16 + r;
+      const float hv = entry_f[2 * e + (u & 1)];
+      job.hatWT[wi] = hv;
+      if (job.dimg_h) {
+        uint32_t hi, lo;
+        bf16_split_bits(job.WT[wi] - hv, hi, lo);
+        const long di = (tile * 16 + r) * job.ldd + col0 + c;
+        job.dimg_h[di] = uint16_t(hi), job.dimg_l[di] = uint16_t(lo);
+      }
     }
     __syncthreads();
   }
@@ -920,6 +929,8 @@ void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const flo
   if (!job.X) {  // LDLQ block: the targets come from the feedback operands
     QTIP_REQUIRE(job.WT && job.L && job.hatWT && ((job.prod64 != nullptr) != (job.prod32 != nullptr)),
                  "viterbi: neither inputs nor complete LDLQ feedback operands");
+    QTIP_REQUIRE((job.dimg_h != nullptr) == (job.dimg_l != nullptr) && (!job.dimg_h || job.ldd >= job.col0 + 16L * job.blocks),
+                 "viterbi: residual images need both parts and rows that hold the block's columns");
     const long nk = job.bufend - job.col0 - 16;
     QTIP_REQUIRE(job.col0 >= 0 && nk >= 0 && nk <= 112 && job.blocks >= 1 && job.col0 + 16 * job.blocks <= job.bufend,
                  "viterbi: column blocks outside their 128-column buffer");

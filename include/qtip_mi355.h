@@ -213,6 +213,15 @@ typedef struct { /* GroupTiming, src/quantizer.hpp:45-47 */
   double load, rht, ldl_cpu, ldlq, viterbi, proxy, pack, total;
 } qtip_timing;
 
+/* The cross-buffer feedback ("prod cache") of one 128-column LDLQ buffer in the arithmetic of ldlq_gpu's update,
+ * src/quantizer.cpp:66-76 (every fp32 operand as bf16 hi + lo, product = lo*hi + hi*lo + hi*hi on the bf16 matrix
+ * cores, fp32 accumulate), in the gathered form qtip_ldlq_dev uses with feedback = 1: all rows quantized so far at once,
+ *   P[r * N + j] = sum over k < K of Lrows[k * ldl + r] * (WT[k * ldw + j] - hatWT[k * ldw + j]),  r < 128, j < N,
+ * where Lrows points at L[bufend][c0] and WT / hatWT at row bufend of the transposed weights.  The order of the fp32
+ * sums is this library's (the reference leaves it to its BLAS).  N and K multiples of 64; synchronous. */
+int qtip_prod_cache_bf16x3_dev(qtip_ctx* ctx, int N, long K, const float* dev_Lrows, long ldl, const float* dev_WT,
+                               const float* dev_hatWT, long ldw, float* dev_P);
+
 /* quantize_group(s, gemm, lins, hp, opt, tm, tag), src/quantizer.cpp:176-346, with the HessPrep fields passed
  * flat: su[n], creg, HRr[n*n], L[n*n] (host; L is read, never freed).  seed gives the SV streams. */
 int qtip_quantize_group(qtip_ctx* ctx, int nlin, const qtip_linear_in* lins, int n, uint64_t seed,

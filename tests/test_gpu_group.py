@@ -141,6 +141,47 @@ def test_ldlq_split_bf16_feedback(qz, oracle, hyb):
         qz.ldlq_dev(dWT, dL, n, m, dH, dQ, feedback=7)
 
 
+def _bf16_parts(x):
+    """hi = bf16(x), lo = bf16(x - hi), both rounded to nearest even, as float32 arrays"""
+    def rne(v):
+        u = np.ascontiguousarray(v, dtype=np.float32).view(np.uint32).astype(np.uint64)
+        u = ((u + 0x7fff + ((u >> 16) & 1)) >> 16) << 16
+        return u.astype(np.uint32).view(np.float32)
+    hi = rne(x)
+    return hi, rne(x - hi)
+
+
+@pytest.mark.parametrize("K,N", [(1408, 192), (8256, 64), (64, 128)])
+def test_prod_cache_split_bf16(qz, K, N):
+    """The gathered cross-buffer product of feedback = 1 (bf16 hi / lo images, three matrix-core terms, fp32 sums)
+    against the same three terms summed in fp64 from operands split on the host (src/quantizer.cpp:66-76 for the
+    terms).  The bound, 2e-6 of sum |a| |b|, is some fifty times the rounding of the fp32 sums and a twentieth of
+    what a dropped lo term, a wrong row or a wrong k would change; the test checks the latter on its own data.
+    Rows padded (ldl, ldw beyond the sizes), N not a multiple of the 128-column tile, K split over workgroups."""
+    import torch
+    say("case: prod cache split bf16 K=%d N=%d" % (K, N))
+    rng = np.random.default_rng(K + N)
+    ldl, ldw = 128 + 64, N + 32
+    Lr = (rng.normal(size=(K, ldl)) * np.exp(rng.normal(size=(K, 1)))).astype(np.float32)
+    WT = rng.normal(size=(K, ldw)).astype(np.float32)
+    HT = (WT + 0.1 * rng.normal(size=(K, ldw))).astype(np.float32)
+    dP = torch.full((128, N), 7.0, device="cuda")
+    qz.prod_cache_bf16x3_dev(N, K, torch.from_numpy(Lr).cuda(), ldl, torch.from_numpy(WT).cuda(),
+                             torch.from_numpy(HT).cuda(), ldw, dP)
+    got = dP.cpu().numpy().astype(np.float64)
+    lh, ll = _bf16_parts(Lr[:, :128])
+    dh, dl = _bf16_parts(WT[:, :N] - HT[:, :N])
+    lh, ll, dh, dl = (v.astype(np.float64) for v in (lh, ll, dh, dl))
+    want = ll.T @ dh + lh.T @ dl + lh.T @ dh
+    bound = 2e-6 * (np.abs(lh).T @ np.abs(dh)) + 1e-30
+    err = np.abs(got - want)
+    say("  largest error over bound %.3f" % (err / bound).max())
+    assert np.all(err <= bound)
+    if K >= 1024:   # what the bound tells apart: two terms only, and a product shifted by one row of k
+        assert np.mean(np.abs(lh.T @ dl + lh.T @ dh - want) > bound) > 0.9
+        assert np.mean(np.abs(np.roll(lh + ll, 1, axis=0).T @ (dh + dl) - want) > bound) > 0.9
+
+
 def test_ldlq_rejects_bad_shapes(qz, pkg):
     import torch
     z = torch.zeros(1, device="cuda")
