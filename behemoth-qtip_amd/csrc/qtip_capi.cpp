@@ -287,11 +287,12 @@ long qtip_selftest_device_alloc_calls(void) { return test_device_alloc_calls(); 
 
 int qtip_set_viterbi_mode(qtip_ctx* ctx, int mode, unsigned margin_units) {
   return guarded([&] {
-    QTIP_REQUIRE(ctx != nullptr && (mode == 0 || mode == 1), "set_viterbi_mode: mode must be 0 or 1");
-    ctx->vit_mode = mode;
+    QTIP_REQUIRE(ctx != nullptr && mode >= 0 && mode <= 3, "set_viterbi_mode: mode must be 0, 1, 2 or 3");
+    ctx->vit_mode = mode == 1 ? 1 : 0;
+    ctx->vit_wide = mode == 2 ? 0 : mode == 3 ? 1 : -1;
     ctx->vit_margin = margin_units ? margin_units : kViterbiMargin;
     for (qtip_ctx* l : ctx->lane)
-      if (l) l->vit_mode = ctx->vit_mode, l->vit_margin = ctx->vit_margin;
+      if (l) l->vit_mode = ctx->vit_mode, l->vit_wide = ctx->vit_wide, l->vit_margin = ctx->vit_margin;
   });
 }
 

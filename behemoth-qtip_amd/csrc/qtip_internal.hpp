@@ -255,6 +255,9 @@ struct TileJob {
   // 0: both passes run on 32-bit metrics first and a pass whose traced decisions are not all won by `margin` units of
   // 2^-25 is run again on fp64 metrics (same results as mode 1, bit for bit); 1: fp64 metrics only
   int mode = 0;
+  // workgroups of 512 threads per tile instead of 256 (mode 0 only; same results): -1 = where the launch has at most
+  // a third as many tiles as the device has workgroup slots, 0 = never, 1 = always
+  int wide = -1;
   uint32_t margin = kViterbiMargin;
   unsigned* stats = nullptr;  // device counters (optional): [0], [1] += passes of the first / second kind run again
 };

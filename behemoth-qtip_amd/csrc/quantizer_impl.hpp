@@ -20,10 +20,12 @@ struct qtip_ctx {
   // Viterbi passes: 0 = 32-bit metrics first, fp64 again where a traced decision is too close (same results);
   // 1 = fp64 only.  vit_stats: two device counters, passes of the first / second kind that were run again.
   int vit_mode = 0;
+  int vit_wide = -1;  // TileJob::wide; a lane runs beside other lanes and keeps to the 256-thread workgroups
   uint32_t vit_margin = qtipmi::kViterbiMargin;
   qtipmi::DBuf<unsigned> vit_stats;
   void viterbi_settings(qtipmi::TileJob& job) const {
     job.mode = vit_mode;
+    job.wide = vit_slots_limit > 0 ? 0 : vit_wide;
     job.margin = vit_margin;
     job.stats = vit_stats.p;
   }

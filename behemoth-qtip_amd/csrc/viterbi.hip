@@ -78,7 +78,15 @@ __device__ __forceinline__ int m_slot(int col, int d) { return m_pos(col) * 16 +
 // addresses: some twenty registers per kind of pass) is then formed where the pass starts instead of once at the top
 // of the kernel, where the three kinds together would sit in registers for the whole launch and push the passes' own
 // values out to scratch memory
+// The wide form of the kernel runs 512 threads per tile: its 32-bit forward passes share the groups out over all of
+// them (opaque_tid_wide), everything else is done twice, by the threads t and t + 256 alike (same reads, same
+// values written to the same places), so that every wave meets every barrier.
 __device__ __forceinline__ int opaque_tid() {
+  int t = threadIdx.x & (kThreads - 1);
+  asm volatile("" : "+v"(t));
+  return t;
+}
+__device__ __forceinline__ int opaque_tid_wide() {
   int t = threadIdx.x;
   asm volatile("" : "+v"(t));
   return t;
@@ -94,7 +102,7 @@ struct Smem {
   double tr_c[2][4];    // trace-back: the four waves' best candidates of a round (cost; d | d1 << 8), two sets
   uint32_t tr_d[2][4];
   uint32_t tr32[2][4][4];  // the same for the 32-bit passes: best, second best, d | d1 << 8, gap inside the best's row
-  uint32_t red32[4][3];    // end of the free 32-bit pass: per wave the best group's metric, the second best, the group
+  uint32_t red32[8][3];    // end of the free 32-bit pass: per wave the best group's metric, the second best, the group
   int overlap;
   uint32_t final_state;
 };
@@ -535,32 +543,30 @@ __device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, d
 // Metrics and error table are double-buffered in LDS (2 x 16 KB, 2 x 8 KB: the footprint of the fp64 arrays): a step
 // reads the present buffers and writes the next metrics and the next step's table, so one barrier per step suffices;
 // a thread keeps its four codebook entries in registers.
-template <bool kSym>
+// kWide: 512 threads; the threads t and t + 256 share the eight groups of a column half, four each (slots 0..3 and
+// 4..7), and the table's 1024 entries two each instead of four.
+template <bool kSym, bool kWide>
 __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restrict__ entry_d, int roll, int ov,
                                                uint32_t* __restrict__ hist, int first_kept) {
-  const int tid = opaque_tid();
+  constexpr int kT = kWide ? 2 * kThreads : kThreads, kSlotsOwn = kWide ? 4 : 8, kEnt = 1024 / kT;
+  const int tfull = kWide ? opaque_tid_wide() : opaque_tid();
+  const int tid = tfull & (kThreads - 1), upper = kWide ? tfull >> 8 : 0;
   const int colA = 4 * (tid & 31) + ((tid >> 5) & 3), colB = 255 - colA;
   const int half = tid >> 7;
   uint32_t* const E32 = reinterpret_cast<uint32_t*>(sm.E);  // [2][32 positions][64 rows]
   uint32_t* const M32 = reinterpret_cast<uint32_t*>(sm.M);  // [2][4096]
   static_assert(sizeof(sm.E) >= 2 * kESlots * sizeof(uint32_t) && sizeof(sm.M) >= 2 * kMSlots * sizeof(uint32_t));
-#ifndef QTIP_V_ENTREG
-#define QTIP_V_ENTREG 1
-#endif
-#ifndef QTIP_V_TABLE_LATE
-#define QTIP_V_TABLE_LATE 0
-#endif
-  double2 ent[4];
-  const double2* __restrict__ entries = reinterpret_cast<const double2*>(entry_d) + tid;
+  double2 ent[kEnt];
+  const double2* __restrict__ entries = reinterpret_cast<const double2*>(entry_d) + tfull;
 #pragma unroll
-  for (int q = 0; q < 4; ++q) ent[q] = entries[256 * q];
-  const int e_wr = (tid >> 6) * 64 + (tid & 63);
-  int ebase[8], wslot[8];
+  for (int q = 0; q < kEnt; ++q) ent[q] = entries[kT * q];
+  const int e_wr = tfull;
+  int ebase[kSlotsOwn], wslot[kSlotsOwn];  // of the slots m0 .. m0 + kSlotsOwn - 1, m0 = 4 upper
 #pragma unroll
-  for (int m = 0; m < 8; ++m) {
-    const uint32_t j = 16u * colA + 8u * uint32_t(half) + m, p = j * (j + 1u);
-    ebase[m] = int((p >> 12) & 15u) * 64 + int((p >> 6) & 63u);
-    wslot[m] = m32_slot(int(j & 255u), int(j >> 8));
+  for (int i = 0; i < kSlotsOwn; ++i) {
+    const uint32_t j = 16u * colA + 8u * uint32_t(half) + uint32_t(i + 4 * upper), p = j * (j + 1u);
+    ebase[i] = int((p >> 12) & 15u) * 64 + int((p >> 6) & 63u);
+    wslot[i] = m32_slot(int(j & 255u), int(j >> 8));
   }
   int xA = m32_pos(colA) * 64 + m32_swz(colA) * 4, xB = m32_pos(colB) * 64 + m32_swz(colB) * 4;  // bytes
   // the error table of step `it` into table buffer it & 1
@@ -569,22 +575,18 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
     const double x0 = double(sm.x[t]), x1 = double(sm.x[t + 1]);
     uint32_t* const Ew = E32 + (it & 1) * kESlots + e_wr;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-#if QTIP_V_ENTREG
+    for (int q = 0; q < kEnt; ++q) {
       const double2 l = ent[q];
-#else
-      const double2 l = entries[256 * q];
-#endif
       const uint32_t v = err_units(l.x, l.y, x0, x1);
-      Ew[256 * q] = v;
-      Ew[256 * q + 1024] = v;
+      Ew[kT * q] = v;
+      Ew[kT * q + 1024] = v;
     }
   };
-  for (int g = tid; g < kGroups; g += kThreads) M32[m32_slot(g & 255, g >> 8)] = (ov < 0 || g == ov) ? 0u : kSat;
+  for (int g = tfull; g < kGroups; g += kT) M32[m32_slot(g & 255, g >> 8)] = (ov < 0 || g == ov) ? 0u : kSat;
   table(0);
   __syncthreads();
 
-  uint32_t fin[8];
+  uint32_t fin[kSlotsOwn];
   // step `it`: metrics of buffer it & 1 and table buffer it & 1 -> metrics of buffer (it + 1) & 1
   auto step = [&](int it, auto kind_tag) __attribute__((always_inline)) {
     constexpr int kind = decltype(kind_tag)::value;  // kDigits: the free pass's last step, results to fin only
@@ -604,22 +606,26 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
         MB[4 * k] = b.x, MB[4 * k + 1] = b.y, MB[4 * k + 2] = b.z, MB[4 * k + 3] = b.w;
       }
     }
-#if !QTIP_V_TABLE_LATE
     if constexpr (kind != kDigits) table(it + 1);
-#endif
-    // the 16 table values of a slot are fetched while the slot before it is worked on
+    // The 16 table values of a slot are fetched while the slot before it is worked on; the value of digit k of slot
+    // m lies (k (2 m + 1)) % 16 positions after the slot's first.  m0: the first slot of this thread, a constant in
+    // each of the two copies of the loop that the wide form needs.
+    auto slots = [&](auto m0_tag) __attribute__((always_inline)) {
+    constexpr int m0 = decltype(m0_tag)::value;
     uint32_t evb[2][16];
 #pragma unroll
-    for (int k = 0; k < 16; ++k) evb[0][k] = Er[ebase[0] + k * 64];  // slot 0: stride 1
+    for (int k = 0; k < 16; ++k) evb[0][k] = Er[ebase[0] + ((k * (2 * m0 + 1)) & 15) * 64];
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
-      if (m < 7) {
-        const int gn = 2 * (m + 1) + 1;
-        const uint32_t* er = Er + ebase[m < 7 ? m + 1 : 7];
+    for (int i = 0; i < kSlotsOwn; ++i) {
+      constexpr int kLast = kSlotsOwn - 1;
+      const int m = i;  // index into this thread's own slots
+      if (i < kLast) {
+        const int gn = 2 * (m0 + i + 1) + 1;
+        const uint32_t* er = Er + ebase[i < kLast ? i + 1 : kLast];
 #pragma unroll
-        for (int k = 0; k < 16; ++k) evb[(m + 1) & 1][k] = er[((k * gn) & 15) * 64];
+        for (int k = 0; k < 16; ++k) evb[(i + 1) & 1][k] = er[((k * gn) & 15) * 64];
       }
-      const uint32_t* ev = evb[m & 1];
+      const uint32_t* ev = evb[i & 1];
       // the table value at position k is the candidate of digit k of the group and of digit 15 - k of its mirror
       uint32_t ba = kSat;
 #pragma unroll
@@ -638,13 +644,17 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
         Mw[wslot[m] ^ kMirror32] = bb;
       }
       if constexpr (kind == kStore) {
-        hs[m * kThreads] = ba;
-        if constexpr (!kSym) hs[(8 + m) * kThreads] = bb;
+        hs[(m0 + m) * kThreads] = ba;
+        if constexpr (!kSym) hs[(8 + m0 + m) * kThreads] = bb;
       }
     }
-#if QTIP_V_TABLE_LATE
-    if constexpr (kind != kDigits) table(it + 1);
-#endif
+    };
+    if constexpr (!kWide) {
+      slots(std::integral_constant<int, 0>{});
+    } else {
+      if (upper) slots(std::integral_constant<int, 4>{});
+      else slots(std::integral_constant<int, 0>{});
+    }
     __syncthreads();
   };
   using Plain = std::integral_constant<int, kPlain>;
@@ -660,8 +670,8 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
     // best final group among the groups below 2048 (each stands for a pair of complementary states), and the runner-up
     uint32_t b1 = kSat, b2 = kSat, bj = 0;
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
-      const uint32_t v = fin[m], j = 16u * colA + 8u * uint32_t(half) + m;
+    for (int m = 0; m < kSlotsOwn; ++m) {
+      const uint32_t v = fin[m], j = 16u * colA + 8u * uint32_t(half) + uint32_t(m + 4 * upper);
       const bool take = v < b1;
       b2 = take ? b1 : min(b2, v);
       bj = take ? j : bj;
@@ -675,11 +685,11 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
       bj = take ? oj : bj;
       b1 = take ? o1 : b1;
     }
-    if ((tid & 63) == 0) sm.red32[tid >> 6][0] = b1, sm.red32[tid >> 6][1] = b2, sm.red32[tid >> 6][2] = bj;
+    if ((tfull & 63) == 0) sm.red32[tfull >> 6][0] = b1, sm.red32[tfull >> 6][1] = b2, sm.red32[tfull >> 6][2] = bj;
     __syncthreads();
     b1 = sm.red32[0][0], b2 = sm.red32[0][1], bj = sm.red32[0][2];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) {
+    for (int w = 1; w < kT / 64; ++w) {
       const uint32_t o1 = sm.red32[w][0], o2 = sm.red32[w][1], oj = sm.red32[w][2];
       const bool take = o1 < b1 || (o1 == b1 && oj < bj);
       b2 = take ? min(b1, o2) : min(b2, o1);
@@ -687,7 +697,7 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
       b1 = take ? o1 : b1;
     }
     __syncthreads();
-    if (tid == 0) sm.red32[0][0] = b1, sm.red32[0][1] = b2 - b1, sm.red32[0][2] = bj;
+    if (tfull == 0) sm.red32[0][0] = b1, sm.red32[0][1] = b2 - b1, sm.red32[0][2] = bj;
     __syncthreads();
   }
 }
@@ -803,11 +813,14 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
   return s;
 }
 
-__global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job, const double* __restrict__ entry_d,
-                                                                 const float* __restrict__ entry_f,
-                                                                 double* __restrict__ hist_all) {
+// kWide: 512 threads per tile, one workgroup per compute unit, for launches that cannot fill the chip anyway (a lone
+// small group): a tile then takes about two thirds of the time.  Same results, bit for bit.
+template <bool kWide>
+__global__ __launch_bounds__(kWide ? 2 * kThreads : kThreads, kWide ? 1 : 3) void viterbi_tiles_kernel(
+    TileJob job, const double* __restrict__ entry_d, const float* __restrict__ entry_f, double* __restrict__ hist_all) {
   __shared__ Smem sm;
-  const int u = threadIdx.x;
+  const int u = threadIdx.x & (kThreads - 1);
+  const bool first_half = threadIdx.x < kThreads;  // global results are written once
   double* hist = hist_all + size_t(blockIdx.x) * kHistWordsPerTile;
   for (long tile = blockIdx.x; tile < job.tiles; tile += gridDim.x)
   for (int blk = job.blocks - 1; blk >= 0; --blk) {
@@ -830,18 +843,18 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
         uint32_t* const hist32 = reinterpret_cast<uint32_t*>(hist);
         uint32_t flag = 0;
         if (pass == 0) {
-          forward_pass32<true>(sm, entry_d, roll, -1, hist32, 62);
+          forward_pass32<true, kWide>(sm, entry_d, roll, -1, hist32, 62);
           flag |= uint32_t(sm.red32[0][1] < job.margin) | uint32_t(sm.red32[0][0] >= kWinnerMax);
           const uint32_t s = trace_back32<true>(sm, entry_d, hist32, roll, sm.red32[0][2], 64, false, job.margin, flag);
           if (!flag && u == 0) sm.overlap = int(s & 0xfffu);  // s is the state of step 63
         } else {
-          forward_pass32<false>(sm, entry_d, roll, ov, hist32, 0);
+          forward_pass32<false, kWide>(sm, entry_d, roll, ov, hist32, 0);
           const uint32_t s = trace_back32<false>(sm, entry_d, hist32, roll, uint32_t(ov), 2, true, job.margin, flag);
           // s is the state of step 1; at step 0 the one predecessor group with a finite initial metric is ov
           if (!flag && u == 0) sm.st[0] = uint16_t((s >> 4) | ((uint32_t(ov) >> 8) << 12));
         }
         done = !flag;
-        if (flag && u == 0 && job.stats) atomicAdd(job.stats + pass, 1u);
+        if (flag && threadIdx.x == 0 && job.stats) atomicAdd(job.stats + pass, 1u);
       }
       if (!done) {
       forward_pass(sm, entry_d, roll, ov, hist, pass == 0 ? 62 : 0);
@@ -864,8 +877,8 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
       ov = sm.overlap;
     }
     // ---- outputs
-    if (job.states && u < kSteps) job.states[(tile * job.q_tile_stride + job.q_offset + blk) * kSteps + u] = sm.st[u];
-    if (job.packed && u < kWords) {
+    if (job.states && first_half && u < kSteps) job.states[(tile * job.q_tile_stride + job.q_offset + blk) * kSteps + u] = sm.st[u];
+    if (job.packed && first_half && u < kWords) {
       uint32_t v;
       if (u == 0) v = sm.st[0];
       else {
@@ -875,7 +888,7 @@ __global__ __launch_bounds__(kThreads, 3) void viterbi_tiles_kernel(TileJob job,
       }
       job.packed[tile * kWords + u] = uint16_t(v);
     }
-    if (job.hatWT) {
+    if (job.hatWT && first_half) {
       const uint32_t s = sm.st[u >> 1];
       const uint32_t e = ((s * (s + 1u)) >> 6) & 1023u;
       const int q = perm_fwd(u), r = q >> 4, c = q & 15;
@@ -913,13 +926,27 @@ __global__ void decode_states_kernel(const uint16_t* __restrict__ st, long count
 
 size_t viterbi_workspace_bytes(int slots) { return size_t(slots) * kHistWordsPerTile * sizeof(double); }
 
+// workgroup slots of the 256-thread kernel on `device`, which must be current (found once per device)
 int viterbi_max_slots(int device) {
+  static std::mutex mu;
+  static int cached[kMaxDevices] = {0};
+  const bool tracked = device >= 0 && device < kMaxDevices;
+  std::lock_guard<std::mutex> lock(mu);
+  if (tracked && cached[device]) return cached[device];
   hipDeviceProp_t prop;
   QTIP_HIP(hipGetDeviceProperties(&prop, device));
   int per_cu = 0;
-  QTIP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, viterbi_tiles_kernel, kThreads, 0));
+  QTIP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, viterbi_tiles_kernel<false>, kThreads, 0));
   if (per_cu < 1) per_cu = 1;
-  return per_cu * prop.multiProcessorCount;
+  const int slots = per_cu * prop.multiProcessorCount;
+  if (tracked) cached[device] = slots;
+  return slots;
+}
+
+static int viterbi_device_slots() {
+  int dev = 0;
+  QTIP_HIP(hipGetDevice(&dev));
+  return viterbi_max_slots(dev);
 }
 
 void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const float* d_entry_f, void* workspace,
@@ -939,13 +966,18 @@ void launch_viterbi_tiles(const TileJob& job, const double* d_entry_d, const flo
   }
   QTIP_REQUIRE(job.blocks == 1 || (!job.X && !job.packed), "viterbi: several blocks per tile row only for LDLQ launches");
   const unsigned grid = unsigned(job.tiles < slots ? job.tiles : slots);
+  // the wide form where the launch leaves two thirds of the chip's workgroup slots empty anyway (and the 32-bit
+  // passes, which are what it shares out over its 512 threads, are in use)
+  const bool wide = job.mode == 0 && (job.wide > 0 || (job.wide < 0 && 3 * job.tiles <= viterbi_device_slots()));
+  const auto kernel = wide ? viterbi_tiles_kernel<true> : viterbi_tiles_kernel<false>;
+  const dim3 block(wide ? 2 * kThreads : kThreads);
   if (start || stop) {
     // the runtime stamps the two events at the kernel's own start and end: the time between them is the kernel's,
     // however late the host got round to queueing it
-    hipExtLaunchKernelGGL(viterbi_tiles_kernel, dim3(grid), dim3(kThreads), 0, s, start, stop, 0, job, d_entry_d,
-                          d_entry_f, static_cast<double*>(workspace));
+    hipExtLaunchKernelGGL(kernel, dim3(grid), block, 0, s, start, stop, 0, job, d_entry_d, d_entry_f,
+                          static_cast<double*>(workspace));
   } else {
-    viterbi_tiles_kernel<<<dim3(grid), dim3(kThreads), 0, s>>>(job, d_entry_d, d_entry_f, static_cast<double*>(workspace));
+    kernel<<<dim3(grid), block, 0, s>>>(job, d_entry_d, d_entry_f, static_cast<double*>(workspace));
   }
   QTIP_HIP(hipGetLastError());
 }

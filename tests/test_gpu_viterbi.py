@@ -163,15 +163,9 @@ def test_non_finite_inputs_leave_other_tiles_alone(qz, oracle, hyb):
     assert np.array_equal(pk[good], oracle.pack_trellis(want))
 
 
-def test_metric_modes_give_the_same_states(qz, oracle, hyb):
-    """The default runs each pass on 32-bit metrics and repeats it on fp64 metrics when a decision on the surviving
-    path is too close to call; fp64-only, and the default with a margin no decision can reach (every pass repeated),
-    must give the same states, the CPU algorithm's, on raw inputs, fp16-rounded inputs (the LDLQ case) and inputs full
-    of exact ties.  The counters say how many passes were repeated."""
-    say("case: 32-bit-first, fp64-only and all-repeated passes agree")
-    qz.set_tlut(None)
+def _mixed_inputs(oracle, B=320):
+    """raw, fp16-rounded, tie-laden and extreme tiles"""
     rng = np.random.default_rng(11)
-    B = 320
     X = oracle.rng_normal(4242, B * 256).astype(np.float32).reshape(B, 256)
     X[64:128] = X[64:128].astype(np.float16).astype(np.float32)           # fp16-representable, as LDLQ feeds them
     X[128:160] = (X[128:160] * np.float32(0.87)).astype(np.float16).astype(np.float32)
@@ -182,6 +176,18 @@ def test_metric_modes_give_the_same_states(qz, oracle, hyb):
     X[179, ::2] = -3.0
     X[180] = X[180] * np.float32(1e-3)
     X[181:192] = rng.standard_t(3, size=(11, 256)).astype(np.float32) * 2
+    return X
+
+
+def test_metric_modes_give_the_same_states(qz, oracle, hyb):
+    """The default runs each pass on 32-bit metrics and repeats it on fp64 metrics when a decision on the surviving
+    path is too close to call; fp64-only, and the default with a margin no decision can reach (every pass repeated),
+    must give the same states, the CPU algorithm's, on raw inputs, fp16-rounded inputs (the LDLQ case) and inputs full
+    of exact ties.  The counters say how many passes were repeated."""
+    say("case: 32-bit-first, fp64-only and all-repeated passes agree")
+    qz.set_tlut(None)
+    B = 320
+    X = _mixed_inputs(oracle, B)
     want = oracle.quantize_tiles(hyb, X, fast=True)
     try:
         qz.viterbi_stats(reset=True)
@@ -205,3 +211,37 @@ def test_metric_modes_give_the_same_states(qz, oracle, hyb):
     # near-ties of 2e-6 relative are rare: the bulk of the passes stands on 32-bit metrics (the tie-laden tiles
     # 160..179 may all be repeated)
     assert r0[0] <= 40 and r0[1] <= 40
+
+
+def test_wide_workgroups_give_the_same_states(qz, oracle, hyb):
+    """A launch that cannot fill the chip gives every tile 512 threads instead of 256 (the 32-bit forward passes
+    share the groups out over all of them; everything else, the fp64 repeat of a pass included, is done by both
+    halves alike).  Forced on and off on the same inputs, with and without every pass repeated: the CPU algorithm's
+    states each time; and benchmark configuration 1 in full through the wide form against the compiled reference's
+    packed words."""
+    say("case: 512-thread workgroups")
+    qz.set_tlut(None)
+    B = 320
+    X = _mixed_inputs(oracle, B)
+    want = oracle.quantize_tiles(hyb, X, fast=True)
+    try:
+        for mode, margin, name in ((2, 0, "256 threads"), (3, 0, "512 threads"), (3, 0xffffffff, "512 threads, all repeated")):
+            qz.viterbi_stats(reset=True)
+            qz.set_viterbi_mode(mode, margin)
+            st, pk = qz.viterbi_tiles(X)
+            r = qz.viterbi_stats(reset=True)
+            say("  %s: %d first and %d second passes repeated" % (name, r[0], r[1]))
+            same = np.all(st == want, axis=1)
+            assert same.all(), "%s: tiles differing from the CPU algorithm: %s" % (name, np.nonzero(~same)[0][:10])
+            assert r == (B, B) if margin else (r[0] <= 40 and r[1] <= 40)
+        meta = json.load(open(os.path.join(GOLDEN, "ref_config1.json")))
+        X1 = oracle.rng_normal(meta["x_seed"], 4096 * 256).astype(np.float32).reshape(4096, 256)
+        qz.set_tlut(oracle.synthetic_tlut(meta["tlut_seed"]))
+        qz.set_viterbi_mode(3)
+        st, pk = qz.viterbi_tiles(X1)
+        want1 = g("ref_config1_packed.bin", np.uint16).reshape(4096, 32)
+        same = np.all(pk == want1, axis=1)
+        assert same.all(), "%d of 4096 tiles differ, first %s" % ((~same).sum(), np.nonzero(~same)[0][:10])
+    finally:
+        qz.set_viterbi_mode(0)
+        qz.set_tlut(None)
