@@ -209,6 +209,7 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
           job.col0 = c0;
           job.blocks = 8;
           c->viterbi_settings(job);
+          if (nch > 1) job.wide = 0;  // the chains fill the chip between them: one launch is not the measure
           hipEvent_t t0 = nullptr, t1 = nullptr;
           if (vit_seconds) t0 = timed.add(hipEventDefault), t1 = timed.add(hipEventDefault);
           launch_viterbi_tiles(job, c->d_entry_d, c->d_entry_f, c->vit_ws.p + viterbi_workspace_bytes(C.slot0), C.slots,

@@ -667,35 +667,34 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
   }
   if constexpr (kSym) {
     step(kSteps - 1, Last{});
-    // best final group among the groups below 2048 (each stands for a pair of complementary states), and the runner-up
+    // Best final group among the groups below 2048 (each stands for a pair of complementary states), and the best
+    // among the groups of other columns (j >> 4): the 16 groups of a column end in final states that differ in their
+    // last digit only where they come from the same predecessor, and which of those wins changes nothing that is
+    // traced back; the trace-back looks at the winner's column itself.  A partial result is (best value, its
+    // smallest group, best value outside that group's column); a thread's own groups are one column.
     uint32_t b1 = kSat, b2 = kSat, bj = 0;
 #pragma unroll
     for (int m = 0; m < kSlotsOwn; ++m) {
       const uint32_t v = fin[m], j = 16u * colA + 8u * uint32_t(half) + uint32_t(m + 4 * upper);
       const bool take = v < b1;
-      b2 = take ? b1 : min(b2, v);
       bj = take ? j : bj;
       b1 = take ? v : b1;
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      const uint32_t o1 = __shfl_xor(b1, off, 64), o2 = __shfl_xor(b2, off, 64), oj = __shfl_xor(bj, off, 64);
-      const bool take = o1 < b1 || (o1 == b1 && oj < bj);  // equal metrics: same choice in both lanes, gap 0 either way
-      b2 = take ? min(b1, o2) : min(b2, o1);
+    auto merge = [&](uint32_t o1, uint32_t o2, uint32_t oj) {
+      const bool same = (oj >> 4) == (bj >> 4);
+      const bool take = o1 < b1 || (o1 == b1 && oj < bj);  // equal metrics: same choice in both lanes
+      const uint32_t out = take ? min(o2, b1) : min(b2, o1);
+      b2 = same ? min(b2, o2) : out;
       bj = take ? oj : bj;
       b1 = take ? o1 : b1;
-    }
+    };
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) merge(__shfl_xor(b1, off, 64), __shfl_xor(b2, off, 64), __shfl_xor(bj, off, 64));
     if ((tfull & 63) == 0) sm.red32[tfull >> 6][0] = b1, sm.red32[tfull >> 6][1] = b2, sm.red32[tfull >> 6][2] = bj;
     __syncthreads();
     b1 = sm.red32[0][0], b2 = sm.red32[0][1], bj = sm.red32[0][2];
 #pragma unroll
-    for (int w = 1; w < kT / 64; ++w) {
-      const uint32_t o1 = sm.red32[w][0], o2 = sm.red32[w][1], oj = sm.red32[w][2];
-      const bool take = o1 < b1 || (o1 == b1 && oj < bj);
-      b2 = take ? min(b1, o2) : min(b2, o1);
-      bj = take ? oj : bj;
-      b1 = take ? o1 : b1;
-    }
+    for (int w = 1; w < kT / 64; ++w) merge(sm.red32[w][0], sm.red32[w][1], sm.red32[w][2]);
     __syncthreads();
     if (tfull == 0) sm.red32[0][0] = b1, sm.red32[0][1] = b2 - b1, sm.red32[0][2] = bj;
     __syncthreads();
@@ -713,8 +712,9 @@ __device__ __forceinline__ uint32_t row_min16_u32(uint32_t c) {
 }
 
 // Trace-back of a 32-bit pass, the scheme of trace_back above with the runner-up of every decision looked at as well.
-// j_last: low 12 bits of the final state (the group the pass ends in).  The decision of step 127 is taken from the
-// metrics entering it (kept slot 63), then two steps per round trip.  flag is raised (in every thread alike) when a
+// j_last: low 12 bits of the final state (the group the pass ends in; for a free pass the best group, of which the
+// column counts).  The decision of step 127 is taken from the metrics entering it (kept slot 63), then two steps
+// per round trip.  flag is raised (in every thread alike) when a
 // decision is won by less than thr units or the winner is not below 2^30.
 // Returns the state of step it_min - 1; record: the states of the steps walked are written to sm.st.
 template <bool kSym>
@@ -742,7 +742,7 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
     return m;
   };
   uint32_t s;
-  {  // step 127: the 16 states (digit << 12) | j_last, one per lane of a row; every row does the same
+  if constexpr (!kSym) {  // step 127: the 16 states (digit << 12) | j_last, one per lane of a row; every row does the same
     const int t = (2 * (kSteps - 1) + roll) & 255;
     const double x0 = double(sm.x[t]), x1 = double(sm.x[t + 1]);
     const uint32_t st = (dp << 12) | j_last;
@@ -751,7 +751,52 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
     const uint32_t m = row_pick(c, k, gap);
     flag |= uint32_t(gap < thr) | uint32_t(m >= kWinnerMax);
     s = (k << 12) | j_last;
-    if (kSym && k >= 8u) s = 65535u - s;  // the smaller state of the pair
+    if (record && threadIdx.x == 0) sm.st[kSteps - 1] = uint16_t(s);
+  } else {
+    // Free pass: the final state is the best of all.  The forward pass has named the best group's column and
+    // vouched for the distance to every other column; here the 256 final states of that column, (digit k << 12) |
+    // column << 4 | last digit e, are weighed: row 4 wave + r of the workgroup takes k, its lanes the 16 e.  The
+    // states of one k come from one predecessor, so only their best counts, and the decision to be won by thr units
+    // is the one between the k: states that share k are traced back alike.
+    const int t = (2 * (kSteps - 1) + roll) & 255;
+    const double x0 = double(sm.x[t]), x1 = double(sm.x[t + 1]);
+    const uint32_t col = j_last >> 4;
+    const uint32_t st = (d << 12) | (col << 4) | dp;
+    const uint32_t c = sat_add(err_of(st, x0, x1), kept(63, st >> 4));
+    uint32_t e1, gap_unused;
+    const uint32_t v = min(row_pick(c, e1, gap_unused), kSat);
+    uint32_t bc = uint32_t(__builtin_amdgcn_readlane(int(v), 0)), sc = kSat, bk = 4u * wave;
+    uint32_t be = uint32_t(__builtin_amdgcn_readlane(int(e1), 0));
+#pragma unroll
+    for (int r = 1; r < 4; ++r) {
+      const uint32_t oc = uint32_t(__builtin_amdgcn_readlane(int(v), 16 * r));
+      const uint32_t oe = uint32_t(__builtin_amdgcn_readlane(int(e1), 16 * r));
+      const bool take = oc < bc;
+      sc = take ? bc : min(sc, oc);
+      bk = take ? 4u * wave + uint32_t(r) : bk;
+      be = take ? oe : be;
+      bc = take ? oc : bc;
+    }
+    if (lane == 0) {
+      sm.tr32[1][wave][0] = bc;
+      sm.tr32[1][wave][1] = sc;
+      sm.tr32[1][wave][2] = bk | (be << 8);
+    }
+    __syncthreads();
+    bc = sm.tr32[1][0][0], sc = sm.tr32[1][0][1];
+    uint32_t bke = sm.tr32[1][0][2];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      const uint32_t oc = sm.tr32[1][w][0], os = sm.tr32[1][w][1];
+      const bool take = oc < bc;
+      sc = take ? min(bc, os) : min(sc, oc);
+      bke = take ? sm.tr32[1][w][2] : bke;
+      bc = take ? oc : bc;
+    }
+    flag |= uint32_t(sc - bc < thr) | uint32_t(bc >= kWinnerMax);
+    const uint32_t k = bke & 15u;
+    s = (k << 12) | (col << 4) | ((bke >> 8) & 15u);
+    if (k >= 8u) s = 65535u - s;  // the smaller state of the pair
     if (record && threadIdx.x == 0) sm.st[kSteps - 1] = uint16_t(s);
   }
   int set = 0;
