@@ -43,6 +43,7 @@
 // and tie rule.  Only the last step tracks its digits (in registers), which the final state needs.
 #include <hip/hip_ext.h>
 
+#include <cstddef>
 #include <mutex>
 #include <type_traits>
 
@@ -717,20 +718,90 @@ __device__ __forceinline__ uint32_t row_min16_u32(uint32_t c) {
 // per round trip.  flag is raised (in every thread alike) when a
 // decision is won by less than thr units or the winner is not below 2^30.
 // Returns the state of step it_min - 1; record: the states of the steps walked are written to sm.st.
-template <bool kSym>
+// kStream (the 512-thread form, whose workgroup has its compute unit to itself): which 256 of a kept step's values a
+// round reads is known only when the round before it is decided, so fetched on demand every round waits for HBM.
+// Whole kept steps are streamed into LDS ahead of the rounds instead (the metric and table arrays are idle now:
+// 48 KB, three steps of 4096 values or six of the 2048 a free pass keeps; direct-to-LDS loads, every wave a share of
+// a step, as many steps in flight as there are buffers beside the one in use), and the codebook is read from a
+// 2 KB table of fp16 pairs in LDS (tl), so that no other vector-memory load waits in line behind the streamed ones.
+// Beside other workgroups the streamed form loses more in their forward passes than it gains (measured), so the
+// 256-thread form fetches on demand.
+template <bool kSym, bool kStream>
 __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restrict__ entry_d,
                                                  const uint32_t* __restrict__ hist, int roll, uint32_t j_last,
-                                                 int it_min, bool record, uint32_t thr, uint32_t& flag) {
+                                                 int it_min, bool record, uint32_t thr, uint32_t& flag,
+                                                 const uint32_t* tl) {
   const uint32_t tid = uint32_t(opaque_tid());
   const uint32_t lane = tid & 63u, wave = tid >> 6, dp = lane & 15u, d = 4u * wave + (lane >> 4);
-  // written by this workgroup's own waves before the barrier that ended the forward pass: workgroup scope suffices
+  // streamed form: kept steps 63, 62, ..., it_min / 2 - 1 are the rows q = 0, 1, ... of a ring of kBufs buffers
+  constexpr int kRowWords = kSym ? kGroups / 2 : kGroups, kBufs = kSym ? 6 : 3;
+  constexpr int kLoads = kStream ? kRowWords / (4 * 2 * kThreads) : 1;  // 16-byte loads per thread and row, 512 threads
+  static_assert(sizeof(sm.E) + sizeof(sm.M) >= size_t(kBufs) * kRowWords * 4 && offsetof(Smem, M) == sizeof(sm.E));
+  static_assert((kBufs - 2) * kLoads <= 15, "the count of outstanding loads must fit the low four bits of the wait");
+  uint32_t* const rows = reinterpret_cast<uint32_t*>(sm.E);
+  const int count = 65 - it_min / 2;
+  int issued = 0, q = 0;  // rows requested so far; the row in use
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  auto issue = [&](int row) {
+    const uint32_t wave8 = threadIdx.x >> 6;  // all eight waves bring a share
+    const uint32_t* g = hist + size_t(63 - row) * kGroups + 4u * lane;
+    uint32_t* l = rows + (row % kBufs) * kRowWords;
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      const uint32_t w0 = (uint32_t(i) * 8u + wave8) * 256u;  // first word of this wave's 1 KB piece
+      __builtin_amdgcn_global_load_lds(g + w0, (lds_ptr)(l + w0), 16, 0, 0);
+    }
+  };
+  // this wave's loads of the rows up to the one wanted have landed: at most `later` rows requested after it are out
+  auto landed = [&](int later) {
+    if (kBufs >= 6 && later >= 4) __builtin_amdgcn_s_waitcnt(0x0F70 | (kBufs >= 6 ? 4 * kLoads : 0));
+    else if (kBufs >= 5 && later == 3) __builtin_amdgcn_s_waitcnt(0x0F70 | (kBufs >= 5 ? 3 * kLoads : 0));
+    else if (kBufs >= 4 && later == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | (kBufs >= 4 ? 2 * kLoads : 0));
+    else if (later >= 1) __builtin_amdgcn_s_waitcnt(0x0F70 | kLoads);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+  };
+  // The barrier of a round.  Streamed: one that orders LDS only (__syncthreads() would wait for the loads in flight);
+  // before it this wave's share of the next row has landed, after it everyone's has, and the buffer of the row in
+  // use, which nobody reads after the barrier, takes the row kBufs further on.
+  auto round_barrier = [&]() {
+    if constexpr (kStream) {
+      const int later = issued - 2 - q;  // rows requested after the next one
+      landed(later > 0 ? later : 0);
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (issued < count) issue(issued++);
+      ++q;
+    } else {
+      __syncthreads();
+    }
+  };
+  if constexpr (kStream) {
+    for (; issued < kBufs && issued < count; ++issued) issue(issued);
+    landed(issued - 1);
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  }
+  // the metrics of kept step `slot` (the row in use, when streamed).  On demand: written by this workgroup's own waves
+  // before the barrier that ended the forward pass, workgroup scope suffices
   auto kept = [&](int slot, uint32_t g) -> uint32_t {
-    return __hip_atomic_load(hist + size_t(slot) * kGroups + hist32_index<kSym>(g), __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_WORKGROUP);
+    if constexpr (kStream) return rows[(q % kBufs) * kRowWords + hist32_index<kSym>(g)];
+    else return __hip_atomic_load(hist + size_t(slot) * kGroups + hist32_index<kSym>(g), __ATOMIC_RELAXED,
+                                  __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   auto err_of = [&](uint32_t st, double x0, double x1) -> uint32_t {
     const uint32_t e = ((st * (st + 1u)) >> 6) & 1023u;
-    return err_units(entry_d[2 * e], entry_d[2 * e + 1], x0, x1);
+    if constexpr (kStream) {
+      const uint32_t w = tl[e & 511u];
+      const uint16_t h0 = uint16_t((w & 0xffffu) ^ ((e >> 9) << 15)), h1 = uint16_t(w >> 16);
+      return err_units(double(float(__builtin_bit_cast(_Float16, h0))), double(float(__builtin_bit_cast(_Float16, h1))),
+                       x0, x1);
+    } else {
+      return err_units(entry_d[2 * e], entry_d[2 * e + 1], x0, x1);
+    }
   };
   // over the 16 lanes of a row: the smallest value (returned), the first lane that holds it, the gap to the runner-up
   auto row_pick = [&](uint32_t c, uint32_t& first, uint32_t& gap) -> uint32_t {
@@ -752,6 +823,7 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
     flag |= uint32_t(gap < thr) | uint32_t(m >= kWinnerMax);
     s = (k << 12) | j_last;
     if (record && threadIdx.x == 0) sm.st[kSteps - 1] = uint16_t(s);
+    if constexpr (kStream) round_barrier();
   } else {
     // Free pass: the final state is the best of all.  The forward pass has named the best group's column and
     // vouched for the distance to every other column; here the 256 final states of that column, (digit k << 12) |
@@ -782,7 +854,7 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
       sm.tr32[1][wave][1] = sc;
       sm.tr32[1][wave][2] = bk | (be << 8);
     }
-    __syncthreads();
+    round_barrier();
     bc = sm.tr32[1][0][0], sc = sm.tr32[1][0][1];
     uint32_t bke = sm.tr32[1][0][2];
 #pragma unroll
@@ -834,7 +906,7 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
       sm.tr32[set][wave][2] = bd | (bd1 << 8);
       sm.tr32[set][wave][3] = bg;
     }
-    __syncthreads();
+    round_barrier();
     bc = sm.tr32[set][0][0], sc = sm.tr32[set][0][1];
     uint32_t bdd = sm.tr32[set][0][2];
     bg = sm.tr32[set][0][3];
@@ -864,8 +936,16 @@ template <bool kWide>
 __global__ __launch_bounds__(kWide ? 2 * kThreads : kThreads, kWide ? 1 : 3) void viterbi_tiles_kernel(
     TileJob job, const double* __restrict__ entry_d, const float* __restrict__ entry_f, double* __restrict__ hist_all) {
   __shared__ Smem sm;
+  __shared__ uint32_t tl[kWide ? 512 : 1];  // wide form: the codebook's 512 value pairs as fp16 bits, for its trace-backs
   const int u = threadIdx.x & (kThreads - 1);
   const bool first_half = threadIdx.x < kThreads;  // global results are written once
+  if constexpr (kWide) {  // the table's values are fp16 values (entry bit 9 is the sign of the first one)
+    const int i = threadIdx.x;
+    const uint32_t h0 = __builtin_bit_cast(uint16_t, _Float16(entry_f[2 * i]));
+    const uint32_t h1 = __builtin_bit_cast(uint16_t, _Float16(entry_f[2 * i + 1]));
+    tl[i] = h0 | (h1 << 16);
+    __syncthreads();
+  }
   double* hist = hist_all + size_t(blockIdx.x) * kHistWordsPerTile;
   for (long tile = blockIdx.x; tile < job.tiles; tile += gridDim.x)
   for (int blk = job.blocks - 1; blk >= 0; --blk) {
@@ -890,11 +970,11 @@ __global__ __launch_bounds__(kWide ? 2 * kThreads : kThreads, kWide ? 1 : 3) voi
         if (pass == 0) {
           forward_pass32<true, kWide>(sm, entry_d, roll, -1, hist32, 62);
           flag |= uint32_t(sm.red32[0][1] < job.margin) | uint32_t(sm.red32[0][0] >= kWinnerMax);
-          const uint32_t s = trace_back32<true>(sm, entry_d, hist32, roll, sm.red32[0][2], 64, false, job.margin, flag);
+          const uint32_t s = trace_back32<true, kWide>(sm, entry_d, hist32, roll, sm.red32[0][2], 64, false, job.margin, flag, tl);
           if (!flag && u == 0) sm.overlap = int(s & 0xfffu);  // s is the state of step 63
         } else {
           forward_pass32<false, kWide>(sm, entry_d, roll, ov, hist32, 0);
-          const uint32_t s = trace_back32<false>(sm, entry_d, hist32, roll, uint32_t(ov), 2, true, job.margin, flag);
+          const uint32_t s = trace_back32<false, kWide>(sm, entry_d, hist32, roll, uint32_t(ov), 2, true, job.margin, flag, tl);
           // s is the state of step 1; at step 0 the one predecessor group with a finite initial metric is ov
           if (!flag && u == 0) sm.st[0] = uint16_t((s >> 4) | ((uint32_t(ov) >> 8) << 12));
         }
