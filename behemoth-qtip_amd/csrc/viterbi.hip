@@ -41,6 +41,14 @@
 // value-major: one contiguous 512-byte store per wave and value) are kept in HBM and the trace-back redoes the
 // add-compare-selects of the path it walks, two steps per round trip, with the forward pass's own fp64 operations
 // and tie rule.  Only the last step tracks its digits (in registers), which the final state needs.
+//
+// The above is the fp64 form.  By default every pass first runs on unsigned 32-bit metrics in units of 2^-25
+// (forward_pass32 / trace_back32 further down: 4-byte table and metrics in the same LDS footprint, double-buffered,
+// one barrier per step; the free pass computes the groups below 2048 only, since complementary states decode alike),
+// its trace-back checks that every decision it takes was won by more than the rounding can move two candidates
+// against each other, and a pass that fails the check is run again through the fp64 form in the same launch: the
+// states are the fp64 form's, bit for bit.  A launch that cannot fill the chip uses the kernel's wide form, 512
+// threads per tile.
 #include <hip/hip_ext.h>
 
 #include <cstddef>
