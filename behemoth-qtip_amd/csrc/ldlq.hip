@@ -292,19 +292,20 @@ int gemm_splitk_splits(long K, int N, int slots) {
   return int(best);
 }
 
-void launch_gemm_tn_f64_gather(int N, long K, const float* A, long lda, const float* B1, const float* B2, long ldb,
-                               double* P, double* partials, int slots, hipStream_t s) {
+int launch_gemm_tn_f64_gather(int N, long K, const float* A, long lda, const float* B1, const float* B2, long ldb,
+                              double* P, double* partials, int slots, hipStream_t s, bool reduce) {
   QTIP_REQUIRE(N >= 4 && K > 0 && K % KC == 0 && N % 4 == 0 && lda % 4 == 0 && ldb % 4 == 0 && B2 != nullptr,
                "fp64 gather GEMM needs 16-byte aligned fp32 rows and K %% 16 == 0");
   const int S = gemm_splitk_splits(K, N, slots);
   dim3 grid(unsigned((N + BN - 1) / BN), unsigned(S));
   gemm_tn_f64_splitk_kernel<<<grid, dim3(256), 0, s>>>(N, K, A, lda, B1, B2, ldb, S == 1 ? P : partials, N);
   QTIP_HIP(hipGetLastError());
-  if (S > 1) {
+  if (S > 1 && reduce) {
     const long count = long(BM) * N;
     sum_splits_kernel<<<dim3(unsigned((count + 255) / 256)), dim3(256), 0, s>>>(partials, S, count, P);
     QTIP_HIP(hipGetLastError());
   }
+  return S;
 }
 
 void launch_split_transpose_bf16(const float* X, const float* X2, long ldx, long rows_k, long cols_i, uint16_t* Th,
@@ -316,19 +317,21 @@ void launch_split_transpose_bf16(const float* X, const float* X2, long ldx, long
   QTIP_HIP(hipGetLastError());
 }
 
-void launch_gemm_img_gather(int N, long K, const uint16_t* Ah, const uint16_t* Al, long lda, const uint16_t* Bh,
-                            const uint16_t* Bl, long ldb, float* P, float* partials, int slots, hipStream_t s) {
+int launch_gemm_img_gather(int N, long K, const uint16_t* Ah, const uint16_t* Al, long lda, const uint16_t* Bh,
+                           const uint16_t* Bl, long ldb, float* P, float* partials, int slots, hipStream_t s,
+                           bool reduce) {
   QTIP_REQUIRE(N > 0 && K > 0 && K % IK == 0 && lda % 8 == 0 && ldb % 8 == 0 && Ah && Al && Bh && Bl,
                "split-bf16 gather GEMM needs K %% 16 == 0 and 16-byte aligned image rows");
   const int S = gemm_splitk_splits(K, N, slots);
   dim3 grid(unsigned((N + SB - 1) / SB), unsigned(S));
   gather_img_kernel<<<grid, dim3(256), 0, s>>>(N, K, Ah, Al, lda, Bh, Bl, ldb, S == 1 ? P : partials, N);
   QTIP_HIP(hipGetLastError());
-  if (S > 1) {
+  if (S > 1 && reduce) {
     const long count = long(SB) * N;
     sum_splits_f32_kernel<<<dim3(unsigned((count + 255) / 256)), dim3(256), 0, s>>>(partials, S, count, P);
     QTIP_HIP(hipGetLastError());
   }
+  return S;
 }
 
 }  // namespace qtipmi

@@ -238,6 +238,10 @@ struct TileJob {
   const float* prod32 = nullptr;
   long prod_row0 = 0;
   long ldp = 0;  // row stride of prod (0: ldw)
+  // prod as the split-K partial slabs of the gathered product: prod[s * prod_split_stride + ...], s < prod_splits,
+  // added in this order (what the product's own reduction kernel would have done)
+  int prod_splits = 1;
+  long prod_split_stride = 0;
   // outputs (any may be null)
   uint16_t* states = nullptr;  // state words of tile t at states[(t * q_tile_stride + q_offset) * 128]
   long q_tile_stride = 1, q_offset = 0;

@@ -177,16 +177,19 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
         // prod[r][:] = sum_{k >= bufend} L[k][c0 + r] (WT - hatWT)[k][:], r < 128
         const float* Lp = L + long(bufend) * n + c0;
         const float *Wp = WT + long(bufend) * m + C.r0, *Hp = hatWT + long(bufend) * m + C.r0;
+        // (the split-K partial slabs are summed by the Viterbi launch as it forms its targets, in the order the
+        // product's own reduction kernel would add them)
+        int splits = 1;
         if (bufend == n) {
           if (feedback == 0) QTIP_HIP(hipMemsetAsync(C.prod, 0, size_t(128) * C.rows * sizeof(double), C.s));
           else QTIP_HIP(hipMemsetAsync(C.prod32, 0, size_t(128) * C.rows * sizeof(float), C.s));
         } else if (feedback == 0) {
-          launch_gemm_tn_f64_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod, C.parts, C.slots, C.s);
+          splits = launch_gemm_tn_f64_gather(int(C.rows), n - bufend, Lp, n, Wp, Hp, m, C.prod, C.parts, C.slots, C.s, false);
         } else {
           const uint16_t* la = limg.p + size_t(c0) * n + bufend;
           const uint16_t* da = dimg.p + size_t(C.r0) * n + bufend;
-          launch_gemm_img_gather(int(C.rows), n - bufend, la, la + size_t(n) * n, n, da, da + size_t(m) * n, n, C.prod32,
-                                 C.parts32, C.slots, C.s);
+          splits = launch_gemm_img_gather(int(C.rows), n - bufend, la, la + size_t(n) * n, n, da, da + size_t(m) * n, n,
+                                          C.prod32, C.parts32, C.slots, C.s, false);
         }
         {
           // one launch per buffer: a workgroup takes its tile row through the 8 column blocks, last to first, and
@@ -197,9 +200,10 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
           job.L = L;
           job.ldl = n;
           job.bufend = bufend;
-          if (feedback == 0) job.prod64 = C.prod;
-          else job.prod32 = C.prod32;
+          if (feedback == 0) job.prod64 = splits > 1 ? C.parts : C.prod;
+          else job.prod32 = splits > 1 ? C.parts32 : C.prod32;
           job.prod_row0 = c0, job.ldp = C.rows;
+          job.prod_splits = splits, job.prod_split_stride = long(128) * C.rows;
           job.states = Q + size_t(C.tile0) * nblk * 128;
           job.q_tile_stride = nblk;
           job.q_offset = c0 / 16;

@@ -376,7 +376,10 @@ __device__ __forceinline__ void tile_targets(Smem& sm, const TileJob& job, long 
   __syncthreads();
   const int q = perm_fwd(u), r = q >> 4, c = q & 15;
   const long col = col0 + c;
-  Acc acc = Acc(job.WT[col * job.ldw + row0 + r]) + prod[(col - job.prod_row0) * (job.ldp ? job.ldp : job.ldw) + row0 + r];
+  const Acc* pp = prod + (col - job.prod_row0) * (job.ldp ? job.ldp : job.ldw) + row0 + r;
+  Acc gathered = pp[0];
+  for (int sp = 1; sp < job.prod_splits; ++sp) gathered += pp[long(sp) * job.prod_split_stride];
+  Acc acc = Acc(job.WT[col * job.ldw + row0 + r]) + gathered;
   for (int kk = 0; kk < nk; ++kk) acc += Acc(Ls[kk * 16 + c]) * (Acc(Ws[kk * 16 + r]) - Acc(Hs[kk * 16 + r]));
   sm.x[u] = float(_Float16(float(acc)));
 }
