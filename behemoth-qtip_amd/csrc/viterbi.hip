@@ -521,6 +521,17 @@ __device__ __forceinline__ int m32_pos(int col) {  // bits 7..0: b7 b6 b5 b4 b1 
 }
 __device__ __forceinline__ int m32_swz(int col) { return (((col >> 4) & 1) << 2) | ((((col >> 5) ^ (col >> 7)) & 1) << 3); }
 __device__ __forceinline__ int m32_slot(int col, int d) { return m32_pos(col) * 16 + (d ^ m32_swz(col)); }
+// The free pass keeps the groups below 2048 only (column c, digits 0..7) in a compact array: 8 slots per column,
+// column c at position [b7 b6 b5 b1 b0 b4 b3^b7 b2^b6], digit d in slot d ^ 4 b5.  The two 16-byte pieces of a
+// column are read by the 16 lanes of a turn from 16 different bank groups, for a thread's own column and for its
+// mirror 255 - c alike (digits 8..15 of column c are digits 7..0 of the mirror), and the 32 lanes of a half-wave
+// write 32 different banks.
+__device__ __forceinline__ int m32c_pos(int col) {
+  return (col & 0xe0) | (((col >> 1) & 1) << 4) | ((col & 1) << 3) | (((col >> 4) & 1) << 2) |
+         ((((col >> 3) ^ (col >> 7)) & 1) << 1) | (((col >> 2) ^ (col >> 6)) & 1);
+}
+__device__ __forceinline__ int m32c_swz(int col) { return ((col >> 5) & 1) << 2; }
+__device__ __forceinline__ int m32c_slot(int col, int d) { return m32c_pos(col) * 8 + (d ^ m32c_swz(col)); }
 // thread that owns group jj < 2048 in the 32-bit passes
 __device__ __forceinline__ uint32_t owner32(uint32_t jj) {
   const uint32_t c = jj >> 4;
@@ -548,8 +559,8 @@ __device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, d
   return uint32_t(__builtin_fmin(v, 2147483647.0));
 }
 
-// One forward pass on 32-bit metrics.  kSym: free ends, the groups below 2048 only (their mirrors get copies), all
-// 128 steps, and the best final group, its metric and the gap to the runner-up are left in sm.red32[0]; otherwise:
+// One forward pass on 32-bit metrics.  kSym: free ends, the groups below 2048 only (a mirror group's metric is read
+// from the group it mirrors), all 128 steps, and the best final group, its metric and the gap to the runner-up are left in sm.red32[0]; otherwise:
 // start in group ov, steps 0 .. 126 (the last step's decision is taken by the trace-back from the metrics entering
 // it).  The results of the even steps first_kept .. 126 (the metrics entering the next, odd step) go to hist.
 // Metrics and error table are double-buffered in LDS (2 x 16 KB, 2 x 8 KB: the footprint of the fp64 arrays): a step
@@ -565,36 +576,77 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
   const int tid = tfull & (kThreads - 1), upper = kWide ? tfull >> 8 : 0;
   const int colA = 4 * (tid & 31) + ((tid >> 5) & 3), colB = 255 - colA;
   const int half = tid >> 7;
-  uint32_t* const E32 = reinterpret_cast<uint32_t*>(sm.E);  // [2][32 positions][64 rows]
-  uint32_t* const M32 = reinterpret_cast<uint32_t*>(sm.M);  // [2][4096]
+  // Tail-biting pass: table [2][32 positions][64 rows] in sm.E, metrics [2][4096] in sm.M.  Free pass: the same 48 KB
+  // hold the table as pairs of neighbouring positions, [2][2 parities][16 pairs][64 rows] x 8 bytes (a lane reads its
+  // 16 positions as eight 8-byte pieces, 333 against 250 B/ns for two-dword reads; parity 0 pairs the positions
+  // (2p, 2p + 1), parity 1 (2p + 1, 2p + 2), the 8 pairs stored twice for the wrap-around), then the compact
+  // metrics [2][2048].
+  constexpr int kEPairWords = 2 * 16 * 64 * 2, kMcSlots = kGroups / 2;
+  uint32_t* const E32 = reinterpret_cast<uint32_t*>(sm.E);
+  uint32_t* const M32 = kSym ? E32 + 2 * kEPairWords : reinterpret_cast<uint32_t*>(sm.M);
   static_assert(sizeof(sm.E) >= 2 * kESlots * sizeof(uint32_t) && sizeof(sm.M) >= 2 * kMSlots * sizeof(uint32_t));
+  static_assert(offsetof(Smem, M) == sizeof(sm.E) &&
+                sizeof(sm.E) + sizeof(sm.M) >= (2 * kEPairWords + 2 * kMcSlots) * sizeof(uint32_t));
   double2 ent[kEnt];
   const double2* __restrict__ entries = reinterpret_cast<const double2*>(entry_d) + tfull;
 #pragma unroll
   for (int q = 0; q < kEnt; ++q) ent[q] = entries[kT * q];
   const int e_wr = tfull;
+  const int e_w = tfull >> 6, e_row = tfull & 63;
+  const int e_wr0 = ((e_w >> 1) * 64 + e_row) * 2 + (e_w & 1);                        // words, free pass
+  const int e_wr1 = ((16 + ((e_w + 1) >> 1) - 1) * 64 + e_row) * 2 + ((e_w & 1) ^ 1);  // floor((w - 1) / 2) = (w + 1) / 2 - 1
   int ebase[kSlotsOwn], wslot[kSlotsOwn];  // of the slots m0 .. m0 + kSlotsOwn - 1, m0 = 4 upper
 #pragma unroll
   for (int i = 0; i < kSlotsOwn; ++i) {
     const uint32_t j = 16u * colA + 8u * uint32_t(half) + uint32_t(i + 4 * upper), p = j * (j + 1u);
-    ebase[i] = int((p >> 12) & 15u) * 64 + int((p >> 6) & 63u);
-    wslot[i] = m32_slot(int(j & 255u), int(j >> 8));
+    const int pos0 = int((p >> 12) & 15u), row = int((p >> 6) & 63u);
+    if constexpr (kSym) {
+      ebase[i] = (((pos0 & 1) * 16 + (pos0 >> 1)) * 64 + row) * 2;  // words: parity, first pair, row
+      wslot[i] = m32c_slot(int(j & 255u), int(j >> 8));
+    } else {
+      ebase[i] = pos0 * 64 + row;
+      wslot[i] = m32_slot(int(j & 255u), int(j >> 8));
+    }
   }
-  int xA = m32_pos(colA) * 64 + m32_swz(colA) * 4, xB = m32_pos(colB) * 64 + m32_swz(colB) * 4;  // bytes
+  // bytes
+  int xA = kSym ? m32c_pos(colA) * 32 + m32c_swz(colA) * 4 : m32_pos(colA) * 64 + m32_swz(colA) * 4;
+  int xB = kSym ? m32c_pos(colB) * 32 + m32c_swz(colB) * 4 : m32_pos(colB) * 64 + m32_swz(colB) * 4;
   // the error table of step `it` into table buffer it & 1
   auto table = [&](int it) __attribute__((always_inline)) {
     const int t = (2 * it + roll) & 255;
     const double x0 = double(sm.x[t]), x1 = double(sm.x[t + 1]);
-    uint32_t* const Ew = E32 + (it & 1) * kESlots + e_wr;
+    if constexpr (kSym) {
+      // thread (w = t / 64, row = t % 64) holds the entries of the positions w + (kT / 64) q.  Parity 0: pair
+      // position / 2, half position % 2; parity 1: pair floor((position - 1) / 2), the other half; pair -1, which
+      // position 0 asks for, is pair 15 of parity 0, which like itself nobody reads.  Every pair a second time 8
+      // further on.  Both addresses advance by kT words per q.
+      uint32_t* const Ew0 = E32 + (it & 1) * kEPairWords + e_wr0;
+      uint32_t* const Ew1 = E32 + (it & 1) * kEPairWords + e_wr1;
 #pragma unroll
-    for (int q = 0; q < kEnt; ++q) {
-      const double2 l = ent[q];
-      const uint32_t v = err_units(l.x, l.y, x0, x1);
-      Ew[kT * q] = v;
-      Ew[kT * q + 1024] = v;
+      for (int q = 0; q < kEnt; ++q) {
+        const double2 l = ent[q];
+        const uint32_t v = err_units(l.x, l.y, x0, x1);
+        Ew0[kT * q] = v;
+        Ew0[kT * q + 8 * 128] = v;
+        Ew1[kT * q] = v;
+        Ew1[kT * q + 8 * 128] = v;
+      }
+    } else {
+      uint32_t* const Ew = E32 + (it & 1) * kESlots + e_wr;
+#pragma unroll
+      for (int q = 0; q < kEnt; ++q) {
+        const double2 l = ent[q];
+        const uint32_t v = err_units(l.x, l.y, x0, x1);
+        Ew[kT * q] = v;
+        Ew[kT * q + 1024] = v;
+      }
     }
   };
-  for (int g = tfull; g < kGroups; g += kT) M32[m32_slot(g & 255, g >> 8)] = (ov < 0 || g == ov) ? 0u : kSat;
+  if constexpr (kSym) {
+    for (int g = tfull; g < kMcSlots; g += kT) M32[g] = 0u;
+  } else {
+    for (int g = tfull; g < kGroups; g += kT) M32[m32_slot(g & 255, g >> 8)] = (ov < 0 || g == ov) ? 0u : kSat;
+  }
   table(0);
   __syncthreads();
 
@@ -604,16 +656,26 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
     constexpr int kind = decltype(kind_tag)::value;  // kDigits: the free pass's last step, results to fin only
     uint32_t* hs = nullptr;
     if constexpr (kind == kStore) hs = hist + size_t(it >> 1) * kGroups + tid;
-    const char* const Mb = reinterpret_cast<const char*>(M32 + (it & 1) * kMSlots);
-    uint32_t* const Mw = M32 + ((it + 1) & 1) * kMSlots;
-    const uint32_t* const Er = E32 + (it & 1) * kESlots;
+    constexpr int kMBuf = kSym ? kMcSlots : kMSlots, kEBuf = kSym ? kEPairWords : kESlots;
+    const char* const Mb = reinterpret_cast<const char*>(M32 + (it & 1) * kMBuf);
+    uint32_t* const Mw = M32 + ((it + 1) & 1) * kMBuf;
+    const uint32_t* const Er = E32 + (it & 1) * kEBuf;
     uint32_t MA[16], MB[16];
     asm volatile("" : "+v"(xA), "+v"(xB));
+    if constexpr (kSym) {
+      // digits 0..7 of the own column, and digits 8..15 as digits 7..0 of the mirror column
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const uint4 a = *reinterpret_cast<const uint4*>(Mb + (xA ^ (16 * k)));
-      MA[4 * k] = a.x, MA[4 * k + 1] = a.y, MA[4 * k + 2] = a.z, MA[4 * k + 3] = a.w;
-      if constexpr (!kSym) {
+      for (int k = 0; k < 2; ++k) {
+        const uint4 a = *reinterpret_cast<const uint4*>(Mb + (xA ^ (16 * k)));
+        MA[4 * k] = a.x, MA[4 * k + 1] = a.y, MA[4 * k + 2] = a.z, MA[4 * k + 3] = a.w;
+        const uint4 b = *reinterpret_cast<const uint4*>(Mb + (xB ^ (16 * k)));
+        MA[15 - 4 * k] = b.x, MA[14 - 4 * k] = b.y, MA[13 - 4 * k] = b.z, MA[12 - 4 * k] = b.w;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint4 a = *reinterpret_cast<const uint4*>(Mb + (xA ^ (16 * k)));
+        MA[4 * k] = a.x, MA[4 * k + 1] = a.y, MA[4 * k + 2] = a.z, MA[4 * k + 3] = a.w;
         const uint4 b = *reinterpret_cast<const uint4*>(Mb + (xB ^ (16 * k)));
         MB[4 * k] = b.x, MB[4 * k + 1] = b.y, MB[4 * k + 2] = b.z, MB[4 * k + 3] = b.w;
       }
@@ -621,27 +683,61 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
     if constexpr (kind != kDigits) table(it + 1);
     // The 16 table values of a slot are fetched while the slot before it is worked on; the value of digit k of slot
     // m lies (k (2 m + 1)) % 16 positions after the slot's first.  m0: the first slot of this thread, a constant in
-    // each of the two copies of the loop that the wide form needs.
+    // each of the two copies of the loop that the wide form needs.  Tail-biting pass: evb[.][k] is the value of digit
+    // k (the offsets of the reads are permuted); free pass: evb[.][t] is the value t positions after the first
+    // (eight 8-byte reads, kept apart: the paired form of the read is the slower one), digit k reads it at
+    // (k (2 m + 1)) % 16.
     auto slots = [&](auto m0_tag) __attribute__((always_inline)) {
     constexpr int m0 = decltype(m0_tag)::value;
-    uint32_t evb[2][16];
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    uint32_t evb[2][kSym ? 1 : 16];  // tail-biting pass: 16 values
+    u32x2 evp[2][kSym ? 8 : 1];      // free pass: 8 pieces of two neighbouring positions
+    auto fetch = [&](int own, int gn, int buf) __attribute__((always_inline)) {
+      const uint32_t* er = Er + ebase[own];
+      if constexpr (kSym) {
+        // written out, so that the eight reads stay eight: the compiler would pair them (ds_read2st64_b64), and the
+        // paired read moves fewer bytes per cycle than two single ones.  It does not know of their latency either:
+        // the wait below is what the uses of the values depend on.
+        const uint32_t a = uint32_t(reinterpret_cast<size_t>(er));
+#define QTIP_READ_PAIR(I) asm volatile("ds_read_b64 %0, %1 offset:" #I "*512" : "=v"(evp[buf][I]) : "v"(a));
+        QTIP_READ_PAIR(0) QTIP_READ_PAIR(1) QTIP_READ_PAIR(2) QTIP_READ_PAIR(3)
+        QTIP_READ_PAIR(4) QTIP_READ_PAIR(5) QTIP_READ_PAIR(6) QTIP_READ_PAIR(7)
+#undef QTIP_READ_PAIR
+      } else {
 #pragma unroll
-    for (int k = 0; k < 16; ++k) evb[0][k] = Er[ebase[0] + ((k * (2 * m0 + 1)) & 15) * 64];
+        for (int k = 0; k < 16; ++k) evb[buf][k] = er[((k * gn) & 15) * 64];
+      }
+    };
+    fetch(0, 2 * m0 + 1, 0);
 #pragma unroll
     for (int i = 0; i < kSlotsOwn; ++i) {
       constexpr int kLast = kSlotsOwn - 1;
       const int m = i;  // index into this thread's own slots
-      if (i < kLast) {
-        const int gn = 2 * (m0 + i + 1) + 1;
-        const uint32_t* er = Er + ebase[i < kLast ? i + 1 : kLast];
-#pragma unroll
-        for (int k = 0; k < 16; ++k) evb[(i + 1) & 1][k] = er[((k * gn) & 15) * 64];
-      }
+      if (i < kLast) fetch(i < kLast ? i + 1 : kLast, 2 * (m0 + i + 1) + 1, (i + 1) & 1);
       const uint32_t* ev = evb[i & 1];
-      // the table value at position k is the candidate of digit k of the group and of digit 15 - k of its mirror
+      u32x2* ep = evp[i & 1];
+      if constexpr (kSym) {
+        // the reads of this slot's values are done when at most the eight issued after them (the next slot's) are
+        // outstanding: LDS operations complete in order
+#define QTIP_EP8 "+v"(ep[0]), "+v"(ep[1]), "+v"(ep[2]), "+v"(ep[3]), "+v"(ep[4]), "+v"(ep[5]), "+v"(ep[6]), "+v"(ep[7])
+        if (i < kLast) asm volatile("s_waitcnt lgkmcnt(8)" : QTIP_EP8);
+        else asm volatile("s_waitcnt lgkmcnt(0)" : QTIP_EP8);
+#undef QTIP_EP8
+      }
+      const int g = 2 * (m0 + i) + 1;
+      // the table value of digit k
+      auto at = [&](int k) -> uint32_t {
+        if constexpr (kSym) {
+          const int t = (k * g) & 15;
+          return (t & 1) ? ep[t >> 1].y : ep[t >> 1].x;
+        } else {
+          return ev[k];
+        }
+      };
+      // the table value of digit k is the candidate of digit k of the group and of digit 15 - k of its mirror
       uint32_t ba = kSat;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) ba = min3u(ba, sat_add(ev[2 * k], MA[2 * k]), sat_add(ev[2 * k + 1], MA[2 * k + 1]));
+      for (int k = 0; k < 8; ++k) ba = min3u(ba, sat_add(at(2 * k), MA[2 * k]), sat_add(at(2 * k + 1), MA[2 * k + 1]));
       uint32_t bb = ba;
       if constexpr (!kSym) {
         bb = kSat;
@@ -653,7 +749,7 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
         fin[m] = ba;
       } else {
         Mw[wslot[m]] = ba;
-        Mw[wslot[m] ^ kMirror32] = bb;
+        if constexpr (!kSym) Mw[wslot[m] ^ kMirror32] = bb;
       }
       if constexpr (kind == kStore) {
         hs[(m0 + m) * kThreads] = ba;
