@@ -587,14 +587,18 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
   static_assert(sizeof(sm.E) >= 2 * kESlots * sizeof(uint32_t) && sizeof(sm.M) >= 2 * kMSlots * sizeof(uint32_t));
   static_assert(offsetof(Smem, M) == sizeof(sm.E) &&
                 sizeof(sm.E) + sizeof(sm.M) >= (2 * kEPairWords + 2 * kMcSlots) * sizeof(uint32_t));
+  // The table entries (position, row) = entry index position * 64 + row a thread forms each step.  Tail-biting
+  // pass: entry t + kT q.  Free pass: row (t % 16) + 16 (t / 32 % 4), positions 2 (t / 128 + (kT / 128) q) + (t / 16
+  // % 2): the 32 lanes of a half-wave then hold both halves of 16 rows' pairs and write 32 different banks.
+  const int e_row = (tfull & 15) | (((tfull >> 5) & 3) << 4), e_h = (tfull >> 4) & 1, e_a = tfull >> 7;
+  const int e_wr = kSym ? (2 * e_a + e_h) * 64 + e_row : tfull;
   double2 ent[kEnt];
-  const double2* __restrict__ entries = reinterpret_cast<const double2*>(entry_d) + tfull;
+  const double2* __restrict__ entries = reinterpret_cast<const double2*>(entry_d) + e_wr;
 #pragma unroll
   for (int q = 0; q < kEnt; ++q) ent[q] = entries[kT * q];
-  const int e_wr = tfull;
-  const int e_w = tfull >> 6, e_row = tfull & 63;
-  const int e_wr0 = ((e_w >> 1) * 64 + e_row) * 2 + (e_w & 1);                        // words, free pass
-  const int e_wr1 = ((16 + ((e_w + 1) >> 1) - 1) * 64 + e_row) * 2 + ((e_w & 1) ^ 1);  // floor((w - 1) / 2) = (w + 1) / 2 - 1
+  // free pass, words: parity 0 holds position 2a + h in pair a, half h; parity 1 in pair a - 1 + h, the other half
+  const int e_wr0 = (e_a * 64 + e_row) * 2 + e_h;
+  const int e_wr1 = ((16 + e_a - 1 + e_h) * 64 + e_row) * 2 + (e_h ^ 1);
   int ebase[kSlotsOwn], wslot[kSlotsOwn];  // of the slots m0 .. m0 + kSlotsOwn - 1, m0 = 4 upper
 #pragma unroll
   for (int i = 0; i < kSlotsOwn; ++i) {
@@ -616,10 +620,9 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
     const int t = (2 * it + roll) & 255;
     const double x0 = double(sm.x[t]), x1 = double(sm.x[t + 1]);
     if constexpr (kSym) {
-      // thread (w = t / 64, row = t % 64) holds the entries of the positions w + (kT / 64) q.  Parity 0: pair
-      // position / 2, half position % 2; parity 1: pair floor((position - 1) / 2), the other half; pair -1, which
-      // position 0 asks for, is pair 15 of parity 0, which like itself nobody reads.  Every pair a second time 8
-      // further on.  Both addresses advance by kT words per q.
+      // Parity 0: pair position / 2, half position % 2; parity 1: pair floor((position - 1) / 2), the other half;
+      // pair -1, which position 0 asks for, is pair 15 of parity 0, which like itself nobody reads.  Every pair a
+      // second time 8 further on.  Both addresses advance by kT words per q (kT / 128 pairs).
       uint32_t* const Ew0 = E32 + (it & 1) * kEPairWords + e_wr0;
       uint32_t* const Ew1 = E32 + (it & 1) * kEPairWords + e_wr1;
 #pragma unroll
