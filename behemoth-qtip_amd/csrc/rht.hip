@@ -197,10 +197,18 @@ __global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict_
   }
 }
 
-__global__ void scale_kernel(float* __restrict__ X, long rows, long cols, long ld, float a) {
-  const long i = long(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i >= rows * cols) return;
-  X[(i / cols) * ld + i % cols] *= a;
+// X[r][c] *= a: a block takes a row segment of 1024 columns, four floats per thread where the row allows it
+__global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ X, long rows, long cols, long ld, float a) {
+  const long r = blockIdx.y;
+  const long c = (long(blockIdx.x) * 256 + threadIdx.x) * 4;
+  float* p = X + r * ld + c;
+  if (c + 4 <= cols && (reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+    float4 v = *reinterpret_cast<float4*>(p);
+    v.x *= a, v.y *= a, v.z *= a, v.w *= a;
+    *reinterpret_cast<float4*>(p) = v;
+  } else {
+    for (int e = 0; e < 4 && c + e < cols; ++e) p[e] *= a;
+  }
 }
 
 __global__ void add_diag_kernel(float* __restrict__ H, long n, float a) {
@@ -230,11 +238,13 @@ __global__ __launch_bounds__(kRedThreads) void reduce_partial_kernel(const float
   const long per = (total + gridDim.x - 1) / gridDim.x;
   const long lo = long(blockIdx.x) * per, hi = lo + per < total ? lo + per : total;
   double acc = 0;
+  // (row, column) of the element i = r cols + c, carried along instead of divided out for every element
+  long r = 0, c = 0;
+  if (mode != 3 && lo + threadIdx.x < hi) r = (lo + threadIdx.x) / cols, c = (lo + threadIdx.x) % cols;
   for (long i = lo + threadIdx.x; i < hi; i += kRedThreads) {
     if (mode == 3) {
       acc += double(A[i * lda + i]);
     } else {
-      const long r = i / cols, c = i % cols;
       const double a = A[r * lda + c];
       if (mode == 0) acc += a * a;
       else {
@@ -242,6 +252,8 @@ __global__ __launch_bounds__(kRedThreads) void reduce_partial_kernel(const float
         if (mode == 1) acc += a * b;
         else acc += (a - b) * (a - b);
       }
+      c += kRedThreads;
+      while (c >= cols) c -= cols, ++r;
     }
   }
   acc = block_sum(acc);
@@ -348,7 +360,10 @@ void Rht::transpose(const float* in, long rows, long cols, long ld_in, float* ou
 
 void Rht::scale(float* X, long rows, long cols, long ld, float a) {
   if (rows * cols <= 0) return;
-  scale_kernel<<<dim3(unsigned((rows * cols + 255) / 256)), dim3(256), 0, s_>>>(X, rows, cols, ld, a);
+  for (long r0 = 0; r0 < rows; r0 += 65535) {  // the grid's second dimension holds 65535 rows
+    const long nr = std::min<long>(65535, rows - r0);
+    scale_kernel<<<dim3(unsigned((cols + 1023) / 1024), unsigned(nr)), dim3(256), 0, s_>>>(X + r0 * ld, nr, cols, ld, a);
+  }
   QTIP_HIP(hipGetLastError());
 }
 
