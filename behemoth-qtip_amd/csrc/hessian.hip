@@ -16,6 +16,7 @@
 // straight into LDS.  Workgroups are numbered so that the 32 that share an XCD (and its L2) at a time form an 8 x 4
 // patch of tiles, which needs 12 operand slices instead of 33.
 #include <mutex>
+#include <type_traits>
 #include <vector>
 
 #include "misc.hpp"
@@ -35,8 +36,9 @@ constexpr int kPatchRows = 8, kPatchCols = 4;             // tiles per XCD patch
 // pieces of a column at position p ^ ((column >> 2) & 3) (free of bank conflicts for the 16-byte fragment reads: the
 // 16 lanes the LDS serves together then touch 16 different 16-byte bank groups).  A stage of an operand is 16 KB of
 // contiguous global memory and goes straight into LDS (global_load_lds_dwordx4, 1 KB per wave and instruction): no
-// staging registers, no transposes, no LDS writes by the waves.  Four stages of LDS; the loads run two stages ahead
-// of the matrix cores, and a wave fetches the fragments of the next 16 k while the 16 MFMAs of the present ones run.
+// staging registers, no transposes, no LDS writes by the waves.  Four stages of LDS; the loads run three stages ahead
+// of the matrix cores, and a wave fetches the fragments of the next 16 k while the 16 MFMAs of the present ones run,
+// every fragment read and every load in the shadow of an MFMA of its own.
 constexpr int IK = 32, ISTAGES = 4;
 constexpr int kImgSliceU16 = kTile * IK;                                  // one operand slice of a stage, 16 KB
 constexpr size_t kImgLdsBytes = size_t(ISTAGES) * 2 * kImgSliceU16 * 2;   // 128 KB
@@ -57,7 +59,8 @@ __global__ __launch_bounds__(256, 1) void syrk_img_kernel(const uint16_t* __rest
   const long ti = (patch / patch_cols) * kPatchRows + within / kPatchCols;
   const long tj = (patch % patch_cols) * kPatchCols + within % kPatchCols;
   if (ti >= tiles || tj > ti) return;  // outside the matrix or above the diagonal
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // uniform: the LDS addresses of the loads stay scalar
   const int wm = wave >> 1, wn = wave & 1;
   const int rl = lane & 31;
 
@@ -79,93 +82,142 @@ __global__ __launch_bounds__(256, 1) void syrk_img_kernel(const uint16_t* __rest
       for (int c = 0; c < 4; ++c) acc[a][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z, z, acc[a][c], 0, 0, 0);
   }
 
-  // wave w brings the 1 KB chunks 4 w .. 4 w + 3 of both operand slices of a stage, 16 bytes per lane
+  // wave w brings the 1 KB chunks 4 w .. 4 w + 3 of both operand slices of a stage, 16 bytes per lane.  pa / pb: this
+  // lane's piece of operand A's / B's slice of stage sa / sb, the stage whose loads are requested next (a quarter of a
+  // slice per instruction: one address and one LDS base per operand and stage, the quarter in the immediate offset)
   const size_t stage_stride = size_t(tiles) * kImgSliceU16;
-  const uint16_t* ga = IA + size_t(ti) * kImgSliceU16 + (wave * 4) * 512 + lane * 8;
-  const uint16_t* gb = IB + size_t(tj) * kImgSliceU16 + (wave * 4) * 512 + lane * 8;
+  const uint16_t* pa = IA + size_t(ti) * kImgSliceU16 + (wave * 4) * 512 + lane * 8;
+  const uint16_t* pb = IB + size_t(tj) * kImgSliceU16 + (wave * 4) * 512 + lane * 8;
+  int sa = 0, sb = 0;
   typedef __attribute__((address_space(3))) void* lds_ptr;
-  auto issue = [&](int st) {
-    uint16_t* la = lds + (st % ISTAGES) * 2 * kImgSliceU16 + (wave * 4) * 512;
-    const size_t off = size_t(st) * stage_stride;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      __builtin_amdgcn_global_load_lds(ga + off + q * 512, (lds_ptr)(la + q * 512), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(gb + off + q * 512, (lds_ptr)(la + kImgSliceU16 + q * 512), 16, 0, 0);
-    }
-  };
-  // fragment of 8 k (piece 2 ks + lane / 32) of column wX * 128 + 32 i + rl
+#define QTIP_LOAD_A(q) \
+  __builtin_amdgcn_global_load_lds(pa, (lds_ptr)(lds + (sa % ISTAGES) * 2 * kImgSliceU16 + (wave * 4) * 512), 16, (q) * 1024, 0)
+#define QTIP_LOAD_B(q)                                                                                                  \
+  __builtin_amdgcn_global_load_lds(pb, (lds_ptr)(lds + (sb % ISTAGES) * 2 * kImgSliceU16 + kImgSliceU16 + (wave * 4) * 512), \
+                                   16, (q) * 1024, 0)
+  auto request_a = [&] { QTIP_LOAD_A(0); QTIP_LOAD_A(1); QTIP_LOAD_A(2); QTIP_LOAD_A(3); pa += stage_stride; ++sa; };
+  auto request_b = [&] { QTIP_LOAD_B(0); QTIP_LOAD_B(1); QTIP_LOAD_B(2); QTIP_LOAD_B(3); pb += stage_stride; ++sb; };
+  // fragment of 8 k (piece 2 ks + lane / 32) of column wX * 128 + 32 i + rl.  read1 fetches fragment j of a step in the
+  // order its MFMAs first use them: a0 b0 b1 b2 b3 a1 a2 a3
   const int offA = (wm * 128 + rl) * IK, offB = (wn * 128 + rl) * IK, sw = (rl >> 2) & 3, hi = lane >> 5;
   bf16x8 fa[2][4], fb[2][4];
-  auto fetch = [&](int st, int ks, int set) {
+  auto read1 = [&](int st, int ks, int set, int j) {
     const uint16_t* As = lds + (st % ISTAGES) * 2 * kImgSliceU16;
     const int piece = ((2 * ks + hi) ^ sw) << 3;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    if (j == 0 || j >= 5) {
+      const int i = j == 0 ? 0 : j - 4;
       fa[set][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + offA + i * 32 * IK + piece));
+    } else {
+      const int i = j - 1;
       fb[set][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(As + kImgSliceU16 + offB + i * 32 * IK + piece));
     }
   };
-  auto mfmas = [&](int set, int half) {  // the 8 MFMAs of row tiles 2 half, 2 half + 1
-#pragma unroll
-    for (int mi = 2 * half; mi < 2 * half + 2; ++mi)
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni)
-        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
+  auto mfma = [&](int set, int j) {  // MFMA j of a step: row tile j / 4, column tile j % 4
+    const int mi = j >> 2, ni = j & 3;
+    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
   };
-  auto landed = [&](int later_stages) {  // this wave's loads of a stage have landed (8 per stage, in order) ...
-    if (later_stages >= 1) __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
-    else __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0)
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();  // ... and so have everyone's (a bare barrier: no wait for the loads in flight)
-    asm volatile("" ::: "memory");
-  };
-  for (int p = 0; p < 2 && p < stages; ++p) issue(p);
-  landed(stages > 1 ? 1 : 0);
-  if (stages > 2) issue(2);
-  fetch(0, 0, 0);
-  // A wave has nothing to hide a wait behind but its own MFMAs, so the fragments of the next 16 k are requested
-  // between the two halves of the 16 MFMAs of the present ones: the wait the compiler puts in front of their first
-  // use then finds them there.
-  for (int st = 0; st < stages; ++st) {
-    mfmas(0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    fetch(st, 1, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    mfmas(0, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    if (st + 1 < stages) {
-      // stage st + 1 is needed next; stage st + 2 may still be on its way; the buffer of stage st - 1, which every
-      // wave has read before this barrier, takes stage st + 3
-      landed(st + 2 < stages ? 1 : 0);
-      if (st + 3 < stages) issue(st + 3);
+
+  // Stages 0..2 requested, stage 0 landed (this wave's loads, then everyone's: a bare barrier, which does not wait
+  // for the loads still in flight), operand A of stage 3 requested, the fragments of stage 0's first 16 k read.
+  const int pre = stages < ISTAGES - 1 ? stages : ISTAGES - 1;
+  for (int p = 0; p < pre; ++p) request_a(), request_b();
+  if (pre >= 3) __builtin_amdgcn_s_waitcnt(0x4F70);       // vmcnt(16)
+  else if (pre == 2) __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
+  else __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0)
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  if (sa < stages) request_a();
+#pragma unroll
+  for (int j = 0; j < 8; ++j) read1(0, 0, 0, j);
+
+  // One stage: 32 MFMAs, two steps of 16 k on fragment sets 0 and 1.  A wave has nothing to hide a wait behind but
+  // its own MFMAs (one wave per SIMD), and an MFMA keeps the matrix core busy for 32 cycles while the wave may issue
+  // other work: so no two memory instructions follow each other.  Under every other MFMA of a step the wave reads one
+  // fragment of the next step, and under MFMAs 1, 5, 9, 13 it requests a quarter of an operand slice three stages
+  // ahead: operand B of stage st + 3 during step 0, then - after the barrier that says stage st + 1 has landed
+  // everywhere and every wave has asked for its last fragments of stage st, whose buffer is therefore free - operand
+  // A of stage st + 4 during step 1.  (The same instructions in bursts - 8 fragment reads, then 8 MFMAs, 8 loads
+  // after the barrier - left the matrix cores idle for a quarter of the loop.)  The scheduling barriers pin the order.
+  // kSteady: every stage asked for exists and two stages beyond st + 1 are on their way, so vmcnt(16) = "stage
+  // st + 1 is here"; the last stages run the same code with the conditions and a full wait.
+#define QTIP_SB __builtin_amdgcn_sched_barrier(0)
+  auto stage = [&](auto steady, int st) {
+    constexpr bool kSteady = decltype(steady)::value;
+    const bool next = kSteady || st + 1 < stages;
+    {
+      const bool go = kSteady || sb < stages;
+#define QTIP_M0(j) { mfma(0, j); QTIP_SB; }
+#define QTIP_R0(j) { mfma(0, j); QTIP_SB; read1(st, 1, 1, (j) / 2); QTIP_SB; }
+#define QTIP_L0(j) { mfma(0, j); QTIP_SB; if (go) QTIP_LOAD_B(((j) - 1) / 4); QTIP_SB; }
+      QTIP_SB;
+      QTIP_R0(0) QTIP_L0(1) QTIP_R0(2) QTIP_M0(3) QTIP_R0(4) QTIP_L0(5) QTIP_R0(6) QTIP_M0(7)
+      QTIP_R0(8) QTIP_L0(9) QTIP_R0(10) QTIP_M0(11) QTIP_R0(12) QTIP_L0(13) QTIP_R0(14) QTIP_M0(15)
+      if (go) pb += stage_stride, ++sb;
     }
-    mfmas(1, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    if (st + 1 < stages) fetch(st + 1, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    mfmas(1, 1);
-    __builtin_amdgcn_sched_barrier(0);
-  }
+    if (next) {
+      if (kSteady) __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16)
+      else __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    }
+    {
+      const bool go = kSteady || sa < stages;
+#define QTIP_M1(j) { mfma(1, j); QTIP_SB; }
+#define QTIP_R1(j) { mfma(1, j); QTIP_SB; if (next) read1(st + 1, 0, 0, (j) / 2); QTIP_SB; }
+#define QTIP_L1(j) { mfma(1, j); QTIP_SB; if (go) QTIP_LOAD_A(((j) - 1) / 4); QTIP_SB; }
+      QTIP_SB;
+      QTIP_R1(0) QTIP_L1(1) QTIP_R1(2) QTIP_M1(3) QTIP_R1(4) QTIP_L1(5) QTIP_R1(6) QTIP_M1(7)
+      QTIP_R1(8) QTIP_L1(9) QTIP_R1(10) QTIP_M1(11) QTIP_R1(12) QTIP_L1(13) QTIP_R1(14) QTIP_M1(15)
+      if (go) pa += stage_stride, ++sa;
+    }
+  };
+  int st = 0;
+  for (; st + 4 < stages; ++st) stage(std::true_type{}, st);
+  for (; st < stages; ++st) stage(std::false_type{}, st);
+#undef QTIP_M0
+#undef QTIP_R0
+#undef QTIP_L0
+#undef QTIP_M1
+#undef QTIP_R1
+#undef QTIP_L1
+#undef QTIP_SB
+#undef QTIP_LOAD_A
+#undef QTIP_LOAD_B
   __syncthreads();
 
   // accumulator element v of a lane: row (v % 4) + 8 (v / 4) + 4 (lane / 32), column lane % 32 of the 32 x 32 tile
   double dot = 0.0;
   if ((ti + 1) * kTile <= n && (tj + 1) * kTile <= n) {
-    float* hb = H + (ti * kTile + wm * 128 + 4 * (lane >> 5)) * n + tj * kTile + wn * 128 + rl;
+    // (the lane number is taken anew: nothing of the addresses below then has to live through the loop above)
+    const int ln = int(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
+    float* hb = H + (ti * kTile + wm * 128 + 4 * (ln >> 5)) * n + tj * kTile + wn * 128 + (ln & 31);
+    // The 16 values of H that go with a 32 x 32 accumulator are fetched together (one predicated load at a time
+    // would be 256 dependent round trips to HBM per tile), and in the accumulating form one accumulator ahead of the
+    // one being added to: a lone wave per SIMD has nothing else to cover the 16 round trips with, and a batch of 8192
+    // rows is only 256 stages of work per tile.  (The proxy's form has 4.5 times the stages and 64-bit sums to hold.
+    // Larger batches - a row of four accumulators, or two accumulators ahead - do not fit the registers.)
+    constexpr int kAheadH = DOT ? 0 : 1;
+    float h[kAheadH + 1][16];
+    auto fetch_h = [&](int blk) {
+      const int mi = blk >> 2, ni = blk & 3;
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
+      for (int v = 0; v < 16; ++v) h[blk % (kAheadH + 1)][v] = hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32];
+    };
+    if (kAheadH) fetch_h(0);
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni) {
-        float h[16];
+    for (int blk = 0; blk < 16; ++blk) {
+      const int mi = blk >> 2, ni = blk & 3;
+      __builtin_amdgcn_sched_barrier(0);
+      if (blk + kAheadH < 16) fetch_h(blk + kAheadH);
+      __builtin_amdgcn_sched_barrier(0);  // all 16 loads are issued before a value (of this or an earlier fetch) is used
 #pragma unroll
-        for (int v = 0; v < 16; ++v) h[v] = hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32];
-        __builtin_amdgcn_sched_barrier(0);  // all 16 loads are issued before the first value is used
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          if (DOT) dot += double(acc[mi][ni][v]) * double(h[v]);
-          else hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32] = h[v] + acc[mi][ni][v];
-        }
+      for (int v = 0; v < 16; ++v) {
+        if (DOT) dot += double(acc[mi][ni][v]) * double(h[blk % (kAheadH + 1)][v]);
+        else hb[long(mi * 32 + (v & 3) + 8 * (v >> 2)) * n + ni * 32] = h[blk % (kAheadH + 1)][v] + acc[mi][ni][v];
       }
+    }
   } else {
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
