@@ -21,6 +21,7 @@ constexpr int kWords = 32;     // packed u16 words per trellis
 constexpr int kLutEntries = 1024;  // distinct codebook entries: bits 6..15 of s*(s+1)
 // A decision of a 32-bit Viterbi pass stands when it is won by this many units of 2^-25: a metric of at most 128
 // rounded terms is within 64 units of the fp64 one, so two candidates 129 units apart are ordered alike in fp64.
+// (The bound of the last step; a step whose candidates have fewer terms is held to as many units less.)
 constexpr uint32_t kViterbiMargin = 160;
 
 struct Error : std::runtime_error {

@@ -491,7 +491,8 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
 // trace-back redoes them from the kept metrics as above and also looks at the runner-up.  If every decision it takes
 // (the final state, and the 16-way choice of each step it walks) is won by at least `thr` > 128 units and the winner is
 // below 2^30 (32.0: nothing on its path was cut off at 64.0), the fp64 recursion takes the same decisions and the
-// pass's result is the fp64 result.  Otherwise the
+// pass's result is the fp64 result.  (thr is what the last step needs, whose candidates are sums of 128 terms; a
+// decision of step t compares sums of t + 1 terms and is held to thr - (127 - t).)  Otherwise the
 // workgroup runs that pass again through the fp64 code above (a fraction of a percent of the passes: near-ties of
 // 5e-6, and the exact ties between states that share predecessor and codebook entry).
 // Integer adds issue at twice the rate of fp64 adds on this chip and a three-way minimum covers two candidates, so an
@@ -1029,7 +1030,10 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
       bg = take ? sm.tr32[set][w][3] : bg;
       bc = take ? oc : bc;
     }
-    flag |= uint32_t(sc - bc < thr) | uint32_t(bg < thr) | uint32_t(bc >= kWinnerMax);
+    // (a candidate of step `it` is a sum of it + 1 rounded terms: what thr allows for 128 terms shrinks by one unit
+    // per term less)
+    const uint32_t fewer = uint32_t(kSteps - 1 - it), thr_it = thr - (fewer < thr ? fewer : thr);
+    flag |= uint32_t(sc - bc < thr_it) | uint32_t(bg < thr_it) | uint32_t(bc >= kWinnerMax);
     const uint32_t s_it = ((bdd & 15u) << 12) | j;
     s = (((bdd >> 8) & 15u) << 12) | (s_it >> 4);
     if (record && threadIdx.x == 0) {
