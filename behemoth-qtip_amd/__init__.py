@@ -341,7 +341,7 @@ class Quantizer:
 
     def set_viterbi_mode(self, mode=0, margin_units=0):
         """0: 32-bit metrics first, fp64 again where a traced decision is closer than margin_units (default 160)
-        units of 2^-25; 1: fp64 metrics only; 2, 3: mode 0 with 256 / 512 threads per tile whatever the size of
+        units of 2^-26; 1: fp64 metrics only; 2, 3: mode 0 with 256 / 512 threads per tile whatever the size of
         the launch (mode 0 picks 512 for launches of at most a third of the device's workgroup slots).  Same states
         in every mode."""
         _check(lib().qtip_set_viterbi_mode(self._h, int(mode), C.c_uint(int(margin_units))))

@@ -19,7 +19,7 @@ constexpr int kStates = 65536; // L = 16
 constexpr int kGroups = 4096;  // states sharing a successor group
 constexpr int kWords = 32;     // packed u16 words per trellis
 constexpr int kLutEntries = 1024;  // distinct codebook entries: bits 6..15 of s*(s+1)
-// A decision of a 32-bit Viterbi pass stands when it is won by this many units of 2^-25: a metric of at most 128
+// A decision of a 32-bit Viterbi pass stands when it is won by this many units of 2^-26: a metric of at most 128
 // rounded terms is within 64 units of the fp64 one, so two candidates 129 units apart are ordered alike in fp64.
 // (The bound of the last step; a step whose candidates have fewer terms is held to as many units less.)
 constexpr uint32_t kViterbiMargin = 160;
@@ -258,7 +258,7 @@ struct TileJob {
   // depend on each other only through that row's own hatWT values, so nothing has to wait for another workgroup
   int blocks = 1;
   // 0: both passes run on 32-bit metrics first and a pass whose traced decisions are not all won by `margin` units of
-  // 2^-25 is run again on fp64 metrics (same results as mode 1, bit for bit); 1: fp64 metrics only
+  // 2^-26 is run again on fp64 metrics (same results as mode 1, bit for bit); 1: fp64 metrics only
   int mode = 0;
   // workgroups of 512 threads per tile instead of 256 (mode 0 only; same results): -1 = where the launch has at most
   // a third as many tiles as the device has workgroup slots, 0 = never, 1 = always

@@ -42,7 +42,7 @@
 // add-compare-selects of the path it walks, two steps per round trip, with the forward pass's own fp64 operations
 // and tie rule.  Only the last step tracks its digits (in registers), which the final state needs.
 //
-// The above is the fp64 form.  By default every pass first runs on unsigned 32-bit metrics in units of 2^-25
+// The above is the fp64 form.  By default every pass first runs on unsigned 32-bit metrics in units of 2^-26
 // (forward_pass32 / trace_back32 further down: 4-byte table and metrics in the same LDS footprint, double-buffered,
 // one barrier per step; the free pass computes the groups below 2048 only, since complementary states decode alike),
 // its trace-back checks that every decision it takes was won by more than the rounding can move two candidates
@@ -483,14 +483,14 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
 
 // ================================================================= the same two passes on 32-bit metrics
 // The fp64 passes above are bound by the issue rate of fp64 vector instructions and, behind it, by 8-byte LDS reads.
-// Both passes are therefore first run on unsigned 32-bit metrics in units of 2^-25: the squared error of a codebook
+// Both passes are therefore first run on unsigned 32-bit metrics in units of 2^-26: the squared error of a codebook
 // entry is formed in fp64 exactly as above and rounded to the nearest unit once (|error| <= 1/2 unit); errors and
-// metrics are held to 2^31 - 1 (= 64.0, which also stands for +inf: every chain of minima starts from it), so the adds
-// are plain integer adds that cannot wrap, and a path metric of n terms differs from the fp64 one by at most n/2
-// units, whatever the path.  Only the decisions on the surviving path matter: the
+// metrics are held to 2^32 - 1 (= 64.0, which also stands for +inf: every chain of minima starts from it; the adds
+// are the integer add with its clamp bit set, which stops there instead of wrapping), and a path metric of n terms
+// differs from the fp64 one by at most n/2 units, whatever the path.  Only the decisions on the surviving path matter: the
 // trace-back redoes them from the kept metrics as above and also looks at the runner-up.  If every decision it takes
 // (the final state, and the 16-way choice of each step it walks) is won by at least `thr` > 128 units and the winner is
-// below 2^30 (32.0: nothing on its path was cut off at 64.0), the fp64 recursion takes the same decisions and the
+// below 2^31 (32.0: nothing on its path was cut off at 64.0), the fp64 recursion takes the same decisions and the
 // pass's result is the fp64 result.  (thr is what the last step needs, whose candidates are sums of 128 terms; a
 // decision of step t compares sums of t + 1 terms and is held to thr - (127 - t).)  Otherwise the
 // workgroup runs that pass again through the fp64 code above (a fraction of a percent of the passes: near-ties of
@@ -512,8 +512,8 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
 // conflicts.  The metric of (column, digit d) sits at pos(column) * 16 + (d ^ swz(column)) with swz a multiple of 4,
 // so a column comes in as four 16-byte reads; pos and swz are chosen so that those reads, the 4-byte writes of a
 // group's result (32 lanes: 4 columns x 8 digits) and of its mirror (slot ^ 0xfeb) are free of bank conflicts.
-constexpr uint32_t kSat = 0x7fffffffu;      // 64.0: the largest metric, and +inf
-constexpr uint32_t kWinnerMax = 0x40000000u;  // 32.0: a decision's winner must be below this
+constexpr uint32_t kSat = 0xffffffffu;      // 64.0: the largest metric, and +inf
+constexpr uint32_t kWinnerMax = 0x80000000u;  // 32.0: a decision's winner must be below this
 constexpr int kMirror32 = 0xfeb;
 static_assert(64 * kGroups <= 2 * kHistWordsPerTile, "the 32-bit kept metrics (64 steps) must fit the fp64 slot");
 
@@ -545,19 +545,20 @@ __device__ __forceinline__ uint32_t hist32_index(uint32_t g) {
   const uint32_t jj = g < 2048u ? g : 4095u - g;
   return ((jj & 7u) + ((kSym || g < 2048u) ? 0u : 8u)) * kThreads + owner32(jj);
 }
-// metrics and errors are at most kSat = 2^31 - 1, so a plain add cannot wrap; every chain of minima starts from kSat
-__device__ __forceinline__ uint32_t sat_add(uint32_t a, uint32_t b) { return a + b; }
+// metrics and errors are at most kSat = 2^32 - 1 and the add stops there (v_add_u32 with clamp); every chain of
+// minima starts from kSat
+__device__ __forceinline__ uint32_t sat_add(uint32_t a, uint32_t b) { return __builtin_elementwise_add_sat(a, b); }
 __device__ __forceinline__ uint32_t min3u(uint32_t a, uint32_t b, uint32_t c) {
   uint32_t r;  // written out: the compiler forms the three-way minimum for only half of the chains
   asm("v_min3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
 }
 // squared error of a codebook entry against the two inputs of a step, the fp64 value of the passes above in units of
-// 2^-25, rounded to nearest; 64.0 and more (and NaN) become 2^31 - 1
+// 2^-26, rounded to nearest; 64.0 and more (and NaN) become 2^32 - 1
 __device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, double x1) {
   const double a = l0 - x0, b = l1 - x1;
-  const double v = __builtin_rint(__builtin_fma(a, a, b * b) * 33554432.0);
-  return uint32_t(__builtin_fmin(v, 2147483647.0));
+  const double v = __builtin_rint(__builtin_fma(a, a, b * b) * 67108864.0);
+  return uint32_t(__builtin_fmin(v, 4294967295.0));
 }
 
 // One forward pass on 32-bit metrics.  kSym: free ends, the groups below 2048 only (a mirror group's metric is read
@@ -827,7 +828,7 @@ __device__ __forceinline__ uint32_t row_min16_u32(uint32_t c) {
 // j_last: low 12 bits of the final state (the group the pass ends in; for a free pass the best group, of which the
 // column counts).  The decision of step 127 is taken from the metrics entering it (kept slot 63), then two steps
 // per round trip.  flag is raised (in every thread alike) when a
-// decision is won by less than thr units or the winner is not below 2^30.
+// decision is won by less than thr units or the winner is not below 2^31.
 // Returns the state of step it_min - 1; record: the states of the steps walked are written to sm.st.
 // kStream (the 512-thread form, whose workgroup has its compute unit to itself): which 256 of a kept step's values a
 // round reads is known only when the round before it is decided, so fetched on demand every round waits for HBM.
