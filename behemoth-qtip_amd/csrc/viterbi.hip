@@ -114,6 +114,7 @@ struct Smem {
   uint32_t red32[8][3];    // end of the free 32-bit pass: per wave the best group's metric, the second best, the group
   int overlap;
   uint32_t final_state;
+  float final_metric;  // the free fp64 pass's best final metric (what later 32-bit passes of the tile row may expect)
 };
 
 __device__ __forceinline__ int perm_fwd(int p) {  // sequence position -> tile index 16*r + c
@@ -342,6 +343,7 @@ __device__ __forceinline__ void forward_pass(Smem& sm, const double* __restrict_
       for (int w = 1; w < 4; ++w)
         if (sm.red_c[w] < c || (sm.red_c[w] == c && sm.red_s[w] < s)) c = sm.red_c[w], s = sm.red_s[w];
       sm.final_state = s & 0xffffu;  // (no comparison succeeds on NaN metrics; the walk needs a 16-bit state anyway)
+      sm.final_metric = float(c);
     }
   } else {
     const uint32_t j = uint32_t(ov), jj = j < 2048u ? j : 4095u - j;
@@ -483,7 +485,8 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
 
 // ================================================================= the same two passes on 32-bit metrics
 // The fp64 passes above are bound by the issue rate of fp64 vector instructions and, behind it, by 8-byte LDS reads.
-// Both passes are therefore first run on unsigned 32-bit metrics in units of 2^-26: the squared error of a codebook
+// Both passes are therefore first run on unsigned 32-bit metrics in units of 2^-26 (or a neighbouring power of two,
+// unit_log2_for below): the squared error of a codebook
 // entry is formed in fp64 exactly as above and rounded to the nearest unit once (|error| <= 1/2 unit); errors and
 // metrics are held to 2^32 - 1 (= 64.0, which also stands for +inf: every chain of minima starts from it; the adds
 // are the integer add with its clamp bit set, which stops there instead of wrapping), and a path metric of n terms
@@ -513,7 +516,23 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
 // so a column comes in as four 16-byte reads; pos and swz are chosen so that those reads, the 4-byte writes of a
 // group's result (32 lanes: 4 columns x 8 digits) and of its mirror (slot ^ 0xfeb) are free of bank conflicts.
 constexpr uint32_t kSat = 0xffffffffu;      // 64.0: the largest metric, and +inf
-constexpr uint32_t kWinnerMax = 0x80000000u;  // 32.0: a decision's winner must be below this
+// A decision's winner must be below this: nothing on its path was then cut off at kSat (a path's metric only grows).
+// A candidate that was cut off is truly larger than it reads, so a margin seen against it is a margin there.
+constexpr uint32_t kWinnerMax = kSat - (1u << 20);
+// The unit of a pass is 2^-k, k chosen per pass so that the winner expected, with room to spare, still fits: the
+// finer the unit, the narrower in value the margin a decision must be won by, the fewer passes repeated - and inputs
+// of another scale than normalized weights (winners near 20) still run on 32-bit metrics.  The tail-biting pass
+// expects the winner of its block's free pass, which ran on the same values (room: an eighth); the free pass that of
+// the tile row's previous column block (room: as much again; k = 26 for winners between 16 and 32).  k = 26 (winners
+// up to 64.0) when nothing is known yet.  A winner that does not fit after all repeats the pass on fp64 metrics.
+constexpr int kUnitLog2Default = 26, kUnitLog2Min = 12, kUnitLog2Max = 30;
+__device__ __forceinline__ int unit_log2_for(float expected_winner, float room) {
+  if (!(expected_winner > 0.f)) return kUnitLog2Default;
+  // largest k with room x winner x 2^k <= 2^32
+  int k = 32 - int(__builtin_ceilf(__builtin_log2f(room * expected_winner)));
+  return k < kUnitLog2Min ? kUnitLog2Min : k > kUnitLog2Max ? kUnitLog2Max : k;
+}
+__device__ __forceinline__ double unit_scale(int k) { return __builtin_bit_cast(double, uint64_t(1023 + k) << 52); }
 constexpr int kMirror32 = 0xfeb;
 static_assert(64 * kGroups <= 2 * kHistWordsPerTile, "the 32-bit kept metrics (64 steps) must fit the fp64 slot");
 
@@ -554,10 +573,11 @@ __device__ __forceinline__ uint32_t min3u(uint32_t a, uint32_t b, uint32_t c) {
   return r;
 }
 // squared error of a codebook entry against the two inputs of a step, the fp64 value of the passes above in units of
-// 2^-26, rounded to nearest; 64.0 and more (and NaN) become 2^32 - 1
-__device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, double x1) {
+// 1 / scale (scale a power of two: the product is exact), rounded to nearest; 2^32 - 1 and more (and NaN) become
+// 2^32 - 1
+__device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, double x1, double scale) {
   const double a = l0 - x0, b = l1 - x1;
-  const double v = __builtin_rint(__builtin_fma(a, a, b * b) * 67108864.0);
+  const double v = __builtin_rint(__builtin_fma(a, a, b * b) * scale);
   return uint32_t(__builtin_fmin(v, 4294967295.0));
 }
 
@@ -572,7 +592,7 @@ __device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, d
 // 4..7), and the table's 1024 entries two each instead of four.
 template <bool kSym, bool kWide>
 __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restrict__ entry_d, int roll, int ov,
-                                               uint32_t* __restrict__ hist, int first_kept) {
+                                               uint32_t* __restrict__ hist, int first_kept, const double scale) {
   constexpr int kT = kWide ? 2 * kThreads : kThreads, kSlotsOwn = kWide ? 4 : 8, kEnt = 1024 / kT;
   const int tfull = kWide ? opaque_tid_wide() : opaque_tid();
   const int tid = tfull & (kThreads - 1), upper = kWide ? tfull >> 8 : 0;
@@ -630,7 +650,7 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
 #pragma unroll
       for (int q = 0; q < kEnt; ++q) {
         const double2 l = ent[q];
-        const uint32_t v = err_units(l.x, l.y, x0, x1);
+        const uint32_t v = err_units(l.x, l.y, x0, x1, scale);
         Ew0[kT * q] = v;
         Ew0[kT * q + 8 * 128] = v;
         Ew1[kT * q] = v;
@@ -641,7 +661,7 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
 #pragma unroll
       for (int q = 0; q < kEnt; ++q) {
         const double2 l = ent[q];
-        const uint32_t v = err_units(l.x, l.y, x0, x1);
+        const uint32_t v = err_units(l.x, l.y, x0, x1, scale);
         Ew[kT * q] = v;
         Ew[kT * q + 1024] = v;
       }
@@ -842,7 +862,7 @@ template <bool kSym, bool kStream>
 __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restrict__ entry_d,
                                                  const uint32_t* __restrict__ hist, int roll, uint32_t j_last,
                                                  int it_min, bool record, uint32_t thr, uint32_t& flag,
-                                                 const uint32_t* tl) {
+                                                 const uint32_t* tl, const double scale) {
   const uint32_t tid = uint32_t(opaque_tid());
   const uint32_t lane = tid & 63u, wave = tid >> 6, dp = lane & 15u, d = 4u * wave + (lane >> 4);
   // streamed form: kept steps 63, 62, ..., it_min / 2 - 1 are the rows q = 0, 1, ... of a ring of kBufs buffers
@@ -910,9 +930,9 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
       const uint32_t w = tl[e & 511u];
       const uint16_t h0 = uint16_t((w & 0xffffu) ^ ((e >> 9) << 15)), h1 = uint16_t(w >> 16);
       return err_units(double(float(__builtin_bit_cast(_Float16, h0))), double(float(__builtin_bit_cast(_Float16, h1))),
-                       x0, x1);
+                       x0, x1, scale);
     } else {
-      return err_units(entry_d[2 * e], entry_d[2 * e + 1], x0, x1);
+      return err_units(entry_d[2 * e], entry_d[2 * e + 1], x0, x1, scale);
     }
   };
   // over the 16 lanes of a row: the smallest value (returned), the first lane that holds it, the gap to the runner-up
@@ -1062,7 +1082,8 @@ __global__ __launch_bounds__(kWide ? 2 * kThreads : kThreads, kWide ? 1 : 3) voi
     __syncthreads();
   }
   double* hist = hist_all + size_t(blockIdx.x) * kHistWordsPerTile;
-  for (long tile = blockIdx.x; tile < job.tiles; tile += gridDim.x)
+  for (long tile = blockIdx.x; tile < job.tiles; tile += gridDim.x) {
+  float expected = 0.f;  // the free pass's winner of this tile row's previous column block (0: none yet)
   for (int blk = job.blocks - 1; blk >= 0; --blk) {
     // the column block of this turn; the hatWT values the previous turn wrote for this tile row are visible after
     // the barrier that ended it
@@ -1082,14 +1103,21 @@ __global__ __launch_bounds__(kWide ? 2 * kThreads : kThreads, kWide ? 1 : 3) voi
       if (job.mode == 0) {
         uint32_t* const hist32 = reinterpret_cast<uint32_t*>(hist);
         uint32_t flag = 0;
+        // (the same in every thread; said so, so that it lives in scalar registers)
+        const int unit_log2 = __builtin_amdgcn_readfirstlane(unit_log2_for(expected, pass == 0 ? 2.f : 1.125f));
+        const double scale = unit_scale(unit_log2);
         if (pass == 0) {
-          forward_pass32<true, kWide>(sm, entry_d, roll, -1, hist32, 62);
-          flag |= uint32_t(sm.red32[0][1] < job.margin) | uint32_t(sm.red32[0][0] >= kWinnerMax);
-          const uint32_t s = trace_back32<true, kWide>(sm, entry_d, hist32, roll, sm.red32[0][2], 64, false, job.margin, flag, tl);
+          forward_pass32<true, kWide>(sm, entry_d, roll, -1, hist32, 62, scale);
+          const uint32_t winner = sm.red32[0][0];
+          flag |= uint32_t(sm.red32[0][1] < job.margin) | uint32_t(winner >= kWinnerMax);
+          const uint32_t s = trace_back32<true, kWide>(sm, entry_d, hist32, roll, sm.red32[0][2], 64, false, job.margin, flag, tl, scale);
           if (!flag && u == 0) sm.overlap = int(s & 0xfffu);  // s is the state of step 63
+          // what the tail-biting pass of this block and the free pass of the next may expect (a winner that did
+          // not fit is replaced by the true one when the pass is repeated on fp64 metrics)
+          expected = __builtin_ldexpf(float(winner), -unit_log2);
         } else {
-          forward_pass32<false, kWide>(sm, entry_d, roll, ov, hist32, 0);
-          const uint32_t s = trace_back32<false, kWide>(sm, entry_d, hist32, roll, uint32_t(ov), 2, true, job.margin, flag, tl);
+          forward_pass32<false, kWide>(sm, entry_d, roll, ov, hist32, 0, scale);
+          const uint32_t s = trace_back32<false, kWide>(sm, entry_d, hist32, roll, uint32_t(ov), 2, true, job.margin, flag, tl, scale);
           // s is the state of step 1; at step 0 the one predecessor group with a finite initial metric is ov
           if (!flag && u == 0) sm.st[0] = uint16_t((s >> 4) | ((uint32_t(ov) >> 8) << 12));
         }
@@ -1098,6 +1126,7 @@ __global__ __launch_bounds__(kWide ? 2 * kThreads : kThreads, kWide ? 1 : 3) voi
       }
       if (!done) {
       forward_pass(sm, entry_d, roll, ov, hist, pass == 0 ? 62 : 0);
+      if (pass == 0) expected = sm.final_metric;  // the true winner, also where a 32-bit pass could not hold it
       {
         const uint32_t s_last = sm.final_state;  // state of step 127
         const uint32_t s = trace_back(sm, entry_d, hist, roll, s_last, pass == 0 ? 64 : 2, pass == 1);
@@ -1143,6 +1172,7 @@ __global__ __launch_bounds__(kWide ? 2 * kThreads : kThreads, kWide ? 1 : 3) voi
       }
     }
     __syncthreads();
+  }
   }
 }
 

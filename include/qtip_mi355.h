@@ -87,8 +87,8 @@ int qtip_viterbi_tiles_dev_noalloc(qtip_ctx* ctx, const float* dev_X, long B, ui
  * reference, whose device kernel scores in fp32 with the predecessor tag in the low mantissa bits and is exact most of
  * the time only (src/viterbi.hip:106-140).
  * mode 0 (default): each pass runs on unsigned 32-bit metrics first (squared errors formed in fp64 as the CPU
- * algorithm forms them, src/qtip_core.cpp:123-127, rounded once to units of 2^-26; saturating integer adds, values held to 2^32 - 1), and its
- * trace-back checks that every decision on the surviving path was won by at least margin_units units, which is more
+ * algorithm forms them, src/qtip_core.cpp:123-127, rounded once to units of 2^-26, or of the power of two that
+ * fits the tile's winner; saturating integer adds, values held to 2^32 - 1), and its trace-back checks that every decision on the surviving path was won by at least margin_units units, which is more
  * than the rounding of 128 terms can move two candidates against each other; a pass that fails the check runs again on
  * fp64 metrics.  The states are those of mode 1 bit for bit.
  * mode 1: fp64 metrics only (viterbi_ref's own arithmetic, src/qtip_core.cpp:129-164).

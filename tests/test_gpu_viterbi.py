@@ -213,6 +213,35 @@ def test_metric_modes_give_the_same_states(qz, oracle, hyb):
     assert r0[0] <= 40 and r0[1] <= 40
 
 
+def test_metric_unit_follows_the_scale_of_the_inputs(qz, oracle, hyb):
+    """The unit of a 32-bit pass is chosen from the winner expected (the free pass's, for the tail-biting pass of the
+    same tile): inputs an eighth or twice the size of normalized weights still give the CPU algorithm's states, and at
+    twice or six times the size - where a free pass in the default unit cannot hold its winner and is repeated on
+    fp64 metrics, which gives the true winner - the tail-biting passes run in a coarser unit instead of being repeated
+    as well."""
+    say("case: inputs of other scales")
+    qz.set_tlut(None)
+    B = 96
+    base = oracle.rng_normal(77, B * 256).astype(np.float32).reshape(B, 256)
+    try:
+        qz.set_viterbi_mode(0)
+        for scale in (0.125, 2.0, 6.0):
+            X = (base * np.float32(scale)).astype(np.float32)
+            want = oracle.quantize_tiles(hyb, X, fast=True)
+            qz.viterbi_stats(reset=True)
+            st, pk = qz.viterbi_tiles(X)
+            r = qz.viterbi_stats(reset=True)
+            say("  x %g: %d first and %d second passes of %d repeated" % (scale, r[0], r[1], B))
+            same = np.all(st == want, axis=1)
+            assert same.all(), "x %g: tiles differing from the CPU algorithm: %s" % (scale, np.nonzero(~same)[0][:10])
+            if scale == 0.125:
+                assert r[0] <= 4 and r[1] <= 4
+            if scale >= 2.0:
+                assert r[1] <= B // 4
+    finally:
+        qz.set_viterbi_mode(0)
+
+
 def test_wide_workgroups_give_the_same_states(qz, oracle, hyb):
     """A launch that cannot fill the chip gives every tile 512 threads instead of 256 (the 32-bit forward passes
     share the groups out over all of them; everything else, the fp64 repeat of a pass included, is done by both
