@@ -485,15 +485,16 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
 
 // ================================================================= the same two passes on 32-bit metrics
 // The fp64 passes above are bound by the issue rate of fp64 vector instructions and, behind it, by 8-byte LDS reads.
-// Both passes are therefore first run on unsigned 32-bit metrics in units of 2^-26 (or a neighbouring power of two,
-// unit_log2_for below): the squared error of a codebook
-// entry is formed in fp64 exactly as above and rounded to the nearest unit once (|error| <= 1/2 unit); errors and
-// metrics are held to 2^32 - 1 (= 64.0, which also stands for +inf: every chain of minima starts from it; the adds
-// are the integer add with its clamp bit set, which stops there instead of wrapping), and a path metric of n terms
-// differs from the fp64 one by at most n/2 units, whatever the path.  Only the decisions on the surviving path matter: the
+// Both passes are therefore first run on unsigned 32-bit metrics in units of 2^-26 (or another even power of two,
+// unit_log2_for below): the squared error of a codebook entry is formed in fp64 (the sum of the two squared
+// differences, as above, on operands scaled by a power of two) and brought to the nearest unit once (|error| <= 1/2
+// unit + 2^-20); errors and metrics are held to 2^32 - 1 (= 64.0 at 2^-26, which also stands for +inf: every chain of
+// minima starts from it; the adds are the integer add with its clamp bit set, which stops there instead of
+// wrapping), and a path metric of n terms differs from the fp64 one by at most n/2 units (and a little), whatever
+// the path.  Only the decisions on the surviving path matter: the
 // trace-back redoes them from the kept metrics as above and also looks at the runner-up.  If every decision it takes
 // (the final state, and the 16-way choice of each step it walks) is won by at least `thr` > 128 units and the winner is
-// below 2^31 (32.0: nothing on its path was cut off at 64.0), the fp64 recursion takes the same decisions and the
+// below 2^32 - 2^20 (nothing on its path was cut off), the fp64 recursion takes the same decisions and the
 // pass's result is the fp64 result.  (thr is what the last step needs, whose candidates are sums of 128 terms; a
 // decision of step t compares sums of t + 1 terms and is held to thr - (127 - t).)  Otherwise the
 // workgroup runs that pass again through the fp64 code above (a fraction of a percent of the passes: near-ties of
@@ -519,20 +520,26 @@ constexpr uint32_t kSat = 0xffffffffu;      // 64.0: the largest metric, and +in
 // A decision's winner must be below this: nothing on its path was then cut off at kSat (a path's metric only grows).
 // A candidate that was cut off is truly larger than it reads, so a margin seen against it is a margin there.
 constexpr uint32_t kWinnerMax = kSat - (1u << 20);
-// The unit of a pass is 2^-k, k chosen per pass so that the winner expected, with room to spare, still fits: the
-// finer the unit, the narrower in value the margin a decision must be won by, the fewer passes repeated - and inputs
-// of another scale than normalized weights (winners near 20) still run on 32-bit metrics.  The tail-biting pass
-// expects the winner of its block's free pass, which ran on the same values (room: an eighth); the free pass that of
-// the tile row's previous column block (room: as much again; k = 26 for winners between 16 and 32).  k = 26 (winners
-// up to 64.0) when nothing is known yet.  A winner that does not fit after all repeats the pass on fp64 metrics.
+// The unit of a pass is 2^-k, k even and chosen per pass so that the winner expected, with room to spare, still
+// fits: the finer the unit, the narrower in value the margin a decision must be won by, the fewer passes repeated -
+// and inputs of another scale than normalized weights (winners near 20 to 25: k = 26) still run on 32-bit metrics.
+// The tail-biting pass expects the winner of its block's free pass, which ran on the same values (room: an eighth);
+// the free pass that of the tile row's previous column block (room: as much again).  k = 26 (winners up to 64.0)
+// when nothing is known yet.  A winner that does not fit after all repeats the pass on fp64 metrics.
 constexpr int kUnitLog2Default = 26, kUnitLog2Min = 12, kUnitLog2Max = 30;
 __device__ __forceinline__ int unit_log2_for(float expected_winner, float room) {
   if (!(expected_winner > 0.f)) return kUnitLog2Default;
-  // largest k with room x winner x 2^k <= 2^32
-  int k = 32 - int(__builtin_ceilf(__builtin_log2f(room * expected_winner)));
+  // largest even k with room x winner x 2^k <= 2^32
+  int k = (32 - int(__builtin_ceilf(__builtin_log2f(room * expected_winner)))) & ~1;
   return k < kUnitLog2Min ? kUnitLog2Min : k > kUnitLog2Max ? kUnitLog2Max : k;
 }
-__device__ __forceinline__ double unit_scale(int k) { return __builtin_bit_cast(double, uint64_t(1023 + k) << 52); }
+// The unit 2^-k as the table's arithmetic wants it (k is even): codebook values and inputs are multiplied by pre =
+// 2^(k/2), which is exact and scales the differences, their squares and the sum of the squares exactly as a
+// multiplication of the sum by 2^k would, so the sum comes out in units.
+struct Unit {
+  double pre;
+};
+__device__ __forceinline__ Unit unit_of(int k) { return Unit{__builtin_bit_cast(double, uint64_t(1023 + k / 2) << 52)}; }
 constexpr int kMirror32 = 0xfeb;
 static_assert(64 * kGroups <= 2 * kHistWordsPerTile, "the 32-bit kept metrics (64 steps) must fit the fp64 slot");
 
@@ -572,12 +579,12 @@ __device__ __forceinline__ uint32_t min3u(uint32_t a, uint32_t b, uint32_t c) {
   asm("v_min3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
 }
-// squared error of a codebook entry against the two inputs of a step, the fp64 value of the passes above in units of
-// 1 / scale (scale a power of two: the product is exact), rounded to nearest; 2^32 - 1 and more (and NaN) become
-// 2^32 - 1
-__device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, double x1, double scale) {
+// Squared error of a codebook entry against the two inputs of a step in units: the fp64 value of the passes above,
+// times 2^k, to the nearest integer (the half is added in fp64 and the conversion cuts off: within 1/2 + 2^-20 of
+// the scaled value); 2^32 - 1 and more (and NaN) become 2^32 - 1.  l and x come multiplied by Unit::pre.
+__device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, double x1) {
   const double a = l0 - x0, b = l1 - x1;
-  const double v = __builtin_rint(__builtin_fma(a, a, b * b) * scale);
+  const double v = __builtin_fma(a, a, __builtin_fma(b, b, 0.5));
   return uint32_t(__builtin_fmin(v, 4294967295.0));
 }
 
@@ -592,7 +599,7 @@ __device__ __forceinline__ uint32_t err_units(double l0, double l1, double x0, d
 // 4..7), and the table's 1024 entries two each instead of four.
 template <bool kSym, bool kWide>
 __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restrict__ entry_d, int roll, int ov,
-                                               uint32_t* __restrict__ hist, int first_kept, const double scale) {
+                                               uint32_t* __restrict__ hist, int first_kept, const Unit unit) {
   constexpr int kT = kWide ? 2 * kThreads : kThreads, kSlotsOwn = kWide ? 4 : 8, kEnt = 1024 / kT;
   const int tfull = kWide ? opaque_tid_wide() : opaque_tid();
   const int tid = tfull & (kThreads - 1), upper = kWide ? tfull >> 8 : 0;
@@ -617,7 +624,7 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
   double2 ent[kEnt];
   const double2* __restrict__ entries = reinterpret_cast<const double2*>(entry_d) + e_wr;
 #pragma unroll
-  for (int q = 0; q < kEnt; ++q) ent[q] = entries[kT * q];
+  for (int q = 0; q < kEnt; ++q) ent[q] = entries[kT * q], ent[q].x *= unit.pre, ent[q].y *= unit.pre;
   // free pass, words: parity 0 holds position 2a + h in pair a, half h; parity 1 in pair a - 1 + h, the other half
   const int e_wr0 = (e_a * 64 + e_row) * 2 + e_h;
   const int e_wr1 = ((16 + e_a - 1 + e_h) * 64 + e_row) * 2 + (e_h ^ 1);
@@ -640,7 +647,8 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
   // the error table of step `it` into table buffer it & 1
   auto table = [&](int it) __attribute__((always_inline)) {
     const int t = (2 * it + roll) & 255;
-    const double x0 = double(sm.x[t]), x1 = double(sm.x[t + 1]);
+    const double x0 = double(sm.x[t]) * unit.pre, x1 = double(sm.x[t + 1]) * unit.pre;
+
     if constexpr (kSym) {
       // Parity 0: pair position / 2, half position % 2; parity 1: pair floor((position - 1) / 2), the other half;
       // pair -1, which position 0 asks for, is pair 15 of parity 0, which like itself nobody reads.  Every pair a
@@ -650,7 +658,7 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
 #pragma unroll
       for (int q = 0; q < kEnt; ++q) {
         const double2 l = ent[q];
-        const uint32_t v = err_units(l.x, l.y, x0, x1, scale);
+        const uint32_t v = err_units(l.x, l.y, x0, x1);
         Ew0[kT * q] = v;
         Ew0[kT * q + 8 * 128] = v;
         Ew1[kT * q] = v;
@@ -661,7 +669,7 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
 #pragma unroll
       for (int q = 0; q < kEnt; ++q) {
         const double2 l = ent[q];
-        const uint32_t v = err_units(l.x, l.y, x0, x1, scale);
+        const uint32_t v = err_units(l.x, l.y, x0, x1);
         Ew[kT * q] = v;
         Ew[kT * q + 1024] = v;
       }
@@ -862,7 +870,7 @@ template <bool kSym, bool kStream>
 __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restrict__ entry_d,
                                                  const uint32_t* __restrict__ hist, int roll, uint32_t j_last,
                                                  int it_min, bool record, uint32_t thr, uint32_t& flag,
-                                                 const uint32_t* tl, const double scale) {
+                                                 const uint32_t* tl, const Unit unit) {
   const uint32_t tid = uint32_t(opaque_tid());
   const uint32_t lane = tid & 63u, wave = tid >> 6, dp = lane & 15u, d = 4u * wave + (lane >> 4);
   // streamed form: kept steps 63, 62, ..., it_min / 2 - 1 are the rows q = 0, 1, ... of a ring of kBufs buffers
@@ -924,16 +932,18 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
     else return __hip_atomic_load(hist + size_t(slot) * kGroups + hist32_index<kSym>(g), __ATOMIC_RELAXED,
                                   __HIP_MEMORY_SCOPE_WORKGROUP);
   };
+  // (the forward pass's own arithmetic: the same products and sums on the same operands give the same integers)
   auto err_of = [&](uint32_t st, double x0, double x1) -> uint32_t {
     const uint32_t e = ((st * (st + 1u)) >> 6) & 1023u;
+    double l0, l1;
     if constexpr (kStream) {
       const uint32_t w = tl[e & 511u];
       const uint16_t h0 = uint16_t((w & 0xffffu) ^ ((e >> 9) << 15)), h1 = uint16_t(w >> 16);
-      return err_units(double(float(__builtin_bit_cast(_Float16, h0))), double(float(__builtin_bit_cast(_Float16, h1))),
-                       x0, x1, scale);
+      l0 = double(float(__builtin_bit_cast(_Float16, h0))), l1 = double(float(__builtin_bit_cast(_Float16, h1)));
     } else {
-      return err_units(entry_d[2 * e], entry_d[2 * e + 1], x0, x1, scale);
+      l0 = entry_d[2 * e], l1 = entry_d[2 * e + 1];
     }
+    return err_units(l0 * unit.pre, l1 * unit.pre, x0 * unit.pre, x1 * unit.pre);
   };
   // over the 16 lanes of a row: the smallest value (returned), the first lane that holds it, the gap to the runner-up
   auto row_pick = [&](uint32_t c, uint32_t& first, uint32_t& gap) -> uint32_t {
@@ -1105,19 +1115,19 @@ __global__ __launch_bounds__(kWide ? 2 * kThreads : kThreads, kWide ? 1 : 3) voi
         uint32_t flag = 0;
         // (the same in every thread; said so, so that it lives in scalar registers)
         const int unit_log2 = __builtin_amdgcn_readfirstlane(unit_log2_for(expected, pass == 0 ? 2.f : 1.125f));
-        const double scale = unit_scale(unit_log2);
+        const Unit unit = unit_of(unit_log2);
         if (pass == 0) {
-          forward_pass32<true, kWide>(sm, entry_d, roll, -1, hist32, 62, scale);
+          forward_pass32<true, kWide>(sm, entry_d, roll, -1, hist32, 62, unit);
           const uint32_t winner = sm.red32[0][0];
           flag |= uint32_t(sm.red32[0][1] < job.margin) | uint32_t(winner >= kWinnerMax);
-          const uint32_t s = trace_back32<true, kWide>(sm, entry_d, hist32, roll, sm.red32[0][2], 64, false, job.margin, flag, tl, scale);
+          const uint32_t s = trace_back32<true, kWide>(sm, entry_d, hist32, roll, sm.red32[0][2], 64, false, job.margin, flag, tl, unit);
           if (!flag && u == 0) sm.overlap = int(s & 0xfffu);  // s is the state of step 63
           // what the tail-biting pass of this block and the free pass of the next may expect (a winner that did
           // not fit is replaced by the true one when the pass is repeated on fp64 metrics)
           expected = __builtin_ldexpf(float(winner), -unit_log2);
         } else {
-          forward_pass32<false, kWide>(sm, entry_d, roll, ov, hist32, 0, scale);
-          const uint32_t s = trace_back32<false, kWide>(sm, entry_d, hist32, roll, uint32_t(ov), 2, true, job.margin, flag, tl, scale);
+          forward_pass32<false, kWide>(sm, entry_d, roll, ov, hist32, 0, unit);
+          const uint32_t s = trace_back32<false, kWide>(sm, entry_d, hist32, roll, uint32_t(ov), 2, true, job.margin, flag, tl, unit);
           // s is the state of step 1; at step 0 the one predecessor group with a finite initial metric is ov
           if (!flag && u == 0) sm.st[0] = uint16_t((s >> 4) | ((uint32_t(ov) >> 8) << 12));
         }

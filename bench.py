@@ -200,7 +200,7 @@ def run_group(args, pkg):
     redone = q.viterbi_stats(reset=True)   # passes of the timed region that were run again on fp64 metrics
     tiles_timed = (sum(ms) // 16) * (n // 16) * args.steps
     vit = dict(viterbi_metrics="fp64" if args.viterbi_fp64 else
-               "u32 in units of 2^-26 or 2^-27 per pass (errors formed in fp64), a pass repeated on fp64 metrics when a traced decision "
+               "u32 in units of 2^-k, k even per pass, 26 for normalized weights (errors formed in fp64), a pass repeated on fp64 metrics when a traced decision "
                "is won by less than 160 units",
                viterbi_first_passes_repeated=redone[0], viterbi_second_passes_repeated=redone[1],
                viterbi_repeated_share=(redone[0] + redone[1]) / (2.0 * tiles_timed))
