@@ -644,8 +644,10 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
   // bytes
   int xA = kSym ? m32c_pos(colA) * 32 + m32c_swz(colA) * 4 : m32_pos(colA) * 64 + m32_swz(colA) * 4;
   int xB = kSym ? m32c_pos(colB) * 32 + m32c_swz(colB) * 4 : m32_pos(colB) * 64 + m32_swz(colB) * 4;
-  // the error table of step `it` into table buffer it & 1
-  auto table = [&](int it) __attribute__((always_inline)) {
+  // the error table of step `it` into table buffer it & 1 (given as a constant: the buffers' offsets then are part
+  // of the instructions)
+  auto table = [&](int it, auto par_tag) __attribute__((always_inline)) {
+    constexpr int tpar = decltype(par_tag)::value;
     const int t = (2 * it + roll) & 255;
     const double x0 = double(sm.x[t]) * unit.pre, x1 = double(sm.x[t + 1]) * unit.pre;
 
@@ -653,8 +655,8 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
       // Parity 0: pair position / 2, half position % 2; parity 1: pair floor((position - 1) / 2), the other half;
       // pair -1, which position 0 asks for, is pair 15 of parity 0, which like itself nobody reads.  Every pair a
       // second time 8 further on.  Both addresses advance by kT words per q (kT / 128 pairs).
-      uint32_t* const Ew0 = E32 + (it & 1) * kEPairWords + e_wr0;
-      uint32_t* const Ew1 = E32 + (it & 1) * kEPairWords + e_wr1;
+      uint32_t* const Ew0 = E32 + tpar * kEPairWords + e_wr0;
+      uint32_t* const Ew1 = E32 + tpar * kEPairWords + e_wr1;
 #pragma unroll
       for (int q = 0; q < kEnt; ++q) {
         const double2 l = ent[q];
@@ -665,7 +667,7 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
         Ew1[kT * q + 8 * 128] = v;
       }
     } else {
-      uint32_t* const Ew = E32 + (it & 1) * kESlots + e_wr;
+      uint32_t* const Ew = E32 + tpar * kESlots + e_wr;
 #pragma unroll
       for (int q = 0; q < kEnt; ++q) {
         const double2 l = ent[q];
@@ -680,19 +682,20 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
   } else {
     for (int g = tfull; g < kGroups; g += kT) M32[m32_slot(g & 255, g >> 8)] = (ov < 0 || g == ov) ? 0u : kSat;
   }
-  table(0);
+  table(0, std::integral_constant<int, 0>{});
   __syncthreads();
 
   uint32_t fin[kSlotsOwn];
-  // step `it`: metrics of buffer it & 1 and table buffer it & 1 -> metrics of buffer (it + 1) & 1
-  auto step = [&](int it, auto kind_tag) __attribute__((always_inline)) {
+  // step `it`: metrics of buffer it & 1 and table buffer it & 1 -> metrics of buffer (it + 1) & 1; par = it & 1
+  auto step = [&](int it, auto kind_tag, auto par_tag) __attribute__((always_inline)) {
     constexpr int kind = decltype(kind_tag)::value;  // kDigits: the free pass's last step, results to fin only
+    constexpr int par = decltype(par_tag)::value;
     uint32_t* hs = nullptr;
     if constexpr (kind == kStore) hs = hist + size_t(it >> 1) * kGroups + tid;
     constexpr int kMBuf = kSym ? kMcSlots : kMSlots, kEBuf = kSym ? kEPairWords : kESlots;
-    const char* const Mb = reinterpret_cast<const char*>(M32 + (it & 1) * kMBuf);
-    uint32_t* const Mw = M32 + ((it + 1) & 1) * kMBuf;
-    const uint32_t* const Er = E32 + (it & 1) * kEBuf;
+    const char* const Mb = reinterpret_cast<const char*>(M32 + par * kMBuf);
+    uint32_t* const Mw = M32 + (par ^ 1) * kMBuf;
+    const uint32_t* const Er = E32 + par * kEBuf;
     uint32_t MA[16], MB[16];
     asm volatile("" : "+v"(xA), "+v"(xB));
     if constexpr (kSym) {
@@ -713,7 +716,7 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
         MB[4 * k] = b.x, MB[4 * k + 1] = b.y, MB[4 * k + 2] = b.z, MB[4 * k + 3] = b.w;
       }
     }
-    if constexpr (kind != kDigits) table(it + 1);
+    if constexpr (kind != kDigits) table(it + 1, std::integral_constant<int, par ^ 1>{});
     // The 16 table values of a slot are fetched while the slot before it is worked on; the value of digit k of slot
     // m lies (k (2 m + 1)) % 16 positions after the slot's first.  m0: the first slot of this thread, a constant in
     // each of the two copies of the loop that the wide form needs.  Tail-biting pass: evb[.][k] is the value of digit
@@ -801,13 +804,19 @@ __device__ __forceinline__ void forward_pass32(Smem& sm, const double* __restric
   using Plain = std::integral_constant<int, kPlain>;
   using Store = std::integral_constant<int, kStore>;
   using Last = std::integral_constant<int, kDigits>;
+  using Even = std::integral_constant<int, 0>;
+  using Odd = std::integral_constant<int, 1>;
+  static_assert((kSteps - 1) % 2 == 1, "steps 0 .. kSteps - 2 are pairs and one more even step");
+  // two steps per turn, so that a step's parity is a constant (first_kept is even: the kept steps are even ones)
 #pragma nounroll
-  for (int it = 0; it < kSteps - 1; ++it) {
-    if (!(it & 1) && it >= first_kept) step(it, Store{});
-    else step(it, Plain{});
+  for (int it = 0; it < kSteps - 2; it += 2) {
+    if (it >= first_kept) step(it, Store{}, Even{});
+    else step(it, Plain{}, Even{});
+    step(it + 1, Plain{}, Odd{});
   }
+  step(kSteps - 2, Store{}, Even{});
   if constexpr (kSym) {
-    step(kSteps - 1, Last{});
+    step(kSteps - 1, Last{}, Odd{});
     // Best final group among the groups below 2048 (each stands for a pair of complementary states), and the best
     // among the groups of other columns (j >> 4): the 16 groups of a column end in final states that differ in their
     // last digit only where they come from the same predecessor, and which of those wins changes nothing that is
