@@ -105,6 +105,7 @@ def lib():
     L.qtip_selftest_device_alloc_calls.restype = l
     L.qtip_set_viterbi_mode.argtypes = [vp, i, C.c_uint]
     L.qtip_viterbi_stats.argtypes = [vp, C.POINTER(C.c_ulonglong), C.POINTER(C.c_ulonglong), i]
+    L.qtip_ldlq_default_chains.argtypes = [vp, C.POINTER(C.c_int)]
     L.qtip_stream_wait.argtypes = [vp, vp]
     L.qtip_stream_signal.argtypes = [vp, vp]
     L.qtip_device_lut.argtypes = [vp, C.POINTER(vp)]
@@ -211,7 +212,7 @@ class QuantOpts:  # src/quantizer.hpp:11-19
     feedback: int = 0          # 0: fp64 feedback (default), 1: fp32 feedback + bf16 hi/lo split MFMA
     skip_proxy: bool = False
     ldl_device_updates: bool = True    # the LDL's trailing updates run on the GPU (same L bit for bit); False: host alone
-    ldlq_chains: int = 0       # independent chains of launches the tile rows are dealt to (0: the library's default: 3 with GPU_MAX_HW_QUEUES >= 6, else 2)
+    ldlq_chains: int = 0       # independent chains of launches the tile rows are dealt to (0: the library's default: 3 where its side streams have hardware queues of their own, else 2: ldlq_default_chains())
     group_lanes: int = 0       # run_groups: groups run side by side on this many lanes (0: as many as fit the chip, 1 for large groups; 1: one after the other)
 
 
@@ -345,6 +346,12 @@ class Quantizer:
         the launch (mode 0 picks 512 for launches of at most a third of the device's workgroup slots).  Same states
         in every mode."""
         _check(lib().qtip_set_viterbi_mode(self._h, int(mode), C.c_uint(int(margin_units))))
+
+    def ldlq_default_chains(self):
+        """What QuantOpts.ldlq_chains = 0 stands for in this context: 2 or 3."""
+        n = C.c_int(0)
+        _check(lib().qtip_ldlq_default_chains(self._h, C.byref(n)))
+        return int(n.value)
 
     def viterbi_stats(self, reset=False):
         """(first passes, second passes) that mode 0 ran again on fp64 metrics."""

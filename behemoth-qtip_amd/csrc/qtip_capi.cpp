@@ -99,6 +99,78 @@ qtip_ctx* make_context(int device, const HostCodebook* cb_from) {
   return c;
 }
 
+// The side streams of a context - two more LDLQ chains and the factorization's - only run beside its own stream
+// and beside each other where each has a hardware queue to itself, and the runtime deals the few queues of a process
+// (four unless the environment said otherwise before it started) to streams as they are made, the caller's own
+// included; nothing tells which stream got which.  Timing does: a wave that sleeps for half a millisecond on each of
+// two streams takes half a millisecond if they have queues of their own and a whole one if they share.  Candidates
+// are made one after the other and kept if such a wave on each of the streams kept so far and on the candidate
+// finishes in well under two delays (the better of two tries: a stream's first launch also sets its queue up); the
+// others are released.  Up to three are kept: chain_stream[0], chain_stream[1], ldl_stream.  With all three LDLQ
+// defaults to three chains whatever the environment says.  The caller's streams may share queues with these: they
+// are idle while a call of this library runs.  Any failure leaves the streams to be made on first use, as before.
+void find_side_streams(qtip_ctx* c) {
+  constexpr int kCandidates = 12;
+  constexpr double kDelayUs = 500.0;
+  std::vector<hipStream_t> kept, dropped;
+  hipStream_t upload = nullptr;
+  try {
+    // a delay on the context's stream, on the first `count` streams kept and on cand, all queued at once: microseconds
+    auto side_by_side_us = [&](size_t count, hipStream_t cand) {
+      auto wait_all = [&] {
+        QTIP_HIP(hipStreamSynchronize(c->stream));
+        for (size_t i = 0; i < count; ++i) QTIP_HIP(hipStreamSynchronize(kept[i]));
+        QTIP_HIP(hipStreamSynchronize(cand));
+      };
+      wait_all();
+      const auto t0 = std::chrono::steady_clock::now();
+      launch_delay(kDelayUs, c->stream);
+      for (size_t i = 0; i < count; ++i) launch_delay(kDelayUs, kept[i]);
+      launch_delay(kDelayUs, cand);
+      wait_all();
+      return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+    };
+    auto beside = [&](size_t count, hipStream_t cand) {
+      const double a = side_by_side_us(count, cand), b = side_by_side_us(count, cand);
+      return (a < b ? a : b) < 1.5 * kDelayUs;
+    };
+    launch_delay(1.0, c->stream);  // the kernel's code is on the device before anything is timed
+    QTIP_HIP(hipStreamSynchronize(c->stream));
+    for (int i = 0; i < kCandidates && kept.size() < 3; ++i) {
+      hipStream_t s = nullptr;
+      QTIP_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+      dropped.push_back(s);  // until shown otherwise
+      if (beside(kept.size(), s)) {
+        dropped.pop_back();
+        kept.push_back(s);
+      }
+    }
+    // The stream that brings host inputs up needs no queue of its own, but it had better share the factorization's,
+    // which has time to spare, than a chain's: a dropped candidate that runs beside the context's stream and the two
+    // chain streams can only have been dropped for sharing the third stream's queue.
+    if (kept.size() == 3)
+      for (size_t i = 0; i < dropped.size() && !upload; ++i)
+        if (beside(2, dropped[i])) {
+          upload = dropped[i];
+          dropped.erase(dropped.begin() + long(i));
+        }
+  } catch (...) {
+    for (hipStream_t s : kept) dropped.push_back(s);
+    kept.clear();
+    if (upload) dropped.push_back(upload);
+    upload = nullptr;
+  }
+  for (hipStream_t s : dropped) {
+    (void)hipStreamSynchronize(s);
+    (void)hipStreamDestroy(s);
+  }
+  if (kept.size() > 0) c->chain_stream[0] = kept[0];
+  if (kept.size() == 2) c->ldl_stream = kept[1];  // two chains and the factorization beside them
+  if (kept.size() == 3) c->chain_stream[1] = kept[1], c->ldl_stream = kept[2];
+  c->upload_stream = upload;
+  c->side_streams = int(kept.size());
+}
+
 void destroy_context(qtip_ctx* ctx) {
   ctx->arena.children.clear();
   for (qtip_ctx*& l : ctx->lane)
@@ -185,6 +257,7 @@ int qtip_create(int device, qtip_ctx** out) {
     qtip_ctx* c = make_context(device, nullptr);
     try {
       viterbi_static_scratch_init(device);
+      find_side_streams(c);
     } catch (...) {
       destroy_context(c);
       throw;
@@ -293,6 +366,13 @@ int qtip_set_viterbi_mode(qtip_ctx* ctx, int mode, unsigned margin_units) {
     ctx->vit_margin = margin_units ? margin_units : kViterbiMargin;
     for (qtip_ctx* l : ctx->lane)
       if (l) l->vit_mode = ctx->vit_mode, l->vit_wide = ctx->vit_wide, l->vit_margin = ctx->vit_margin;
+  });
+}
+
+int qtip_ldlq_default_chains(qtip_ctx* ctx, int* chains) {
+  return guarded([&] {
+    QTIP_REQUIRE(ctx != nullptr && chains != nullptr, "ldlq_default_chains: null argument");
+    *chains = ldlq_default_chains(ctx);
   });
 }
 

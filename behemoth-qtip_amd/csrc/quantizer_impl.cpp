@@ -91,6 +91,15 @@ void ldl_hessian_impl(const float* host_HRr, int n, int threads, float* host_L) 
 // apart and keep that distance: while the workgroups of one chain walk their trace-backs (a chain of HBM round
 // trips during which they issue next to nothing), those of the other two, resident on the same compute units, run
 // their forward passes.  One chain alone leaves the chip idle for the length of every trace-back.
+int ldlq_default_chains(qtip_ctx* c) {
+  static const int env_chains = [] {
+    const char* q = getenv("GPU_MAX_HW_QUEUES");
+    return q && atoi(q) >= 6 ? 3 : 2;
+  }();
+  if (c->default_chains == 0) c->default_chains = c->side_streams >= 3 ? 3 : env_chains;
+  return c->default_chains;
+}
+
 void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, float* hatWT, uint16_t* Q, int feedback,
                double* vit_seconds, int chains) {
   QTIP_REQUIRE(n % 128 == 0, "LDLQ needs n %% 128 == 0 (n = %ld)", n);
@@ -100,18 +109,13 @@ void ldlq_impl(qtip_ctx* c, const float* WT, const float* L, long n, long m, flo
   hipStream_t s = c->stream;
   ensure_viterbi_workspace(c);
   const long ntr = m / 16, nblk = n / 16;
-  // chains: only where every chain still fills its share of the chip.  Default: three where the process was given
-  // enough hardware queues for them (context stream, two chain streams, the LDL's stream and the caller's own: with
-  // HIP's default of four queues two of these would share one and run one after the other), else two.
-  // The library cannot see how many queues the runtime was started with, only what the environment says now, so a
-  // default of three is on probation: the first call that runs three chains looks at its launches' own time stamps
-  // and the context goes back to two for good when the first launches of the chains ran one after the other.
-  static const int env_chains = [] {
-    const char* q = getenv("GPU_MAX_HW_QUEUES");
-    return q && atoi(q) >= 6 ? 3 : 2;
-  }();
-  if (c->default_chains == 0) c->default_chains = env_chains;
-  int nch = chains == 0 ? c->default_chains : chains;
+  // chains: only where every chain still fills its share of the chip.  Default: three where the context found its two
+  // chain streams and the LDL's stream running beside its own stream and beside each other when it was made (each on
+  // a hardware queue of its own), or where the environment says the process was given six queues or more; else two.
+  // Either way a default of three is on probation: the first call that runs three chains looks at its launches' own
+  // time stamps and the context goes back to two for good when the first launches of the chains ran one after the
+  // other.
+  int nch = chains == 0 ? ldlq_default_chains(c) : chains;
   while (nch > 1 && ntr < long(nch) * (c->vit_slots / nch)) --nch;
   struct Chain {
     hipStream_t s;

@@ -39,7 +39,9 @@ struct qtip_ctx {
   // so that one chain's trace-backs and gathers run under the others' forward passes
   static constexpr int kMaxChains = 3;
   hipStream_t chain_stream[kMaxChains - 1] = {};
-  int default_chains = 0;       // 0: not decided yet (the environment's queue count decides, then the first call checks)
+  int default_chains = 0;       // 0: not decided yet (side_streams or the environment's queue count decides, then the first call checks)
+  int side_streams = 0;         // how many of chain_stream[0], chain_stream[1], ldl_stream (in this order) were found
+                                // to run beside the context's stream and beside each other when the context was made
   bool chains_checked = false;
   double vit_tile_us = 800.0;   // a resident Viterbi workgroup's time per tile, from the last timed LDLQ call
   qtipmi::Rht rht;
@@ -71,6 +73,7 @@ void nvfp4_prepare_assisted_impl(qtip_ctx* c, const float* host_H, int n, double
                                  float* host_dw);
 void ldlq_impl(qtip_ctx* c, const float* dWT, const float* dL, long n, long m, float* d_hatWT, uint16_t* dQ,
                int feedback, double* vit_seconds, int chains);
+int ldlq_default_chains(qtip_ctx* c);  // what chains = 0 stands for in this context (decided on the first call)
 // what a group carries from one phase of its quantization to the next (device buffers, offsets of its linears, times)
 struct GroupWork {
   long mt = 0;

@@ -222,8 +222,8 @@ def run_group(args, pkg):
                                                      for a, b in zip(fres[-1][0], stats["cmp_outs3"]))))
         del fres
     if args.chains == 0 and not args.no_chains2_leg:
-        # beside it: three groups with two LDLQ chains, what a caller gets whose process runs on HIP's default of four
-        # hardware queues (the third chain needs GPU_MAX_HW_QUEUES >= 6 in the environment when the runtime starts)
+        # beside it: three groups with two LDLQ chains, what a caller gets whose context found fewer than three side
+        # streams with hardware queues of their own when it was made
         kc = min(args.steps, 3)
         copt = pkg.QuantOpts(ldl_threads=args.ldl_threads, skip_proxy=False, feedback=args.feedback,
                              ldl_device_updates=not args.host_ldl, ldlq_chains=2, group_lanes=args.lanes)
@@ -298,9 +298,10 @@ def run_group(args, pkg):
     stats.pop("cmp_outs3", None)
     ntr = sum(ms) // 16
     launches = n // 128   # one Viterbi launch per 128-column buffer and chain: a workgroup takes its tile row through 8 column blocks
-    # the library's rule: three chains with at least 6 hardware queues, else two; a chain must fill its share of the
-    # 768 resident workgroups
-    nch = args.chains or (3 if int(os.environ.get("GPU_MAX_HW_QUEUES", "4")) >= 6 else 2)
+    # the library's rule: three chains where its side streams have hardware queues of their own (it times them when
+    # the context is made) or the environment promises 6 queues, else two; a chain must fill its share of the 768
+    # resident workgroups
+    nch = args.chains or q.ldlq_default_chains()
     while nch > 1 and ntr < 768:
         nch -= 1
     # groups too small to fill the chip run side by side (qtip_opts.group_lanes): that many times as many launches
@@ -404,9 +405,9 @@ def main():
                          "for the large configurations; 1: one after the other)")
     ap.add_argument("--hw-queues", type=int, default=None,
                     help="GPU_MAX_HW_QUEUES for this process (set before the HIP runtime starts; 0: leave the environment "
-                         "alone; default: 8, and 16 for --config 2).  With HIP's default of 4 the library runs two chains "
-                         "of launches per group, with 6 or more three; small groups run side by side on as many lanes "
-                         "as there are queues")
+                         "alone; default: 0, and 16 for --config 2).  The three chains of launches of a large group "
+                         "find their hardware queues among HIP's default of 4 (the library times its side streams "
+                         "when a context is made); small groups run side by side on as many lanes as there are queues")
     ap.add_argument("--viterbi-fp64", action="store_true",
                     help="fp64 path metrics only (default: 32-bit metrics first, a pass repeated on fp64 metrics when a "
                          "traced decision is too close; same codes)")
@@ -423,7 +424,7 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     if args.hw_queues is None:
-        args.hw_queues = 16 if args.config == 2 else 8
+        args.hw_queues = 16 if args.config == 2 else 0
     if args.steps is None:
         args.steps = 48 if args.config == 2 else 16
     if args.warmup is None:

@@ -102,6 +102,9 @@ int qtip_set_viterbi_mode(qtip_ctx* ctx, int mode, unsigned margin_units);
  * first passes (free ends, on the rotated sequence) and second passes (tail-biting).  Waits for the device.
  * Either pointer may be NULL. */
 int qtip_viterbi_stats(qtip_ctx* ctx, unsigned long long* redone_first, unsigned long long* redone_second, int reset);
+/* What qtip_opts.ldlq_chains = 0 stands for in this context: 2 or 3 (see there).  No counterpart in the reference,
+ * whose LDLQ is one sequence of launches (src/quantizer.cpp:42-108). */
+int qtip_ldlq_default_chains(qtip_ctx* ctx, int* chains);
 
 /* hat[i] = lut[state[i]] (k_decode_states, src/viterbi.hip:231-238): B x 128 states -> B x 256 fp32 */
 int qtip_decode_states_dev(qtip_ctx* ctx, const uint16_t* dev_states, long B, float* dev_hat);
@@ -197,9 +200,11 @@ typedef struct { /* QuantOpts, src/quantizer.hpp:11-19 */
   int ldlq_chains;       /* LDLQ deals the tile rows of a group to this many independent chains of launches (each on
                             a stream of its own inside ctx), so that the trace-backs of one run under the forward
                             passes of the others; same codes whatever the number.  At most 3.  0 (default): 3 if the
-                            environment gave the process at least 6 hardware queues (GPU_MAX_HW_QUEUES, read by
-                            the HIP runtime when it starts), else 2 - with HIP's default of four queues a third
-                            chain would share a queue with another stream and run after it, not beside it */
+                            context, when it was made, found three side streams that run beside its own stream and
+                            beside each other (each on a hardware queue of its own: qtip_create times them), or if
+                            the environment gave the process at least 6 hardware queues (GPU_MAX_HW_QUEUES, read by
+                            the HIP runtime when it starts); else 2 - a chain whose stream shares a queue with
+                            another stream runs after it, not beside it.  qtip_ldlq_default_chains tells which */
   int group_lanes;       /* qtip_run_groups runs this many groups side by side, each on a lane of its own inside ctx
                             (one stream, workspaces, staging), group g on lane g mod lanes; same results whatever
                             the number.  At most 12.  1: one group after the other, as the reference schedules them.

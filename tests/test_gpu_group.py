@@ -267,6 +267,14 @@ def test_group_small_end_to_end(qz, oracle, pkg, hyb, synth):
     assert tm.total > 0 and tm.ldlq > 0 and tm.viterbi > 0
 
 
+def test_default_chain_count(qz):
+    """A context times its side streams when it is made and runs three LDLQ chains by default where three of them
+    have hardware queues of their own, else two (unless the environment promises six queues or more)."""
+    n = qz.ldlq_default_chains()
+    say("default LDLQ chains of this context: %d" % n)
+    assert n in (2, 3)
+
+
 def test_ldlq_chains_give_the_same_codes(qz, oracle, pkg, hyb):
     """The tile rows of a group are dealt to 1, 2 or 3 independent chains of launches (streams of their own, feedback
     slabs of their own, ragged shares of rows with two linears of different height): every packed word, Wscale and
