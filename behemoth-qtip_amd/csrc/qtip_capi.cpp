@@ -105,7 +105,7 @@ qtip_ctx* make_context(int device, const HostCodebook* cb_from) {
 // included; nothing tells which stream got which.  Timing does: a wave that sleeps for half a millisecond on each of
 // two streams takes half a millisecond if they have queues of their own and a whole one if they share.  Candidates
 // are made one after the other and kept if such a wave on each of the streams kept so far and on the candidate
-// finishes in well under two delays (the better of two tries: a stream's first launch also sets its queue up); the
+// finishes in well under two delays (in one of three tries: a stream's first launch also sets its queue up); the
 // others are released.  Up to three are kept: chain_stream[0], chain_stream[1], ldl_stream.  With all three LDLQ
 // defaults to three chains whatever the environment says.  The caller's streams may share queues with these: they
 // are idle while a call of this library runs.  Any failure leaves the streams to be made on first use, as before.
@@ -131,8 +131,9 @@ void find_side_streams(qtip_ctx* c) {
       return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
     };
     auto beside = [&](size_t count, hipStream_t cand) {
-      const double a = side_by_side_us(count, cand), b = side_by_side_us(count, cand);
-      return (a < b ? a : b) < 1.5 * kDelayUs;
+      for (int attempt = 0; attempt < 3; ++attempt)  // the first launch on a stream also sets its queue up
+        if (side_by_side_us(count, cand) < 1.5 * kDelayUs) return true;
+      return false;
     };
     launch_delay(1.0, c->stream);  // the kernel's code is on the device before anything is timed
     QTIP_HIP(hipStreamSynchronize(c->stream));
