@@ -147,14 +147,21 @@ void find_side_streams(qtip_ctx* c) {
       }
     }
     // The stream that brings host inputs up needs no queue of its own, but it had better share the factorization's,
-    // which has time to spare, than a chain's: a dropped candidate that runs beside the context's stream and the two
-    // chain streams can only have been dropped for sharing the third stream's queue.
-    if (kept.size() == 3)
+    // which has time to spare, than a chain's: a candidate that runs beside the context's stream and the two chain
+    // streams shares the third stream's queue or none of these four.
+    if (kept.size() == 3) {
       for (size_t i = 0; i < dropped.size() && !upload; ++i)
         if (beside(2, dropped[i])) {
           upload = dropped[i];
           dropped.erase(dropped.begin() + long(i));
         }
+      for (int i = 0; i < 8 && !upload; ++i) {  // none among them: a few more candidates, for this alone
+        hipStream_t s = nullptr;
+        QTIP_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+        if (beside(2, s)) upload = s;
+        else dropped.push_back(s);
+      }
+    }
   } catch (...) {
     for (hipStream_t s : kept) dropped.push_back(s);
     kept.clear();
