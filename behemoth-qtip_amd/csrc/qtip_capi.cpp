@@ -158,8 +158,11 @@ void find_side_streams(qtip_ctx* c) {
       for (int i = 0; i < 8 && !upload; ++i) {  // none among them: a few more candidates, for this alone
         hipStream_t s = nullptr;
         QTIP_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-        if (beside(2, s)) upload = s;
-        else dropped.push_back(s);
+        dropped.push_back(s);  // until shown otherwise
+        if (beside(2, s)) {
+          dropped.pop_back();
+          upload = s;
+        }
       }
     }
   } catch (...) {
