@@ -516,7 +516,7 @@ __device__ __forceinline__ uint32_t trace_back(Smem& sm, const double* __restric
 // conflicts.  The metric of (column, digit d) sits at pos(column) * 16 + (d ^ swz(column)) with swz a multiple of 4,
 // so a column comes in as four 16-byte reads; pos and swz are chosen so that those reads, the 4-byte writes of a
 // group's result (32 lanes: 4 columns x 8 digits) and of its mirror (slot ^ 0xfeb) are free of bank conflicts.
-constexpr uint32_t kSat = 0xffffffffu;      // 64.0: the largest metric, and +inf
+constexpr uint32_t kSat = 0xffffffffu;      // the largest metric (64.0 in units of 2^-26), and +inf
 // A decision's winner must be below this: nothing on its path was then cut off at kSat (a path's metric only grows).
 // A candidate that was cut off is truly larger than it reads, so a margin seen against it is a margin there.
 constexpr uint32_t kWinnerMax = kSat - (1u << 20);
@@ -865,7 +865,7 @@ __device__ __forceinline__ uint32_t row_min16_u32(uint32_t c) {
 // j_last: low 12 bits of the final state (the group the pass ends in; for a free pass the best group, of which the
 // column counts).  The decision of step 127 is taken from the metrics entering it (kept slot 63), then two steps
 // per round trip.  flag is raised (in every thread alike) when a
-// decision is won by less than thr units or the winner is not below 2^31.
+// decision is won by less than thr units or the winner is not below kWinnerMax.
 // Returns the state of step it_min - 1; record: the states of the steps walked are written to sm.st.
 // kStream (the 512-thread form, whose workgroup has its compute unit to itself): which 256 of a kept step's values a
 // round reads is known only when the round before it is decided, so fetched on demand every round waits for HBM.
