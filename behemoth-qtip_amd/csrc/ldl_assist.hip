@@ -88,7 +88,7 @@ __device__ __forceinline__ void subtract_tile(const double4_t (&acc)[4][4], doub
 // of LDS each, three per CU), so this one stays within 168 registers and 48 KB of LDS and takes the place of one of
 // them, not two: the operand slices go from global memory straight into LDS (global_load_lds_dwordx4: a wave's 64
 // lanes fill one 1 KB row of 128 doubles), eight columns of the panel per stage, three stages in flight, one
-// barrier per stage, no staging registers.
+// barrier per stage, no staging registers; fragment reads and loads go one at a time under the MFMAs (see the loop).
 // Lanes beyond nr in the last tile row read whatever follows in Xt (the caller's buffer extends at least 128 doubles
 // beyond the last row read); those columns only feed outputs that are never stored.
 constexpr int UT = 128;
@@ -111,54 +111,126 @@ __global__ __launch_bounds__(256, 3) void rank_update_lower_kernel(const double*
   }
   const int i0 = bi * UT, j0 = bj * UT;
   __shared__ __attribute__((aligned(16))) double S[VSTAGES][2][VK][UT];  // [stage][Xi | Xj][k][column]
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), wm = wave >> 1, wn = wave & 1;
   double4_t acc[4][4];
 #pragma unroll
   for (int a = 0; a < 4; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = double4_t{0, 0, 0, 0};
-  // wave w brings rows 2w and 2w + 1 of a stage's Xi and Xj slices
+  // wave w brings rows 2w and 2w + 1 of a stage's Xi and Xj slices; gi / gj: this lane's piece of the next slice to
+  // be requested, `asked` its number
   const double* gi = Xt + long(2 * wave) * ldx + i0 + 2 * lane;
   const double* gj = Xt + long(2 * wave) * ldx + j0 + 2 * lane;
+  const long slice_stride = long(VK) * ldx;
+  int asked = 0;
   typedef __attribute__((address_space(3))) void* lds_ptr;
-  auto issue = [&](int slice) {
-    const int st = slice % VSTAGES;
-    const long off = long(slice) * VK * ldx;
-#pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      __builtin_amdgcn_global_load_lds(gi + off + r * ldx, (lds_ptr)&S[st][0][2 * wave + r][0], 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(gj + off + r * ldx, (lds_ptr)&S[st][1][2 * wave + r][0], 16, 0, 0);
-    }
+  auto load1 = [&](int st, int q) {  // into stage st; q = 0, 1: rows 2w, 2w + 1 of Xi; 2, 3: of Xj
+    const int r = q & 1;
+    if (q < 2) __builtin_amdgcn_global_load_lds(gi + r * ldx, (lds_ptr)&S[st][0][2 * wave + r][0], 16, 0, 0);
+    else __builtin_amdgcn_global_load_lds(gj + r * ldx, (lds_ptr)&S[st][1][2 * wave + r][0], 16, 0, 0);
+  };
+  auto asked_one = [&] {
+    gi += slice_stride, gj += slice_stride, ++asked;
+    // the two running pointers as they are: without this the compiler keeps one pointer per load of the unrolled
+    // loop, two dozen registers that the accumulators leave no room for
+    asm volatile("" : "+v"(gi), "+v"(gj));
   };
   const int slices = kb / VK;  // kb is a multiple of 16
-  issue(0);
-  if (slices > 1) issue(1);
-  for (int sl = 0; sl < slices; ++sl) {
-    // this wave's loads of slice sl have landed when at most the 4 of slice sl + 1 are outstanding
-    if (sl + 1 < slices) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
-    else __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
-    // everyone's have, and everyone is done reading the stage that slice sl + 2 overwrites (a barrier that orders
-    // LDS only: __syncthreads() would also wait for the loads of slice sl + 1)
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    if (sl + 2 < slices) issue(sl + 2);
-    const int st = sl % VSTAGES;
-#pragma unroll
-    for (int kk = 0; kk < VK; kk += 4) {
-      const int kr = kk + (lane >> 4), c = lane & 15;
-      double a[4], b[4];
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) a[mi] = S[st][0][kr][wm * 64 + mi * 16 + c];
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni) b[ni] = S[st][1][kr][wn * 64 + ni * 16 + c];
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+  // fragments of the 4 k of step ks (0, 1) of the slice in stage st: a[set][mi], b[set][ni]
+  const int c16 = lane & 15, kq = lane >> 4;
+  double fa[2][4], fb[2][4];
+  auto read1 = [&](int st, int ks, int set, int j) {  // j = 0..7 in the order the MFMAs first use them: a0 b0 b1 b2 b3 a1 a2 a3
+    const int kr = 4 * ks + kq;
+    if (j == 0 || j >= 5) {
+      const int mi = j == 0 ? 0 : j - 4;
+      fa[set][mi] = S[st][0][kr][wm * 64 + mi * 16 + c16];
+    } else {
+      const int ni = j - 1;
+      fb[set][ni] = S[st][1][kr][wn * 64 + ni * 16 + c16];
     }
+  };
+  auto mfma = [&](int set, int j) {
+    const int mi = j >> 2, ni = j & 3;
+    acc[mi][ni] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[set][mi], fb[set][ni], acc[mi][ni], 0, 0, 0);
+  };
+  // Slices 0 and 1 requested, slice 0 landed (this wave's loads, then everyone's: a bare barrier, which does not wait
+  // for the loads still in flight), slice 2 requested, the fragments of slice 0's first 4 k read.
+  load1(0, 0), load1(0, 1), load1(0, 2), load1(0, 3);
+  asked_one();
+  if (slices > 1) {
+    load1(1, 0), load1(1, 1), load1(1, 2), load1(1, 3);
+    asked_one();
   }
-  subtract_tile(acc, C, ldc, nr, i0 + wm * 64, j0 + wn * 64, lane);
+  if (slices > 1) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
+  else __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  if (asked < slices) {
+    load1(2, 0), load1(2, 1), load1(2, 2), load1(2, 3);
+    asked_one();
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) read1(0, 0, 0, j);
+  // One slice: 32 MFMAs, two steps of 4 k on fragment sets 0 and 1.  The workgroup runs beside the Viterbi kernel's,
+  // one wave per SIMD with nothing to hide a wait behind but its own MFMAs (32 cycles each, during which the wave may
+  // issue other work): under every other MFMA of a step it reads one fragment of the next step, and under MFMAs 1, 5,
+  // 9, 13 of the second step it requests one row of slice sl + 3 - after the barrier in the middle, which says slice
+  // sl + 1 has landed everywhere and every wave has asked for its last fragments of slice sl, whose stage is
+  // therefore free.  The scheduling barriers pin that order.  kSteady: every slice asked for exists and one more is
+  // on its way beyond sl + 1, so vmcnt(4) = "slice sl + 1 is here"; the last slices run the same code with the
+  // conditions and a full wait.
+#define QTIP_SB __builtin_amdgcn_sched_barrier(0)
+  auto slice = [&](auto steady, auto stage, int sl) {  // slice sl, which lies in stage sl % VSTAGES = stage
+    constexpr bool kSteady = decltype(steady)::value;
+    constexpr int st = decltype(stage)::value, nst = (st + 1) % VSTAGES;
+    const bool next = kSteady || sl + 1 < slices;
+#define QTIP_M0(j) { mfma(0, j); QTIP_SB; }
+#define QTIP_R0(j) { mfma(0, j); QTIP_SB; read1(st, 1, 1, (j) / 2); QTIP_SB; }
+    QTIP_SB;
+    QTIP_R0(0) QTIP_M0(1) QTIP_R0(2) QTIP_M0(3) QTIP_R0(4) QTIP_M0(5) QTIP_R0(6) QTIP_M0(7)
+    QTIP_R0(8) QTIP_M0(9) QTIP_R0(10) QTIP_M0(11) QTIP_R0(12) QTIP_M0(13) QTIP_R0(14) QTIP_M0(15)
+    if (next) {
+      // this wave's part of slice sl + 1 has landed and its reads of slice sl have returned
+      if (kSteady) __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+      else __builtin_amdgcn_s_waitcnt(0x0070);          // vmcnt(0) lgkmcnt(0)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    }
+    const bool go = kSteady || asked < slices;
+#define QTIP_M1(j) { mfma(1, j); QTIP_SB; }
+#define QTIP_R1(j) { mfma(1, j); QTIP_SB; if (next) read1(nst, 0, 0, (j) / 2); QTIP_SB; }
+#define QTIP_L1(j) { mfma(1, j); QTIP_SB; if (go) load1(st, ((j) - 1) / 4); QTIP_SB; }
+    QTIP_SB;
+    QTIP_R1(0) QTIP_L1(1) QTIP_R1(2) QTIP_M1(3) QTIP_R1(4) QTIP_L1(5) QTIP_R1(6) QTIP_M1(7)
+    QTIP_R1(8) QTIP_L1(9) QTIP_R1(10) QTIP_M1(11) QTIP_R1(12) QTIP_L1(13) QTIP_R1(14) QTIP_M1(15)
+    if (go) asked_one();
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  using S2 = std::integral_constant<int, 2>;
+  static_assert(VSTAGES == 3);
+  int sl = 0;
+  for (; sl + 5 < slices; sl += 3) {
+    slice(std::true_type{}, S0{}, sl);
+    slice(std::true_type{}, S1{}, sl + 1);
+    slice(std::true_type{}, S2{}, sl + 2);
+  }
+  for (; sl < slices; sl += 3) {  // the last 3 to 5 slices (or all, of fewer)
+    slice(std::false_type{}, S0{}, sl);
+    if (sl + 1 < slices) slice(std::false_type{}, S1{}, sl + 1);
+    if (sl + 2 < slices) slice(std::false_type{}, S2{}, sl + 2);
+  }
+#undef QTIP_M0
+#undef QTIP_R0
+#undef QTIP_M1
+#undef QTIP_R1
+#undef QTIP_L1
+#undef QTIP_SB
+  // the lane number anew: the loop leaves no register to keep it in
+  const int ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  subtract_tile(acc, C, ldc, nr, i0 + wm * 64, j0 + wn * 64, ln);
 }
 
 // The panels travel one ahead of the updates: as soon as panel k is solved its rows go up, the update of the next
