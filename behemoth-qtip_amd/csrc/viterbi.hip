@@ -942,9 +942,9 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
                                   __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   // (the forward pass's own arithmetic: the same products and sums on the same operands give the same integers)
-  auto err_of = [&](uint32_t st, double x0, double x1) -> uint32_t {
+  // the codebook entry of a state, and its error against two inputs
+  auto entry_of = [&](uint32_t st, double& l0, double& l1) {
     const uint32_t e = ((st * (st + 1u)) >> 6) & 1023u;
-    double l0, l1;
     if constexpr (kStream) {
       const uint32_t w = tl[e & 511u];
       const uint16_t h0 = uint16_t((w & 0xffffu) ^ ((e >> 9) << 15)), h1 = uint16_t(w >> 16);
@@ -952,7 +952,14 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
     } else {
       l0 = entry_d[2 * e], l1 = entry_d[2 * e + 1];
     }
+  };
+  auto err_at = [&](double l0, double l1, double x0, double x1) -> uint32_t {
     return err_units(l0 * unit.pre, l1 * unit.pre, x0 * unit.pre, x1 * unit.pre);
+  };
+  auto err_of = [&](uint32_t st, double x0, double x1) -> uint32_t {
+    double l0, l1;
+    entry_of(st, l0, l1);
+    return err_at(l0, l1, x0, x1);
   };
   // over the 16 lanes of a row: the smallest value (returned), the first lane that holds it, the gap to the runner-up
   auto row_pick = [&](uint32_t c, uint32_t& first, uint32_t& gap) -> uint32_t {
@@ -1031,11 +1038,18 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
     const double xb0 = double(sm.x[tb]), xb1 = double(sm.x[tb + 1]);
     const uint32_t g = (d << 8) | (j >> 4);
     const uint32_t s1 = (dp << 12) | g;
-    const uint32_t c1 = sat_add(err_of(s1, xa0, xa1), kept(it / 2 - 1, s1 >> 4));
+    // A round's three loads all at once, the two codebook entries (cached) before the kept metric (from HBM): the
+    // kept metric is read with an atomic load, which the compiler moves nothing across, so written in the order of
+    // use a round would wait for one entry, then for the metric, then for the other entry.
+    double la0, la1, lb0, lb1;
+    entry_of(s1, la0, la1);
+    entry_of((d << 12) | j, lb0, lb1);
+    const uint32_t kv = kept(it / 2 - 1, s1 >> 4);
+    const uint32_t c1 = sat_add(err_at(la0, la1, xa0, xa1), kv);
     uint32_t k1, gap1;
     // the metric of group g entering step it, as the forward pass had it
     const uint32_t m1 = min(row_pick(c1, k1, gap1), kSat);
-    const uint32_t c0 = sat_add(err_of((d << 12) | j, xb0, xb1), m1);
+    const uint32_t c0 = sat_add(err_at(lb0, lb1, xb0, xb1), m1);
     // every lane of row r holds that row's (c0, k1, gap1) for d = 4 wave + r: best and runner-up of the wave's four
     uint32_t bc = uint32_t(__builtin_amdgcn_readlane(int(c0), 0)), sc = kSat, bd = 4u * wave;
     uint32_t bd1 = uint32_t(__builtin_amdgcn_readlane(int(k1), 0)), bg = uint32_t(__builtin_amdgcn_readlane(int(gap1), 0));
