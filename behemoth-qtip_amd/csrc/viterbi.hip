@@ -110,7 +110,7 @@ struct Smem {
   uint32_t red_s[4];
   double tr_c[2][4];    // trace-back: the four waves' best candidates of a round (cost; d | d1 << 8), two sets
   uint32_t tr_d[2][4];
-  uint32_t tr32[2][4][4];  // the same for the 32-bit passes: best, second best, d | d1 << 8, gap inside the best's row
+  alignas(16) uint32_t tr32[2][4][4];  // the same for the 32-bit passes: best, second best, d | d1 << 8, gap inside the best's row
   uint32_t red32[8][3];    // end of the free 32-bit pass: per wave the best group's metric, the second best, the group
   int overlap;
   uint32_t final_state;
@@ -1072,16 +1072,25 @@ __device__ __forceinline__ uint32_t trace_back32(Smem& sm, const double* __restr
       sm.tr32[set][wave][3] = bg;
     }
     round_barrier();
-    bc = sm.tr32[set][0][0], sc = sm.tr32[set][0][1];
-    uint32_t bdd = sm.tr32[set][0][2];
-    bg = sm.tr32[set][0][3];
+    // The four waves' entries in four 16-byte reads, all asked for before the first is looked at: the values are the
+    // same in every lane, and left to itself the compiler turns the choices below into branches around single
+    // 4-byte reads, one LDS round trip after the other.
+    uint4 q[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) q[w] = *reinterpret_cast<const uint4*>(sm.tr32[set][w]);
+    asm volatile("" : "+v"(q[0].x), "+v"(q[0].y), "+v"(q[0].z), "+v"(q[0].w), "+v"(q[1].x), "+v"(q[1].y), "+v"(q[1].z),
+                 "+v"(q[1].w), "+v"(q[2].x), "+v"(q[2].y), "+v"(q[2].z), "+v"(q[2].w), "+v"(q[3].x), "+v"(q[3].y),
+                 "+v"(q[3].z), "+v"(q[3].w));
+    bc = q[0].x, sc = q[0].y;
+    uint32_t bdd = q[0].z;
+    bg = q[0].w;
 #pragma unroll
     for (int w = 1; w < 4; ++w) {
-      const uint32_t oc = sm.tr32[set][w][0], os = sm.tr32[set][w][1];
+      const uint32_t oc = q[w].x, os = q[w].y;
       const bool take = oc < bc;
       sc = take ? min(bc, os) : min(sc, oc);
-      bdd = take ? sm.tr32[set][w][2] : bdd;
-      bg = take ? sm.tr32[set][w][3] : bg;
+      bdd = take ? q[w].z : bdd;
+      bg = take ? q[w].w : bg;
       bc = take ? oc : bc;
     }
     // (a candidate of step `it` is a sum of it + 1 rounded terms: what thr allows for 128 terms shrinks by one unit
