@@ -16,14 +16,11 @@
 namespace qtipmi {
 namespace {
 
-// the scalar codec (nvfp4_codec.hpp) under the names the kernels use
-__device__ __forceinline__ float nv_fp8_dec(unsigned c) { return nvcodec::e4m3_value(c); }           // code <= 126 -> value
-__device__ __forceinline__ unsigned nv_fp8_enc(float x) { return nvcodec::e4m3_of_magnitude(x); }    // finite x -> code of |x|
-__device__ __forceinline__ float nv_bf16_round(float f) { return nvcodec::through_bf16(f); }
-__device__ __forceinline__ float nv_level(int c) { return nvcodec::e2m1_value(unsigned(c)); }
-__device__ __forceinline__ int nv_fp4_code(float a) { return int(nvcodec::e2m1_of_magnitude(a)); }  // a >= 0
+// The scalar codec is nvfp4_codec.hpp's: e4m3_value (code <= 126 -> value), e4m3_of_magnitude (finite x -> code of |x|),
+// through_bf16, e2m1_value and e2m1_of_magnitude (a >= 0 -> code).
+namespace nvc = nvcodec;
 
-constexpr int kCand = 11;       // scale candidates of the search: the plain one, 8 shrink factors, one code down, one up
+constexpr int kScaleTries = 11;  // scale candidates of the search: the plain one, 8 shrink factors, one code down, one up
 constexpr int kBlockRows = 64;  // matrix rows per workgroup: one per lane
 
 // Block scale candidate number `which` (uniform over a wave) of a row whose 16 targets have the largest magnitude
@@ -41,9 +38,9 @@ __device__ __forceinline__ unsigned nv_candidate(int which, float amax, float gl
       case 7: shrink = 1.00f; break;
       default: break;
     }
-    return nv_fp8_enc(amax * shrink / (6.f * global));
+    return nvc::e4m3_of_magnitude(amax * shrink / (6.f * global));
   }
-  const unsigned plain = nv_fp8_enc(amax / (6.f * global));
+  const unsigned plain = nvc::e4m3_of_magnitude(amax / (6.f * global));
   if (which == 9) return plain > 0 ? plain - 1 : 0;
   if (which == 10) return plain < 126 ? plain + 1 : 126;
   return plain;
@@ -54,23 +51,23 @@ __device__ __forceinline__ unsigned nv_candidate(int which, float amax, float gl
 // with the winner (src/nvfp4_gpu.hip:66-158); here the ncand waves of a workgroup round the same 64 rows at the same
 // time, each under its own candidate, leave their costs in LDS, and the wave whose candidate wins a row (smallest cost,
 // the earliest candidate among equals) writes that row's result.  With s the candidate's scale:
-//   t_k  = W[k] + F[k] + sum_{j > k in block} d_j Lb[j][k]   target after the feedback, j ascending
+//   t_k  = W[k] + F[k] + sum_{j > k in block} d_j Ltile[j][k]   target after the feedback, j ascending
 //   q_k  = bf16(level * dec(s) * global)                       what execution sees
 //   d_k  = W[k] - q_k                                          error fed back
 //   cost = sum_k dw[k] (t_k - q_k)^2                           proxy increment, k descending
 // WT, FT: [n][m].  packedT: [n/2][m], scalesT: [n/16][m], E: [16][m].
-__global__ __launch_bounds__(kBlockRows * kCand) void nv_block_kernel(
+__global__ __launch_bounds__(kBlockRows * kScaleTries) void nv_block_kernel(
     const float* __restrict__ WT, const float* __restrict__ FT, long m, long n, long c0, const float* __restrict__ L,
     const float* __restrict__ dw, float global, int calibrate, int ncand, uint8_t* __restrict__ packedT,
     uint8_t* __restrict__ scalesT, float* __restrict__ E) {
-  __shared__ float Lb[16][16];
-  __shared__ float Dw[16];
-  __shared__ float costs[kCand][kBlockRows];
+  __shared__ float Ltile[16][16];
+  __shared__ float colw[16];
+  __shared__ float costs[kScaleTries][kBlockRows];
   const int lane = threadIdx.x & 63;
   const int which = __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6));
   for (int idx = threadIdx.x; idx < 256; idx += blockDim.x)
-    Lb[idx >> 4][idx & 15] = calibrate ? L[(c0 + (idx >> 4)) * n + c0 + (idx & 15)] : 0.f;
-  if (threadIdx.x < 16) Dw[threadIdx.x] = dw ? dw[c0 + threadIdx.x] : 1.f;
+    Ltile[idx >> 4][idx & 15] = calibrate ? L[(c0 + (idx >> 4)) * n + c0 + (idx & 15)] : 0.f;
+  if (threadIdx.x < 16) colw[threadIdx.x] = dw ? dw[c0 + threadIdx.x] : 1.f;
   __syncthreads();
   const long r = long(blockIdx.x) * kBlockRows + lane;
   const bool live = r < m;
@@ -83,8 +80,8 @@ __global__ __launch_bounds__(kBlockRows * kCand) void nv_block_kernel(
     amax = fmaxf(amax, fabsf(calibrate ? t0[k] : w[k]));
   }
   const unsigned code8 = nv_candidate(which, amax, global);
-  const float sd = nv_fp8_dec(code8);
-  const float scale = sd * global;
+  const float sd = nvc::e4m3_value(code8);
+  const float step = sd * global;
   float cost = 0.f;
   uint32_t nib_lo = 0, nib_hi = 0;  // E2M1 codes of columns 0..7 and 8..15, 4 bits each
 #pragma unroll
@@ -92,14 +89,14 @@ __global__ __launch_bounds__(kBlockRows * kCand) void nv_block_kernel(
     float t = t0[k];
     if (calibrate) {
 #pragma unroll
-      for (int j = k + 1; j < 16; ++j) t = fmaf(err[j], Lb[j][k], t);
+      for (int j = k + 1; j < 16; ++j) t = fmaf(err[j], Ltile[j][k], t);
     }
-    const float x = scale != 0.f ? t / scale : 0.f;
-    const int code = nv_fp4_code(fabsf(x));
-    const float q = nv_bf16_round((x < 0 ? -1.f : 1.f) * nv_level(code) * sd * global);
-    cost = fmaf(Dw[k] * (t - q), t - q, cost);
+    const float x = step != 0.f ? t / step : 0.f;
+    const unsigned mag = nvc::e2m1_of_magnitude(fabsf(x));
+    const float q = nvc::through_bf16((x < 0 ? -1.f : 1.f) * nvc::e2m1_value(mag) * sd * global);
+    cost = fmaf(colw[k] * (t - q), t - q, cost);
     err[k] = w[k] - q;
-    const uint32_t nib = uint32_t(code) | ((__float_as_uint(x) >> 31) << 3);
+    const uint32_t nib = mag | ((__float_as_uint(x) >> 31) << 3);
     if (k < 8) nib_lo |= nib << (4 * k);
     else nib_hi |= nib << (4 * (k - 8));
   }
@@ -206,7 +203,7 @@ __global__ __launch_bounds__(256) void transpose_u8_kernel(const uint8_t* __rest
 void launch_nvfp4_block(const float* WT, const float* FT, long m, long n, long c0, const float* L, const float* dw,
                         float global, bool calibrate, bool search, uint8_t* packedT, uint8_t* scalesT, float* E,
                         hipStream_t s) {
-  const int ncand = search ? kCand : 1;
+  const int ncand = search ? kScaleTries : 1;
   nv_block_kernel<<<dim3(unsigned((m + kBlockRows - 1) / kBlockRows)), dim3(unsigned(kBlockRows * ncand)), 0, s>>>(
       WT, FT, m, n, c0, L, dw, global, calibrate ? 1 : 0, ncand, packedT, scalesT, E);
   QTIP_HIP(hipGetLastError());
