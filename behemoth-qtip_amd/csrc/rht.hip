@@ -14,6 +14,7 @@
 //     flips the sign bit of a value before a plain add.  Longer rows take a second kernel for the mix.
 #include <mutex>
 
+#include "data/qtip_tables.h"
 #include "qtip_internal.hpp"
 #include "rht.hpp"
 
@@ -160,6 +161,149 @@ __global__ __launch_bounds__(kRowThreads) void rht_rows_kernel(float* __restrict
   }
 }
 
+// ---- rows of K chunks of 1024 values (every large layer here: 12288 = 12 x 1024, 28672 = 28 x 1024): one resident
+// workgroup per compute unit walks its share of the rows and has the next row on its way from HBM while it mixes
+// the present one.  The form above gives a row to a workgroup that loads, transforms, mixes and stores it, one phase
+// after the other, with nothing else resident beside it (a row fills most of the LDS): each phase leaves the other
+// pipes idle.  Here
+//   * a wave holds a 1024-point chunk in 16 registers per lane; the loads of the next row's chunks are issued before
+//     the present row's mix and land while its 784 (K = 28) signed adds per thread run;
+//   * the exchanges between lanes 1, 2, 4 and 8 apart are DPP moves in the vector pipe, only those 16 and 32 apart go
+//     through the LDS crossbar;
+//   * the signs of the mixing matrix are compile-time constants: a term of the mix is one add or one subtract
+//     (s - y and s + (-y) are the same sum), with no sign table read and no sign-bit arithmetic.
+// Same sums in the same order as the form above, so the same bits.
+template <int K>
+struct HadRows {
+  uint64_t minus[K];  // bit k of minus[k2]: entry (k2, k) of the mixing matrix is -1
+};
+template <int K, bool kTranspose>
+constexpr HadRows<K> had_rows() {
+  HadRows<K> r{};
+  const uint32_t* bits = K == 12 ? qtip_had12_bits : K == 20 ? qtip_had20_bits : K == 28 ? qtip_had28_bits : qtip_had36_bits;
+  constexpr int wpr = (K + 31) / 32;
+  for (int k2 = 0; k2 < K; ++k2)
+    for (int k = 0; k < K; ++k) {
+      const int row = kTranspose ? k : k2, col = kTranspose ? k2 : k;
+      const bool plus = (bits[row * wpr + (col >> 5)] >> (col & 31)) & 1u;
+      if (!plus) r.minus[k2] |= uint64_t(1) << k;
+    }
+  return r;
+}
+template <int K, bool kTranspose>
+inline constexpr HadRows<K> kHadRows = had_rows<K, kTranspose>();
+
+// the value of the lane whose index differs in bit log2(MASK), MASK <= 8: within a row of 16 lanes, by DPP
+template <int MASK>
+__device__ __forceinline__ float row_partner(float v) {
+  const int x = __builtin_bit_cast(int, v);
+  int y;
+  if constexpr (MASK == 1) y = __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xf, 0xf, false);        // quad_perm [1, 0, 3, 2]
+  else if constexpr (MASK == 2) y = __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xf, 0xf, false);   // quad_perm [2, 3, 0, 1]
+  else if constexpr (MASK == 4)                                                                 // i ^ 3, then i ^ 7
+    y = __builtin_amdgcn_update_dpp(0, __builtin_amdgcn_update_dpp(0, x, 0x1B, 0xf, 0xf, false), 0x141, 0xf, 0xf, false);
+  else y = __builtin_amdgcn_update_dpp(0, x, 0x128, 0xf, 0xf, false);                           // row_ror:8
+  return __builtin_bit_cast(float, y);
+}
+
+// natural-order 1024-point transform of the 16 consecutive values per lane of one wave
+__device__ __forceinline__ void fwht_wave1024(float (&r)[16], int lane) {
+  fwht_registers<16>(r);
+#define QTIP_ROW_STAGE(MASK)                                                    \
+  {                                                                             \
+    const uint32_t neg = (lane & MASK) ? 0x80000000u : 0u;                      \
+    _Pragma("unroll") for (int e = 0; e < 16; ++e) r[e] = row_partner<MASK>(r[e]) + flip(r[e], neg); \
+  }
+  QTIP_ROW_STAGE(1)
+  QTIP_ROW_STAGE(2)
+  QTIP_ROW_STAGE(4)
+  QTIP_ROW_STAGE(8)
+#undef QTIP_ROW_STAGE
+#pragma unroll
+  for (int mask = 16; mask <= 32; mask <<= 1) {
+    const uint32_t neg = (lane & mask) ? 0x80000000u : 0u;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) r[e] = __shfl_xor(r[e], mask, 64) + flip(r[e], neg);
+  }
+}
+
+// X: rows of KT * 1024 values, 16-byte aligned (ld % 4 == 0).  gridDim.x workgroups share the rows out in turn.
+template <int KT, bool kTranspose>
+__global__ __launch_bounds__(kRowThreads) void rht_rows_p1024_kernel(float* __restrict__ X, long ld, long rows,
+                                                                    float scale, const float* __restrict__ rs,
+                                                                    const float* __restrict__ cs) {
+  extern __shared__ float v[];
+  constexpr int kWaves = kRowThreads / 64;
+  constexpr int kTurns = (KT + kWaves - 1) / kWaves;  // chunks a wave takes at most
+  constexpr HadRows<KT> kHad = kHadRows<KT, kTranspose>;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // A lane's 16 values leave as four 16-byte writes, 64 bytes from the neighbouring lane's: the four pieces of lane l
+  // change places by (l / 4 % 4) ^ (l & 2), so that 8 neighbouring lanes write 8 different 16-byte columns of 128
+  // bytes of banks and 16 lanes 16 of 256; the mix reads value i of a chunk at i with bits 2..3 changed accordingly
+  // (64 neighbouring i: 64 neighbouring words).
+  const int swz = ((lane >> 2) & 3) ^ (lane & 2);
+  float4 in[kTurns][4];
+  auto fetch = [&](long row) {
+    const float* x = X + row * ld + lane * 16;
+#pragma unroll
+    for (int j = 0; j < kTurns; ++j) {
+      const int chunk = wave + kWaves * j;
+      if (chunk < KT) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) in[j][q] = *reinterpret_cast<const float4*>(x + chunk * 1024 + 4 * q);
+      }
+    }
+  };
+  long row = blockIdx.x;
+  if (row < rows) fetch(row);
+  for (; row < rows; row += gridDim.x) {
+    const float rsv = rs ? rs[row] : 1.0f;
+#pragma unroll
+    for (int j = 0; j < kTurns; ++j) {
+      const int chunk = wave + kWaves * j;
+      if (chunk < KT) {
+        float r[16];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) r[4 * q] = in[j][q].x, r[4 * q + 1] = in[j][q].y, r[4 * q + 2] = in[j][q].z, r[4 * q + 3] = in[j][q].w;
+        if (rs || cs) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) r[e] *= rsv;
+          if (cs) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float4 c = *reinterpret_cast<const float4*>(cs + chunk * 1024 + lane * 16 + 4 * q);
+              r[4 * q] *= c.x, r[4 * q + 1] *= c.y, r[4 * q + 2] *= c.z, r[4 * q + 3] *= c.w;
+            }
+          }
+        }
+        fwht_wave1024(r, lane);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<float4*>(v + chunk * 1024 + lane * 16 + 4 * (q ^ swz)) = make_float4(r[4 * q], r[4 * q + 1], r[4 * q + 2], r[4 * q + 3]);
+      }
+    }
+    __syncthreads();
+    const int i = threadIdx.x;
+    float y[KT];
+#pragma unroll
+    for (int k = 0; k < KT; ++k) y[k] = v[k * 1024 + (i ^ ((((i >> 6) & 3) ^ ((i >> 4) & 2)) << 2))];
+    __syncthreads();  // the next row's chunks may now be written over this one
+    const long next = row + gridDim.x;
+    if (next < rows) fetch(next);
+    float* x = X + row * ld + i;
+#pragma unroll
+    for (int k2 = 0; k2 < KT; ++k2) {
+      float s = 0.0f;
+#pragma unroll
+      for (int k = 0; k < KT; ++k) {
+        if ((kHad.minus[k2] >> k) & 1) s -= y[k];
+        else s += y[k];
+      }
+      x[k2 * 1024] = s * scale;
+    }
+  }
+}
+
 // The mix for rows too long for LDS, in place on transformed chunks: one wave per 64 values of i, the K inputs of a
 // lane parked in LDS (ys[k][lane]) because the outputs overwrite them.
 __global__ __launch_bounds__(kMixLanes) void had_mix_long_rows_kernel(float* __restrict__ X, long ld, int P, int K,
@@ -274,6 +418,8 @@ void Rht::init(int device, hipStream_t stream) {
   dev_ = device;
   s_ = stream;
   partial_.alloc(kRedBlocks + 1);
+  QTIP_HIP(hipDeviceGetAttribute(&cus_, hipDeviceAttributeMultiprocessorCount, device));
+  if (cus_ <= 0) cus_ = 1;
 }
 
 // sign bits of the mixing matrix (hadK, or its transpose), row k2 in (K + 31) / 32 words: bit k set = entry -1
@@ -305,6 +451,16 @@ RowKernel row_kernel(int K) {
     default: return rht_rows_kernel<0>;
   }
 }
+using PipeKernel = void (*)(float*, long, long, float, const float*, const float*);
+PipeKernel pipe_kernel(int K, bool transpose) {
+  switch (K) {
+    case 12: return transpose ? rht_rows_p1024_kernel<12, true> : rht_rows_p1024_kernel<12, false>;
+    case 20: return transpose ? rht_rows_p1024_kernel<20, true> : rht_rows_p1024_kernel<20, false>;
+    case 28: return transpose ? rht_rows_p1024_kernel<28, true> : rht_rows_p1024_kernel<28, false>;
+    case 36: return transpose ? rht_rows_p1024_kernel<36, true> : rht_rows_p1024_kernel<36, false>;
+    default: return nullptr;
+  }
+}
 // the row kernels may use all of the LDS; told to the runtime once per device
 void allow_full_lds() {
   static std::mutex mu;
@@ -317,6 +473,10 @@ void allow_full_lds() {
   for (int K : {0, 12, 20, 28, 36})
     QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(row_kernel(K)),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, kRowLdsFloats * int(sizeof(float))));
+  for (int K : {12, 20, 28, 36})
+    for (bool t : {false, true})
+      QTIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(pipe_kernel(K, t)),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, kRowLdsFloats * int(sizeof(float))));
   configured[size_t(dev)] = true;
 }
 }  // namespace
@@ -330,6 +490,18 @@ void Rht::hadamard_rows(float* X, long rows, int n, long ld, bool transpose, con
   if (rows <= 0) return;
   allow_full_lds();
   const float sc = 1.0f / std::sqrt(float(n));
+  // rows of K x 1024 values that are 16-byte aligned: the form that keeps the next row in flight
+  const auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  if (P == 1024 && pipe_kernel(K, transpose) && n <= kRowLdsFloats && ld % 4 == 0 && aligned16(X) && aligned16(cs)) {
+    // as many workgroups as are resident at once (a K = 12 row leaves room for two per compute unit)
+    int per_cu = 1;
+    QTIP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(pipe_kernel(K, transpose)),
+                                                          kRowThreads, size_t(n) * sizeof(float)));
+    const unsigned grid = unsigned(std::min<long>(rows, long(cus_) * std::max(per_cu, 1)));
+    pipe_kernel(K, transpose)<<<dim3(grid), dim3(kRowThreads), size_t(n) * sizeof(float), s_>>>(X, ld, rows, sc, rs, cs);
+    QTIP_HIP(hipGetLastError());
+    return;
+  }
   const uint32_t* neg = K > 1 ? device_had(K, transpose) : nullptr;
   // a row that fits in LDS is transformed and mixed in one pass; a longer one goes chunk group by chunk group and is
   // mixed by a second kernel

@@ -24,6 +24,7 @@ class Rht {
  private:
   const uint32_t* device_had(int K, bool transpose);
   int dev_ = 0;
+  int cus_ = 1;  // compute units of the device: resident workgroups of the row kernel that walks rows
   hipStream_t s_ = nullptr;
   DBuf<double> partial_;
   std::vector<std::pair<int, std::unique_ptr<DBuf<uint32_t>>>> had_;

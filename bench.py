@@ -25,6 +25,7 @@ sys.path.insert(0, ROOT)
 FLOP_PER_WEIGHT = 393216.0      # 2^16 add-compare-selects per weight, counted as 6 flop each
 PEAK_FP64_TFLOPS = 78.6         # MI355X vector fp64
 PEAK_32BIT_TFLOPS = 157.3       # MI355X vector fp32: the rate of 32-bit lanes, which the u32 path metrics run on
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 HBM_BYTES_PER_WEIGHT = 2040.0   # algorithmic HBM traffic of the Viterbi per weight (4-bit back-pointers of two passes + X)
 
 
@@ -374,6 +375,34 @@ def run_ldl_only(args, pkg):
                       "same_factor_bits": same and same_resident, "ldl_threads": args.ldl_threads}), flush=True)
 
 
+def run_rht_only(args, pkg):
+    """The row transform alone (hadK (x) H_1024 over rows resident in HBM, in place): milliseconds per pass and the
+    HBM rate of one read and one write of the matrix, for the shapes the large configurations transform."""
+    import torch
+    q = pkg.Quantizer(0)
+    out = []
+    for rows, n in ((28672, 28672), (12288, 28672), (28672, 12288), (12288, 12288)):
+        X = torch.randn(rows, n, device="cuda")
+        q.hadamard_rows_dev(X, rows, n, n, True)
+        q.synchronize()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(max(args.steps, 3)):
+            t0 = time.time()
+            q.hadamard_rows_dev(X, rows, n, n, True)
+            q.synchronize()
+            torch.cuda.synchronize()
+            dt = time.time() - t0
+            best = dt if best is None else min(best, dt)
+        nbytes = 2.0 * rows * n * 4
+        out.append({"rows": rows, "n": n, "ms": best * 1e3, "bytes": nbytes,
+                    "roofline": {"bound": "hbm", "achieved": nbytes / best / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                 "frac": nbytes / best / 1e9 / PEAK_HBM_GBS}})
+        del X
+    print(json.dumps({"workload": "RHT rows alone (sign-free pass, transposed factor), best of %d" % max(args.steps, 3),
+                      "passes": out}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -389,6 +418,9 @@ def main():
     ap.add_argument("--ldl-only", action="store_true",
                     help="time the block LDL of the configuration's rotated Hessian by itself, three times each: host panels "
                          "with GPU trailing updates, and host alone (not the contract's metric; one line of JSON)")
+    ap.add_argument("--rht-only", action="store_true",
+                    help="time the row transform by itself on the large configurations' shapes (not the contract's "
+                         "metric; one line of JSON with the HBM rate of each pass)")
     ap.add_argument("--host-ldl-once", action="store_true", help="with --ldl-only: one host-only factorization instead of three")
     ap.add_argument("--no-host-input-leg", action="store_true",
                     help="skip the extra groups with W and H passed as host pointers reported beside the default run")
@@ -445,6 +477,8 @@ def main():
         del a, b
     if args.ldl_only:
         return run_ldl_only(args, pkg)
+    if args.rht_only:
+        return run_rht_only(args, pkg)
     res = run_viterbi_only(args, pkg) if args.config == 1 else run_group(args, pkg)
     value = res["weights"] / res["wall"] / 1e6
     achieved = res["vit_launch_weights"] * FLOP_PER_WEIGHT / res["vit_launch_s"] / 1e12

@@ -25,7 +25,13 @@ def main():
     out.append("#define QTIP_TABLES_H_")
     out.append("#include <stdint.h>")
     out.append("#define QTIP_NUM_HAD %d" % len(order))
-    out.append("static const int qtip_had_order[QTIP_NUM_HAD] = {%s};" % ",".join(map(str, order)))
+    out.append("/* in C++ the tables can be read in constant expressions */")
+    out.append("#ifdef __cplusplus")
+    out.append("#define QTIP_TABLE static constexpr")
+    out.append("#else")
+    out.append("#define QTIP_TABLE static const")
+    out.append("#endif")
+    out.append("QTIP_TABLE int qtip_had_order[QTIP_NUM_HAD] = {%s};" % ",".join(map(str, order)))
     for K in order:
         body = re.search(r"kHad%d\[\d+\]\s*=\s*\{([^}]*)\}" % K, src).group(1)
         vals = [int(v) for v in body.split(",")]
@@ -40,7 +46,7 @@ def main():
                     if k < K and vals[r * K + k] > 0:
                         x |= 1 << b
                 words.append("0x%08xu" % x)
-        out.append("static const uint32_t qtip_had%d_bits[%d] = {" % (K, len(words)))
+        out.append("QTIP_TABLE uint32_t qtip_had%d_bits[%d] = {" % (K, len(words)))
         for i in range(0, len(words), 8):
             out.append("  " + ",".join(words[i:i + 8]) + ",")
         out.append("};")
@@ -59,7 +65,7 @@ def main():
     body = re.search(r"kTlutF32Bits\[1024\]\s*=\s*\{([^}]*)\}", src).group(1)
     vals = [v.strip() for v in body.split(",") if v.strip()]
     assert len(vals) == 1024
-    out.append("static const uint32_t qtip_hyb_tlut_bits[1024] = {")
+    out.append("QTIP_TABLE uint32_t qtip_hyb_tlut_bits[1024] = {")
     for i in range(0, 1024, 8):
         out.append("  " + ",".join(v + "u" for v in vals[i:i + 8]) + ",")
     out.append("};")
