@@ -5,10 +5,11 @@
 #include <algorithm>
 #include <chrono>
 #include <cmath>
-
 #include <cstdlib>
 #include <cstring>
+#include <exception>
 #include <mutex>
+#include <thread>
 #include <vector>
 
 namespace qtipmi {
@@ -387,6 +388,38 @@ void group_finish(qtip_ctx* c, GroupWork& w, int nlin, const qtip_linear_in* lin
   DBuf<float>&WT = w.WT, &hatWT = w.hatWT, &d_su = w.d_su, &d_sv = w.d_sv;
   DBuf<uint16_t>& Q = w.Q;
   double t0 = now_s();
+  // ---- states -> packed trellis in kernel layout, src/quantizer.cpp:305-320 (packed on the device).  The packing
+  // kernel is small and the copy to the caller's (pageable) memory is the copy engines' and a host thread's work:
+  // where a chain's stream exists (idle now: LDLQ has been waited for) both run there, from a helper thread, beside
+  // the proxy's matrix-core kernels instead of after them.
+  const long nblk = n / 16;
+  DBuf<uint16_t> tr(size_t(mt / 16) * nblk * 32);
+  auto pack_to_host = [&](hipStream_t st) {
+    for (int li = 0; li < nlin; ++li) {
+      const long m = lins[li].m;
+      const size_t tile0 = size_t(off[li] / 16) * nblk;
+      launch_pack_swizzle(Q + tile0 * 128, m, n, tr + tile0 * 32, st);
+      QTIP_HIP(hipMemcpyAsync(outs[li].trellis, tr + tile0 * 32, size_t(m / 16) * nblk * 32 * 2, hipMemcpyDeviceToHost, st));
+    }
+    QTIP_HIP(hipStreamSynchronize(st));
+  };
+  struct Packer {  // joined whatever ends this scope
+    std::thread t;
+    std::exception_ptr err;
+    ~Packer() {
+      if (t.joinable()) t.join();
+    }
+  } packer;
+  const bool pack_beside = !opt.skip_proxy && c->chain_stream[0] != nullptr;
+  if (pack_beside)
+    packer.t = std::thread([&] {
+      try {
+        QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
+        pack_to_host(c->chain_stream[0]);
+      } catch (...) {
+        packer.err = std::current_exception();
+      }
+    });
   // ---- proxy (rotated, scaled domain; Wscale cancels), src/quantizer.cpp:268-303
   if (!opt.skip_proxy) {
     // the rotated Hessian: the caller's device copy if it kept one, else uploaded
@@ -410,17 +443,11 @@ void group_finish(qtip_ctx* c, GroupWork& w, int nlin, const qtip_linear_in* lin
   T.proxy += now_s() - t0;
   t0 = now_s();
 
-  // ---- states -> packed trellis in kernel layout, src/quantizer.cpp:305-320 (packed on the device)
-  {
-    const long nblk = n / 16;
-    DBuf<uint16_t> tr(size_t(mt / 16) * nblk * 32);
-    for (int li = 0; li < nlin; ++li) {
-      const long m = lins[li].m;
-      const size_t tile0 = size_t(off[li] / 16) * nblk;
-      launch_pack_swizzle(Q + tile0 * 128, m, n, tr + tile0 * 32, s);
-      QTIP_HIP(hipMemcpyAsync(outs[li].trellis, tr + tile0 * 32, size_t(m / 16) * nblk * 32 * 2, hipMemcpyDeviceToHost, s));
-    }
-    QTIP_HIP(hipStreamSynchronize(s));
+  if (pack_beside) {
+    packer.t.join();
+    if (packer.err) std::rethrow_exception(packer.err);
+  } else {
+    pack_to_host(s);
   }
   // ---- optional reconstruction in the original domain, src/quantizer.cpp:321-338:
   //      hatW = diag(SV) U_m (hatWr * Wscale) U_n^T diag(SU)
