@@ -24,7 +24,8 @@ def synth(pkg):
     return mod
 
 
-@pytest.mark.parametrize("n", [12, 64, 96, 80, 448, 864, 1024, 2304, 3328, 4096, 8192, 12288, 28672, 49152, 53248, 57344])
+@pytest.mark.parametrize("n", [12, 64, 96, 80, 448, 864, 1024, 2304, 3328, 4096, 8192, 12288, 20480, 28672, 36864, 49152,
+                               53248, 57344])
 def test_hadamard_rows(qz, oracle, n):
     """Bit-identical to the fp32 dataflow of the reference's kernels (restated on the CPU) and within 2e-5 of the
     fp64 definition (tests/test_gpu.cpp:27-50); strided rows keep their padding."""
@@ -44,6 +45,25 @@ def test_hadamard_rows(qz, oracle, n):
         oracle.lib().qo_hadamard_rows(w64, rows, n, ld, tr)
         assert np.max(np.abs(y[:, :n] - w64.reshape(rows, ld)[:, :n])) < 2e-5
         assert np.array_equal(y[:, n:], x[:, n:])
+
+
+@pytest.mark.parametrize("n", [12288, 20480, 28672, 36864])
+def test_hadamard_many_rows(qz, oracle, n):
+    """Rows of K x 1024 values, more of them than workgroups are resident: every workgroup walks several rows with the
+    next one in flight.  Bit-identical to the fp32 dataflow of the reference's kernels; the last rows, which some
+    workgroups no longer have, included."""
+    import torch
+    say("case: hadamard many rows n=%d" % n)
+    rows = 2 * 256 * 2 + 37
+    x = oracle.rng_normal(7 + n, rows * n).astype(np.float32).reshape(rows, n)
+    for tr in (0, 1):
+        d = torch.from_numpy(x).cuda()
+        qz.hadamard_rows_dev(d, rows, n, n, tr)
+        qz.synchronize()
+        y = d.cpu().numpy()
+        w32 = x.copy().reshape(-1)
+        assert oracle.lib().qo_hadamard_rows_f32(w32, rows, n, n, tr) == 0
+        assert np.array_equal(y.view(np.uint32), w32.reshape(rows, n).view(np.uint32)), (n, tr)
 
 
 def test_hadamard_rejects_unsupported(qz, pkg):
