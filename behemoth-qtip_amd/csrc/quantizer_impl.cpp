@@ -410,7 +410,9 @@ void group_finish(qtip_ctx* c, GroupWork& w, int nlin, const qtip_linear_in* lin
       if (t.joinable()) t.join();
     }
   } packer;
-  const bool pack_beside = !opt.skip_proxy && c->chain_stream[0] != nullptr;
+  // (not on a lane: the lanes' own streams already share the hardware queues, and one more stream per lane makes
+  // lanes wait for each other)
+  const bool pack_beside = !opt.skip_proxy && c->chain_stream[0] != nullptr && c->vit_slots_limit == 0;
   if (pack_beside)
     packer.t = std::thread([&] {
       try {
