@@ -74,7 +74,7 @@ void order_streams(hipStream_t first, hipStream_t then) {
 
 namespace {
 // a context on the current device: stream, codebook (cb_from's, or the default one), Hadamard tables
-qtip_ctx* make_context(int device, const HostCodebook* cb_from) {
+qtip_ctx* make_context(int device, const HostCodebook* cb_from, hipStream_t own_stream = nullptr) {
   struct Cleanup {
     qtip_ctx* c;
     ~Cleanup() {
@@ -86,7 +86,8 @@ qtip_ctx* make_context(int device, const HostCodebook* cb_from) {
   } guard{new qtip_ctx()};
   qtip_ctx* c = guard.c;
   c->device = device;
-  QTIP_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+  c->stream = own_stream;  // a stream the caller made for this context (released with it), else one made here
+  if (!c->stream) QTIP_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   c->arena.streams.push_back(&c->stream);
   for (hipStream_t& cs : c->chain_stream) c->arena.streams.push_back(&cs);
   if (cb_from) c->cb = *cb_from;
@@ -214,10 +215,69 @@ void destroy_context(qtip_ctx* ctx) {
 }
 }  // namespace
 
+// A stream for lane k that runs beside the streams of the lanes made before it, found by timing as the side streams
+// of a context are: lanes only share the chip if each has a hardware queue of its own, and which queue a new stream
+// gets is the runtime's choice (with 16 queues asked for, twelve streams made in a row came out with shared queues
+// on some boxes and not on others: 141-151 against 215 Mweights/s for twelve lanes of 1024 x 1024 groups).  The
+// parent's own streams may share a lane's queue: they are idle while lanes run.  Null when no candidate passed (the
+// process has fewer queues than lanes): the search is then given up for the later lanes too.
+hipStream_t lane_stream_beside(qtip_ctx* parent, int k) {
+  constexpr int kCandidates = 24;
+  constexpr double kDelayUs = 500.0;
+  std::vector<hipStream_t> others;
+  for (int j = 0; j < k; ++j)
+    if (parent->lane[j]) others.push_back(parent->lane[j]->stream);
+  if (others.empty() || parent->lane_streams_exhausted) return nullptr;
+  std::vector<hipStream_t> dropped;
+  hipStream_t found = nullptr;
+  try {
+    auto wait_all = [&](hipStream_t cand) {
+      for (hipStream_t o : others) QTIP_HIP(hipStreamSynchronize(o));
+      QTIP_HIP(hipStreamSynchronize(cand));
+    };
+    auto beside = [&](hipStream_t cand) {
+      for (int attempt = 0; attempt < 3; ++attempt) {  // the first launch on a stream also sets its queue up
+        wait_all(cand);
+        const auto t0 = std::chrono::steady_clock::now();
+        for (hipStream_t o : others) launch_delay(kDelayUs, o);
+        launch_delay(kDelayUs, cand);
+        wait_all(cand);
+        if (std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count() < 1.5 * kDelayUs)
+          return true;
+      }
+      return false;
+    };
+    for (int i = 0; i < kCandidates && !found; ++i) {
+      hipStream_t s = nullptr;
+      QTIP_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+      dropped.push_back(s);  // until shown otherwise
+      if (beside(s)) {
+        dropped.pop_back();
+        found = s;
+      }
+    }
+  } catch (...) {
+    if (found) dropped.push_back(found);
+    found = nullptr;
+  }
+  for (hipStream_t s : dropped) {
+    (void)hipStreamSynchronize(s);
+    (void)hipStreamDestroy(s);
+  }
+  if (!found) parent->lane_streams_exhausted = true;
+  return found;
+}
+
 qtip_ctx* lane_context(qtip_ctx* parent, int k) {
   QTIP_REQUIRE(k >= 0 && k < qtip_ctx::kMaxLanes, "lane %d of %d", k, qtip_ctx::kMaxLanes);
   if (!parent->lane[k]) {
-    parent->lane[k] = make_context(parent->device, &parent->cb);
+    hipStream_t own = lane_stream_beside(parent, k);
+    try {
+      parent->lane[k] = make_context(parent->device, &parent->cb, own);
+    } catch (...) {
+      if (own) (void)hipStreamDestroy(own);
+      throw;
+    }
     // one stream per lane, the factorization's work included: a stream only runs beside the others if it has a
     // hardware queue to itself, and a process has few of them (GPU_MAX_HW_QUEUES, 4 unless the environment says
     // more); with a stream more per lane for the factorization 1024 x 1024 groups ran at 59 instead of 134 Mweights/s
@@ -232,6 +292,7 @@ qtip_ctx* lane_context(qtip_ctx* parent, int k) {
 
 void release_lanes(qtip_ctx* parent) {
   parent->arena.children.clear();
+  parent->lane_streams_exhausted = false;
   for (qtip_ctx*& l : parent->lane)
     if (l) {
       destroy_context(l);

@@ -34,6 +34,7 @@ struct qtip_ctx {
   // (streams, workspaces, rings) made on first use, kept here and released with this context
   static constexpr int kMaxLanes = 12;
   qtip_ctx* lane[kMaxLanes] = {};
+  bool lane_streams_exhausted = false;  // a lane found no stream that runs beside the earlier lanes': no search for the later ones
 
   // LDLQ runs its tile rows as up to kMaxChains independent chains of launches, on the context's stream and these,
   // so that one chain's trace-backs and gathers run under the others' forward passes
