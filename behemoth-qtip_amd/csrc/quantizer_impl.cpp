@@ -9,6 +9,7 @@
 #include <cstring>
 #include <exception>
 #include <mutex>
+#include <system_error>
 #include <thread>
 #include <vector>
 
@@ -412,16 +413,21 @@ void group_finish(qtip_ctx* c, GroupWork& w, int nlin, const qtip_linear_in* lin
   } packer;
   // (not on a lane: the lanes' own streams already share the hardware queues, and one more stream per lane makes
   // lanes wait for each other)
-  const bool pack_beside = !opt.skip_proxy && c->chain_stream[0] != nullptr && c->vit_slots_limit == 0;
-  if (pack_beside)
-    packer.t = std::thread([&] {
-      try {
-        QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
-        pack_to_host(c->chain_stream[0]);
-      } catch (...) {
-        packer.err = std::current_exception();
-      }
-    });
+  bool pack_beside = !opt.skip_proxy && c->chain_stream[0] != nullptr && c->vit_slots_limit == 0;
+  if (pack_beside) {
+    try {
+      packer.t = std::thread([&] {
+        try {
+          QTIP_HIP(hipSetDevice(c->device));  // this thread's own current device
+          pack_to_host(c->chain_stream[0]);
+        } catch (...) {
+          packer.err = std::current_exception();
+        }
+      });
+    } catch (const std::system_error&) {
+      pack_beside = false;  // no thread to be had: after the proxy, on this one
+    }
+  }
   // ---- proxy (rotated, scaled domain; Wscale cancels), src/quantizer.cpp:268-303
   if (!opt.skip_proxy) {
     // the rotated Hessian: the caller's device copy if it kept one, else uploaded
